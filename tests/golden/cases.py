@@ -1,0 +1,95 @@
+"""Case table shared by the fixture generator and the tests that read the
+fixtures.  Inputs are regenerated from integer hashes (exactly reproducible),
+so the fixtures hold expected OUTPUTS only."""
+from __future__ import annotations
+
+import numpy as np
+
+from wayruntime_amd import synth
+
+# name, seq_q, nq, nkv, hd, rows (allocated), seq_k (cursor or None = rows),
+# scale_override, window, kv dtype
+ATTN_CASES = [
+    # workload shapes (BASELINE.json configs 2, 3, 5)
+    ("qwen3_ctx128",   1, 16, 8, 128,  128, None, 0.0, 0, "f16"),
+    ("qwen3_ctx512",   1, 16, 8, 128,  512, None, 0.0, 0, "f16"),
+    ("qwen3_ctx2048",  1, 16, 8, 128, 2048, None, 0.0, 0, "f16"),
+    ("qwen3_ctx8192",  1, 16, 8, 128, 8192, None, 0.0, 0, "f16"),
+    ("llama3_ctx4096", 1, 32, 8, 128, 4096, None, 0.0, 0, "f16"),
+    ("llama3_ctx301_cursor", 1, 32, 8, 128, 512, 301, 0.0, 0, "f16"),
+    ("gemma_ctx1000_scale1_win512", 1, 8, 4, 256, 1000, None, 1.0, 512, "f16"),
+    ("gemma_ctx1000_scale1", 1, 8, 4, 256, 1000, None, 1.0, 0, "f16"),
+    # tile-boundary and masking behaviour (flash tile = 64 keys)
+    ("small_ctx1",     1, 4, 2, 32,    1, None, 0.0, 0, "f16"),
+    ("small_ctx63",    1, 4, 2, 32,   63, None, 0.0, 0, "f16"),
+    ("small_ctx64",    1, 4, 2, 32,   64, None, 0.0, 0, "f16"),
+    ("small_ctx65",    1, 4, 2, 32,   65, None, 0.0, 0, "f16"),
+    ("small_ctx200_win16",  1, 4, 2, 32, 200, None, 0.0, 16, "f16"),
+    ("small_ctx200_win64",  1, 4, 2, 32, 200, None, 0.0, 64, "f16"),
+    ("small_ctx200_win72",  1, 4, 2, 32, 200, None, 0.0, 72, "f16"),
+    ("small_ctx200_win999", 1, 4, 2, 32, 200, None, 0.0, 999, "f16"),
+    ("small_ctx200_scale025", 1, 4, 2, 32, 200, None, 0.25, 0, "f16"),
+    ("small_cursor150_of_200", 1, 4, 2, 32, 200, 150, 0.0, 0, "f16"),
+    ("mha_hd64_ctx130", 1, 4, 4, 64, 130, None, 0.0, 0, "f16"),
+    ("g8_hd64_ctx257",  1, 8, 1, 64, 257, None, 0.0, 0, "f16"),
+    # seq_q > 1 is NON-causal in the reference op
+    ("seqq3_ctx100",   3, 4, 2, 32,  100, None, 0.0, 0, "f16"),
+    # F32 K/V, the dtype the reference's own self-tests use
+    ("f32kv_ctx96",    2, 2, 1, 16,   96, None, 0.0, 0, "f32"),
+]
+
+
+def attn_inputs(case):
+    """(q float32 [seq_q,nq,hd], k, v [rows,nkv,hd] uint16 or float32)."""
+    name, seq_q, nq, nkv, hd, rows, _seq_k, _sc, _win, kvdt = case
+    base = (sum(ord(c) * (i + 1) for i, c in enumerate(name)) * 2654435761) & 0xFFFFFFFF
+    q = synth.hash_bell(base + 1, (seq_q, nq, hd))
+    k = synth.hash_bell(base + 2, (rows, nkv, hd))
+    v = synth.hash_bell(base + 3, (rows, nkv, hd))
+    if kvdt == "f16":
+        k = synth.f32_to_f16_trunc(k)
+        v = synth.f32_to_f16_trunc(v)
+    return q, k, v
+
+
+# name, seq, heads, hd, pos, theta, n_rot_pairs
+ROPE_CASES = [
+    ("qwen3_q_pos0",    4, 16, 128,    0, 1e6, 0),
+    ("qwen3_k_pos1000", 3,  8, 128, 1000, 1e6, 0),
+    ("llama3_pos4090",  8,  8, 128, 4090, 5e5, 0),
+    ("gemma_partial",   2,  4, 256,   77, 1e6, 32),
+    ("theta_default",   2,  2,   8,    5, 0.0, 0),
+]
+
+
+def rope_input(case):
+    name, seq, heads, hd, _pos, _theta, _nrot = case
+    base = (sum(ord(c) * (i + 3) for i, c in enumerate(name)) * 40503) & 0xFFFFFFFF
+    return synth.hash_bell(base, (seq, heads, hd))
+
+
+def math_grid(fn: str) -> np.ndarray:
+    """Exactly reproducible float32 argument grids for the scalar math pins."""
+    i = np.arange(8192, dtype=np.float32)
+    if fn == "exp":       # covers both clamps and every k in [-127, 127]
+        return (i - np.float32(4096.0)) * np.float32(0.0224)
+    if fn == "log":
+        return (i + np.float32(1.0)) * np.float32(137.53)
+    if fn == "sqrt":
+        return i * i * np.float32(0.0371) + np.float32(1e-6)
+    if fn in ("sin", "cos"):
+        return (i - np.float32(4096.0)) * np.float32(0.0119)
+    raise KeyError(fn)
+
+
+def f16_encode_bits() -> np.ndarray:
+    """uint32 float bit patterns for the truncating-encode pin: hashed
+    patterns over the whole float32 space plus the edges around the binary16
+    normal range."""
+    h = synth._hash32(0xF16F16, 16384)
+    edges = np.array([0x00000000, 0x80000000, 0x3F800000, 0x3F801800, 0x3F801FFF,
+                      0x387FFFFF, 0x38800000, 0x38800001, 0x33800000, 0x477FE000,
+                      0x477FFFFF, 0x47800000, 0x7F800000, 0xFF800000, 0x7FC00000,
+                      0x7F800001, 0x00000001, 0x007FFFFF, 0xC0000000, 0x3F7FFFFF],
+                     dtype=np.uint32)
+    return np.concatenate([edges, h])

@@ -1,0 +1,80 @@
+#!/usr/bin/env python3
+"""Writes the fixtures in this directory from the COMPILED REFERENCE
+(``oracle/_ref/libwayref.so``, built by ``make -C oracle ref`` from the
+reference's own sources).  Run from the repository root where the reference
+tree is available:
+
+    python tests/golden/make_golden.py
+
+Inputs come from tests/golden/cases.py (integer-hash fills, regenerated
+bit-for-bit by the tests), so the files hold expected outputs only:
+
+    attn_golden.npz   one float32 array per attention case
+    rope_golden.npz   one float32 array per RoPE case
+    mathx_golden.npz  exp/log/sqrt/sin/cos on fixed grids
+    f16_golden.npz    truncating encode of fixed float32 bit patterns,
+                      decode of all 65536 binary16 patterns (as uint32 bits)
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import sys
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+sys.path.insert(0, ROOT)
+
+import oracle  # noqa: E402
+from tests.golden import cases  # noqa: E402
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def main() -> None:
+    oracle.build(ref=True)
+    if not oracle.have_ref():
+        raise SystemExit("reference build not available; cannot write fixtures")
+    ref = oracle.ref()
+
+    attn = {}
+    for case in cases.ATTN_CASES:
+        name, _sq, _nq, _nkv, _hd, _rows, seq_k, sc, win, _dt = case
+        q, k, v = cases.attn_inputs(case)
+        rc, out = oracle.ref_attention(q, k, v, seq_k=seq_k, scale_override=sc, window=win)
+        assert rc == 0, (name, rc)
+        attn[name] = out
+    np.savez(os.path.join(HERE, "attn_golden.npz"), **attn)
+
+    rope = {}
+    for case in cases.ROPE_CASES:
+        name, _seq, _heads, _hd, pos, theta, nrot = case
+        x = cases.rope_input(case)
+        y = np.empty_like(x)
+        tx, ty = oracle.wrap(x), oracle.wrap(y)
+        rc = ref.wri_op_rope(C.byref(tx), C.byref(ty), pos, theta, nrot)
+        assert rc == 0, (name, rc)
+        rope[name] = y
+    np.savez(os.path.join(HERE, "rope_golden.npz"), **rope)
+
+    mathx = {}
+    for fn in ("exp", "log", "sqrt", "sin", "cos"):
+        f = getattr(ref, "wri_" + fn)
+        mathx[fn] = np.array([f(float(x)) for x in cases.math_grid(fn)], dtype=np.float32)
+    np.savez_compressed(os.path.join(HERE, "mathx_golden.npz"), **mathx)
+
+    bits = cases.f16_encode_bits()
+    # exact bit patterns (NaN payloads included) go in as raw 4-byte buffers
+    enc = np.array([ref.wri_f32_to_f16(C.c_float.from_buffer_copy(int(b).to_bytes(4, "little")))
+                    for b in bits], dtype=np.uint16)
+    dec = np.array([ref.wri_f16_to_f32(h) for h in range(65536)], dtype=np.float32).view(np.uint32)
+    np.savez_compressed(os.path.join(HERE, "f16_golden.npz"), encode=enc, decode_bits=dec)
+
+    for f in sorted(os.listdir(HERE)):
+        if f.endswith(".npz"):
+            print(f, os.path.getsize(os.path.join(HERE, f)), "bytes")
+
+
+if __name__ == "__main__":
+    main()

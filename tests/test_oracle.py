@@ -1,0 +1,384 @@
+"""Pins the CPU oracle: against the fixtures written from the compiled
+reference, against the reference's own self-test vectors (re-derived here from
+the closed forms in its source), against mathematics, and — where the
+reference build is present — against the reference itself by memcmp."""
+import ctypes as C
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from tests.golden import cases
+from wayruntime_amd import synth
+
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+
+
+def _npz(name):
+    return np.load(os.path.join(GOLD, name))
+
+
+def _oracle_case(case):
+    name, seq_q, nq, nkv, hd, rows, seq_k, sc, win, kvdt = case
+    q, k, v = cases.attn_inputs(case)
+    out = np.empty_like(q)
+    flags = oracle.GROWABLE if seq_k is not None else 0
+    tq = oracle.wrap(q)
+    tk = oracle.wrap(k, flags=flags, valid_rows=seq_k or 0)
+    tv = oracle.wrap(v, flags=flags, valid_rows=seq_k or 0)
+    tc = oracle.wrap(out)
+    rc = oracle.lib().wro_op_gqa_attention(C.byref(tq), C.byref(tk), C.byref(tv), C.byref(tc),
+                                           sc, win, None)
+    return rc, out
+
+
+# ------------------------------------------------------------- fixtures ----
+
+@pytest.fixture(scope="module", autouse=True)
+def _cap():
+    oracle.set_attn_max_seq(32768)
+    yield
+    oracle.set_attn_max_seq(4096)
+
+
+@pytest.mark.parametrize("case", cases.ATTN_CASES, ids=[c[0] for c in cases.ATTN_CASES])
+def test_attention_bit_exact_vs_reference_fixture(case):
+    gold = _npz("attn_golden.npz")[case[0]]
+    rc, out = _oracle_case(case)
+    assert rc == 0
+    assert out.tobytes() == gold.tobytes()
+
+
+@pytest.mark.parametrize("case", cases.ROPE_CASES, ids=[c[0] for c in cases.ROPE_CASES])
+def test_rope_bit_exact_vs_reference_fixture(case):
+    name, _seq, _heads, _hd, pos, theta, nrot = case
+    gold = _npz("rope_golden.npz")[name]
+    out = oracle.rope(cases.rope_input(case), pos, theta, nrot)
+    assert out.tobytes() == gold.tobytes()
+
+
+@pytest.mark.parametrize("fn", ["exp", "log", "sqrt", "sin", "cos"])
+def test_scalar_math_bit_exact_vs_reference_fixture(fn):
+    gold = _npz("mathx_golden.npz")[fn]
+    f = getattr(oracle.lib(), "wro_" + fn)
+    got = np.array([f(float(x)) for x in cases.math_grid(fn)], dtype=np.float32)
+    assert got.tobytes() == gold.tobytes()
+
+
+def test_scalar_math_close_to_libm():
+    # closed forms: the polynomials are ~1e-6 (exp, sqrt, log) / ~1e-4 (sin, cos
+    # near +-pi) approximations of the textbook functions
+    x = cases.math_grid("exp")
+    x = x[(x > -80) & (x < 80)]
+    got = np.array([oracle.lib().wro_exp(float(v)) for v in x], dtype=np.float64)
+    assert np.max(np.abs(got / np.exp(x.astype(np.float64)) - 1)) < 2e-5
+    x = cases.math_grid("sqrt")
+    got = np.array([oracle.lib().wro_sqrt(float(v)) for v in x], dtype=np.float64)
+    assert np.max(np.abs(got / np.sqrt(x.astype(np.float64)) - 1)) < 1e-6
+    x = cases.math_grid("sin")
+    gs = np.array([oracle.lib().wro_sin(float(v)) for v in x], dtype=np.float64)
+    gc = np.array([oracle.lib().wro_cos(float(v)) for v in x], dtype=np.float64)
+    assert np.max(np.abs(gs - np.sin(x.astype(np.float64)))) < 0.1    # 7th-order Taylor at +-pi: pi^9/9!
+    assert np.max(np.abs(gc - np.cos(x.astype(np.float64)))) < 0.25   # pi^8/8!
+    inner = np.abs(((x + np.pi) % (2 * np.pi)) - np.pi) < 1.5
+    assert np.max(np.abs(gs - np.sin(x.astype(np.float64)))[inner]) < 3e-4
+    assert oracle.lib().wro_exp(-88.5) == 0.0 and oracle.lib().wro_exp(88.5) == np.float32(1e38)
+
+
+def test_f16_codecs_vs_fixture_and_ieee():
+    g = _npz("f16_golden.npz")
+    bits = cases.f16_encode_bits()
+    lib = oracle.lib()
+    enc = np.array([lib.wro_f32_to_f16(C.c_float.from_buffer_copy(int(b).to_bytes(4, "little")))
+                    for b in bits], dtype=np.uint16)
+    assert np.array_equal(enc, g["encode"])
+    dec = np.array([lib.wro_f16_to_f32(h) for h in range(65536)], dtype=np.float32)
+    assert np.array_equal(dec.view(np.uint32), g["decode_bits"])
+    # IEEE: decode equals numpy's exact binary16 -> binary32 widening (NaN payloads aside)
+    ieee = np.arange(65536, dtype=np.uint16).view(np.float16).astype(np.float32)
+    finite = np.isfinite(ieee)
+    assert np.array_equal(dec[finite].view(np.uint32), ieee[finite].view(np.uint32))
+    # vectorised helper used to fill caches == scalar codec
+    assert np.array_equal(synth.f32_to_f16_trunc(bits.view(np.float32)), g["encode"])
+
+
+def test_f16_reference_unit_test_known_answers():
+    # test/unit_tests.c:100-107
+    lib = oracle.lib()
+    assert lib.wro_f32_to_f16(1.0) == 0x3C00
+    assert lib.wro_f32_to_f16(1.000732421875) == 0x3C00      # round-to-nearest would give 0x3C01
+    assert lib.wro_f16_to_f32(0x3C00) == 1.0
+    assert lib.wro_f16_to_f32(0xC000) == -2.0
+
+
+def test_f16_truncation_is_round_toward_zero_and_idempotent():
+    lib = oracle.lib()
+    allh = np.arange(65536, dtype=np.uint16)
+    dec = allh.view(np.float16).astype(np.float32)
+    back = synth.f32_to_f16_trunc(dec)
+    e = (allh >> 10) & 0x1F
+    normal = (e > 0) & (e < 31)
+    assert np.array_equal(back[normal], allh[normal])              # exact values survive
+    sub = (e == 0)
+    assert np.array_equal(back[sub], allh[sub] & 0x8000)           # subnormals flush to +-0
+    nan = (e == 31) & ((allh & 0x3FF) != 0)
+    assert np.array_equal(back[nan], (allh[nan] & 0x8000) | 0x7C00)  # NaN collapses to inf
+    # magnitude never grows, and is within one half-ulp step of the input
+    x = synth.normal(7, (20000,), std=3.0)
+    t = synth.f32_to_f16_trunc(x).view(np.float16).astype(np.float32)
+    big = np.abs(x) >= 2.0 ** -14
+    assert np.all(np.abs(t[big]) <= np.abs(x[big]))
+    assert np.all(np.abs(x[big]) - np.abs(t[big]) < np.abs(x[big]) * 2.0 ** -10)
+    assert lib.wro_f32_to_f16(1e-8) == 0 and lib.wro_f32_to_f16(-1e-8) == 0x8000
+    assert lib.wro_f32_to_f16(1e9) == 0x7C00 and lib.wro_f32_to_f16(-1e9) == 0xFC00
+
+
+# ---------------------------------------- the reference's own self-tests ----
+
+def _materialised_f64(q, k, v, scale, key_lo=0):
+    """Textbook softmax attention in float64, one KV head."""
+    s = (q.astype(np.float64) @ k.astype(np.float64).T) * scale
+    s[:, :key_lo] = -np.inf
+    s -= s.max(axis=1, keepdims=True)
+    p = np.exp(s)
+    p /= p.sum(axis=1, keepdims=True)
+    return p @ v.astype(np.float64)
+
+
+def test_reference_flash_attn_fixture_small():
+    # src/core/kernels.c:1909-1974: SQ=2, SK=8, D=4, literal Q, closed-form K/V,
+    # default scale / scale override 0.25 / sliding window 4; tolerance 1e-4
+    q = np.array([[0.1, 0.2, 0.3, 0.4], [0.5, 0.6, 0.7, 0.8]], dtype=np.float32).reshape(2, 1, 4)
+    i = np.arange(32)
+    k = (((i * 7 + 3) % 13).astype(np.float32) * np.float32(0.1)).reshape(8, 1, 4)
+    v = (((i * 5 + 1) % 11).astype(np.float32) * np.float32(0.1)).reshape(8, 1, 4)
+    for sc, win in ((0.0, 0), (0.25, 0), (0.0, 4)):
+        out = np.empty_like(q)
+        tq, tk, tv, tc = oracle.wrap(q), oracle.wrap(k), oracle.wrap(v), oracle.wrap(out)
+        rc = oracle.lib().wro_op_gqa_attention(C.byref(tq), C.byref(tk), C.byref(tv),
+                                               C.byref(tc), sc, win, None)
+        assert rc == 0
+        scale = sc if sc > 0 else 0.5
+        want = _materialised_f64(q[:, 0], k[:, 0], v[:, 0], scale, key_lo=(8 - win) if win else 0)
+        assert np.max(np.abs(out[:, 0] - want)) < 1e-4
+
+
+def test_reference_flash_attn_fixture_long_growable():
+    # src/core/kernels.c:1979-2036: LQ=2, LD=8, GROWABLE F32 K/V with
+    # valid_rows in {64,256,1024,4096}, integer-hash fills
+    LQ, LD, SK_MAX = 2, 8, 4096
+    qi = np.arange(LQ * LD)
+    q = (((qi * 11 + 3) % 17).astype(np.float32) * np.float32(0.05)).reshape(LQ, 1, LD)
+    with np.errstate(over="ignore"):
+        s = np.arange(SK_MAX * LD, dtype=np.uint32) * np.uint32(2654435761) + np.uint32(0x9E3779B9)
+    k = (((s & 0xFFFF).astype(np.int32).astype(np.float32) / np.float32(32768.0) - np.float32(1.0))
+         * np.float32(0.3)).reshape(SK_MAX, 1, LD)
+    v = ((((s >> 16) & 0xFFFF).astype(np.int32).astype(np.float32) / np.float32(32768.0)
+          - np.float32(1.0)) * np.float32(0.3)).reshape(SK_MAX, 1, LD)
+    for sk in (64, 256, 1024, 4096):
+        out = np.empty_like(q)
+        tq, tc = oracle.wrap(q), oracle.wrap(out)
+        tk = oracle.wrap(k, flags=oracle.GROWABLE, valid_rows=sk)
+        tv = oracle.wrap(v, flags=oracle.GROWABLE, valid_rows=sk)
+        rc = oracle.lib().wro_op_gqa_attention(C.byref(tq), C.byref(tk), C.byref(tv),
+                                               C.byref(tc), 0.0, 0, None)
+        assert rc == 0
+        want = _materialised_f64(q[:, 0], k[:sk, 0], v[:sk, 0], 1.0 / np.sqrt(LD))
+        assert np.max(np.abs(out[:, 0] - want)) < 1e-4
+
+
+def test_reference_ops_test_gqa_head_map():
+    # src/core/kernels.c:2185-2208: one key => each output row is the V row of kv head qh // group
+    q = np.ones((1, 4, 2), dtype=np.float32)
+    k = np.ones((1, 2, 2), dtype=np.float32)
+    v = np.array([10, 20, 30, 40], dtype=np.float32).reshape(1, 2, 2)
+    out = np.empty_like(q)
+    tq, tk, tv, tc = oracle.wrap(q), oracle.wrap(k), oracle.wrap(v), oracle.wrap(out)
+    assert oracle.lib().wro_op_gqa_attention(C.byref(tq), C.byref(tk), C.byref(tv),
+                                             C.byref(tc), 0.0, 0, None) == 0
+    assert np.array_equal(out.reshape(-1), [10, 20, 10, 20, 30, 40, 30, 40])
+
+
+def test_error_contract_and_counter():
+    # src/core/kernels.c:1418-1454, 2039-2059
+    lib = oracle.lib()
+    oracle.set_attn_max_seq(4096)
+    try:
+        ctr = C.c_uint64(0)
+        q = np.ones((1, 1, 1), dtype=np.float32)
+        kv = np.zeros((4097, 1, 1), dtype=np.float32)
+        out = np.empty_like(q)
+        tq, tk, tv, tc = oracle.wrap(q), oracle.wrap(kv), oracle.wrap(kv), oracle.wrap(out)
+        call = lambda a, b, c, d, s=0.0, w=0: lib.wro_op_gqa_attention(  # noqa: E731
+            C.byref(a), C.byref(b), C.byref(c), C.byref(d), s, w, C.byref(ctr))
+        assert call(tq, tk, tv, tc) == oracle.WRO_ERR_LIMIT            # over the cap: refused
+        assert ctr.value == 1                                          # counted before shape checks
+        # GROWABLE cursor inside the cap is fine
+        tk2 = oracle.wrap(kv, flags=oracle.GROWABLE, valid_rows=4096)
+        tv2 = oracle.wrap(kv, flags=oracle.GROWABLE, valid_rows=4096)
+        assert call(tq, tk2, tv2, tc) == 0
+        # nq % nkv != 0
+        q3 = np.ones((1, 3, 2), dtype=np.float32)
+        k2 = np.ones((4, 2, 2), dtype=np.float32)
+        o3 = np.empty_like(q3)
+        assert call(oracle.wrap(q3), oracle.wrap(k2), oracle.wrap(k2), oracle.wrap(o3)) == oracle.WRO_ERR_INVAL
+        # head_dim mismatch between Q and K
+        q4 = np.ones((1, 2, 4), dtype=np.float32)
+        o4 = np.empty_like(q4)
+        assert call(oracle.wrap(q4), oracle.wrap(k2), oracle.wrap(k2), oracle.wrap(o4)) == oracle.WRO_ERR_INVAL
+        # ndim < 3 is refused BEFORE the counter bump
+        before = ctr.value
+        q2d = oracle.wrap(np.ones((2, 2), dtype=np.float32))
+        assert call(q2d, oracle.wrap(k2), oracle.wrap(k2), oracle.wrap(o4)) == oracle.WRO_ERR_INVAL
+        assert ctr.value == before
+        # NULL data
+        tn = oracle.wrap(np.ones((1, 2, 2), dtype=np.float32))
+        tn.data = None
+        assert call(tn, oracle.wrap(k2), oracle.wrap(k2), oracle.wrap(o4)) == oracle.WRO_ERR_INVAL
+        # output too small
+        small = oracle.wrap(np.empty((1, 1, 2), dtype=np.float32))
+        q22 = oracle.wrap(np.ones((1, 2, 2), dtype=np.float32))
+        assert call(q22, oracle.wrap(k2), oracle.wrap(k2), small) == oracle.WRO_ERR_INVAL
+        # head_dim over the flash cap
+        qb = np.ones((1, 1, 1025), dtype=np.float32)
+        kb = np.ones((1, 1, 1025), dtype=np.float32)
+        ob = np.empty_like(qb)
+        assert call(oracle.wrap(qb), oracle.wrap(kb), oracle.wrap(kb), oracle.wrap(ob)) == oracle.WRO_ERR_LIMIT
+    finally:
+        oracle.set_attn_max_seq(32768)
+
+
+def test_growable_zero_cursor_falls_back_to_allocated_rows():
+    # src/core/kernels.c:1437-1438
+    q = synth.hash_bell(1, (1, 2, 8))
+    k = synth.f32_to_f16_trunc(synth.hash_bell(2, (10, 1, 8)))
+    v = synth.f32_to_f16_trunc(synth.hash_bell(3, (10, 1, 8)))
+    out = np.empty_like(q)
+    tk = oracle.wrap(k, flags=oracle.GROWABLE, valid_rows=0)
+    tv = oracle.wrap(v, flags=oracle.GROWABLE, valid_rows=0)
+    tq, tc = oracle.wrap(q), oracle.wrap(out)
+    assert oracle.lib().wro_op_gqa_attention(C.byref(tq), C.byref(tk), C.byref(tv), C.byref(tc),
+                                             0.0, 0, None) == 0
+    assert np.array_equal(out, oracle.attention(q, k, v, seq_k=10))
+
+
+# ----------------------------------------------------------- mathematics ----
+
+def _f64_gqa(q, k16, v16, seq_k, scale, key_lo=0):
+    k = k16[:seq_k].view(np.float16).astype(np.float64)
+    v = v16[:seq_k].view(np.float16).astype(np.float64)
+    nq, nkv = q.shape[1], k.shape[1]
+    g = nq // nkv
+    out = np.empty(q.shape, dtype=np.float64)
+    for h in range(nq):
+        out[:, h] = _materialised_f64(q[:, h], k[:, h // g], v[:, h // g], scale, key_lo)
+    return out
+
+
+@pytest.mark.parametrize("nq,nkv,hd,ctx", [(16, 8, 128, 777), (32, 8, 128, 1300), (8, 4, 256, 515)])
+def test_attention_matches_float64_softmax(nq, nkv, hd, ctx):
+    q = synth.normal(11, (1, nq, hd))
+    k = synth.f32_to_f16_trunc(synth.normal(12, (ctx, nkv, hd)))
+    v = synth.f32_to_f16_trunc(synth.normal(13, (ctx, nkv, hd)))
+    got = oracle.attention(q, k, v)
+    want = _f64_gqa(q, k, v, ctx, 1.0 / np.sqrt(hd))
+    assert np.max(np.abs(got - want)) < 2e-5
+    # sliding window == float64 softmax over the last `window` keys only
+    got_w = oracle.attention(q, k, v, window=200)
+    want_w = _f64_gqa(q, k, v, ctx, 1.0 / np.sqrt(hd), key_lo=ctx - 200)
+    assert np.max(np.abs(got_w - want_w)) < 2e-5
+    # window >= seq_k is the same as no window, bit for bit
+    assert np.array_equal(oracle.attention(q, k, v, window=ctx), got)
+    assert np.array_equal(oracle.attention(q, k, v, window=ctx + 5), got)
+
+
+def test_attention_invariants():
+    nq, nkv, hd = 4, 2, 32
+    q = synth.normal(21, (1, nq, hd))
+    k = synth.f32_to_f16_trunc(synth.normal(22, (50, nkv, hd)))
+    v = synth.f32_to_f16_trunc(synth.normal(23, (50, nkv, hd)))
+    # one key: output is that V row
+    one = oracle.attention(q, k, v, seq_k=1)
+    vrow = v[0].view(np.float16).astype(np.float32)
+    assert np.allclose(one[0], np.repeat(vrow, nq // nkv, axis=0), rtol=0, atol=1e-6)
+    # identical keys: uniform weights, output is the mean of V
+    ku = np.broadcast_to(k[:1], k.shape).copy()
+    mean = v.view(np.float16).astype(np.float64).mean(axis=0)
+    uni = oracle.attention(q, ku, v)
+    assert np.allclose(uni[0], np.repeat(mean, nq // nkv, axis=0), atol=1e-5)
+    # rows past the cursor are never read
+    k2, v2 = k.copy(), v.copy()
+    k2[30:] = 0x7E00  # NaN
+    v2[30:] = 0x7E00
+    assert np.array_equal(oracle.attention(q, k2, v2, seq_k=30), oracle.attention(q, k, v, seq_k=30))
+
+
+def test_causal_prefill_definition_and_batched_loop():
+    nq, nkv, hd, p0, T = 4, 2, 32, 5, 70
+    q = synth.normal(31, (T, nq, hd))
+    k = synth.f32_to_f16_trunc(synth.normal(32, (p0 + T, nkv, hd)))
+    v = synth.f32_to_f16_trunc(synth.normal(33, (p0 + T, nkv, hd)))
+    pre = oracle.causal_prefill(q, k, v, p0=p0)
+    for i in (0, 1, 58, 59, 69):
+        assert np.array_equal(pre[i:i + 1], oracle.attention(q[i:i + 1], k, v, seq_k=p0 + i + 1))
+    # the last row sees everything: equals the non-causal op on that row
+    assert np.array_equal(pre[-1:], oracle.attention(q[-1:], k, v))
+    # threaded and sampled evaluation agree with the serial loop
+    assert np.array_equal(oracle.causal_prefill(q, k, v, p0=p0, threads=3), pre)
+    samp = oracle.causal_prefill(q, k, v, p0=p0, rows=[3, 40])
+    assert np.array_equal(samp[[3, 40]], pre[[3, 40]]) and np.isnan(samp[0]).all()
+
+
+def test_kv_append_row_cursor_and_bits():
+    nkv, hd, cap = 2, 8, 3
+    store = np.zeros((cap, nkv, hd), dtype=np.uint16)
+    t = oracle.wrap(store, flags=oracle.GROWABLE)
+    lib = oracle.lib()
+    rows = synth.normal(41, (cap + 1, nkv * hd), std=2.0)
+    for i in range(cap):
+        assert lib.wro_kv_append_row(C.byref(t), rows[i], nkv, hd) == 0
+        assert t.valid_rows == i + 1
+    assert np.array_equal(store.reshape(cap, -1), synth.f32_to_f16_trunc(rows[:cap]))
+    before = store.copy()
+    assert lib.wro_kv_append_row(C.byref(t), rows[cap], nkv, hd) == oracle.WRO_ERR_CTX_FULL
+    assert t.valid_rows == cap and np.array_equal(store, before)          # consumed nothing
+    assert lib.wro_tensor_set_valid_rows(C.byref(t), 1) == 0 and t.valid_rows == 1   # rollback
+    assert lib.wro_tensor_set_valid_rows(C.byref(t), cap + 1) == oracle.WRO_ERR_INVAL
+    fixed = oracle.wrap(store)
+    assert lib.wro_tensor_set_valid_rows(C.byref(fixed), 1) == oracle.WRO_ERR_INVAL
+
+
+def test_rope_known_answers():
+    # src/core/kernels.c:2160-2183
+    x = np.arange(1, 9, dtype=np.float32).reshape(2, 1, 4)
+    y = oracle.rope(x, 0, 10000.0, 0)
+    assert abs(y[0, 0, 0] - 1.0) < 0.01 and abs(y[0, 0, 2] - 3.0) < 0.01
+    assert abs(y[1, 0, 0] - (5 * 0.5403 - 7 * 0.8415)) < 0.05
+    y2 = oracle.rope(x, 0, 10000.0, 1)
+    assert y2[1, 0, 1] == 6.0 and y2[1, 0, 3] == 8.0
+    # position 0 is the identity, exactly (cos 0 = 1, sin 0 = 0 in the polynomials)
+    z = synth.normal(5, (1, 2, 64))
+    assert np.array_equal(oracle.rope(z, 0, 1e6, 0), z)
+    # small angles: pair norms are preserved to polynomial accuracy (the
+    # truncated series drift near +-pi, so only the slow pairs are checked)
+    r = oracle.rope(z, 3, 1e6, 0)
+    n0 = z[..., 16:32] ** 2 + z[..., 48:] ** 2
+    n1 = r[..., 16:32] ** 2 + r[..., 48:] ** 2
+    assert np.allclose(n0, n1, rtol=1e-4, atol=1e-6)
+
+
+# ------------------------------------------ live memcmp vs the reference ----
+
+@pytest.mark.skipif(not oracle.have_ref(), reason="compiled reference not built here")
+@pytest.mark.parametrize("nq,nkv,hd,ctx,sc,win", [
+    (16, 8, 128, 333, 0.0, 0), (32, 8, 128, 1111, 0.0, 0), (8, 4, 256, 700, 1.0, 256),
+    (4, 1, 64, 65, 0.3, 3), (2, 2, 16, 5000, 0.0, 1000)])
+def test_oracle_equals_compiled_reference_on_normal_inputs(nq, nkv, hd, ctx, sc, win):
+    q = synth.normal(51, (1, nq, hd))
+    k = synth.f32_to_f16_trunc(synth.normal(52, (ctx, nkv, hd)))
+    v = synth.f32_to_f16_trunc(synth.normal(53, (ctx, nkv, hd)))
+    rc, want = oracle.ref_attention(q, k, v, scale_override=sc, window=win)
+    assert rc == 0
+    got = oracle.attention(q, k, v, scale_override=sc, window=win)
+    assert got.tobytes() == want.tobytes()
