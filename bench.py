@@ -1,0 +1,210 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention path on one MI355X.
+
+Headline workload (the configuration the metric is quoted on): batched decode
+attention, Llama-3-8B head shape (32 query / 8 KV heads, head_dim 128),
+16 sessions, every session at 4096 cached positions, F16 cache resident in HBM,
+F32 queries resident in HBM.  One "step" is one batched attention launch over
+one layer of all 16 caches; successive steps walk through `--layers` distinct
+layers so the working set (268 MB per layer) cannot sit in the last-level
+cache.
+
+Prints ONE JSON line.  `value` is algorithmic K/V bytes per step divided by
+wall time per step (whole step: split-K kernel + combine).  `roofline` is for
+the split-K kernel alone, timed with per-launch events.  `cpu_baseline` is the
+CPU oracle (a bit-exact restatement of the reference op) on the same data, one
+core, on a bounded sample.  `prefill` reports causal prefill attention.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0           # MI355X HBM3E
+MFMA_F16_PEAK_TFLOPS = 2500.0   # MI355X dense f16
+
+
+def pooled16(pool16: np.ndarray, salt: int, n: int) -> np.ndarray:
+    """n F16 bit patterns drawn from a pool of truncated N(0,1) samples at a
+    salted offset, sign-flipped for odd salts: distinct per (session, layer),
+    still N(0,1), and cheap to make."""
+    off = (salt * 2654435761) % (pool16.size - n)
+    x = pool16[off:off + n].copy()
+    if salt & 1:
+        x ^= np.uint16(0x8000)
+    return x
+
+
+def main() -> None:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--layers", type=int, default=8,
+                    help="distinct cache layers walked by successive steps")
+    ap.add_argument("--sessions", type=int, default=16)
+    ap.add_argument("--ctx", type=int, default=4096)
+    ap.add_argument("--cpu-seconds", type=float, default=12.0,
+                    help="budget for the CPU baseline sample (0 disables it)")
+    ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--keys-per-wg", type=int, default=0)
+    args = ap.parse_args()
+
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU; --gpus %d is not supported "
+              "(nothing here uses a second device)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    from wayruntime_amd import hipattn, synth
+
+    hipattn.init(0)
+    nq, nkv, hd = 32, 8, 128
+    S, ctx, L = args.sessions, args.ctx, args.layers
+    row = nkv * hd
+
+    t0 = time.time()
+    pool16 = synth.f32_to_f16_trunc(synth.normal(synth.config_seed(3, 0), (1 << 24,)))
+    caches = []
+    host_kv = {}                                    # (session) -> (k16, v16) of layer 0, for checks
+    for s in range(S):
+        kv = hipattn.KVCache(L, hd, nkv, ctx)
+        for layer in range(L):
+            k16 = pooled16(pool16, 1 + 2 * (s * L + layer), ctx * row)
+            v16 = pooled16(pool16, 2 + 2 * (s * L + layer), ctx * row)
+            k16 = k16.reshape(ctx, nkv, hd)
+            v16 = v16.reshape(ctx, nkv, hd)
+            kv.write_f16(layer, 0, k16, v16)
+            if layer == 0:
+                host_kv[s] = (k16, v16)
+        caches.append(kv)
+    q_host = synth.normal(synth.config_seed(3, 1), (L, S, nq, hd))
+    q_dev = hipattn.DeviceBuffer.from_host(q_host)
+    out_dev = hipattn.DeviceBuffer(S * nq * hd * 4)
+    seq_k = [ctx] * S
+    step_q_bytes = S * nq * hd * 4
+    setup_s = time.time() - t0
+
+    if args.keys_per_wg:
+        hipattn.set_tuning(args.keys_per_wg, False)
+
+    class _Off:                                     # device pointer at an offset
+        def __init__(self, p):
+            self.p = p
+
+    def step(i: int) -> None:
+        layer = i % L
+        hipattn.decode_batched_dev(caches, layer, seq_k, _Off(q_dev.p + layer * step_q_bytes),
+                                   out_dev, nq)
+
+    # ---- correctness of what is being timed: session 0, layer 0 vs the oracle
+    import oracle
+    oracle.set_attn_max_seq(1 << 20)
+    step(0)
+    hipattn.sync()
+    got = out_dev.to_host((S, nq, hd))
+    want0 = oracle.attention(q_host[0, 0][None], host_kv[0][0], host_kv[0][1])[0]
+    max_abs = float(np.max(np.abs(got[0] - want0)))
+    rel_l2 = float(np.linalg.norm(got[0] - want0) / np.linalg.norm(want0))
+    if not (max_abs <= 2e-3 and rel_l2 <= 1e-3):
+        print("bench.py: device output outside tolerance: max_abs=%g rel_l2=%g" % (max_abs, rel_l2),
+              file=sys.stderr)
+        sys.exit(1)
+
+    # ---- timed region
+    for i in range(args.warmup):
+        step(i)
+    hipattn.sync()
+    t = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    hipattn.sync()
+    wall = time.perf_counter() - t
+    ms_per_step = wall * 1e3 / args.steps
+    bytes_per_step = 2 * 2 * nkv * hd * ctx * S              # K and V, two bytes each
+    value = bytes_per_step / (ms_per_step * 1e-3) / 1e9
+
+    # ---- dominant kernel alone, per-launch events
+    n_prof = min(args.steps, 512)
+    hipattn.profile_begin(n_prof)
+    for i in range(n_prof):
+        step(i)
+    kern_ms, n_timed = hipattn.profile_end()
+    kern_avg_ms = kern_ms / max(n_timed, 1)
+    achieved = bytes_per_step / (kern_avg_ms * 1e-3) / 1e9
+    roofline = {"bound": "hbm", "kernel": "decode_mfma_kernel<128>", "achieved": round(achieved, 1),
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                "traffic": None, "kernel_avg_us": round(kern_avg_ms * 1e3, 2),
+                "bytes_per_launch": bytes_per_step}
+
+    # ---- causal prefill (secondary figure of the metric)
+    prefill = None
+    if not args.no_prefill:
+        T = 2048
+        qp = synth.normal(synth.config_seed(4, 1), (T, nq, hd))
+        qp_dev = hipattn.DeviceBuffer.from_host(qp)
+        op_dev = hipattn.DeviceBuffer(qp.nbytes)
+        reps = 5
+        hipattn.prefill_dev(caches[0], 0, 0, T, qp_dev, op_dev, nq)
+        hipattn.profile_begin(reps)
+        for _ in range(reps):
+            hipattn.prefill_dev(caches[0], 0, 0, T, qp_dev, op_dev, nq)
+        pms, pn = hipattn.profile_end()
+        flops = 4.0 * nq * hd * T * (T + 1) / 2.0
+        p_avg = pms / max(pn, 1)
+        tfl = flops / (p_avg * 1e-3) / 1e12
+        gotp = op_dev.to_host((T, nq, hd))
+        rows = [0, 1, 31, 32, 777, 2047]
+        wantp = oracle.causal_prefill(qp, host_kv[0][0], host_kv[0][1], p0=0, rows=rows)
+        perr = float(np.max(np.abs(gotp[rows] - wantp[rows])))
+        prefill = {"workload": "causal prefill, 32/8/128, T=2048, empty cache", "tflops": round(tfl, 2),
+                   "ms": round(p_avg, 4), "frac_of_f16_mfma_peak": round(tfl / MFMA_F16_PEAK_TFLOPS, 4),
+                   "max_abs_err_sampled_rows": perr}
+        qp_dev.free()
+        op_dev.free()
+
+    # ---- CPU baseline: the oracle on the same data, one core, bounded sample
+    cpu = None
+    if args.cpu_seconds > 0:
+        done_bytes, t_cpu, n_calls = 0, 0.0, 0
+        s = 0
+        while t_cpu < args.cpu_seconds and n_calls < 3 * S:
+            k16, v16 = host_kv[s % S]
+            tc = time.perf_counter()
+            oracle.attention(q_host[0, s % S][None], k16, v16)
+            t_cpu += time.perf_counter() - tc
+            done_bytes += 2 * 2 * nkv * hd * ctx
+            n_calls += 1
+            s += 1
+        cpu = {"value": round(done_bytes / t_cpu / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+               "sample": "%d single-session calls of the same workload (32/8/128, ctx %d), "
+                         "%.1f s of CPU time, host has %d cpus" % (n_calls, ctx, t_cpu, os.cpu_count())}
+
+    line = {
+        "metric": "decode-attn HBM GB/s (% peak) at 16 sess x 4K ctx; prefill attn TFLOP/s",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f16 cache, f32 accumulate",
+        "data": "synthetic",
+        "config": {"workload": "batched decode attention, Llama-3-8B head shape 32/8/128, "
+                               "%d sessions x %d ctx, %d cache layers walked" % (S, ctx, L),
+                   "sessions": S, "ctx": ctx, "layers": L},
+        "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
+        "roofline": roofline, "cpu_baseline": cpu, "prefill": prefill,
+        "check": {"max_abs": max_abs, "rel_l2": rel_l2},
+        "device": hipattn.device_name(), "setup_s": round(setup_s, 1),
+    }
+    print(json.dumps(line), flush=True)
+    for kv in caches:
+        kv.close()
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,186 @@
+/*
+ * wr_hip_attn.h — C ABI of the MI355X (gfx950) attention path.
+ *
+ * A C11 host engine calls these in place of the reference's CPU attention
+ * op, its KV append and its KV storage.  Plain C linkage, plain pointers and
+ * sizes, int returns; no C++ or framework types cross this boundary.
+ *
+ * Each entry point names the reference interface it replaces (paths relative
+ * to the reference tree).
+ *
+ * Conventions (reference: include/wayruntime/wayruntime.h:82-107):
+ *   - return 0 (WR_OK) on success, a negative wr_status value on failure;
+ *   - nothing is ever truncated or clamped: a sequence above the cap is
+ *     WR_HIP_ERR_LIMIT, a full cache is WR_HIP_ERR_CTX_FULL;
+ *   - a failed call leaves cache contents below the caller's cursor intact.
+ *     The cursor itself (how many rows are valid) is owned by the caller, as
+ *     the reference keeps it in the session (src/core/session.c:160-168):
+ *     rollback is "reset the cursor"; rows above it are never read;
+ *   - host-pointer entry points are synchronous: results are in the caller's
+ *     buffer on return.  `_dev` entry points take device pointers, enqueue on
+ *     the library stream and return without waiting;
+ *   - thread safety: calls on DIFFERENT wr_hip_kv objects may run concurrently
+ *     from different threads (reference threading contract,
+ *     include/wayruntime/wayruntime.h:29-40); calls on one object must be
+ *     serialised by the caller (the session lock does that).
+ */
+#ifndef WR_HIP_ATTN_H
+#define WR_HIP_ATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* wr_status values used on this path (wayruntime.h:82-107). */
+#define WR_HIP_OK               0
+#define WR_HIP_ERR_UNSUPPORTED (-3)
+#define WR_HIP_ERR_INVAL       (-4)
+#define WR_HIP_ERR_NOMEM       (-5)
+#define WR_HIP_ERR_CTX_FULL    (-6)
+#define WR_HIP_ERR_STATE       (-7)
+#define WR_HIP_ERR_LIMIT       (-8)
+#define WR_HIP_ERR_INTERNAL    (-10)
+
+/* Limits.  WR_HIP_ATTN_MAX_SEQ plays the role of WR_ATTN_MAX_SEQ
+ * (src/core/internal.h:186-193) raised for the long-context workloads;
+ * WR_HIP_BATCH_MAX == WR_BATCH_MAX (wayruntime.h:423);
+ * WR_HIP_FLASH_D_MAX == WR_FLASH_D_MAX (internal.h:197). */
+#define WR_HIP_ATTN_MAX_SEQ   131072u
+#define WR_HIP_BATCH_MAX      16u
+#define WR_HIP_FLASH_D_MAX    1024u
+#define WR_HIP_MAX_LAYERS     64u        /* WR_MAX_LAYERS, internal.h:184 */
+
+/* Per-session device KV cache (opaque). */
+typedef struct wr_hip_kv wr_hip_kv;
+
+/* Log sink with the signature of wr_log_fn (wayruntime.h:126-130); device
+ * errors are reported through it like session.c:170-174 reports op failures. */
+typedef void (*wr_hip_log_fn)(int level, const char *msg, void *user);
+
+/* ---- lifecycle ----------------------------------------------------------
+ * Replaces: nothing on the CPU path; attaches where the engine is created and
+ * destroyed (src/core/engine.c:119-178, 180).  One init per process; a second
+ * init without shutdown returns WR_HIP_ERR_STATE (single engine per process,
+ * engine.c:125-129).  Fails with WR_HIP_ERR_UNSUPPORTED when no gfx950 device
+ * is present: there is no CPU fallback. */
+int  wr_hip_attn_init(int device);
+void wr_hip_attn_shutdown(void);
+void wr_hip_attn_set_log(wr_hip_log_fn fn, void *user);
+/* Number of attention calls issued, one per session-layer, the quantity the
+ * reference counts in WR_CTR_ATTENTION_CALLS (src/core/kernels.c:1423). */
+uint64_t wr_hip_attn_calls(void);
+/* "gfx950 ..." description of the device in use (static storage). */
+const char *wr_hip_attn_device_name(void);
+
+/* ---- KV storage ---------------------------------------------------------
+ * Replaces the KV half of session_build / wr_map_alloc / wr_map_free
+ * (src/core/session.c:640-674, 775, 811): one device allocation per session,
+ * made once, never grown.  Layers whose hd_per_layer entry is 0 get no
+ * storage (KV-shared layers alias another layer, session.c:652-658; pass the
+ * source layer's index to the other calls).  Allocation failure is
+ * WR_HIP_ERR_NOMEM; max_ctx above the cap is WR_HIP_ERR_LIMIT
+ * (session.c:755). */
+int  wr_hip_attn_kv_create(uint32_t n_layers, const uint32_t *hd_per_layer,
+                           uint32_t nkv, uint32_t max_ctx, wr_hip_kv **out);
+void wr_hip_attn_kv_destroy(wr_hip_kv *kv);
+uint64_t wr_hip_attn_kv_bytes(const wr_hip_kv *kv);
+
+/* ---- append -------------------------------------------------------------
+ * Replaces kv_append_row (src/core/session.c:139-154) for n_rows consecutive
+ * positions: k_f32 / v_f32 are host F32 [n_rows, nkv, hd_layer]; the rows are
+ * copied up and converted on the device with the reference's TRUNCATING
+ * F32->F16 rule (src/core/quant.c:121-136) into rows pos .. pos+n_rows-1.
+ * pos + n_rows > max_ctx is WR_HIP_ERR_CTX_FULL and writes nothing. */
+int wr_hip_attn_append(wr_hip_kv *kv, uint32_t layer, uint32_t pos,
+                       uint32_t n_rows, const float *k_f32,
+                       const float *v_f32);
+
+/* Test / tooling access to the cache in the reference's layout: F16 bit
+ * patterns, position-major [n_rows, nkv, hd_layer] (the layout of the
+ * reference's kv_k / kv_v tensors, src/core/internal.h:492-497).
+ * kv_write stores already-converted rows verbatim. */
+int wr_hip_attn_kv_read(wr_hip_kv *kv, uint32_t layer, uint32_t pos,
+                        uint32_t n_rows, uint16_t *k_f16, uint16_t *v_f16);
+int wr_hip_attn_kv_write(wr_hip_kv *kv, uint32_t layer, uint32_t pos,
+                         uint32_t n_rows, const uint16_t *k_f16,
+                         const uint16_t *v_f16);
+
+/* ---- decode -------------------------------------------------------------
+ * Replaces wri_op_gqa_attention with seq_q = 1 (src/core/kernels.c:1414-1527,
+ * contract src/core/internal.h:325-338) at its two call sites
+ * (src/core/session.c:341, 493).  q and out are host F32 [nq, hd_layer];
+ * seq_k is the number of valid rows (the K tensor's valid_rows);
+ * scale_override <= 0 means 1/sqrt(hd); window > 0 keeps only the last
+ * `window` keys.  seq_k == 0 or nq % nkv != 0 is WR_HIP_ERR_INVAL; seq_k above
+ * max_ctx is WR_HIP_ERR_INVAL (capacity), above the cap WR_HIP_ERR_LIMIT. */
+int wr_hip_attn_decode(wr_hip_kv *kv, uint32_t layer, uint32_t seq_k,
+                       const float *q, float *out, uint32_t nq,
+                       float scale_override, uint32_t window);
+
+/* One launch for n <= WR_HIP_BATCH_MAX sessions with ragged seq_k.
+ * Replaces the per-session attention calls inside the batched step
+ * (src/core/batch.c:156-164) when the host loop runs layer-major.  All caches
+ * must have the same nkv and the same head_dim at `layer`.  n == 0 or
+ * n > WR_HIP_BATCH_MAX is WR_HIP_ERR_LIMIT (batch.c:129). */
+int wr_hip_attn_decode_batched(uint32_t n, wr_hip_kv *const *kv,
+                               uint32_t layer, const uint32_t *seq_k,
+                               const float *const *q, float *const *out,
+                               uint32_t nq, float scale_override,
+                               uint32_t window);
+
+/* ---- causal prefill -----------------------------------------------------
+ * Replaces the loop of seq_q = 1 attention calls that prefill runs
+ * (src/core/session.c:615-625): rows p0 .. p0+T-1 have already been appended;
+ * row i of q [T, nq, hd_layer] attends keys 0 .. p0+i (with `window` > 0, the
+ * last `window` of those).  out is host F32 [T, nq, hd_layer]. */
+int wr_hip_attn_prefill(wr_hip_kv *kv, uint32_t layer, uint32_t p0,
+                        uint32_t T, const float *q, float *out, uint32_t nq,
+                        float scale_override, uint32_t window);
+
+/* ---- device-resident forms (measurement, device-side callers) ------------
+ * Same semantics, but q / out / k_f32 / v_f32 are DEVICE pointers obtained
+ * from wr_hip_attn_dev_alloc, the work is enqueued on the library stream and
+ * the call returns without waiting; wr_hip_attn_sync waits.  For the batched
+ * form q_dev and out_dev are [n, nq, hd] contiguous. */
+void *wr_hip_attn_dev_alloc(size_t bytes);
+void  wr_hip_attn_dev_free(void *p);
+int   wr_hip_attn_h2d(void *dst_dev, const void *src_host, size_t bytes);
+int   wr_hip_attn_d2h(void *dst_host, const void *src_dev, size_t bytes);
+int   wr_hip_attn_sync(void);
+void *wr_hip_attn_stream(void);          /* hipStream_t of the library */
+
+int wr_hip_attn_append_dev(wr_hip_kv *kv, uint32_t layer, uint32_t pos,
+                           uint32_t n_rows, const float *k_f32_dev,
+                           const float *v_f32_dev);
+int wr_hip_attn_decode_batched_dev(uint32_t n, wr_hip_kv *const *kv,
+                                   uint32_t layer, const uint32_t *seq_k,
+                                   const float *q_dev, float *out_dev,
+                                   uint32_t nq, float scale_override,
+                                   uint32_t window);
+int wr_hip_attn_prefill_dev(wr_hip_kv *kv, uint32_t layer, uint32_t p0,
+                            uint32_t T, const float *q_dev, float *out_dev,
+                            uint32_t nq, float scale_override,
+                            uint32_t window);
+
+/* Tuning knobs for measurement (0 = automatic): keys handled per workgroup in
+ * the split-K decode kernel, and a switch forcing the generic (non-MFMA)
+ * kernels.  Not needed by a normal caller. */
+void wr_hip_attn_set_tuning(uint32_t decode_keys_per_wg, int force_generic);
+
+/* Kernel timing for the roofline figure.  Between profile_begin and
+ * profile_end every launch of the MAIN kernel of a call (the split-K decode
+ * kernel, or the prefill kernel; not the small combine / append kernels) is
+ * bracketed by its own pair of events, so the sum is pure kernel time as a
+ * profiler would report it.  profile_end waits for the stream, then returns
+ * the summed milliseconds and the number of launches timed.  At most
+ * max_launches launches are timed; further ones run untimed. */
+int wr_hip_attn_profile_begin(uint32_t max_launches);
+int wr_hip_attn_profile_end(double *total_ms, uint32_t *n_launches);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* WR_HIP_ATTN_H */

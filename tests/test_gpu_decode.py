@@ -1,0 +1,272 @@
+"""Device decode attention and cache append against the CPU oracle, through
+the C ABI.  Tolerance: max-abs 2e-3 and rel-L2 1e-3 on the attention outputs
+(float32 accumulate), bit-exact on the cache contents."""
+import numpy as np
+import pytest
+
+import oracle
+from tests import util
+from tests.golden import cases
+from wayruntime_amd import hipattn, synth
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _device():
+    hipattn.init()
+    print("device:", hipattn.device_name(), flush=True)
+    yield
+    hipattn.set_tuning(0, False)
+
+
+# ------------------------------------------------------------------ append --
+
+@pytest.mark.parametrize("nkv,hd,max_ctx,chunks", [
+    (8, 128, 200, [1, 1, 1, 30, 1, 64, 33, 69]),      # crosses 32-position blocks at every offset
+    (4, 256, 70, [70]),
+    (2, 32, 40, [5, 35]),
+    (1, 20, 9, [1] * 9),                               # head_dim that is no multiple of 16
+])
+def test_append_is_bit_exact_and_leaves_neighbours_alone(nkv, hd, max_ctx, chunks):
+    kv = hipattn.KVCache(2, hd, nkv, max_ctx)
+    k32 = synth.normal(100, (max_ctx, nkv, hd), std=3.0)
+    v32 = synth.normal(101, (max_ctx, nkv, hd), std=3.0)
+    # values that exercise the codec edges: overflow, subnormal range, signed zero, NaN
+    k32.reshape(-1)[:6] = [1e6, -1e6, 3e-6, -3e-6, -0.0, np.nan]
+    v32.reshape(-1)[:4] = [65504.0, 65520.0, 6.1e-5, 6.0e-5]
+    pos = 0
+    for n in chunks:
+        print("append", nkv, hd, "pos", pos, "n", n, flush=True)
+        assert kv.append(1, pos, k32[pos:pos + n], v32[pos:pos + n]) == hipattn.OK
+        pos += n
+        gk, gv = kv.read_f16(1, 0, pos)
+        assert np.array_equal(gk, synth.f32_to_f16_trunc(k32[:pos]))
+        assert np.array_equal(gv, synth.f32_to_f16_trunc(v32[:pos]))
+    # the other layer is untouched (zero-filled at creation)
+    zk, zv = kv.read_f16(0, 0, max_ctx)
+    assert not zk.any() and not zv.any()
+    # a full cache refuses and writes nothing
+    before = kv.read_f16(1, 0, max_ctx)
+    assert kv.append(1, max_ctx, k32[:1], v32[:1]) == hipattn.ERR_CTX_FULL
+    assert kv.append(1, max_ctx - 1, k32[:2], v32[:2]) == hipattn.ERR_CTX_FULL
+    after = kv.read_f16(1, 0, max_ctx)
+    assert np.array_equal(before[0], after[0]) and np.array_equal(before[1], after[1])
+    kv.close()
+
+
+def test_append_matches_oracle_append_row():
+    import ctypes as C
+    nkv, hd, cap = 2, 64, 37
+    kv = hipattn.KVCache(1, hd, nkv, cap)
+    rows_k = synth.normal(7, (cap, nkv * hd), std=2.0)
+    rows_v = synth.normal(8, (cap, nkv * hd), std=2.0)
+    ok = np.zeros((cap, nkv, hd), dtype=np.uint16)
+    ov = np.zeros((cap, nkv, hd), dtype=np.uint16)
+    tk, tv = oracle.wrap(ok, flags=oracle.GROWABLE), oracle.wrap(ov, flags=oracle.GROWABLE)
+    for i in range(cap):
+        assert oracle.lib().wro_kv_append_row(C.byref(tk), rows_k[i], nkv, hd) == 0
+        assert oracle.lib().wro_kv_append_row(C.byref(tv), rows_v[i], nkv, hd) == 0
+        assert kv.append(0, i, rows_k[i].reshape(1, nkv, hd), rows_v[i].reshape(1, nkv, hd)) == 0
+    gk, gv = kv.read_f16(0, 0, cap)
+    assert np.array_equal(gk, ok) and np.array_equal(gv, ov)
+    kv.close()
+
+
+# ------------------------------------------------------------------ decode --
+
+def _run_decode(nq, nkv, hd, ctx, sc=0.0, win=0, seed=1, rows=None, generic=False, keys_per_wg=0):
+    rows = rows or ctx
+    q = synth.normal(seed, (nq, hd))
+    _k32, _v32, k16, v16 = util.make_kv(seed + 10, rows, nkv, hd)
+    kv = hipattn.KVCache(1, hd, nkv, rows)
+    kv.write_f16(0, 0, k16, v16)
+    hipattn.set_tuning(keys_per_wg, generic)
+    got = kv.decode(0, ctx, q, sc, win)
+    hipattn.set_tuning(0, False)
+    want = util.oracle_decode(q, k16, v16, ctx, sc, win)
+    kv.close()
+    return got, want
+
+
+@pytest.mark.parametrize("ctx", [128, 512, 2048, 8192])
+def test_decode_qwen3_shape_context_sweep(ctx):
+    print("decode 16/8/128 ctx", ctx, flush=True)
+    got, want = _run_decode(16, 8, 128, ctx, seed=synth.config_seed(2, ctx % 251))
+    print("  errors", util.assert_close(got, want, f"ctx={ctx}"), flush=True)
+
+
+@pytest.mark.parametrize("nq,nkv,hd,ctx,sc,win", [
+    (32, 8, 128, 4096, 0.0, 0),        # Llama-3-8B shape
+    (32, 8, 128, 1000, 0.0, 0),        # ragged: not a multiple of the 32-key tile
+    (8, 4, 256, 3000, 0.0, 0),         # Gemma-class shape
+    (8, 4, 256, 3000, 1.0, 1024),      # explicit scale 1.0 and sliding window
+    (4, 4, 64, 777, 0.0, 0),           # MHA, head_dim 64
+    (8, 1, 64, 300, 0.0, 0),           # group of 8
+    (16, 8, 128, 1, 0.0, 0),           # a single key: output is the V row
+    (16, 8, 128, 33, 0.0, 0),
+    (16, 8, 128, 2048, 0.0, 100),      # window inside one workgroup's span
+    (16, 8, 128, 2048, 0.0, 1999),
+    (16, 8, 128, 2048, 0.0, 5000),     # window larger than the context: no masking
+    (16, 8, 128, 700, 0.25, 0),        # scale override
+])
+def test_decode_shapes_windows_scales(nq, nkv, hd, ctx, sc, win):
+    print("decode", nq, nkv, hd, ctx, sc, win, flush=True)
+    got, want = _run_decode(nq, nkv, hd, ctx, sc, win, seed=ctx + win)
+    print("  errors", util.assert_close(got, want), flush=True)
+
+
+@pytest.mark.parametrize("nq,nkv,hd,ctx,sc,win", [
+    (4, 2, 32, 200, 0.0, 16),          # head_dim 32: generic kernel
+    (2, 1, 16, 96, 0.0, 0),
+    (4, 1, 4, 8, 0.0, 4),              # the reference self-test's tiny shape
+    (3, 3, 20, 50, 0.0, 0),            # odd head_dim
+    (32, 2, 128, 500, 0.0, 0),         # group of 16: beyond the MFMA kernel's group limit
+    (2, 1, 1024, 70, 0.0, 0),          # largest head_dim
+])
+def test_decode_generic_shapes(nq, nkv, hd, ctx, sc, win):
+    print("decode generic", nq, nkv, hd, ctx, sc, win, flush=True)
+    got, want = _run_decode(nq, nkv, hd, ctx, sc, win, seed=ctx)
+    print("  errors", util.assert_close(got, want), flush=True)
+
+
+@pytest.mark.parametrize("keys_per_wg", [32, 128, 4096, 1 << 20])
+def test_split_k_partition_does_not_change_the_result(keys_per_wg):
+    # any partition of the keys must give the unsplit result within tolerance;
+    # one split (direct write) and many splits (partials + combine) both covered
+    print("split-K keys_per_wg", keys_per_wg, flush=True)
+    got, want = _run_decode(32, 8, 128, 3001, seed=5, keys_per_wg=keys_per_wg)
+    util.assert_close(got, want)
+    got_g, _ = _run_decode(32, 8, 128, 3001, seed=5, keys_per_wg=keys_per_wg, generic=True)
+    util.assert_close(got_g, want, "generic")
+    # the two device implementations agree far inside the tolerance
+    assert util.errors(got, got_g)[0] < 2e-4
+
+
+def test_rows_above_the_cursor_are_never_trusted():
+    nq, nkv, hd, rows, ctx = 16, 8, 128, 512, 300
+    q = synth.normal(3, (nq, hd))
+    _a, _b, k16, v16 = util.make_kv(30, rows, nkv, hd)
+    k_bad, v_bad = k16.copy(), v16.copy()
+    k_bad[ctx:] = 0x7E00          # NaN bit patterns above the cursor
+    v_bad[ctx:] = 0x7C00          # +inf
+    kv = hipattn.KVCache(1, hd, nkv, rows)
+    kv.write_f16(0, 0, k_bad, v_bad)
+    got = kv.decode(0, ctx, q)
+    util.assert_close(got, util.oracle_decode(q, k16, v16, ctx))
+    kv.close()
+
+
+@pytest.mark.parametrize("case", [c for c in cases.ATTN_CASES if c[9] == "f16" and c[1] == 1],
+                         ids=lambda c: c[0])
+def test_decode_against_reference_golden_outputs(case):
+    # expected outputs written by the compiled reference (tests/golden)
+    name, _sq, nq, nkv, hd, rows, seq_k, sc, win, _dt = case
+    print("golden", name, flush=True)
+    import os
+    gold = np.load(os.path.join(os.path.dirname(__file__), "golden", "attn_golden.npz"))[name]
+    q, k16, v16 = cases.attn_inputs(case)
+    kv = hipattn.KVCache(1, hd, nkv, rows)
+    kv.write_f16(0, 0, k16, v16)
+    got = kv.decode(0, seq_k or rows, q[0], sc, win)
+    util.assert_close(got, gold[0], name)
+    kv.close()
+
+
+# ----------------------------------------------------------------- batched --
+
+def test_batched_ragged_llama_shape_equals_serial_and_oracle():
+    nq, nkv, hd, S = 32, 8, 128, 16
+    ctxs = synth.ragged_contexts(synth.config_seed(3, 0), S, 256, 4096)
+    print("batched ctx", ctxs.tolist(), flush=True)
+    caches, qs, kvs = [], [], []
+    for i, ctx in enumerate(ctxs):
+        q = synth.normal(synth.config_seed(3, 10 + i), (nq, hd))
+        _a, _b, k16, v16 = util.make_kv(synth.config_seed(3, 40 + 2 * i), int(ctx), nkv, hd)
+        kv = hipattn.KVCache(1, hd, nkv, int(ctx))
+        kv.write_f16(0, 0, k16, v16)
+        caches.append(kv); qs.append(q); kvs.append((k16, v16))
+    outs = hipattn.decode_batched(caches, 0, ctxs, qs)
+    for i in range(S):
+        want = util.oracle_decode(qs[i], kvs[i][0], kvs[i][1], int(ctxs[i]))
+        util.assert_close(outs[i], want, f"session {i}")
+    # serial per-session stepping: within rounding of the batched result under
+    # the automatic partition, and bit-identical when both use the same key
+    # partition (sessions never share arithmetic)
+    for i in range(S):
+        single = caches[i].decode(0, int(ctxs[i]), qs[i])
+        assert util.errors(single, outs[i])[0] < 1e-5, f"session {i}"
+    hipattn.set_tuning(256, False)
+    outs_fixed = hipattn.decode_batched(caches, 0, ctxs, qs)
+    for i in range(S):
+        single = caches[i].decode(0, int(ctxs[i]), qs[i])
+        assert np.array_equal(single, outs_fixed[i]), f"session {i}"
+    hipattn.set_tuning(0, False)
+    for kv in caches:
+        kv.close()
+
+
+def test_decode_step_loop_append_then_attend():
+    # eight decode steps, each appending one position per session and then
+    # attending (the long-context workload's step shape, at a short context)
+    nq, nkv, hd, S, base = 8, 4, 256, 3, 250
+    caches, k16s, v16s = [], [], []
+    for i in range(S):
+        kv = hipattn.KVCache(1, hd, nkv, base + 8)
+        _a, _b, k16, v16 = util.make_kv(900 + i, base + 8, nkv, hd)
+        kv.write_f16(0, 0, k16[:base], v16[:base])
+        caches.append(kv); k16s.append(k16); v16s.append(v16)
+    for step in range(8):
+        qs = [synth.normal(1000 + 10 * step + i, (nq, hd)) for i in range(S)]
+        for i in range(S):
+            kn = synth.normal(2000 + 10 * step + i, (1, nkv, hd))
+            vn = synth.normal(3000 + 10 * step + i, (1, nkv, hd))
+            assert caches[i].append(0, base + step, kn, vn) == hipattn.OK
+            k16s[i][base + step] = synth.f32_to_f16_trunc(kn)[0]
+            v16s[i][base + step] = synth.f32_to_f16_trunc(vn)[0]
+        outs = hipattn.decode_batched(caches, 0, [base + step + 1] * S, qs)
+        for i in range(S):
+            util.assert_close(outs[i], util.oracle_decode(qs[i], k16s[i], v16s[i], base + step + 1),
+                              f"step {step} session {i}")
+    for kv in caches:
+        kv.close()
+
+
+# ---------------------------------------------------------- error contract --
+
+def test_error_contract():
+    import ctypes as C
+    lib = hipattn.lib()
+    kv = hipattn.KVCache(2, [128, 0], 8, 64)      # layer 1 has no storage (shared layer)
+    q = np.zeros((16, 128), dtype=np.float32)
+    out = np.zeros_like(q)
+    dec = lambda layer, seq_k, nq=16, qq=q: lib.wr_hip_attn_decode(      # noqa: E731
+        kv.h, layer, seq_k, qq.ctypes.data, out.ctypes.data, nq, 0.0, 0)
+    assert dec(0, 0) == hipattn.ERR_INVAL                    # empty sequence
+    assert dec(0, 65) == hipattn.ERR_INVAL                   # beyond the allocation
+    assert dec(0, hipattn.ATTN_MAX_SEQ + 1) == hipattn.ERR_LIMIT     # cap: refused, never clamped
+    assert dec(1, 10) == hipattn.ERR_INVAL                   # layer without storage
+    assert dec(2, 10) == hipattn.ERR_INVAL
+    assert dec(0, 10, nq=12) == hipattn.ERR_INVAL            # nq % nkv != 0
+    assert lib.wr_hip_attn_decode(kv.h, 0, 10, None, out.ctypes.data, 16, 0.0, 0) == hipattn.ERR_INVAL
+    calls = lib.wr_hip_attn_calls()
+    assert dec(0, 10) == hipattn.OK
+    assert lib.wr_hip_attn_calls() == calls + 1              # one count per session-layer call
+    h = C.c_void_p()
+    hd = (C.c_uint32 * 1)(128)
+    assert lib.wr_hip_attn_kv_create(1, hd, 8, hipattn.ATTN_MAX_SEQ + 1, C.byref(h)) == hipattn.ERR_LIMIT
+    assert lib.wr_hip_attn_kv_create(65, hd, 8, 16, C.byref(h)) == hipattn.ERR_LIMIT
+    assert lib.wr_hip_attn_kv_create(1, hd, 0, 16, C.byref(h)) == hipattn.ERR_INVAL
+    big = (C.c_uint32 * 1)(2048)
+    assert lib.wr_hip_attn_kv_create(1, big, 8, 16, C.byref(h)) == hipattn.ERR_LIMIT
+    # batch limits: 0 and 17 sessions are refused (reference batch.c:129)
+    kvp = (C.c_void_p * 17)(*([kv.h] * 17))
+    sk = (C.c_uint32 * 17)(*([10] * 17))
+    ptrs = (C.c_void_p * 17)(*([q.ctypes.data] * 17))
+    outs = (C.c_void_p * 17)(*([out.ctypes.data] * 17))
+    assert lib.wr_hip_attn_decode_batched(0, kvp, 0, sk, ptrs, outs, 16, 0.0, 0) == hipattn.ERR_LIMIT
+    assert lib.wr_hip_attn_decode_batched(17, kvp, 0, sk, ptrs, outs, 16, 0.0, 0) == hipattn.ERR_LIMIT
+    # the same session twice in one batch is refused (reference batch.c:135-136)
+    assert lib.wr_hip_attn_decode_batched(2, kvp, 0, sk, ptrs, outs, 16, 0.0, 0) == hipattn.ERR_INVAL
+    assert lib.wr_hip_attn_init(0) == hipattn.ERR_STATE      # single engine per process
+    kv.close()

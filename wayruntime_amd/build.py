@@ -1,0 +1,52 @@
+"""Builds the gfx950 shared library in-tree (``wayruntime_amd/libwr_hip_attn.so``).
+
+    python -m wayruntime_amd.build            # compile
+    python -m wayruntime_amd.build --temps    # also keep ISA / resource usage under _work/temps
+"""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(PKG)
+HIP_SO = os.path.join(PKG, "libwr_hip_attn.so")
+HIP_SRC = os.path.join(PKG, "csrc", "wr_hip_attn.hip")
+
+HIPCC_FLAGS = [
+    "-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-shared",
+    # no packed-FP32 VALU forms in device code
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-function",
+]
+
+
+def build_hip(keep_temps: bool = False) -> str:
+    cmd = ["hipcc"] + HIPCC_FLAGS
+    if keep_temps:
+        tmp = os.path.join(ROOT, "_work", "temps")
+        os.makedirs(tmp, exist_ok=True)
+        cmd += ["-save-temps=obj"]
+    cmd += ["-o", HIP_SO, HIP_SRC]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    noise = "is not a recognized feature for this target"
+    err = "\n".join(l for l in res.stderr.splitlines() if noise not in l)
+    if err.strip():
+        sys.stderr.write(err + "\n")
+    if res.returncode != 0:
+        raise RuntimeError("hipcc failed building " + HIP_SO)
+    if keep_temps:
+        for f in os.listdir(PKG):
+            if f.startswith("wr_hip_attn-") or f.startswith("wr_hip_attn.hip-"):
+                os.replace(os.path.join(PKG, f), os.path.join(ROOT, "_work", "temps", f))
+    return HIP_SO
+
+
+def build_all(keep_temps: bool = False) -> None:
+    build_hip(keep_temps)
+
+
+if __name__ == "__main__":
+    build_all("--temps" in sys.argv)
+    print("built", HIP_SO)

@@ -1,0 +1,96 @@
+// Cache append / import / export kernels.
+//
+// append: F32 rows [n_rows][nkv][hd] -> truncated F16 into rows pos.. of K and
+// of the block-transposed Vt (layout in common.hip.h).  The conversion is the
+// reference's truncating rule (reference: src/core/session.c:139-154 calling
+// src/core/quant.c:121-136), done with integer ops so the stored bits equal
+// the reference's bit for bit.  HBM-bound byte work: 6 bytes moved per element
+// (4 read, 2 written).
+#pragma once
+
+#include "common.hip.h"
+
+namespace wr {
+
+template <typename Src>
+__device__ __forceinline__ uint16_t to_cache_bits(Src v);
+template <>
+__device__ __forceinline__ uint16_t to_cache_bits<float>(float v) { return f32_to_f16_trunc(v); }
+template <>
+__device__ __forceinline__ uint16_t to_cache_bits<uint16_t>(uint16_t v) { return v; }
+
+// K side: one thread per element; reads and writes are both unit-stride in d.
+template <typename Src>
+__global__ __launch_bounds__(256) void append_k_kernel(const Src* __restrict__ src,
+                                                       uint16_t* __restrict__ k, uint32_t pos,
+                                                       uint32_t n_rows, uint32_t nkv, uint32_t hd,
+                                                       uint32_t ctx_pad)
+{
+    const size_t total = (size_t)n_rows * nkv * hd;
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const uint32_t d = (uint32_t)(idx % hd);
+    const uint32_t kvh = (uint32_t)((idx / hd) % nkv);
+    const uint32_t r = (uint32_t)(idx / ((size_t)hd * nkv));
+    k[k_row_offset(kvh, ctx_pad, pos + r, hd) + d] = to_cache_bits<Src>(src[idx]);
+}
+
+// V side: a workgroup owns a 32-position x 64-dimension tile of one KV head.
+// It reads the source unit-stride in d, turns the tile through LDS and writes
+// each dimension's 32 positions as one contiguous 64-byte run.  Positions of
+// the block that lie outside [pos, pos + n_rows) are left untouched, so a
+// one-row decode append never disturbs its neighbours.
+template <typename Src>
+__global__ __launch_bounds__(256) void append_v_kernel(const Src* __restrict__ src,
+                                                       uint16_t* __restrict__ vt, uint32_t pos,
+                                                       uint32_t n_rows, uint32_t nkv, uint32_t hd,
+                                                       uint32_t ctx_pad)
+{
+    __shared__ uint16_t tile[64][kVBlock + 2];
+    const uint32_t d0 = blockIdx.x * 64;
+    const uint32_t kvh = blockIdx.y;
+    const uint32_t blk = pos / kVBlock + blockIdx.z;
+    const uint32_t t = threadIdx.x;
+    const uint32_t end = pos + n_rows;
+
+    const uint32_t dl = t & 63;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const uint32_t pl = i * 4 + (t >> 6);
+        const uint32_t p = blk * kVBlock + pl;
+        uint16_t bits = 0;
+        if (p >= pos && p < end && d0 + dl < hd)
+            bits = to_cache_bits<Src>(src[((size_t)(p - pos) * nkv + kvh) * hd + d0 + dl]);
+        tile[dl][pl] = bits;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const uint32_t idx = i * 256 + t;
+        const uint32_t dl2 = idx / kVBlock;
+        const uint32_t pl2 = idx % kVBlock;
+        const uint32_t p = blk * kVBlock + pl2;
+        if (p >= pos && p < end && d0 + dl2 < hd)
+            vt[vt_offset(kvh, ctx_pad, p, d0 + dl2, hd)] = tile[dl2][pl2];
+    }
+}
+
+// Export rows back in position-major order [n_rows][nkv][hd] (tests, tooling).
+__global__ __launch_bounds__(256) void export_kv_kernel(const uint16_t* __restrict__ k,
+                                                        const uint16_t* __restrict__ vt,
+                                                        uint16_t* __restrict__ k_out,
+                                                        uint16_t* __restrict__ v_out, uint32_t pos,
+                                                        uint32_t n_rows, uint32_t nkv, uint32_t hd,
+                                                        uint32_t ctx_pad)
+{
+    const size_t total = (size_t)n_rows * nkv * hd;
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const uint32_t d = (uint32_t)(idx % hd);
+    const uint32_t kvh = (uint32_t)((idx / hd) % nkv);
+    const uint32_t r = (uint32_t)(idx / ((size_t)hd * nkv));
+    k_out[idx] = k[k_row_offset(kvh, ctx_pad, pos + r, hd) + d];
+    v_out[idx] = vt[vt_offset(kvh, ctx_pad, pos + r, d, hd)];
+}
+
+}  // namespace wr

@@ -1,0 +1,753 @@
+// C ABI of the MI355X attention path: device state, cache slabs, argument
+// checking and kernel launches.  Declarations and the reference interfaces
+// each entry point stands in for are in include/wr_hip_attn.h.
+//
+// There is no CPU path in this file: without a gfx950 device init fails and
+// every other entry point returns WR_HIP_ERR_STATE.
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
+
+#include <atomic>
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <new>
+#include <vector>
+
+#include "../../include/wr_hip_attn.h"
+#include "common.hip.h"
+#include "kernels_append.hip.h"
+#include "kernels_decode.hip.h"
+#include "kernels_prefill.hip.h"
+
+using namespace wr;
+
+struct wr_hip_kv {
+    uint32_t n_layers, nkv, max_ctx, ctx_pad;
+    uint32_t hd[WR_HIP_MAX_LAYERS];
+    size_t k_off[WR_HIP_MAX_LAYERS];     // byte offsets into slab
+    size_t vt_off[WR_HIP_MAX_LAYERS];
+    uint8_t* slab;
+    size_t bytes;
+};
+
+namespace {
+
+struct Buffer {
+    void* p = nullptr;
+    size_t cap = 0;
+};
+
+struct Lib {
+    std::mutex mu;               // serialises submissions and workspace growth
+    bool inited = false;
+    int device = -1;
+    hipStream_t stream = nullptr;
+    char name[320] = "uninitialised";
+    Buffer d_stage;              // device staging for host-pointer entry points
+    Buffer d_part;               // split-K partials
+    Buffer h_pin;                // pinned host staging
+    std::atomic<uint64_t> calls{0};
+    wr_hip_log_fn log_fn = nullptr;
+    void* log_user = nullptr;
+    uint32_t tune_keys_per_wg = 0;
+    int force_generic = 0;
+    std::vector<hipEvent_t> ev;
+    uint32_t ev_used = 0;
+    bool profiling = false;
+} g;
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr size_t kPinSmall = 1u << 20;      // host copies up to this size go through pinned staging
+
+void logmsg(int level, const char* fmt, ...)
+{
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    if (g.log_fn)
+        g.log_fn(level, buf, g.log_user);
+    else
+        fprintf(stderr, "[wr_hip_attn] %s\n", buf);
+}
+
+int hip_fail(hipError_t e, const char* what, uint32_t layer)
+{
+    logmsg(0, "hip: %s failed at layer %u: %s", what, layer, hipGetErrorString(e));
+    return (e == hipErrorOutOfMemory) ? WR_HIP_ERR_NOMEM : WR_HIP_ERR_INTERNAL;
+}
+
+#define HIP_TRY(expr, what, layer)                                   \
+    do {                                                             \
+        hipError_t e_ = (expr);                                      \
+        if (e_ != hipSuccess) return hip_fail(e_, what, layer);      \
+    } while (0)
+
+int ensure_device(Buffer& b, size_t need)
+{
+    if (need <= b.cap) return WR_HIP_OK;
+    HIP_TRY(hipStreamSynchronize(g.stream), "sync before workspace growth", 0);
+    if (b.p) (void)hipFree(b.p);
+    b.p = nullptr;
+    b.cap = 0;
+    const size_t want = need + need / 2 + 4096;
+    HIP_TRY(hipMalloc(&b.p, want), "workspace alloc", 0);
+    b.cap = want;
+    return WR_HIP_OK;
+}
+
+int ensure_pinned(Buffer& b, size_t need)
+{
+    if (need <= b.cap) return WR_HIP_OK;
+    HIP_TRY(hipStreamSynchronize(g.stream), "sync before pinned growth", 0);
+    if (b.p) (void)hipHostFree(b.p);
+    b.p = nullptr;
+    b.cap = 0;
+    const size_t want = need + need / 2 + 4096;
+    HIP_TRY(hipHostMalloc(&b.p, want, hipHostMallocDefault), "pinned alloc", 0);
+    b.cap = want;
+    return WR_HIP_OK;
+}
+
+// Host -> device / device -> host on the library stream.  Small transfers go
+// through pinned staging (predictable latency); large ones are handed to the
+// runtime directly.  Both leave the stream synchronised for the host buffer.
+int copy_up(void* dst_dev, const void* src_host, size_t bytes, size_t pin_off)
+{
+    if (bytes == 0) return WR_HIP_OK;
+    if (pin_off + bytes <= g.h_pin.cap && bytes <= kPinSmall) {
+        memcpy((uint8_t*)g.h_pin.p + pin_off, src_host, bytes);
+        HIP_TRY(hipMemcpyAsync(dst_dev, (uint8_t*)g.h_pin.p + pin_off, bytes,
+                               hipMemcpyHostToDevice, g.stream), "h2d", 0);
+    } else {
+        HIP_TRY(hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, g.stream),
+                "h2d", 0);
+        HIP_TRY(hipStreamSynchronize(g.stream), "h2d sync", 0);
+    }
+    return WR_HIP_OK;
+}
+
+int copy_down_sync(void* dst_host, const void* src_dev, size_t bytes)
+{
+    if (bytes == 0) return hipStreamSynchronize(g.stream) == hipSuccess ? WR_HIP_OK
+                                                                         : WR_HIP_ERR_INTERNAL;
+    if (bytes <= g.h_pin.cap && bytes <= kPinSmall) {
+        HIP_TRY(hipMemcpyAsync(g.h_pin.p, src_dev, bytes, hipMemcpyDeviceToHost, g.stream),
+                "d2h", 0);
+        HIP_TRY(hipStreamSynchronize(g.stream), "d2h sync", 0);
+        memcpy(dst_host, g.h_pin.p, bytes);
+    } else {
+        HIP_TRY(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, g.stream),
+                "d2h", 0);
+        HIP_TRY(hipStreamSynchronize(g.stream), "d2h sync", 0);
+    }
+    return WR_HIP_OK;
+}
+
+template <typename Kern, typename Args>
+void launch_main(Kern kernel, dim3 grid, dim3 block, const Args& args)
+{
+    if (g.profiling && g.ev_used + 2 <= g.ev.size()) {
+        hipExtLaunchKernelGGL(kernel, grid, block, 0, g.stream, g.ev[g.ev_used],
+                              g.ev[g.ev_used + 1], 0, args);
+        g.ev_used += 2;
+    } else {
+        hipLaunchKernelGGL(kernel, grid, block, 0, g.stream, args);
+    }
+}
+
+bool mfma_shape(uint32_t hd, uint32_t group)
+{
+    return !g.force_generic && (hd == 64 || hd == 128 || hd == 256) && group <= kMaxGroupMfma;
+}
+
+int check_layer(const wr_hip_kv* kv, uint32_t layer)
+{
+    if (!kv) return WR_HIP_ERR_INVAL;
+    if (layer >= kv->n_layers || kv->hd[layer] == 0) return WR_HIP_ERR_INVAL;
+    return WR_HIP_OK;
+}
+
+uint32_t key_lo_for(uint32_t window, uint32_t seq_k)
+{
+    return (window > 0 && seq_k > window) ? seq_k - window : 0;
+}
+
+// ------------------------------------------------------------------------
+// Unlocked bodies (caller holds g.mu and has set the device).
+
+template <typename Src>
+int append_rows_locked(wr_hip_kv* kv, uint32_t layer, uint32_t pos, uint32_t n_rows,
+                       const Src* k_dev, const Src* v_dev)
+{
+    const uint32_t hd = kv->hd[layer], nkv = kv->nkv;
+    uint16_t* kbase = reinterpret_cast<uint16_t*>(kv->slab + kv->k_off[layer]);
+    uint16_t* vbase = reinterpret_cast<uint16_t*>(kv->slab + kv->vt_off[layer]);
+    const size_t total = (size_t)n_rows * nkv * hd;
+    const uint32_t blocks = (uint32_t)((total + 255) / 256);
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(append_k_kernel<Src>), dim3(blocks), dim3(256), 0, g.stream,
+                       k_dev, kbase, pos, n_rows, nkv, hd, kv->ctx_pad);
+    const uint32_t nblk = (pos + n_rows - 1) / kVBlock - pos / kVBlock + 1;
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(append_v_kernel<Src>), dim3((hd + 63) / 64, nkv, nblk),
+                       dim3(256), 0, g.stream, v_dev, vbase, pos, n_rows, nkv, hd, kv->ctx_pad);
+    HIP_TRY(hipGetLastError(), "append launch", layer);
+    return WR_HIP_OK;
+}
+
+int check_append(const wr_hip_kv* kv, uint32_t layer, uint32_t pos, uint32_t n_rows,
+                 const void* k, const void* v)
+{
+    if (!g.inited) return WR_HIP_ERR_STATE;
+    int rc = check_layer(kv, layer);
+    if (rc) return rc;
+    if (n_rows == 0) return WR_HIP_OK;
+    if (!k || !v) return WR_HIP_ERR_INVAL;
+    if ((uint64_t)pos + n_rows > kv->max_ctx) return WR_HIP_ERR_CTX_FULL;
+    return WR_HIP_OK;
+}
+
+int decode_locked(uint32_t n, wr_hip_kv* const* kv, uint32_t layer, const uint32_t* seq_k,
+                  const float* q_dev, float* out_dev, uint32_t nq, float scale_override,
+                  uint32_t window)
+{
+    const uint32_t hd = kv[0]->hd[layer], nkv = kv[0]->nkv;
+    const uint32_t group = nq / nkv;
+    const bool use_mfma = mfma_shape(hd, group);
+
+    DecodeArgs a;
+    memset(&a, 0, sizeof a);
+    uint64_t tiles_total = 0;
+    uint32_t tiles[kBatchMax];
+    for (uint32_t i = 0; i < n; i++) {
+        DecodeSession& s = a.s[i];
+        s.k = reinterpret_cast<const uint16_t*>(kv[i]->slab + kv[i]->k_off[layer]);
+        s.vt = reinterpret_cast<const uint16_t*>(kv[i]->slab + kv[i]->vt_off[layer]);
+        s.seq_k = seq_k[i];
+        s.key_lo = key_lo_for(window, seq_k[i]);
+        s.ctx_pad = kv[i]->ctx_pad;
+        tiles[i] = (s.seq_k + kTileKeys - 1) / kTileKeys - s.key_lo / kTileKeys;
+        tiles_total += tiles[i];
+    }
+
+    // Keys per workgroup: enough workgroups to fill 256 CUs several times over,
+    // but at least one tile per wave so the per-workgroup merge stays small
+    // next to the data it streams.
+    uint32_t tiles_per_wg;
+    if (g.tune_keys_per_wg) {
+        tiles_per_wg = g.tune_keys_per_wg / kTileKeys;
+        if (tiles_per_wg == 0) tiles_per_wg = 1;
+    } else {
+        const uint64_t units = tiles_total * (use_mfma ? nkv : nq);
+        tiles_per_wg = (uint32_t)((units + 2047) / 2048);
+        tiles_per_wg = (tiles_per_wg + 3) & ~3u;
+        if (tiles_per_wg < 4) tiles_per_wg = 4;
+    }
+    uint32_t max_splits = 1;
+    for (uint32_t i = 0; i < n; i++) {
+        a.s[i].n_splits = (tiles[i] + tiles_per_wg - 1) / tiles_per_wg;
+        if (a.s[i].n_splits > max_splits) max_splits = a.s[i].n_splits;
+    }
+    a.q = q_dev;
+    a.out = out_dev;
+    a.nq = nq;
+    a.nkv = nkv;
+    a.group = group;
+    a.hd = hd;
+    a.tiles_per_wg = tiles_per_wg;
+    a.max_splits = max_splits;
+    a.direct = (max_splits == 1) ? 1u : 0u;
+    const float scale = (scale_override > 0.0f) ? scale_override : 1.0f / sqrtf((float)hd);
+    a.qscale = scale * kLog2e;
+
+    if (!a.direct) {
+        const size_t po = (size_t)n * nq * max_splits * hd * sizeof(float);
+        const size_t pml = (size_t)n * nq * max_splits * 2 * sizeof(float);
+        int rc = ensure_device(g.d_part, po + pml);
+        if (rc) return rc;
+        a.part_o = reinterpret_cast<float*>(g.d_part.p);
+        a.part_ml = reinterpret_cast<float*>((uint8_t*)g.d_part.p + po);
+    }
+
+    if (use_mfma) {
+        const dim3 grid(max_splits, nkv, n), block(kDecodeThreads);
+        if (hd == 64)
+            launch_main(decode_mfma_kernel<64>, grid, block, a);
+        else if (hd == 128)
+            launch_main(decode_mfma_kernel<128>, grid, block, a);
+        else
+            launch_main(decode_mfma_kernel<256>, grid, block, a);
+    } else {
+        launch_main(decode_generic_kernel, dim3(max_splits, nq, n), dim3(kDecodeThreads), a);
+    }
+    if (!a.direct)
+        hipLaunchKernelGGL(decode_combine_kernel, dim3(nq, n), dim3(128), 0, g.stream, a);
+    HIP_TRY(hipGetLastError(), "decode launch", layer);
+    g.calls.fetch_add(n, std::memory_order_relaxed);
+    return WR_HIP_OK;
+}
+
+int check_decode(uint32_t n, wr_hip_kv* const* kv, uint32_t layer, const uint32_t* seq_k,
+                 const void* q, const void* out, uint32_t nq)
+{
+    if (!g.inited) return WR_HIP_ERR_STATE;
+    if (!kv || !seq_k || !q || !out) return WR_HIP_ERR_INVAL;
+    if (n == 0 || n > WR_HIP_BATCH_MAX) return WR_HIP_ERR_LIMIT;
+    for (uint32_t i = 0; i < n; i++) {
+        int rc = check_layer(kv[i], layer);
+        if (rc) return rc;
+        if (kv[i]->nkv != kv[0]->nkv || kv[i]->hd[layer] != kv[0]->hd[layer])
+            return WR_HIP_ERR_INVAL;
+        for (uint32_t j = 0; j < i; j++)
+            if (kv[i] == kv[j]) return WR_HIP_ERR_INVAL;
+    }
+    if (nq == 0 || nq % kv[0]->nkv != 0) return WR_HIP_ERR_INVAL;
+    for (uint32_t i = 0; i < n; i++) {
+        if (seq_k[i] == 0) return WR_HIP_ERR_INVAL;
+        if (seq_k[i] > WR_HIP_ATTN_MAX_SEQ) return WR_HIP_ERR_LIMIT;
+        if (seq_k[i] > kv[i]->max_ctx) return WR_HIP_ERR_INVAL;
+    }
+    return WR_HIP_OK;
+}
+
+int prefill_locked(wr_hip_kv* kv, uint32_t layer, uint32_t p0, uint32_t T, const float* q_dev,
+                   float* out_dev, uint32_t nq, float scale_override, uint32_t window)
+{
+    const uint32_t hd = kv->hd[layer];
+    PrefillArgs a;
+    memset(&a, 0, sizeof a);
+    a.k = reinterpret_cast<const uint16_t*>(kv->slab + kv->k_off[layer]);
+    a.vt = reinterpret_cast<const uint16_t*>(kv->slab + kv->vt_off[layer]);
+    a.q = q_dev;
+    a.out = out_dev;
+    a.p0 = p0;
+    a.T = T;
+    a.nq = nq;
+    a.nkv = kv->nkv;
+    a.group = nq / kv->nkv;
+    a.hd = hd;
+    a.ctx_pad = kv->ctx_pad;
+    a.window = window;
+    const float scale = (scale_override > 0.0f) ? scale_override : 1.0f / sqrtf((float)hd);
+    a.qscale = scale * kLog2e;
+    launch_main(prefill_generic_kernel, dim3(T, nq), dim3(kDecodeThreads), a);
+    HIP_TRY(hipGetLastError(), "prefill launch", layer);
+    g.calls.fetch_add(T, std::memory_order_relaxed);
+    return WR_HIP_OK;
+}
+
+int check_prefill(const wr_hip_kv* kv, uint32_t layer, uint32_t p0, uint32_t T, const void* q,
+                  const void* out, uint32_t nq)
+{
+    if (!g.inited) return WR_HIP_ERR_STATE;
+    int rc = check_layer(kv, layer);
+    if (rc) return rc;
+    if (!q || !out) return WR_HIP_ERR_INVAL;
+    if (T == 0) return WR_HIP_ERR_INVAL;
+    if (nq == 0 || nq % kv->nkv != 0) return WR_HIP_ERR_INVAL;
+    if ((uint64_t)p0 + T > WR_HIP_ATTN_MAX_SEQ) return WR_HIP_ERR_LIMIT;
+    if ((uint64_t)p0 + T > kv->max_ctx) return WR_HIP_ERR_INVAL;
+    return WR_HIP_OK;
+}
+
+struct Locked {
+    std::lock_guard<std::mutex> lk;
+    Locked() : lk(g.mu)
+    {
+        if (g.inited) (void)hipSetDevice(g.device);
+    }
+};
+
+}  // namespace
+
+// ======================================================================= ABI
+
+extern "C" {
+
+int wr_hip_attn_init(int device)
+{
+    std::lock_guard<std::mutex> lk(g.mu);
+    if (g.inited) return WR_HIP_ERR_STATE;
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess || count <= 0) {
+        logmsg(0, "init: no HIP device visible; this library has no CPU path");
+        return WR_HIP_ERR_UNSUPPORTED;
+    }
+    if (device < 0 || device >= count) return WR_HIP_ERR_INVAL;
+    hipDeviceProp_t prop;
+    HIP_TRY(hipSetDevice(device), "set device", 0);
+    HIP_TRY(hipGetDeviceProperties(&prop, device), "device properties", 0);
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+        logmsg(0, "init: device %d is %s; the kernels are built for gfx950 only", device,
+               prop.gcnArchName);
+        return WR_HIP_ERR_UNSUPPORTED;
+    }
+    HIP_TRY(hipStreamCreateWithFlags(&g.stream, hipStreamNonBlocking), "stream create", 0);
+    g.device = device;
+    snprintf(g.name, sizeof g.name, "%s %s, %d CUs, %.1f GiB", prop.gcnArchName, prop.name,
+             prop.multiProcessorCount, (double)prop.totalGlobalMem / (1024.0 * 1024.0 * 1024.0));
+    g.inited = true;
+    g.calls.store(0);
+    int rc = ensure_pinned(g.h_pin, 2 * kPinSmall);
+    if (rc == WR_HIP_OK) rc = ensure_device(g.d_stage, 2 * kPinSmall);
+    if (rc != WR_HIP_OK) {
+        g.inited = false;
+        (void)hipStreamDestroy(g.stream);
+        g.stream = nullptr;
+    }
+    return rc;
+}
+
+void wr_hip_attn_shutdown(void)
+{
+    std::lock_guard<std::mutex> lk(g.mu);
+    if (!g.inited) return;
+    (void)hipSetDevice(g.device);
+    (void)hipStreamSynchronize(g.stream);
+    for (hipEvent_t e : g.ev) (void)hipEventDestroy(e);
+    g.ev.clear();
+    g.ev_used = 0;
+    g.profiling = false;
+    if (g.d_stage.p) (void)hipFree(g.d_stage.p);
+    if (g.d_part.p) (void)hipFree(g.d_part.p);
+    if (g.h_pin.p) (void)hipHostFree(g.h_pin.p);
+    g.d_stage = Buffer();
+    g.d_part = Buffer();
+    g.h_pin = Buffer();
+    (void)hipStreamDestroy(g.stream);
+    g.stream = nullptr;
+    g.inited = false;
+    g.device = -1;
+    g.tune_keys_per_wg = 0;
+    g.force_generic = 0;
+}
+
+void wr_hip_attn_set_log(wr_hip_log_fn fn, void* user)
+{
+    g.log_fn = fn;
+    g.log_user = user;
+}
+
+uint64_t wr_hip_attn_calls(void) { return g.calls.load(std::memory_order_relaxed); }
+
+const char* wr_hip_attn_device_name(void) { return g.name; }
+
+void wr_hip_attn_set_tuning(uint32_t decode_keys_per_wg, int force_generic)
+{
+    std::lock_guard<std::mutex> lk(g.mu);
+    g.tune_keys_per_wg = decode_keys_per_wg;
+    g.force_generic = force_generic;
+}
+
+// ---------------------------------------------------------------- storage --
+
+int wr_hip_attn_kv_create(uint32_t n_layers, const uint32_t* hd_per_layer, uint32_t nkv,
+                          uint32_t max_ctx, wr_hip_kv** out)
+{
+    if (!out) return WR_HIP_ERR_INVAL;
+    *out = nullptr;
+    if (!g.inited) return WR_HIP_ERR_STATE;
+    if (!hd_per_layer || n_layers == 0 || nkv == 0 || max_ctx == 0) return WR_HIP_ERR_INVAL;
+    if (n_layers > WR_HIP_MAX_LAYERS) return WR_HIP_ERR_LIMIT;
+    if (max_ctx > WR_HIP_ATTN_MAX_SEQ) return WR_HIP_ERR_LIMIT;
+    for (uint32_t L = 0; L < n_layers; L++)
+        if (hd_per_layer[L] > WR_HIP_FLASH_D_MAX) return WR_HIP_ERR_LIMIT;
+
+    wr_hip_kv* kv = new (std::nothrow) wr_hip_kv();
+    if (!kv) return WR_HIP_ERR_NOMEM;
+    kv->n_layers = n_layers;
+    kv->nkv = nkv;
+    kv->max_ctx = max_ctx;
+    kv->ctx_pad = (max_ctx + kVBlock - 1) / kVBlock * kVBlock;
+    size_t cur = 0;
+    bool any = false;
+    for (uint32_t L = 0; L < n_layers; L++) {
+        kv->hd[L] = hd_per_layer[L];
+        if (kv->hd[L] == 0) continue;
+        any = true;
+        const size_t side = ((size_t)nkv * kv->ctx_pad * kv->hd[L] * 2 + 255) & ~(size_t)255;
+        kv->k_off[L] = cur;
+        cur += side;
+        kv->vt_off[L] = cur;
+        cur += side;
+    }
+    if (!any) {
+        delete kv;
+        return WR_HIP_ERR_INVAL;
+    }
+    kv->bytes = cur;
+
+    Locked lk;
+    hipError_t e = hipMalloc((void**)&kv->slab, cur);
+    if (e != hipSuccess) {
+        logmsg(0, "session: device slab alloc failed (%zu bytes): %s", cur, hipGetErrorString(e));
+        delete kv;
+        return WR_HIP_ERR_NOMEM;
+    }
+    e = hipMemsetAsync(kv->slab, 0, cur, g.stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(g.stream);
+    if (e != hipSuccess) {
+        (void)hipFree(kv->slab);
+        delete kv;
+        return hip_fail(e, "slab clear", 0);
+    }
+    *out = kv;
+    return WR_HIP_OK;
+}
+
+void wr_hip_attn_kv_destroy(wr_hip_kv* kv)
+{
+    if (!kv) return;
+    if (g.inited) {
+        Locked lk;
+        (void)hipStreamSynchronize(g.stream);
+        if (kv->slab) (void)hipFree(kv->slab);
+    }
+    delete kv;
+}
+
+uint64_t wr_hip_attn_kv_bytes(const wr_hip_kv* kv) { return kv ? kv->bytes : 0; }
+
+// ----------------------------------------------------------------- append --
+
+int wr_hip_attn_append_dev(wr_hip_kv* kv, uint32_t layer, uint32_t pos, uint32_t n_rows,
+                           const float* k_f32_dev, const float* v_f32_dev)
+{
+    int rc = check_append(kv, layer, pos, n_rows, k_f32_dev, v_f32_dev);
+    if (rc || n_rows == 0) return rc;
+    Locked lk;
+    return append_rows_locked<float>(kv, layer, pos, n_rows, k_f32_dev, v_f32_dev);
+}
+
+int wr_hip_attn_append(wr_hip_kv* kv, uint32_t layer, uint32_t pos, uint32_t n_rows,
+                       const float* k_f32, const float* v_f32)
+{
+    int rc = check_append(kv, layer, pos, n_rows, k_f32, v_f32);
+    if (rc || n_rows == 0) return rc;
+    const size_t bytes = (size_t)n_rows * kv->nkv * kv->hd[layer] * sizeof(float);
+    Locked lk;
+    rc = ensure_device(g.d_stage, 2 * bytes);
+    if (rc) return rc;
+    float* dk = reinterpret_cast<float*>(g.d_stage.p);
+    float* dv = reinterpret_cast<float*>((uint8_t*)g.d_stage.p + bytes);
+    rc = copy_up(dk, k_f32, bytes, 0);
+    if (rc == WR_HIP_OK) rc = copy_up(dv, v_f32, bytes, bytes);
+    if (rc == WR_HIP_OK) rc = append_rows_locked<float>(kv, layer, pos, n_rows, dk, dv);
+    // the staging buffers are reused by the next call: wait for the kernels
+    if (rc == WR_HIP_OK) HIP_TRY(hipStreamSynchronize(g.stream), "append sync", layer);
+    return rc;
+}
+
+int wr_hip_attn_kv_write(wr_hip_kv* kv, uint32_t layer, uint32_t pos, uint32_t n_rows,
+                         const uint16_t* k_f16, const uint16_t* v_f16)
+{
+    int rc = check_append(kv, layer, pos, n_rows, k_f16, v_f16);
+    if (rc || n_rows == 0) return rc;
+    const size_t bytes = (size_t)n_rows * kv->nkv * kv->hd[layer] * sizeof(uint16_t);
+    Locked lk;
+    rc = ensure_device(g.d_stage, 2 * bytes);
+    if (rc) return rc;
+    uint16_t* dk = reinterpret_cast<uint16_t*>(g.d_stage.p);
+    uint16_t* dv = reinterpret_cast<uint16_t*>((uint8_t*)g.d_stage.p + bytes);
+    rc = copy_up(dk, k_f16, bytes, 0);
+    if (rc == WR_HIP_OK) rc = copy_up(dv, v_f16, bytes, bytes);
+    if (rc == WR_HIP_OK) rc = append_rows_locked<uint16_t>(kv, layer, pos, n_rows, dk, dv);
+    if (rc == WR_HIP_OK) HIP_TRY(hipStreamSynchronize(g.stream), "kv_write sync", layer);
+    return rc;
+}
+
+int wr_hip_attn_kv_read(wr_hip_kv* kv, uint32_t layer, uint32_t pos, uint32_t n_rows,
+                        uint16_t* k_f16, uint16_t* v_f16)
+{
+    if (!g.inited) return WR_HIP_ERR_STATE;
+    int rc = check_layer(kv, layer);
+    if (rc) return rc;
+    if (n_rows == 0) return WR_HIP_OK;
+    if (!k_f16 || !v_f16) return WR_HIP_ERR_INVAL;
+    if ((uint64_t)pos + n_rows > kv->max_ctx) return WR_HIP_ERR_INVAL;
+    const uint32_t hd = kv->hd[layer], nkv = kv->nkv;
+    const size_t total = (size_t)n_rows * nkv * hd;
+    const size_t bytes = total * sizeof(uint16_t);
+    Locked lk;
+    rc = ensure_device(g.d_stage, 2 * bytes);
+    if (rc) return rc;
+    uint16_t* dk = reinterpret_cast<uint16_t*>(g.d_stage.p);
+    uint16_t* dv = reinterpret_cast<uint16_t*>((uint8_t*)g.d_stage.p + bytes);
+    hipLaunchKernelGGL(export_kv_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0,
+                       g.stream,
+                       reinterpret_cast<const uint16_t*>(kv->slab + kv->k_off[layer]),
+                       reinterpret_cast<const uint16_t*>(kv->slab + kv->vt_off[layer]), dk, dv, pos,
+                       n_rows, nkv, hd, kv->ctx_pad);
+    HIP_TRY(hipGetLastError(), "export launch", layer);
+    rc = copy_down_sync(k_f16, dk, bytes);
+    if (rc == WR_HIP_OK) rc = copy_down_sync(v_f16, dv, bytes);
+    return rc;
+}
+
+// ----------------------------------------------------------------- decode --
+
+int wr_hip_attn_decode_batched_dev(uint32_t n, wr_hip_kv* const* kv, uint32_t layer,
+                                   const uint32_t* seq_k, const float* q_dev, float* out_dev,
+                                   uint32_t nq, float scale_override, uint32_t window)
+{
+    int rc = check_decode(n, kv, layer, seq_k, q_dev, out_dev, nq);
+    if (rc) return rc;
+    Locked lk;
+    return decode_locked(n, kv, layer, seq_k, q_dev, out_dev, nq, scale_override, window);
+}
+
+int wr_hip_attn_decode_batched(uint32_t n, wr_hip_kv* const* kv, uint32_t layer,
+                               const uint32_t* seq_k, const float* const* q, float* const* out,
+                               uint32_t nq, float scale_override, uint32_t window)
+{
+    int rc = check_decode(n, kv, layer, seq_k, q, out, nq);
+    if (rc) return rc;
+    for (uint32_t i = 0; i < n; i++)
+        if (!q[i] || !out[i]) return WR_HIP_ERR_INVAL;
+    const size_t row = (size_t)nq * kv[0]->hd[layer] * sizeof(float);
+    Locked lk;
+    rc = ensure_device(g.d_stage, 2 * n * row);
+    if (rc) return rc;
+    rc = ensure_pinned(g.h_pin, n * row);
+    if (rc) return rc;
+    float* dq = reinterpret_cast<float*>(g.d_stage.p);
+    float* dout = reinterpret_cast<float*>((uint8_t*)g.d_stage.p + n * row);
+    for (uint32_t i = 0; i < n; i++) memcpy((uint8_t*)g.h_pin.p + i * row, q[i], row);
+    HIP_TRY(hipMemcpyAsync(dq, g.h_pin.p, n * row, hipMemcpyHostToDevice, g.stream), "q h2d",
+            layer);
+    rc = decode_locked(n, kv, layer, seq_k, dq, dout, nq, scale_override, window);
+    if (rc) return rc;
+    HIP_TRY(hipMemcpyAsync(g.h_pin.p, dout, n * row, hipMemcpyDeviceToHost, g.stream), "out d2h",
+            layer);
+    HIP_TRY(hipStreamSynchronize(g.stream), "decode sync", layer);
+    for (uint32_t i = 0; i < n; i++) memcpy(out[i], (uint8_t*)g.h_pin.p + i * row, row);
+    return WR_HIP_OK;
+}
+
+int wr_hip_attn_decode(wr_hip_kv* kv, uint32_t layer, uint32_t seq_k, const float* q, float* out,
+                       uint32_t nq, float scale_override, uint32_t window)
+{
+    wr_hip_kv* kvs[1] = {kv};
+    const float* qs[1] = {q};
+    float* outs[1] = {out};
+    if (!kv || !q || !out) return g.inited ? WR_HIP_ERR_INVAL : WR_HIP_ERR_STATE;
+    return wr_hip_attn_decode_batched(1, kvs, layer, &seq_k, qs, outs, nq, scale_override, window);
+}
+
+// ---------------------------------------------------------------- prefill --
+
+int wr_hip_attn_prefill_dev(wr_hip_kv* kv, uint32_t layer, uint32_t p0, uint32_t T,
+                            const float* q_dev, float* out_dev, uint32_t nq, float scale_override,
+                            uint32_t window)
+{
+    int rc = check_prefill(kv, layer, p0, T, q_dev, out_dev, nq);
+    if (rc) return rc;
+    Locked lk;
+    return prefill_locked(kv, layer, p0, T, q_dev, out_dev, nq, scale_override, window);
+}
+
+int wr_hip_attn_prefill(wr_hip_kv* kv, uint32_t layer, uint32_t p0, uint32_t T, const float* q,
+                        float* out, uint32_t nq, float scale_override, uint32_t window)
+{
+    int rc = check_prefill(kv, layer, p0, T, q, out, nq);
+    if (rc) return rc;
+    const size_t bytes = (size_t)T * nq * kv->hd[layer] * sizeof(float);
+    Locked lk;
+    rc = ensure_device(g.d_stage, 2 * bytes);
+    if (rc) return rc;
+    float* dq = reinterpret_cast<float*>(g.d_stage.p);
+    float* dout = reinterpret_cast<float*>((uint8_t*)g.d_stage.p + bytes);
+    rc = copy_up(dq, q, bytes, 0);
+    if (rc == WR_HIP_OK)
+        rc = prefill_locked(kv, layer, p0, T, dq, dout, nq, scale_override, window);
+    if (rc == WR_HIP_OK) rc = copy_down_sync(out, dout, bytes);
+    return rc;
+}
+
+// ------------------------------------------------------- device utilities --
+
+void* wr_hip_attn_dev_alloc(size_t bytes)
+{
+    if (!g.inited || bytes == 0) return nullptr;
+    Locked lk;
+    void* p = nullptr;
+    if (hipMalloc(&p, bytes) != hipSuccess) return nullptr;
+    return p;
+}
+
+void wr_hip_attn_dev_free(void* p)
+{
+    if (!g.inited || !p) return;
+    Locked lk;
+    (void)hipStreamSynchronize(g.stream);
+    (void)hipFree(p);
+}
+
+int wr_hip_attn_h2d(void* dst_dev, const void* src_host, size_t bytes)
+{
+    if (!g.inited) return WR_HIP_ERR_STATE;
+    if (!dst_dev || !src_host) return WR_HIP_ERR_INVAL;
+    Locked lk;
+    HIP_TRY(hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, g.stream), "h2d", 0);
+    HIP_TRY(hipStreamSynchronize(g.stream), "h2d sync", 0);
+    return WR_HIP_OK;
+}
+
+int wr_hip_attn_d2h(void* dst_host, const void* src_dev, size_t bytes)
+{
+    if (!g.inited) return WR_HIP_ERR_STATE;
+    if (!dst_host || !src_dev) return WR_HIP_ERR_INVAL;
+    Locked lk;
+    HIP_TRY(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, g.stream), "d2h", 0);
+    HIP_TRY(hipStreamSynchronize(g.stream), "d2h sync", 0);
+    return WR_HIP_OK;
+}
+
+int wr_hip_attn_sync(void)
+{
+    if (!g.inited) return WR_HIP_ERR_STATE;
+    Locked lk;
+    HIP_TRY(hipStreamSynchronize(g.stream), "sync", 0);
+    return WR_HIP_OK;
+}
+
+void* wr_hip_attn_stream(void) { return g.inited ? (void*)g.stream : nullptr; }
+
+int wr_hip_attn_profile_begin(uint32_t max_launches)
+{
+    if (!g.inited) return WR_HIP_ERR_STATE;
+    Locked lk;
+    HIP_TRY(hipStreamSynchronize(g.stream), "sync", 0);
+    while (g.ev.size() < 2 * (size_t)max_launches) {
+        hipEvent_t e;
+        HIP_TRY(hipEventCreate(&e), "event create", 0);
+        g.ev.push_back(e);
+    }
+    g.ev_used = 0;
+    g.profiling = true;
+    return WR_HIP_OK;
+}
+
+int wr_hip_attn_profile_end(double* total_ms, uint32_t* n_launches)
+{
+    if (!g.inited) return WR_HIP_ERR_STATE;
+    Locked lk;
+    HIP_TRY(hipStreamSynchronize(g.stream), "sync", 0);
+    double sum = 0.0;
+    for (uint32_t i = 0; i + 1 < g.ev_used; i += 2) {
+        float ms = 0.f;
+        HIP_TRY(hipEventElapsedTime(&ms, g.ev[i], g.ev[i + 1]), "event elapsed", 0);
+        sum += ms;
+    }
+    if (total_ms) *total_ms = sum;
+    if (n_launches) *n_launches = g.ev_used / 2;
+    g.profiling = false;
+    g.ev_used = 0;
+    return WR_HIP_OK;
+}
+
+}  // extern "C"
