@@ -41,9 +41,16 @@ ATTN_CASES = [
 
 def attn_inputs(case):
     """(q float32 [seq_q,nq,hd], k, v [rows,nkv,hd] uint16 or float32)."""
-    name, seq_q, nq, nkv, hd, rows, _seq_k, _sc, _win, kvdt = case
+    name, seq_q, nq, nkv, hd, rows, _seq_k, sc, _win, kvdt = case
     base = (sum(ord(c) * (i + 1) for i, c in enumerate(name)) * 2654435761) & 0xFFFFFFFF
     q = synth.hash_bell(base + 1, (seq_q, nq, hd))
+    if sc >= 1.0:
+        # An explicit scale of 1.0 on unit-variance inputs spreads the scores
+        # over more than 88 nats.  The reference's polynomial exp returns ~1
+        # instead of ~0 for arguments in [-88, -87.68] (src/core/mathx.c:50 skips
+        # the exponent add when k = -127), so such inputs test that defect, not
+        # attention.  Shrink q (exact power of two) to keep scores in range.
+        q = q * np.float32(0.125)
     k = synth.hash_bell(base + 2, (rows, nkv, hd))
     v = synth.hash_bell(base + 3, (rows, nkv, hd))
     if kvdt == "f16":

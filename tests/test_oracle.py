@@ -86,6 +86,19 @@ def test_scalar_math_close_to_libm():
     assert oracle.lib().wro_exp(-88.5) == 0.0 and oracle.lib().wro_exp(88.5) == np.float32(1e38)
 
 
+def test_reference_exp_defect_band_is_restated():
+    # src/core/mathx.c:43-55: for x in [-88, -87.68] the split gives k = -127,
+    # the exponent add is skipped and the bare polynomial (~1.03 .. 1.41) comes
+    # back instead of ~1e-38.  The oracle restates it (it is bit-compared with
+    # the compiled reference above); the device kernels do NOT imitate it, so
+    # parity inputs keep score spreads below 87 nats.
+    lib = oracle.lib()
+    assert 1.0 < lib.wro_exp(-87.9) < 1.5
+    assert 1.0 < lib.wro_exp(-87.7) < 1.5
+    assert lib.wro_exp(-87.6) < 1e-37
+    assert lib.wro_exp(-88.01) == 0.0
+
+
 def test_f16_codecs_vs_fixture_and_ieee():
     g = _npz("f16_golden.npz")
     bits = cases.f16_encode_bits()
