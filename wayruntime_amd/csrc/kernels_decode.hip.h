@@ -11,9 +11,12 @@
 // owns ONE KV head of one session over a contiguous run of 32-key tiles and
 // serves the whole GQA group from it, so every K and V byte is fetched from
 // HBM exactly once.  Its four waves take tiles round-robin and keep private
-// online-softmax state (m, l, O); they merge through LDS at the end and the
-// workgroup writes either the final rows (single split) or one partial
-// (m, l, unnormalised O) per head that decode_combine_kernel merges.
+// online-softmax state (m, l, O); they merge through LDS at the end.  A
+// session with one split gets its final rows written directly; otherwise the
+// workgroup publishes a partial (m, l, unnormalised O) per head, takes a
+// ticket from a per-(session, KV head) counter, and the workgroup that draws
+// the last ticket merges all partials and writes the rows.  One launch, no
+// second pass.
 //
 // HBM-bound: algorithmic bytes per launch = 4 * nkv * hd * sum(seq_k)
 // (K and V, two bytes each); Q, O and partials are <1 %.
@@ -21,16 +24,19 @@
 // Inside a wave the two contractions run on the matrix cores only to take the
 // arithmetic off the vector ALUs (a 4-head group would otherwise need ~100
 // VALU ops per 32 bytes loaded, which caps bandwidth).  Accuracy is kept at
-// F32 level by splitting the F32 operands into two halves-precision terms:
-// q = q_hi + q_lo and p = p_hi + p_lo, each term a separate MFMA into the same
-// F32 accumulator.  K and V are already F16, so nothing is lost there.
+// F32 level by splitting each F32 operand into two half-precision terms,
+// x = x_hi + x_lo, and giving the two terms their own COLUMNS of the same
+// MFMA: column h carries the hi term of head h, column h + G the lo term.
+// The two columns are added after the first contraction (scores) and at the
+// very end of the second (outputs).  K and V are already F16, nothing is lost
+// there.
 //
-//   S^T[key][head] = K[key][:] . Q^T[:][head]      v_mfma_f32_16x16x32_f16
-//   O^T[dim][head] += Vt[dim][key] . P^T[key][head]
+//   S^T[key][col] = K[key][:] . Q^T[:][col]        v_mfma_f32_16x16x32_f16
+//   O^T[dim][col] += Vt[dim][key] . P^T[key][col]
 //
-// Orientation is chosen so a head is a COLUMN: lane l owns column l%16 in
-// both accumulators, so max / sum / rescale of one head never leave the lane
-// except for one exchange across the four 16-lane groups.
+// A head is a COLUMN: lane l owns column l%16 in both accumulators, so max,
+// sum and rescale of one head stay inside the lane except for one exchange
+// across the four 16-lane groups and one with the partner column.
 #pragma once
 
 #include "common.hip.h"
@@ -40,8 +46,9 @@ namespace wr {
 constexpr int kDecodeThreads = 256;
 constexpr int kDecodeWaves = 4;
 constexpr int kTileKeys = 32;
-constexpr int kMaxGroupMfma = 8;      // heads per KV head the MFMA kernel serves
+constexpr int kMaxGroupMfma = 8;      // heads per KV head the MFMA kernel serves (2G <= 16 columns)
 constexpr int kBatchMax = 16;
+constexpr int kFlashDMax = 1024;      // largest head_dim (reference: WR_FLASH_D_MAX)
 
 struct DecodeSession {
     const uint16_t* k;       // K of this layer
@@ -58,10 +65,10 @@ struct DecodeArgs {
     float* out;              // [n][nq][hd]
     float* part_o;           // [n][nq][max_splits][hd], unnormalised
     float* part_ml;          // [n][nq][max_splits][2] = (m in log2 units, l)
+    uint32_t* counters;      // tickets, zero between launches: [n][nkv] (MFMA) or [n][nq] (generic)
     uint32_t nq, nkv, group, hd;
     uint32_t tiles_per_wg;   // 32-key tiles per workgroup
     uint32_t max_splits;
-    uint32_t direct;         // 1: every session has one split, write final rows
     float qscale;            // softmax scale * log2(e)
 };
 
@@ -80,6 +87,98 @@ __device__ __forceinline__ TileRange split_tiles(const DecodeSession& S, uint32_
     return r;
 }
 
+// Called by every thread of a workgroup after it has stored its partial rows
+// for heads [head0, head0 + nh) of `sess` at its split index.  The workgroup
+// that draws the last of the n_splits tickets merges the partials of those
+// heads (log-sum-exp over the split maxima, one normalisation), writes the
+// final rows and puts the counter back to zero for the next launch.
+constexpr int kMaxSplits = 64;        // key splits per session (host picks tiles_per_wg to respect it)
+
+// Partial rows cross workgroups (and XCDs, each with its own L2) inside one
+// launch.  They are written and read with agent-scope relaxed atomics: on
+// gfx950 those are write-through stores / L2-coherent loads (sc1), so the data
+// itself never sits dirty in one XCD's L2.  Ordering against the ticket comes
+// from waiting for the stores to be acknowledged (workgroup-scope release =
+// s_waitcnt vmcnt(0)) and a workgroup barrier before one thread takes the
+// ticket.  A device-wide release fence instead would write back the whole L2
+// (buffer_wbl2) from every workgroup: measured at 5-10x the kernel's run time.
+__device__ __forceinline__ float part_load(const float* p)
+{
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void part_store(float* p, float v)
+{
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Called by every thread of a workgroup after it has stored its partial rows
+// for heads [head0, head0 + nh) of `sess` at its split index.  The workgroup
+// that draws the last of the n_splits tickets merges the partials of those
+// heads (log-sum-exp over the split maxima, one normalisation), writes the
+// final rows and puts the counter back to zero for the next launch.
+// `scratch` is LDS the caller no longer needs: 3 * nh * kMaxSplits floats.
+__device__ __forceinline__ void publish_and_merge(const DecodeArgs& a, uint32_t sess,
+                                                  uint32_t head0, uint32_t nh, uint32_t n_splits,
+                                                  uint32_t counter_idx, float* scratch)
+{
+    __shared__ uint32_t s_ticket;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");   // own partial stores acknowledged
+    __syncthreads();
+    if (threadIdx.x == 0)
+        s_ticket = __hip_atomic_fetch_add(&a.counters[counter_idx], 1u, __ATOMIC_RELAXED,
+                                          __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (s_ticket != n_splits - 1) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+
+    float* s_m = scratch;                       // [nh][kMaxSplits]
+    float* s_l = scratch + nh * kMaxSplits;
+    float* s_w = scratch + 2 * nh * kMaxSplits;
+    for (uint32_t idx = threadIdx.x; idx < nh * n_splits; idx += blockDim.x) {
+        const uint32_t h = idx / n_splits, i = idx % n_splits;
+        const size_t pi = ((size_t)sess * a.nq + head0 + h) * a.max_splits + i;
+        s_m[h * kMaxSplits + i] = part_load(&a.part_ml[pi * 2]);
+        s_l[h * kMaxSplits + i] = part_load(&a.part_ml[pi * 2 + 1]);
+    }
+    __syncthreads();
+    if (threadIdx.x < nh) {
+        const uint32_t h = threadIdx.x;
+        float M = -INFINITY;
+        for (uint32_t i = 0; i < n_splits; i++) M = fmaxf(M, s_m[h * kMaxSplits + i]);
+        float L = 0.f;
+        for (uint32_t i = 0; i < n_splits; i++) {
+            const float f = fast_exp2(s_m[h * kMaxSplits + i] - M);
+            s_w[h * kMaxSplits + i] = f;
+            L += s_l[h * kMaxSplits + i] * f;
+        }
+        const float inv = (L > 0.f) ? 1.0f / L : 0.f;
+        for (uint32_t i = 0; i < n_splits; i++) s_w[h * kMaxSplits + i] *= inv;
+    }
+    __syncthreads();
+
+    const uint32_t hd = a.hd;
+    for (uint32_t idx = threadIdx.x; idx < nh * hd; idx += blockDim.x) {
+        const uint32_t h = idx / hd, d = idx % hd;
+        const float* po = a.part_o + (((size_t)sess * a.nq + head0 + h) * a.max_splits) * hd + d;
+        const float* w = s_w + h * kMaxSplits;
+        float acc0 = 0.f, acc1 = 0.f, acc2 = 0.f, acc3 = 0.f;
+        uint32_t i = 0;
+        for (; i + 4 <= n_splits; i += 4) {
+            const float v0 = part_load(po + (size_t)(i + 0) * hd);
+            const float v1 = part_load(po + (size_t)(i + 1) * hd);
+            const float v2 = part_load(po + (size_t)(i + 2) * hd);
+            const float v3 = part_load(po + (size_t)(i + 3) * hd);
+            acc0 += v0 * w[i + 0];
+            acc1 += v1 * w[i + 1];
+            acc2 += v2 * w[i + 2];
+            acc3 += v3 * w[i + 3];
+        }
+        for (; i < n_splits; i++) acc0 += part_load(po + (size_t)i * hd) * w[i];
+        a.out[((size_t)sess * a.nq + head0 + h) * hd + d] = (acc0 + acc1) + (acc2 + acc3);
+    }
+    if (threadIdx.x == 0) a.counters[counter_idx] = 0;
+}
+
 // ------------------------------------------------------------------ MFMA --
 
 template <int HD>
@@ -87,6 +186,10 @@ struct DecodeFrag {
     half8 k[2][HD / 32];     // two 16-key sub-tiles x (HD/32) contraction steps
     half8 v[HD / 16];        // HD/16 dimension tiles x 32 keys
 };
+
+// The cache is read exactly once per launch: non-temporal loads keep it from
+// displacing anything useful in the caches.
+__device__ __forceinline__ half8 stream_load(const half8* p) { return __builtin_nontemporal_load(p); }
 
 template <int HD>
 __device__ __forceinline__ void load_frag(DecodeFrag<HD>& f, const uint16_t* __restrict__ kbase,
@@ -103,25 +206,26 @@ __device__ __forceinline__ void load_frag(DecodeFrag<HD>& f, const uint16_t* __r
         const uint32_t key = kb + 8 * (m >> 2) + 4 * t + (m & 3);
         const half8* row = reinterpret_cast<const half8*>(kbase + (size_t)key * HD);
 #pragma unroll
-        for (int s = 0; s < HD / 32; s++) f.k[t][s] = row[s * 4 + g];
+        for (int s = 0; s < HD / 32; s++) f.k[t][s] = stream_load(&row[s * 4 + g]);
     }
     const half8* vb = reinterpret_cast<const half8*>(vtbase + (size_t)tile * HD * kVBlock);
 #pragma unroll
-    for (int dt = 0; dt < HD / 16; dt++) f.v[dt] = vb[(dt * 16 + m) * 4 + g];
+    for (int dt = 0; dt < HD / 16; dt++) f.v[dt] = stream_load(&vb[(dt * 16 + m) * 4 + g]);
 }
 
 template <int HD>
 struct DecodeState {
-    f32x4 o[HD / 16];        // O^T: dim = dt*16 + 4g + r, head = lane%16
+    f32x4 o[HD / 16];        // O^T: dim = dt*16 + 4g + r, column = lane%16
     float m;                 // running max (log2 units), common to the 4 groups
     float l;                 // this lane group's share of the denominator
 };
 
+// col_kind: 0 = hi column of a head, 1 = lo column, 2 = unused column.
 template <int HD>
 __device__ __forceinline__ void process_tile(DecodeState<HD>& st, DecodeFrag<HD>& f,
-                                             const half8 (&qhi)[HD / 32],
-                                             const half8 (&qlo)[HD / 32], uint32_t tile,
-                                             uint32_t key_lo, uint32_t seq_k, int lane)
+                                             const half8 (&qop)[HD / 32], uint32_t tile,
+                                             uint32_t key_lo, uint32_t seq_k, int lane,
+                                             int partner_addr, int col_kind)
 {
     const int g = lane >> 4;
     const uint32_t kb = tile * kTileKeys;
@@ -131,14 +235,18 @@ __device__ __forceinline__ void process_tile(DecodeState<HD>& st, DecodeFrag<HD>
     for (int t = 0; t < 2; t++) {
         c[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int s = 0; s < HD / 32; s++) {
-            c[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(f.k[t][s], qhi[s], c[t], 0, 0, 0);
-            c[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(f.k[t][s], qlo[s], c[t], 0, 0, 0);
-        }
+        for (int s = 0; s < HD / 32; s++)
+            c[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(f.k[t][s], qop[s], c[t], 0, 0, 0);
     }
+    // score = hi column + lo column; both columns of a head end up with the sum
     float sc[8];
 #pragma unroll
-    for (int j = 0; j < 8; j++) sc[j] = c[j >> 2][j & 3];
+    for (int j = 0; j < 8; j++) {
+        const float own = c[j >> 2][j & 3];
+        const float other = __int_as_float(
+            __builtin_amdgcn_ds_bpermute(partner_addr, __float_as_int(own)));
+        sc[j] = (col_kind == 2) ? own : own + other;
+    }
 
     const bool boundary = (kb < key_lo) || (kb + kTileKeys > seq_k);
     if (boundary) {
@@ -170,23 +278,22 @@ __device__ __forceinline__ void process_tile(DecodeState<HD>& st, DecodeFrag<HD>
     const float alpha = fast_exp2(st.m - m_new);
     st.m = m_new;
 
-    half8 phi, plo;
+    half8 pop;
     float psum = 0.f;
 #pragma unroll
     for (int j = 0; j < 8; j++) {
         const float p = fast_exp2(sc[j] - m_new);
         psum += p;
         const _Float16 h = (_Float16)p;
-        phi[j] = h;
-        plo[j] = (_Float16)(p - (float)h);
+        const _Float16 lo = (_Float16)(p - (float)h);
+        pop[j] = (col_kind == 0) ? h : ((col_kind == 1) ? lo : (_Float16)0.0f);
     }
     st.l = st.l * alpha + psum;
 
 #pragma unroll
     for (int dt = 0; dt < HD / 16; dt++) {
         st.o[dt] *= alpha;
-        st.o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(f.v[dt], phi, st.o[dt], 0, 0, 0);
-        st.o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(f.v[dt], plo, st.o[dt], 0, 0, 0);
+        st.o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(f.v[dt], pop, st.o[dt], 0, 0, 0);
     }
 }
 
@@ -206,25 +313,34 @@ void decode_mfma_kernel(const DecodeArgs a)
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n = lane & 15, g = lane >> 4;
-    const uint32_t G = a.group;
+    const int G = (int)a.group;
     const TileRange tr = split_tiles(S, split, a.tiles_per_wg);
 
-    // Q^T operand: column n is head kvh*G + n (zero beyond the group), scaled
-    // into log2 units and split into two half-precision terms.
-    half8 qhi[HD / 32], qlo[HD / 32];
+    // Q^T operand through LDS: row c of lds_q is MFMA column c.  Columns
+    // 0..G-1 hold the hi terms of the group's heads, G..2G-1 the lo terms,
+    // the rest zero; values are pre-multiplied by scale*log2(e).
+    __shared__ __attribute__((aligned(16))) _Float16 lds_q[16][HD + 8];
     {
-        const float* qrow = a.q + ((size_t)sess * a.nq + kvh * G + (n < (int)G ? n : 0)) * HD;
-#pragma unroll
-        for (int s = 0; s < HD / 32; s++) {
-#pragma unroll
-            for (int j = 0; j < 8; j++) {
-                float x = (n < (int)G) ? qrow[s * 32 + g * 8 + j] * a.qscale : 0.f;
-                const _Float16 h = (_Float16)x;
-                qhi[s][j] = h;
-                qlo[s][j] = (_Float16)(x - (float)h);
-            }
+        const float* qg = a.q + ((size_t)sess * a.nq + kvh * G) * HD;     // G contiguous rows
+        for (int idx = threadIdx.x; idx < G * HD; idx += kDecodeThreads) {
+            const int h = idx / HD, d = idx % HD;
+            const float x = qg[idx] * a.qscale;
+            const _Float16 hi = (_Float16)x;
+            lds_q[h][d] = hi;
+            lds_q[h + G][d] = (_Float16)(x - (float)hi);
         }
+        for (int idx = threadIdx.x; idx < (16 - 2 * G) * HD; idx += kDecodeThreads)
+            lds_q[2 * G + idx / HD][idx % HD] = (_Float16)0.0f;
     }
+    __syncthreads();
+    half8 qop[HD / 32];
+#pragma unroll
+    for (int s = 0; s < HD / 32; s++)
+        qop[s] = *reinterpret_cast<const half8*>(&lds_q[n][s * 32 + g * 8]);
+
+    const int col_kind = (n < G) ? 0 : ((n < 2 * G) ? 1 : 2);
+    const int partner = (n < G) ? lane + G : ((n < 2 * G) ? lane - G : lane);
+    const int partner_addr = partner * 4;
 
     DecodeState<HD> st;
 #pragma unroll
@@ -242,11 +358,11 @@ void decode_mfma_kernel(const DecodeArgs a)
         for (;;) {
             const uint32_t t1 = t + kDecodeWaves;
             if (t1 < tr.t_end) load_frag<HD>(fb, kbase, vtbase, t1, lane);
-            process_tile<HD>(st, fa, qhi, qlo, t, S.key_lo, S.seq_k, lane);
+            process_tile<HD>(st, fa, qop, t, S.key_lo, S.seq_k, lane, partner_addr, col_kind);
             if (t1 >= tr.t_end) break;
             const uint32_t t2 = t1 + kDecodeWaves;
             if (t2 < tr.t_end) load_frag<HD>(fa, kbase, vtbase, t2, lane);
-            process_tile<HD>(st, fb, qhi, qlo, t1, S.key_lo, S.seq_k, lane);
+            process_tile<HD>(st, fb, qop, t1, S.key_lo, S.seq_k, lane, partner_addr, col_kind);
             if (t2 >= tr.t_end) break;
             t = t2;
         }
@@ -254,11 +370,18 @@ void decode_mfma_kernel(const DecodeArgs a)
     // denominator: add the four lane groups' shares
     st.l += wave_xor_f32(st.l, 16);
     st.l += wave_xor_f32(st.l, 32);
+    // outputs: hi column + lo column
+#pragma unroll
+    for (int dt = 0; dt < HD / 16; dt++)
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+            st.o[dt][r] += __int_as_float(
+                __builtin_amdgcn_ds_bpermute(partner_addr, __float_as_int(st.o[dt][r])));
 
     __shared__ float lds_o[kDecodeWaves][kMaxGroupMfma][HD];
     __shared__ float lds_m[kDecodeWaves][kMaxGroupMfma];
     __shared__ float lds_l[kDecodeWaves][kMaxGroupMfma];
-    if (n < (int)G) {
+    if (n < G) {
 #pragma unroll
         for (int dt = 0; dt < HD / 16; dt++)
 #pragma unroll
@@ -270,7 +393,8 @@ void decode_mfma_kernel(const DecodeArgs a)
     }
     __syncthreads();
 
-    for (uint32_t idx = threadIdx.x; idx < G * HD; idx += kDecodeThreads) {
+    const bool direct = (S.n_splits == 1);
+    for (uint32_t idx = threadIdx.x; idx < (uint32_t)G * HD; idx += kDecodeThreads) {
         const uint32_t h = idx / HD, d = idx % HD;
         float M = lds_m[0][h];
 #pragma unroll
@@ -283,16 +407,20 @@ void decode_mfma_kernel(const DecodeArgs a)
             L += lds_l[w][h] * fct;
         }
         const uint32_t head = kvh * G + h;
-        if (a.direct) {
+        if (direct) {
             a.out[((size_t)sess * a.nq + head) * HD + d] = (L > 0.f) ? acc / L : 0.f;
         } else {
             const size_t pi = ((size_t)sess * a.nq + head) * a.max_splits + split;
-            a.part_o[pi * HD + d] = acc;
+            part_store(&a.part_o[pi * HD + d], acc);
             if (d == 0) {
-                a.part_ml[pi * 2 + 0] = M;
-                a.part_ml[pi * 2 + 1] = L;
+                part_store(&a.part_ml[pi * 2 + 0], M);
+                part_store(&a.part_ml[pi * 2 + 1], L);
             }
         }
+    }
+    if (!direct) {
+        __syncthreads();      // lds_o is reused as merge scratch
+        publish_and_merge(a, sess, kvh * G, G, S.n_splits, sess * a.nkv + kvh, &lds_o[0][0][0]);
     }
 }
 
@@ -303,7 +431,6 @@ void decode_mfma_kernel(const DecodeArgs a)
 // the MFMA kernel against.
 
 constexpr int kGenericMaxPerLane = 16;      // 1024 / 64
-constexpr int kFlashDMax = 1024;            // largest head_dim (reference: WR_FLASH_D_MAX)
 
 struct GenericShared {
     float o[kDecodeWaves][kFlashDMax];
@@ -403,46 +530,25 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_generic_kernel(const De
                       a.q + ((size_t)sess * a.nq + head) * hd, a.qscale);
     const GenericMerge g = merge_generic(sh);
 
+    const bool direct = (S.n_splits == 1);
     for (uint32_t d = threadIdx.x; d < hd; d += kDecodeThreads) {
         float acc = 0.f;
 #pragma unroll
         for (int w = 0; w < kDecodeWaves; w++) acc += sh.o[w][d] * g.fct[w];
-        if (a.direct) {
+        if (direct) {
             a.out[((size_t)sess * a.nq + head) * hd + d] = (g.L > 0.f) ? acc / g.L : 0.f;
         } else {
             const size_t pi = ((size_t)sess * a.nq + head) * a.max_splits + split;
-            a.part_o[pi * hd + d] = acc;
+            part_store(&a.part_o[pi * hd + d], acc);
             if (d == 0) {
-                a.part_ml[pi * 2 + 0] = g.M;
-                a.part_ml[pi * 2 + 1] = g.L;
+                part_store(&a.part_ml[pi * 2 + 0], g.M);
+                part_store(&a.part_ml[pi * 2 + 1], g.L);
             }
         }
     }
-}
-
-// --------------------------------------------------------------- combine --
-// Merges the per-split partials of one (session, head): log-sum-exp over the
-// split maxima, then one normalisation.  grid = (nq, sessions).
-
-__global__ __launch_bounds__(128) void decode_combine_kernel(const DecodeArgs a)
-{
-    const uint32_t head = blockIdx.x, sess = blockIdx.y;
-    const uint32_t ns = a.s[sess].n_splits;
-    const uint32_t hd = a.hd;
-    const size_t base = ((size_t)sess * a.nq + head) * a.max_splits;
-
-    float M = -INFINITY;
-    for (uint32_t i = 0; i < ns; i++) M = fmaxf(M, a.part_ml[(base + i) * 2]);
-    float L = 0.f;
-    for (uint32_t i = 0; i < ns; i++)
-        L += a.part_ml[(base + i) * 2 + 1] * fast_exp2(a.part_ml[(base + i) * 2] - M);
-    const float inv = (L > 0.f) ? 1.0f / L : 0.f;
-
-    for (uint32_t d = threadIdx.x; d < hd; d += blockDim.x) {
-        float acc = 0.f;
-        for (uint32_t i = 0; i < ns; i++)
-            acc += a.part_o[(base + i) * hd + d] * fast_exp2(a.part_ml[(base + i) * 2] - M);
-        a.out[((size_t)sess * a.nq + head) * hd + d] = acc * inv;
+    if (!direct) {
+        __syncthreads();      // sh.o is reused as merge scratch
+        publish_and_merge(a, sess, head, 1, S.n_splits, sess * a.nq + head, &sh.o[0][0]);
     }
 }
 

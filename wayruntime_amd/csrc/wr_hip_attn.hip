@@ -49,6 +49,7 @@ struct Lib {
     char name[320] = "uninitialised";
     Buffer d_stage;              // device staging for host-pointer entry points
     Buffer d_part;               // split-K partials
+    uint32_t* d_counters = nullptr;   // split-K tickets, zero whenever no launch is in flight
     Buffer h_pin;                // pinned host staging
     std::atomic<uint64_t> calls{0};
     wr_hip_log_fn log_fn = nullptr;
@@ -61,6 +62,8 @@ struct Lib {
 } g;
 
 constexpr float kLog2e = 1.4426950408889634f;
+constexpr uint32_t kTargetWorkgroups = 256;  // split-K decode: about one workgroup per CU
+constexpr uint32_t kMaxHeads = 4096;        // query heads per session the ticket array is sized for
 constexpr size_t kPinSmall = 1u << 20;      // host copies up to this size go through pinned staging
 
 void logmsg(int level, const char* fmt, ...)
@@ -238,15 +241,21 @@ int decode_locked(uint32_t n, wr_hip_kv* const* kv, uint32_t layer, const uint32
     // but at least one tile per wave so the per-workgroup merge stays small
     // next to the data it streams.
     uint32_t tiles_per_wg;
+    uint32_t tiles_max = 1;
+    for (uint32_t i = 0; i < n; i++)
+        if (tiles[i] > tiles_max) tiles_max = tiles[i];
     if (g.tune_keys_per_wg) {
         tiles_per_wg = g.tune_keys_per_wg / kTileKeys;
         if (tiles_per_wg == 0) tiles_per_wg = 1;
     } else {
         const uint64_t units = tiles_total * (use_mfma ? nkv : nq);
-        tiles_per_wg = (uint32_t)((units + 2047) / 2048);
+        tiles_per_wg = (uint32_t)((units + kTargetWorkgroups - 1) / kTargetWorkgroups);
         tiles_per_wg = (tiles_per_wg + 3) & ~3u;
         if (tiles_per_wg < 4) tiles_per_wg = 4;
     }
+    // the in-kernel merge handles at most kMaxSplits partials per head
+    const uint32_t floor_tiles = (tiles_max + kMaxSplits - 1) / kMaxSplits;
+    if (tiles_per_wg < floor_tiles) tiles_per_wg = floor_tiles;
     uint32_t max_splits = 1;
     for (uint32_t i = 0; i < n; i++) {
         a.s[i].n_splits = (tiles[i] + tiles_per_wg - 1) / tiles_per_wg;
@@ -260,11 +269,11 @@ int decode_locked(uint32_t n, wr_hip_kv* const* kv, uint32_t layer, const uint32
     a.hd = hd;
     a.tiles_per_wg = tiles_per_wg;
     a.max_splits = max_splits;
-    a.direct = (max_splits == 1) ? 1u : 0u;
+    a.counters = g.d_counters;
     const float scale = (scale_override > 0.0f) ? scale_override : 1.0f / sqrtf((float)hd);
     a.qscale = scale * kLog2e;
 
-    if (!a.direct) {
+    if (max_splits > 1) {
         const size_t po = (size_t)n * nq * max_splits * hd * sizeof(float);
         const size_t pml = (size_t)n * nq * max_splits * 2 * sizeof(float);
         int rc = ensure_device(g.d_part, po + pml);
@@ -284,8 +293,6 @@ int decode_locked(uint32_t n, wr_hip_kv* const* kv, uint32_t layer, const uint32
     } else {
         launch_main(decode_generic_kernel, dim3(max_splits, nq, n), dim3(kDecodeThreads), a);
     }
-    if (!a.direct)
-        hipLaunchKernelGGL(decode_combine_kernel, dim3(nq, n), dim3(128), 0, g.stream, a);
     HIP_TRY(hipGetLastError(), "decode launch", layer);
     g.calls.fetch_add(n, std::memory_order_relaxed);
     return WR_HIP_OK;
@@ -306,6 +313,7 @@ int check_decode(uint32_t n, wr_hip_kv* const* kv, uint32_t layer, const uint32_
             if (kv[i] == kv[j]) return WR_HIP_ERR_INVAL;
     }
     if (nq == 0 || nq % kv[0]->nkv != 0) return WR_HIP_ERR_INVAL;
+    if (nq > kMaxHeads) return WR_HIP_ERR_LIMIT;
     for (uint32_t i = 0; i < n; i++) {
         if (seq_k[i] == 0) return WR_HIP_ERR_INVAL;
         if (seq_k[i] > WR_HIP_ATTN_MAX_SEQ) return WR_HIP_ERR_LIMIT;
@@ -394,6 +402,13 @@ int wr_hip_attn_init(int device)
     g.calls.store(0);
     int rc = ensure_pinned(g.h_pin, 2 * kPinSmall);
     if (rc == WR_HIP_OK) rc = ensure_device(g.d_stage, 2 * kPinSmall);
+    if (rc == WR_HIP_OK) {
+        const size_t cb = (size_t)WR_HIP_BATCH_MAX * kMaxHeads * sizeof(uint32_t);
+        hipError_t e = hipMalloc((void**)&g.d_counters, cb);
+        if (e == hipSuccess) e = hipMemsetAsync(g.d_counters, 0, cb, g.stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(g.stream);
+        if (e != hipSuccess) rc = hip_fail(e, "ticket array", 0);
+    }
     if (rc != WR_HIP_OK) {
         g.inited = false;
         (void)hipStreamDestroy(g.stream);
@@ -414,6 +429,8 @@ void wr_hip_attn_shutdown(void)
     g.profiling = false;
     if (g.d_stage.p) (void)hipFree(g.d_stage.p);
     if (g.d_part.p) (void)hipFree(g.d_part.p);
+    if (g.d_counters) (void)hipFree(g.d_counters);
+    g.d_counters = nullptr;
     if (g.h_pin.p) (void)hipHostFree(g.h_pin.p);
     g.d_stage = Buffer();
     g.d_part = Buffer();

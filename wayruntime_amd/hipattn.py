@@ -11,7 +11,7 @@ import os
 import numpy as np
 
 PKG = os.path.dirname(os.path.abspath(__file__))
-HIP_SO = os.path.join(PKG, "libwr_hip_attn.so")
+HIP_SO = os.environ.get("WR_HIP_ATTN_LIB") or os.path.join(PKG, "libwr_hip_attn.so")
 
 OK = 0
 ERR_UNSUPPORTED, ERR_INVAL, ERR_NOMEM, ERR_CTX_FULL = -3, -4, -5, -6
