@@ -1,0 +1,147 @@
+"""Causal prefill on the device against the CPU oracle (a loop of seq_q = 1
+attention calls, the reference's prefill semantics), through the C ABI.
+Tolerance: max-abs 2e-3, rel-L2 1e-3."""
+import numpy as np
+import pytest
+
+import oracle
+from tests import util
+from wayruntime_amd import hipattn, synth
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _device():
+    hipattn.init()
+    oracle.set_attn_max_seq(1 << 20)
+    yield
+    hipattn.set_tuning(0, False)
+
+
+def _setup(nq, nkv, hd, p0, T, seed, theta=None, extra_rows=0):
+    """Cache with p0 + T appended rows (through the F32 append path), q [T,nq,hd]."""
+    rows = p0 + T
+    k32 = synth.normal(seed, (rows, nkv, hd))
+    v32 = synth.normal(seed + 1, (rows, nkv, hd))
+    q = synth.normal(seed + 2, (T, nq, hd))
+    if theta:
+        # inputs "after RoPE": rotate K at positions 0.. and Q at p0..
+        k32 = oracle.rope(k32, 0, theta)
+        q = oracle.rope(q, p0, theta)
+    kv = hipattn.KVCache(1, hd, nkv, rows + extra_rows)
+    assert kv.append(0, 0, k32, v32) == hipattn.OK
+    return kv, q, synth.f32_to_f16_trunc(k32), synth.f32_to_f16_trunc(v32)
+
+
+@pytest.mark.parametrize("nq,nkv,hd,p0,T,win", [
+    (16, 8, 128, 0, 512, 0),        # Qwen3 shape, empty cache
+    (32, 8, 128, 0, 512, 0),        # Llama-3 shape
+    (32, 8, 128, 100, 300, 0),      # chunk appended to a non-empty cache, ragged sizes
+    (8, 4, 256, 0, 200, 0),         # Gemma-class
+    (4, 4, 64, 7, 130, 0),          # MHA
+    (8, 1, 64, 0, 97, 0),           # group of 8: two head chunks per KV head
+    (16, 8, 128, 0, 1, 0),          # a single row
+    (16, 8, 128, 31, 2, 0),
+    (16, 8, 128, 0, 33, 0),
+    (16, 8, 128, 0, 400, 64),       # sliding window
+    (32, 8, 128, 50, 300, 33),
+    (8, 4, 256, 0, 300, 100),
+])
+def test_prefill_matches_serial_stepping_oracle(nq, nkv, hd, p0, T, win):
+    print("prefill", nq, nkv, hd, p0, T, win, flush=True)
+    kv, q, k16, v16 = _setup(nq, nkv, hd, p0, T, seed=1000 + T + p0)
+    got = kv.prefill(0, p0, q, 0.0, win)
+    want = oracle.causal_prefill(q, k16, v16, p0=p0, window=win, threads=8)
+    print("  errors", util.assert_close(got, want), flush=True)
+    kv.close()
+
+
+@pytest.mark.parametrize("nq,nkv,hd,p0,T,win", [
+    (4, 2, 32, 3, 70, 0),           # head_dim 32: generic kernel
+    (6, 2, 64, 0, 40, 0),           # group of 3
+    (3, 3, 20, 0, 25, 8),
+])
+def test_prefill_generic_shapes(nq, nkv, hd, p0, T, win):
+    print("prefill generic", nq, nkv, hd, p0, T, win, flush=True)
+    kv, q, k16, v16 = _setup(nq, nkv, hd, p0, T, seed=77 + T)
+    got = kv.prefill(0, p0, q, 0.0, win)
+    want = oracle.causal_prefill(q, k16, v16, p0=p0, window=win)
+    util.assert_close(got, want)
+    kv.close()
+
+
+def test_prefill_row_equals_decode_call_and_last_row_sees_everything():
+    nq, nkv, hd, p0, T = 16, 8, 128, 40, 100
+    kv, q, k16, v16 = _setup(nq, nkv, hd, p0, T, seed=5)
+    got = kv.prefill(0, p0, q)
+    for i in (0, 1, 31, 32, 63, 99):
+        dec = kv.decode(0, p0 + i + 1, q[i])             # definition: row i == decode at seq_k = p0+i+1
+        assert util.errors(got[i], dec)[0] < 2e-3
+        util.assert_close(got[i], util.oracle_decode(q[i], k16, v16, p0 + i + 1), f"row {i}")
+    # the last row equals the reference op (non-causal) over the whole cache
+    util.assert_close(got[-1], oracle.attention(q[-1:], k16, v16)[0])
+    kv.close()
+
+
+def test_prefill_mfma_and_generic_kernels_agree():
+    nq, nkv, hd, p0, T = 32, 8, 128, 10, 150
+    kv, q, k16, v16 = _setup(nq, nkv, hd, p0, T, seed=9)
+    a = kv.prefill(0, p0, q)
+    hipattn.set_tuning(0, True)
+    b = kv.prefill(0, p0, q)
+    hipattn.set_tuning(0, False)
+    assert util.errors(a, b)[0] < 2e-3
+    util.assert_close(b, oracle.causal_prefill(q, k16, v16, p0=p0, threads=8), "generic")
+    kv.close()
+
+
+def test_prefill_ignores_rows_that_were_never_appended():
+    nq, nkv, hd, T = 16, 8, 128, 70
+    kv, q, k16, v16 = _setup(nq, nkv, hd, 0, T, seed=21, extra_rows=58)
+    bad = np.full((58, nkv, hd), 0x7E00, dtype=np.uint16)       # NaN patterns above the chunk
+    kv.write_f16(0, T, bad, bad)
+    got = kv.prefill(0, 0, q)
+    util.assert_close(got, oracle.causal_prefill(q, k16, v16, threads=8))
+    kv.close()
+
+
+@pytest.mark.parametrize("nq,nkv,theta,T", [(16, 8, 1e6, 2048), (32, 8, 5e5, 2048), (32, 8, 5e5, 4096)])
+def test_prefill_workload_sizes_after_rope_sampled_rows(nq, nkv, theta, T):
+    # the prefill workload: Q/K/V N(0,1), rotated (theta 1e6 Qwen3, 5e5 Llama-3),
+    # appended to an empty cache; the CPU loop is quadratic, so the oracle checks a
+    # spread of rows and properties cover the rest
+    hd = 128
+    print("prefill workload", nq, nkv, T, flush=True)
+    kv, q, k16, v16 = _setup(nq, nkv, hd, 0, T, seed=synth.config_seed(4, nq + T % 97), theta=theta)
+    got = kv.prefill(0, 0, q)
+    assert not np.isnan(got).any()
+    rows = sorted(set([0, 1, 31, 32, 33, 63, 64, 127, 128, 500, 1023, 1024, T // 2 + 17, T - 2, T - 1]))
+    want = oracle.causal_prefill(q, k16, v16, rows=rows, threads=8)
+    print("  errors", util.assert_close(got[rows], want[rows]), flush=True)
+    # row 0 sees one key: its output is V row 0 of the matching KV head
+    v0 = v16[0].view(np.float16).astype(np.float32)
+    assert np.allclose(got[0], np.repeat(v0, nq // nkv, axis=0), atol=1e-5)
+    # every output is a convex combination of V rows: bounded by the per-dim extremes
+    v = v16.view(np.float16).astype(np.float32)
+    vmax = np.repeat(np.maximum.accumulate(v, axis=0), nq // nkv, axis=1)
+    vmin = np.repeat(np.minimum.accumulate(v, axis=0), nq // nkv, axis=1)
+    assert np.all(got <= vmax + 1e-3) and np.all(got >= vmin - 1e-3)
+    kv.close()
+
+
+def test_prefill_error_contract():
+    lib = hipattn.lib()
+    kv = hipattn.KVCache(1, 128, 8, 64)
+    q = np.zeros((4, 16, 128), dtype=np.float32)
+    out = np.zeros_like(q)
+    pre = lambda p0, T, nq=16: lib.wr_hip_attn_prefill(kv.h, 0, p0, T, q.ctypes.data,   # noqa: E731
+                                                        out.ctypes.data, nq, 0.0, 0)
+    assert pre(0, 0) == hipattn.ERR_INVAL
+    assert pre(62, 4) == hipattn.ERR_INVAL                 # runs past the allocation
+    assert pre(hipattn.ATTN_MAX_SEQ, 4) == hipattn.ERR_LIMIT
+    assert pre(0, 4, nq=12) == hipattn.ERR_INVAL
+    calls = lib.wr_hip_attn_calls()
+    assert pre(0, 4) == hipattn.OK
+    assert lib.wr_hip_attn_calls() == calls + 4            # one per token, as the serial loop counts
+    kv.close()

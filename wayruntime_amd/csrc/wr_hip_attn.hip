@@ -342,7 +342,22 @@ int prefill_locked(wr_hip_kv* kv, uint32_t layer, uint32_t p0, uint32_t T, const
     a.window = window;
     const float scale = (scale_override > 0.0f) ? scale_override : 1.0f / sqrtf((float)hd);
     a.qscale = scale * kLog2e;
-    launch_main(prefill_generic_kernel, dim3(T, nq), dim3(kDecodeThreads), a);
+    const uint32_t G = a.group;
+    const bool mfma = !g.force_generic && (hd == 64 || hd == 128 || hd == 256) &&
+                      (G == 1 || G == 2 || G == 4 || G == 8);
+    if (mfma) {
+        const uint32_t Gw = G < 4 ? G : 4;
+        const uint32_t BP = 32 * (4 / Gw);
+        const dim3 grid((T + BP - 1) / BP, kv->nkv * (G / Gw)), block(kPrefillThreads);
+        if (hd == 64)
+            launch_main(prefill_mfma_kernel<64>, grid, block, a);
+        else if (hd == 128)
+            launch_main(prefill_mfma_kernel<128>, grid, block, a);
+        else
+            launch_main(prefill_mfma_kernel<256>, grid, block, a);
+    } else {
+        launch_main(prefill_generic_kernel, dim3(T, nq), dim3(kDecodeThreads), a);
+    }
     HIP_TRY(hipGetLastError(), "prefill launch", layer);
     g.calls.fetch_add(T, std::memory_order_relaxed);
     return WR_HIP_OK;
