@@ -22,9 +22,13 @@ DTYPE_F32, DTYPE_F16 = 0, 1
 GROWABLE = 1 << 1
 
 
+HOSTCPU_SO = os.path.join(_HERE, "libwayruntime_cpuattn.so")
+
+
 def build(ref: bool = True) -> None:
-    """Compile the oracle (and the reference when its tree is present)."""
-    subprocess.check_call(["make", "-s", "-C", _HERE, "oracle"] + (["ref"] if ref else []))
+    """Compile the oracle, the host engine on the CPU test double, and the
+    reference when its tree is present."""
+    subprocess.check_call(["make", "-s", "-C", _HERE, "oracle", "hostcpu"] + (["ref"] if ref else []))
 
 
 class Tensor(C.Structure):

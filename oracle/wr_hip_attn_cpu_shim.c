@@ -1,0 +1,184 @@
+/*
+ * wr_hip_attn_cpu_shim.c — TEST DOUBLE of the device attention library.
+ * TEST INFRASTRUCTURE, never shipped: it exists so the C11 host engine's own
+ * logic (locking, all-or-nothing rollback, context limits, layer-major batch
+ * and prefill drivers, the GGUF loader) can be exercised on a machine without
+ * a GPU.  It implements the wr_hip_attn_* entry points the host engine calls
+ * on top of the CPU oracle (wr_oracle.c) and is linked ONLY into
+ * oracle/libwayruntime_cpuattn.so, which only the tests load.
+ */
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "../include/wr_hip_attn.h"
+#include "wr_oracle.h"
+
+struct wr_hip_kv {
+    uint32_t n_layers, nkv, max_ctx;
+    uint32_t hd[WR_HIP_MAX_LAYERS];
+    uint16_t *k[WR_HIP_MAX_LAYERS], *v[WR_HIP_MAX_LAYERS];   /* position-major [max_ctx][nkv][hd] */
+    uint64_t bytes;
+};
+
+static int g_inited;
+static uint64_t g_calls;
+
+int wr_hip_attn_init(int device)
+{
+    (void)device;
+    if (g_inited) return WR_HIP_ERR_STATE;
+    g_inited = 1;
+    g_calls = 0;
+    wro_set_attn_max_seq(WR_HIP_ATTN_MAX_SEQ);
+    return WR_HIP_OK;
+}
+
+void wr_hip_attn_shutdown(void) { g_inited = 0; }
+void wr_hip_attn_set_log(wr_hip_log_fn fn, void *user) { (void)fn; (void)user; }
+uint64_t wr_hip_attn_calls(void) { return g_calls; }
+const char *wr_hip_attn_device_name(void) { return "cpu test double (oracle)"; }
+
+int wr_hip_attn_kv_create(uint32_t n_layers, const uint32_t *hd, uint32_t nkv, uint32_t max_ctx,
+                          wr_hip_kv **out)
+{
+    if (!out) return WR_HIP_ERR_INVAL;
+    *out = NULL;
+    if (!g_inited) return WR_HIP_ERR_STATE;
+    if (!hd || !n_layers || !nkv || !max_ctx) return WR_HIP_ERR_INVAL;
+    if (n_layers > WR_HIP_MAX_LAYERS || max_ctx > WR_HIP_ATTN_MAX_SEQ) return WR_HIP_ERR_LIMIT;
+    wr_hip_kv *kv = calloc(1, sizeof *kv);
+    if (!kv) return WR_HIP_ERR_NOMEM;
+    kv->n_layers = n_layers;
+    kv->nkv = nkv;
+    kv->max_ctx = max_ctx;
+    for (uint32_t L = 0; L < n_layers; L++) {
+        kv->hd[L] = hd[L];
+        if (!hd[L]) continue;
+        const size_t n = (size_t)max_ctx * nkv * hd[L];
+        kv->k[L] = calloc(n, 2);
+        kv->v[L] = calloc(n, 2);
+        kv->bytes += 4 * n;
+        if (!kv->k[L] || !kv->v[L]) {
+            wr_hip_attn_kv_destroy(kv);
+            return WR_HIP_ERR_NOMEM;
+        }
+    }
+    *out = kv;
+    return WR_HIP_OK;
+}
+
+void wr_hip_attn_kv_destroy(wr_hip_kv *kv)
+{
+    if (!kv) return;
+    for (uint32_t L = 0; L < kv->n_layers; L++) {
+        free(kv->k[L]);
+        free(kv->v[L]);
+    }
+    free(kv);
+}
+
+uint64_t wr_hip_attn_kv_bytes(const wr_hip_kv *kv) { return kv ? kv->bytes : 0; }
+
+static int layer_ok(const wr_hip_kv *kv, uint32_t layer)
+{
+    return kv && layer < kv->n_layers && kv->hd[layer] != 0;
+}
+
+int wr_hip_attn_append(wr_hip_kv *kv, uint32_t layer, uint32_t pos, uint32_t n_rows,
+                       const float *k, const float *v)
+{
+    if (!g_inited) return WR_HIP_ERR_STATE;
+    if (!layer_ok(kv, layer)) return WR_HIP_ERR_INVAL;
+    if (n_rows == 0) return WR_HIP_OK;
+    if (!k || !v) return WR_HIP_ERR_INVAL;
+    if ((uint64_t)pos + n_rows > kv->max_ctx) return WR_HIP_ERR_CTX_FULL;
+    const size_t row = (size_t)kv->nkv * kv->hd[layer];
+    for (size_t i = 0; i < (size_t)n_rows * row; i++) {
+        kv->k[layer][(size_t)pos * row + i] = wro_f32_to_f16(k[i]);
+        kv->v[layer][(size_t)pos * row + i] = wro_f32_to_f16(v[i]);
+    }
+    return WR_HIP_OK;
+}
+
+int wr_hip_attn_kv_read(wr_hip_kv *kv, uint32_t layer, uint32_t pos, uint32_t n_rows,
+                        uint16_t *k, uint16_t *v)
+{
+    if (!g_inited) return WR_HIP_ERR_STATE;
+    if (!layer_ok(kv, layer) || !k || !v || (uint64_t)pos + n_rows > kv->max_ctx)
+        return WR_HIP_ERR_INVAL;
+    const size_t row = (size_t)kv->nkv * kv->hd[layer];
+    memcpy(k, kv->k[layer] + (size_t)pos * row, (size_t)n_rows * row * 2);
+    memcpy(v, kv->v[layer] + (size_t)pos * row, (size_t)n_rows * row * 2);
+    return WR_HIP_OK;
+}
+
+int wr_hip_attn_kv_write(wr_hip_kv *kv, uint32_t layer, uint32_t pos, uint32_t n_rows,
+                         const uint16_t *k, const uint16_t *v)
+{
+    if (!g_inited) return WR_HIP_ERR_STATE;
+    if (!layer_ok(kv, layer) || !k || !v) return WR_HIP_ERR_INVAL;
+    if ((uint64_t)pos + n_rows > kv->max_ctx) return WR_HIP_ERR_CTX_FULL;
+    const size_t row = (size_t)kv->nkv * kv->hd[layer];
+    memcpy(kv->k[layer] + (size_t)pos * row, k, (size_t)n_rows * row * 2);
+    memcpy(kv->v[layer] + (size_t)pos * row, v, (size_t)n_rows * row * 2);
+    return WR_HIP_OK;
+}
+
+static int check_decode(const wr_hip_kv *kv, uint32_t layer, uint32_t seq_k, uint32_t nq)
+{
+    if (!layer_ok(kv, layer)) return WR_HIP_ERR_INVAL;
+    if (nq == 0 || nq % kv->nkv) return WR_HIP_ERR_INVAL;
+    if (seq_k == 0) return WR_HIP_ERR_INVAL;
+    if (seq_k > WR_HIP_ATTN_MAX_SEQ) return WR_HIP_ERR_LIMIT;
+    if (seq_k > kv->max_ctx) return WR_HIP_ERR_INVAL;
+    return WR_HIP_OK;
+}
+
+int wr_hip_attn_decode(wr_hip_kv *kv, uint32_t layer, uint32_t seq_k, const float *q, float *out,
+                       uint32_t nq, float scale_override, uint32_t window)
+{
+    if (!g_inited) return WR_HIP_ERR_STATE;
+    if (!kv || !q || !out) return WR_HIP_ERR_INVAL;
+    int rc = check_decode(kv, layer, seq_k, nq);
+    if (rc) return rc;
+    wro_attention_f16kv(q, kv->k[layer], kv->v[layer], out, 1, nq, kv->nkv, kv->hd[layer], seq_k,
+                        scale_override, window);
+    g_calls++;
+    return WR_HIP_OK;
+}
+
+int wr_hip_attn_decode_batched(uint32_t n, wr_hip_kv *const *kv, uint32_t layer,
+                               const uint32_t *seq_k, const float *const *q, float *const *out,
+                               uint32_t nq, float scale_override, uint32_t window)
+{
+    if (!g_inited) return WR_HIP_ERR_STATE;
+    if (!kv || !seq_k || !q || !out) return WR_HIP_ERR_INVAL;
+    if (n == 0 || n > WR_HIP_BATCH_MAX) return WR_HIP_ERR_LIMIT;
+    for (uint32_t i = 0; i < n; i++) {
+        int rc = check_decode(kv[i], layer, seq_k[i], nq);
+        if (rc) return rc;
+        for (uint32_t j = 0; j < i; j++)
+            if (kv[i] == kv[j]) return WR_HIP_ERR_INVAL;
+    }
+    for (uint32_t i = 0; i < n; i++) {
+        wro_attention_f16kv(q[i], kv[i]->k[layer], kv[i]->v[layer], out[i], 1, nq, kv[i]->nkv,
+                            kv[i]->hd[layer], seq_k[i], scale_override, window);
+        g_calls++;
+    }
+    return WR_HIP_OK;
+}
+
+int wr_hip_attn_prefill(wr_hip_kv *kv, uint32_t layer, uint32_t p0, uint32_t T, const float *q,
+                        float *out, uint32_t nq, float scale_override, uint32_t window)
+{
+    if (!g_inited) return WR_HIP_ERR_STATE;
+    if (!layer_ok(kv, layer) || !q || !out || T == 0) return WR_HIP_ERR_INVAL;
+    if (nq == 0 || nq % kv->nkv) return WR_HIP_ERR_INVAL;
+    if ((uint64_t)p0 + T > WR_HIP_ATTN_MAX_SEQ) return WR_HIP_ERR_LIMIT;
+    if ((uint64_t)p0 + T > kv->max_ctx) return WR_HIP_ERR_INVAL;
+    wro_causal_prefill(q, kv->k[layer], kv->v[layer], out, p0, T, nq, kv->nkv, kv->hd[layer],
+                       scale_override, window);
+    g_calls += T;
+    return WR_HIP_OK;
+}

@@ -1,0 +1,123 @@
+"""End to end on the device: the C11 host engine (wr_engine / wr_model /
+wr_session API) with attention and the KV cache on the GPU, against the greedy
+token stream the compiled reference produced for the same random-init model
+(tests/golden/e2e_*_golden.npz, written by tests/golden/make_e2e_golden.py)."""
+import os
+
+import numpy as np
+import pytest
+
+from tests.golden.make_e2e_golden import TINY, file_crc, workload
+from wayruntime_amd import engine as E, gguf_writer as gw, hipattn
+
+pytestmark = pytest.mark.gpu
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+
+
+@pytest.fixture(scope="module")
+def eng():
+    hipattn.shutdown()              # the engine owns the device library in this module
+    e = E.Engine(E.HOST_SO)
+    yield e
+    e.close()
+
+
+def _run_stream(model, g, n_prompt):
+    prompt = workload(gw.ModelShape(vocab=model.vocab), n_prompt)
+    assert np.array_equal(prompt, g["prompt"])
+    n_steps = len(g["tokens"])
+    probe_idx = np.linspace(0, model.vocab - 1, 8).astype(int)
+    # free-running greedy: step for step against the reference's stream
+    s = model.session(n_prompt + n_steps - 1)
+    assert s.prefill(prompt[:-1]) == n_prompt - 1
+    tok, got, worst_probe = int(prompt[-1]), [], 0.0
+    for step in range(n_steps):
+        logits = s.step(tok)
+        assert logits is not None, f"step {step}: status {s.status}"
+        worst_probe = max(worst_probe, float(np.max(np.abs(logits[probe_idx] - g["probes"][step]))))
+        tok = int(np.argmax(logits))            # first maximum: ties keep the lower id
+        got.append(tok)
+    s.close()
+    # teacher-forced: feed the reference's own tokens, compare the argmax at each step
+    t = model.session(n_prompt + n_steps - 1)
+    assert t.prefill(prompt[:-1]) == n_prompt - 1
+    feed, forced = int(prompt[-1]), 0
+    for step in range(n_steps):
+        logits = t.step(feed)
+        forced += int(np.argmax(logits)) == int(g["tokens"][step])
+        feed = int(g["tokens"][step])
+    t.close()
+    return np.array(got), forced, worst_probe
+
+
+def test_tiny_model_stream_on_device(eng, tmp_path):
+    g = np.load(os.path.join(GOLD, "e2e_tiny_golden.npz"))
+    p = str(tmp_path / "tiny.gguf")
+    gw.write_model(p, TINY)
+    m = eng.load(p)
+    got, forced, probe = _run_stream(m, g, len(g["prompt"]))
+    print("tiny: forced", forced, "probe err", probe, flush=True)
+    assert forced == len(g["tokens"]) and np.array_equal(got, g["tokens"]) and probe < 1e-4
+    m.close()
+
+
+def test_qwen3_0_6b_greedy_stream_matches_reference(eng, tmp_path):
+    # 28 layers, hidden 1024, 16/8 heads, head_dim 128, F16 weights N(0, 0.02):
+    # 127-token prefill, then 129 greedy steps
+    g = np.load(os.path.join(GOLD, "e2e_qwen3_golden.npz"))
+    p = str(tmp_path / "qwen3.gguf")
+    print("writing model ...", flush=True)
+    gw.write_model(p, gw.QWEN3_0_6B)
+    if file_crc(p) != int(g["model_crc"][0]):
+        pytest.skip("random-init model file differs from the one the golden stream was made with "
+                    "(different numpy build?): inputs differ, nothing to compare")
+    m = eng.load(p, max_context=512)
+    before = eng.counters()[E.WR_CTR_ATTENTION_CALLS]
+    got, forced, probe = _run_stream(m, g, 128)
+    n = len(g["tokens"])
+    print(f"qwen3: teacher-forced {forced}/{n}, probe logit err {probe:.2e}, "
+          f"min reference top-2 gap {float(g['gaps'].min()):.4f}", flush=True)
+    assert forced == n                                   # argmax agrees at every step
+    assert np.array_equal(got, g["tokens"])              # and the free-running stream is identical
+    assert probe < 1e-3
+    # one attention per session-layer-token, as the reference counts them: two runs of 127 + 129
+    assert eng.counters()[E.WR_CTR_ATTENTION_CALLS] - before == 2 * 28 * (127 + 129)
+    m.close()
+    os.remove(p)
+
+
+def test_batched_step_equals_serial_on_device(eng, tmp_path):
+    p = str(tmp_path / "tiny.gguf")
+    gw.write_model(p, TINY)
+    m = eng.load(p)
+    n = 5
+    prompts = [workload(TINY, 4 + 7 * i) for i in range(n)]
+    batch = [m.session(128) for _ in range(n)]
+    serial = [m.session(128) for _ in range(n)]
+    for i in range(n):
+        assert batch[i].prefill(prompts[i]) == len(prompts[i])
+        assert serial[i].prefill(prompts[i]) == len(prompts[i])
+    toks = list(range(10, 10 + n))
+    for _ in range(6):
+        rc, lb = E.batch_step(batch, toks)
+        assert rc == n
+        ls = [serial[i].step(toks[i]) for i in range(n)]
+        for i in range(n):
+            assert lb[i].tobytes() == ls[i].tobytes(), f"session {i}"
+        toks = [int(np.argmax(x)) for x in lb]
+    # context full in one session refuses the whole batch; nobody advances
+    small = m.session(2)
+    assert small.prefill([1, 2]) == 2
+    pos = [s.pos for s in batch]
+    assert E.batch_step(batch + [small], toks + [1])[0] == E.WR_ERR_CTX_FULL
+    assert [s.pos for s in batch] == pos
+    # injected failure mid-stack: rollback, then the retry equals the serial twins
+    eng.lib.wrh_debug_fail_attention_at(1)
+    assert E.batch_step(batch, toks)[0] == E.WR_ERR_INTERNAL
+    assert [s.pos for s in batch] == pos
+    rc, lb = E.batch_step(batch, toks)
+    ls = [serial[i].step(toks[i]) for i in range(n)]
+    assert rc == n and all(lb[i].tobytes() == ls[i].tobytes() for i in range(n))
+    for s in batch + serial + [small]:
+        s.close()
+    m.close()

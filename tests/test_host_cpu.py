@@ -1,0 +1,207 @@
+"""Host engine logic on the CPU test double (oracle/libwayruntime_cpuattn.so:
+the C11 host engine linked against an oracle-backed stand-in for the device
+library).  Covers what needs no GPU: the GGUF loader, the greedy token stream of
+a toy model against the compiled reference's golden stream, context limits,
+all-or-nothing rollback, batched == serial, and the error contract."""
+import os
+import struct
+
+import numpy as np
+import pytest
+
+import oracle
+from tests.golden.make_e2e_golden import TINY, workload
+from wayruntime_amd import engine as E, gguf_writer as gw
+
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+
+
+@pytest.fixture(scope="module")
+def eng():
+    oracle.build(ref=False)
+    e = E.Engine(oracle.HOSTCPU_SO, threads=4)
+    yield e
+    e.close()
+
+
+@pytest.fixture(scope="module")
+def tiny_path(tmp_path_factory):
+    p = str(tmp_path_factory.mktemp("gguf") / "tiny.gguf")
+    gw.write_model(p, TINY)
+    return p
+
+
+@pytest.fixture()
+def model(eng, tiny_path):
+    m = eng.load(tiny_path)
+    yield m
+    m.close()
+
+
+def test_model_info_matches_file(model):
+    i = model.info
+    assert (i.arch, i.quant) == (b"qwen3", b"F16")
+    assert (i.n_layers, i.n_q_heads, i.n_kv_heads, i.head_dim) == (2, 4, 2, 32)
+    assert (i.hidden_dim, i.ffn_dim, i.vocab_size, i.train_context, i.max_context) == (64, 128, 300, 512, 512)
+    assert abs(i.rope_freq_base - 1e6) < 1 and abs(i.rms_eps - 1e-6) < 1e-12
+    assert i.has_qk_norm == 1 and i.tied_lm_head == 1 and i.is_gemma == 0
+
+
+def test_greedy_stream_matches_reference_golden(model):
+    # tests/golden/e2e_tiny_golden.npz was written by the compiled reference
+    g = np.load(os.path.join(GOLD, "e2e_tiny_golden.npz"))
+    prompt = workload(TINY, len(g["prompt"]))
+    assert np.array_equal(prompt, g["prompt"])
+    s = model.session(len(prompt) + len(g["tokens"]) - 1)
+    assert s.prefill(prompt[:-1]) == len(prompt) - 1
+    tok, probe_idx = int(prompt[-1]), np.linspace(0, TINY.vocab - 1, 8).astype(int)
+    for step, want in enumerate(g["tokens"]):
+        logits = s.step(tok)
+        assert logits is not None
+        assert np.max(np.abs(logits[probe_idx] - g["probes"][step])) < 2e-5
+        tok = int(np.argmax(logits))
+        assert tok == int(want), f"step {step}"
+    s.close()
+
+
+def test_prefill_equals_token_by_token_steps(model):
+    ids = workload(TINY, 40)
+    a, b = model.session(64), model.session(64)
+    assert a.prefill(ids[:39]) == 39
+    for t in ids[:39]:
+        assert b.step(t) is not None
+    la, lb = a.step(ids[39]), b.step(ids[39])
+    assert a.pos == b.pos == 40
+    assert np.array_equal(la, lb)          # same per-row arithmetic, bit for bit (CPU double)
+    a.close(); b.close()
+
+
+def test_context_is_a_hard_boundary(model):
+    # the reference's llm_step fixture (src/core/session.c:946-985) on this engine
+    s = model.session(16)
+    assert s.pos == 0
+    assert s.step(5) is not None and s.pos == 1                 # cursor 0 -> 1
+    assert s.step(TINY.vocab) is None                           # out-of-vocabulary: refused
+    assert s.status == E.WR_ERR_INVAL and s.pos == 1            # ... and nothing consumed
+    assert s.prefill(list(range(14))) == 14 and s.pos == 15
+    assert s.prefill([1, 2]) == E.WR_ERR_CTX_FULL and s.pos == 15   # all or nothing
+    assert s.step(7) is not None and s.pos == 16
+    assert s.step(7) is None and s.status == E.WR_ERR_CTX_FULL and s.pos == 16
+    assert s.prefill([]) == 0
+    assert s.prefill([1, TINY.vocab + 3]) < 0 and s.pos == 16
+    s.close()
+
+
+def test_prefill_with_bad_token_consumes_nothing(model):
+    s = model.session(32)
+    assert s.prefill([1, 2, 3]) == 3
+    assert s.prefill([4, 5, 9999, 6]) == E.WR_ERR_INVAL
+    assert s.pos == 3 and s.status == E.WR_ERR_INVAL
+    ref = model.session(32)
+    assert ref.prefill([1, 2, 3]) == 3
+    assert np.array_equal(s.step(8), ref.step(8))               # state is as if the call never happened
+    s.close(); ref.close()
+
+
+def test_injected_attention_failure_rolls_back(eng, model):
+    s, twin = model.session(32), model.session(32)
+    for sess in (s, twin):
+        assert sess.prefill([3, 1, 4, 1, 5]) == 5
+    eng.lib.wrh_debug_fail_attention_at(1)                      # layer 1 fails once, on the host
+    assert s.step(9) is None
+    assert s.status == E.WR_ERR_INTERNAL and s.pos == 5
+    assert np.array_equal(s.step(9), twin.step(9))              # retry equals an undisturbed twin
+    eng.lib.wrh_debug_fail_attention_at(0)
+    assert s.prefill([2, 6]) == E.WR_ERR_INTERNAL and s.pos == 6
+    assert twin.prefill([2, 6]) == 2 and s.prefill([2, 6]) == 2
+    assert np.array_equal(s.step(1), twin.step(1))
+    s.close(); twin.close()
+
+
+def test_batched_step_equals_serial_steps_bit_for_bit(model):
+    # reference: wri_self_test_batch_step (src/core/batch.c:257-390)
+    n = 3
+    prompts = [workload(TINY, 5 + 3 * i) for i in range(n)]
+    batch = [model.session(64) for _ in range(n)]
+    serial = [model.session(64) for _ in range(n)]
+    for i in range(n):
+        assert batch[i].prefill(prompts[i]) == len(prompts[i])
+        assert serial[i].prefill(prompts[i]) == len(prompts[i])
+    toks = [11, 22, 33]
+    for _ in range(5):
+        rc, lb = E.batch_step(batch, toks)
+        assert rc == n
+        ls = [serial[i].step(toks[i]) for i in range(n)]
+        for i in range(n):
+            assert lb[i].tobytes() == ls[i].tobytes()
+            assert batch[i].pos == serial[i].pos
+        toks = [int(np.argmax(x)) for x in lb]
+    for s in batch + serial:
+        s.close()
+
+
+def test_batch_contract(eng, model):
+    a, b = model.session(4), model.session(8)
+    assert E.batch_step([a, a], [1, 2])[0] == E.WR_ERR_INVAL            # same session twice
+    sessions = [model.session(4) for _ in range(17)]
+    assert E.batch_step(sessions, [1] * 17)[0] == E.WR_ERR_LIMIT       # more than WR_BATCH_MAX
+    for s in sessions:
+        s.close()
+    for _ in range(4):
+        assert E.batch_step([a, b], [1, 2])[0] == 2
+    # a is full: the whole batch is refused and b does not advance
+    assert E.batch_step([a, b], [1, 2])[0] == E.WR_ERR_CTX_FULL
+    assert (a.pos, b.pos) == (4, 4) and b.status == E.WR_ERR_CTX_FULL
+    # an out-of-vocabulary token in one row refuses the batch
+    c = model.session(8)
+    assert E.batch_step([b, c], [1, 100000])[0] == E.WR_ERR_INVAL and (b.pos, c.pos) == (4, 0)
+    # injected failure: nobody advances, and the next batch matches fresh twins
+    eng.lib.wrh_debug_fail_attention_at(1)
+    assert E.batch_step([b, c], [1, 2])[0] == E.WR_ERR_INTERNAL and (b.pos, c.pos) == (4, 0)
+    assert E.batch_step([b, c], [1, 2])[0] == 2 and (b.pos, c.pos) == (5, 1)
+    for s in (a, b, c):
+        s.close()
+
+
+def test_attention_counter_counts_session_layer_calls(eng, model):
+    s = model.session(16)
+    before = eng.counters()[E.WR_CTR_ATTENTION_CALLS]
+    s.step(1)
+    assert eng.counters()[E.WR_CTR_ATTENTION_CALLS] == before + TINY.n_layers
+    s.prefill([1, 2, 3])
+    assert eng.counters()[E.WR_CTR_ATTENTION_CALLS] == before + TINY.n_layers * 4
+    s.close()
+
+
+def test_loader_refusals(eng, tiny_path, tmp_path):
+    raw = open(tiny_path, "rb").read()
+
+    def load(data, name):
+        p = str(tmp_path / name)
+        open(p, "wb").write(data)
+        with pytest.raises(E.EngineError) as ei:
+            eng.load(p)
+        return ei.value.rc
+
+    assert load(b"GGUX" + raw[4:], "magic.gguf") == E.WR_ERR_FORMAT
+    assert load(raw[:4] + struct.pack("<I", 7) + raw[8:], "version.gguf") == E.WR_ERR_FORMAT
+    assert load(raw[:1000], "short.gguf") == E.WR_ERR_FORMAT
+    assert load(raw.replace(b"qwen3", b"gemma"), "arch.gguf") == E.WR_ERR_UNSUPPORTED
+    assert load(raw.replace(b"blk.1.attn_q.weight", b"blk.1.attn_x.weight"), "missing.gguf") == E.WR_ERR_FORMAT
+    with pytest.raises(E.EngineError) as ei:
+        eng.load(str(tmp_path / "nope.gguf"))
+    assert ei.value.rc == E.WR_ERR_IO
+    with pytest.raises(E.EngineError) as ei:
+        eng.load(tiny_path, max_context=1 << 20)                # above the cap: refused, not clamped
+    assert ei.value.rc == E.WR_ERR_LIMIT
+    m = eng.load(tiny_path, max_context=64)
+    with pytest.raises(E.EngineError) as ei:
+        m.session(65)                                           # above the model bound
+    assert ei.value.rc == E.WR_ERR_INVAL
+    m.close()
+
+
+def test_single_engine_per_process(eng):
+    import ctypes as C
+    h = C.c_void_p()
+    assert eng.lib.wr_engine_create(None, C.byref(h)) == E.WR_ERR_STATE

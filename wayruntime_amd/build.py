@@ -43,10 +43,29 @@ def build_hip(keep_temps: bool = False) -> str:
     return HIP_SO
 
 
+HOST_SO = os.path.join(PKG, "libwayruntime_amd.so")
+HOST_DIR = os.path.join(PKG, "host")
+HOST_SRCS = ["wr_math.c", "wr_ops.c", "wr_model.c", "wr_session.c"]
+# -ffp-contract=off: the scalar ops keep the reference's multiply-then-add
+# rounding; the matmul uses explicit FMA intrinsics and is not affected.
+HOST_CFLAGS = ["-std=c11", "-O3", "-mavx2", "-mfma", "-mf16c", "-ffp-contract=off", "-fopenmp",
+               "-fPIC", "-shared", "-Wall", "-Wextra", "-Wshadow", "-Wvla"]
+
+
+def build_host() -> str:
+    """The C11 host engine, linked against the device library next to it."""
+    cmd = (["gcc"] + HOST_CFLAGS + ["-I" + os.path.join(HOST_DIR, "include"), "-o", HOST_SO]
+           + [os.path.join(HOST_DIR, f) for f in HOST_SRCS]
+           + ["-L" + PKG, "-lwr_hip_attn", "-Wl,-rpath,$ORIGIN", "-lpthread"])
+    subprocess.check_call(cmd)
+    return HOST_SO
+
+
 def build_all(keep_temps: bool = False) -> None:
     build_hip(keep_temps)
+    build_host()
 
 
 if __name__ == "__main__":
     build_all("--temps" in sys.argv)
-    print("built", HIP_SO)
+    print("built", HIP_SO, HOST_SO)

@@ -57,6 +57,8 @@ struct DecodeSession {
     uint32_t key_lo;         // first visible key (sliding window), else 0
     uint32_t ctx_pad;        // rows allocated per KV head (multiple of 32)
     uint32_t n_splits;       // workgroups along the key axis
+    uint32_t tiles_per_wg;   // 32-key tiles per workgroup (a function of this session only)
+    uint32_t pad_;
 };
 
 struct DecodeArgs {
@@ -67,7 +69,6 @@ struct DecodeArgs {
     float* part_ml;          // [n][nq][max_splits][2] = (m in log2 units, l)
     uint32_t* counters;      // tickets, zero between launches: [n][nkv] (MFMA) or [n][nq] (generic)
     uint32_t nq, nkv, group, hd;
-    uint32_t tiles_per_wg;   // 32-key tiles per workgroup
     uint32_t max_splits;
     float qscale;            // softmax scale * log2(e)
 };
@@ -76,9 +77,9 @@ struct TileRange {
     uint32_t t_begin, t_end;      // tiles [t_begin, t_end)
 };
 
-__device__ __forceinline__ TileRange split_tiles(const DecodeSession& S, uint32_t split,
-                                                 uint32_t tiles_per_wg)
+__device__ __forceinline__ TileRange split_tiles(const DecodeSession& S, uint32_t split)
 {
+    const uint32_t tiles_per_wg = S.tiles_per_wg;
     const uint32_t first = S.key_lo / kTileKeys;
     const uint32_t last = (S.seq_k + kTileKeys - 1) / kTileKeys;
     TileRange r;
@@ -314,7 +315,16 @@ void decode_mfma_kernel(const DecodeArgs a)
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n = lane & 15, g = lane >> 4;
     const int G = (int)a.group;
-    const TileRange tr = split_tiles(S, split, a.tiles_per_wg);
+    const TileRange tr = split_tiles(S, split);
+
+    const uint16_t* kbase = S.k + (size_t)kvh * S.ctx_pad * HD;
+    const uint16_t* vtbase = S.vt + (size_t)kvh * (S.ctx_pad / kVBlock) * HD * kVBlock;
+
+    // The first tile's loads go out before anything else: the HBM latency
+    // then overlaps the staging of Q.
+    DecodeFrag<HD> fa, fb;
+    uint32_t t = tr.t_begin + wave;
+    if (t < tr.t_end) load_frag<HD>(fa, kbase, vtbase, t, lane);
 
     // Q^T operand through LDS: row c of lds_q is MFMA column c.  Columns
     // 0..G-1 hold the hi terms of the group's heads, G..2G-1 the lo terms,
@@ -348,13 +358,7 @@ void decode_mfma_kernel(const DecodeArgs a)
     st.m = -INFINITY;
     st.l = 0.f;
 
-    const uint16_t* kbase = S.k + (size_t)kvh * S.ctx_pad * HD;
-    const uint16_t* vtbase = S.vt + (size_t)kvh * (S.ctx_pad / kVBlock) * HD * kVBlock;
-
-    uint32_t t = tr.t_begin + wave;
     if (t < tr.t_end) {
-        DecodeFrag<HD> fa, fb;
-        load_frag<HD>(fa, kbase, vtbase, t, lane);
         for (;;) {
             const uint32_t t1 = t + kDecodeWaves;
             if (t1 < tr.t_end) load_frag<HD>(fb, kbase, vtbase, t1, lane);
@@ -521,7 +525,7 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_generic_kernel(const De
     if (split >= S.n_splits) return;
     const uint32_t hd = a.hd;
     const uint32_t kvh = head / a.group;
-    const TileRange tr = split_tiles(S, split, a.tiles_per_wg);
+    const TileRange tr = split_tiles(S, split);
     const uint32_t key_begin = max(tr.t_begin * kTileKeys, S.key_lo);
     const uint32_t key_end = min(tr.t_end * kTileKeys, S.seq_k);
 

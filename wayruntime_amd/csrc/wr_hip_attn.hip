@@ -62,7 +62,7 @@ struct Lib {
 } g;
 
 constexpr float kLog2e = 1.4426950408889634f;
-constexpr uint32_t kTargetWorkgroups = 256;  // split-K decode: about one workgroup per CU
+constexpr uint32_t kDefaultTilesPerWg = 64;  // split-K decode: 2048 keys per workgroup
 constexpr uint32_t kMaxHeads = 4096;        // query heads per session the ticket array is sized for
 constexpr size_t kPinSmall = 1u << 20;      // host copies up to this size go through pinned staging
 
@@ -237,28 +237,22 @@ int decode_locked(uint32_t n, wr_hip_kv* const* kv, uint32_t layer, const uint32
         tiles_total += tiles[i];
     }
 
-    // Keys per workgroup: enough workgroups to fill 256 CUs several times over,
-    // but at least one tile per wave so the per-workgroup merge stays small
-    // next to the data it streams.
-    uint32_t tiles_per_wg;
-    uint32_t tiles_max = 1;
-    for (uint32_t i = 0; i < n; i++)
-        if (tiles[i] > tiles_max) tiles_max = tiles[i];
-    if (g.tune_keys_per_wg) {
-        tiles_per_wg = g.tune_keys_per_wg / kTileKeys;
-        if (tiles_per_wg == 0) tiles_per_wg = 1;
-    } else {
-        const uint64_t units = tiles_total * (use_mfma ? nkv : nq);
-        tiles_per_wg = (uint32_t)((units + kTargetWorkgroups - 1) / kTargetWorkgroups);
-        tiles_per_wg = (tiles_per_wg + 3) & ~3u;
-        if (tiles_per_wg < 4) tiles_per_wg = 4;
-    }
-    // the in-kernel merge handles at most kMaxSplits partials per head
-    const uint32_t floor_tiles = (tiles_max + kMaxSplits - 1) / kMaxSplits;
-    if (tiles_per_wg < floor_tiles) tiles_per_wg = floor_tiles;
+    // Keys per workgroup.  The rule looks at ONE session only (its own visible
+    // key range), never at the rest of the batch: a session's arithmetic is then
+    // the same whether it is stepped alone or with others, which is what makes
+    // the batched step bit-identical to serial steps (reference contract:
+    // src/core/batch.c:15-19).  2048 keys (64 tiles) per workgroup measured best
+    // for the 16-session workload; the floor keeps the in-kernel merge within
+    // kMaxSplits partials for very long contexts.
+    (void)tiles_total;
     uint32_t max_splits = 1;
     for (uint32_t i = 0; i < n; i++) {
-        a.s[i].n_splits = (tiles[i] + tiles_per_wg - 1) / tiles_per_wg;
+        uint32_t tpw = g.tune_keys_per_wg ? g.tune_keys_per_wg / kTileKeys : kDefaultTilesPerWg;
+        if (tpw == 0) tpw = 1;
+        const uint32_t floor_tiles = (tiles[i] + kMaxSplits - 1) / kMaxSplits;
+        if (tpw < floor_tiles) tpw = floor_tiles;
+        a.s[i].tiles_per_wg = tpw;
+        a.s[i].n_splits = (tiles[i] + tpw - 1) / tpw;
         if (a.s[i].n_splits > max_splits) max_splits = a.s[i].n_splits;
     }
     a.q = q_dev;
@@ -267,7 +261,6 @@ int decode_locked(uint32_t n, wr_hip_kv* const* kv, uint32_t layer, const uint32
     a.nkv = nkv;
     a.group = group;
     a.hd = hd;
-    a.tiles_per_wg = tiles_per_wg;
     a.max_splits = max_splits;
     a.counters = g.d_counters;
     const float scale = (scale_override > 0.0f) ? scale_override : 1.0f / sqrtf((float)hd);

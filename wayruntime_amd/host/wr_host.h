@@ -1,0 +1,124 @@
+/*
+ * wr_host.h — internal contracts of the C11 host engine.
+ *
+ * The engine keeps the reference's decode structure (reference:
+ * src/core/session.c, src/core/batch.c) but drives it layer-major over a set
+ * of ROWS, so that one attention launch per layer serves a whole prefill chunk
+ * or a whole batch of sessions.  A row is one token of one session at one
+ * position; every CPU op here is row-wise, so the per-row arithmetic is the
+ * same whether a row travels alone (wr_step), with its prompt neighbours
+ * (wr_prefill) or with other sessions (wr_batch_step).
+ */
+#ifndef WR_HOST_H
+#define WR_HOST_H
+
+#include <pthread.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include <wayruntime/wayruntime.h>
+
+#include "../../include/wr_hip_attn.h"
+
+#define WRH_MAX_LAYERS   64          /* reference: WR_MAX_LAYERS, src/core/internal.h:184 */
+#define WRH_DEFAULT_CTX  4096        /* reference: WR_DEFAULT_MAX_CONTEXT, internal.h:194 */
+#define WRH_PREFILL_CHUNK 256        /* rows per layer-major prefill pass */
+
+/* ---- scalar math with the reference's polynomials (wr_math.c) ------------- */
+float wrh_exp(float x);
+float wrh_log(float x);
+float wrh_sqrt(float x);
+float wrh_sin(float x);
+float wrh_cos(float x);
+
+/* ---- weights ------------------------------------------------------------- */
+typedef struct wrh_weight {
+    const void *data;        /* points into the mapped file */
+    uint32_t    rows, cols;  /* [rows][cols], cols contiguous: W[out][in] or table[token][hidden] */
+    uint8_t     is_f16;      /* 1 = binary16, 0 = float32 */
+} wrh_weight;
+
+typedef struct wrh_vec {
+    const float *data;
+    uint32_t     n;
+} wrh_vec;
+
+struct wr_engine {
+    wr_engine_config cfg;
+    int      n_threads;
+    uint32_t models_live;
+    uint64_t ctr[WR_COUNTER_COUNT];
+};
+
+struct wr_model {
+    wr_engine *engine;
+    char       arch[32];
+    uint32_t   n_layers, n_q, n_kv, head_dim, hidden, ffn, vocab;
+    uint32_t   train_context, max_context, n_rot_pairs;
+    float      rms_eps, rope_base;
+    uint8_t    has_qk_norm, tied_head, all_f16;
+
+    wrh_weight embed, lm_head;
+    wrh_vec    final_norm;
+    wrh_vec    attn_norm[WRH_MAX_LAYERS], ffn_norm[WRH_MAX_LAYERS];
+    wrh_vec    q_norm[WRH_MAX_LAYERS], k_norm[WRH_MAX_LAYERS];
+    wrh_weight wq[WRH_MAX_LAYERS], wk[WRH_MAX_LAYERS], wv[WRH_MAX_LAYERS], wo[WRH_MAX_LAYERS];
+    wrh_weight w_gate[WRH_MAX_LAYERS], w_up[WRH_MAX_LAYERS], w_down[WRH_MAX_LAYERS];
+
+    void           *map;         /* mmap of the GGUF file */
+    size_t          map_bytes;
+    pthread_mutex_t lock;        /* guards session_refs */
+    uint32_t        session_refs;
+};
+
+/* Scratch for R rows of the forward pass. */
+typedef struct wrh_workspace {
+    uint32_t rows_cap;
+    float *residual, *normed;            /* [R][hidden] */
+    float *q, *attn;                     /* [R][n_q*hd]  */
+    float *k, *v;                        /* [R][n_kv*hd] */
+    float *gate, *up;                    /* [R][ffn]     */
+    float *proj;                         /* [R][hidden]  */
+    void  *block;
+} wrh_workspace;
+
+struct wr_session {
+    wr_model       *model;
+    pthread_mutex_t lock;
+    uint32_t        max_context;
+    uint32_t        pos;                     /* tokens in the cache == next position */
+    wr_status       last_status;
+    wr_hip_kv      *kv;                      /* device cache */
+    uint32_t        kv_rows[WRH_MAX_LAYERS]; /* per-layer cursor (the reference's valid_rows) */
+    float          *logits;                  /* [vocab] */
+    wrh_workspace   ws1;                     /* one-row scratch for wr_step */
+};
+
+/* ---- ops (wr_ops.c) -------------------------------------------------------
+ * All row-wise over R rows; `ld` is the row stride in floats. */
+int  wrh_embed(const wrh_weight *table, uint32_t token, float *out_row);
+void wrh_rmsnorm(const float *x, const float *w, uint32_t wn, float *out, uint32_t rows,
+                 uint32_t dim, float eps);
+/* C[r][j] = sum_k A[r][k] * W[j][k]; each output column is reduced whole in one
+ * thread, so results do not depend on the thread count or on R. */
+void wrh_matmul(wr_engine *e, const float *A, uint32_t R, uint32_t lda, const wrh_weight *W,
+                float *C, uint32_t ldc);
+void wrh_rope(float *x, uint32_t heads, uint32_t hd, uint32_t pos, float theta,
+              uint32_t n_rot_pairs);
+void wrh_swiglu(wr_engine *e, float *gate, const float *up, uint64_t n);
+void wrh_add(float *acc, const float *x, uint64_t n);
+
+/* ---- model / gguf (wr_model.c) -------------------------------------------- */
+void wrh_logf(wr_engine *e, int level, const char *fmt, ...) __attribute__((format(printf, 3, 4)));
+extern wr_engine *wrh_engine;           /* the process engine, NULL when none */
+
+/* ---- forward (wr_session.c) ------------------------------------------------ */
+int  wrh_workspace_init(wrh_workspace *ws, const wr_model *m, uint32_t rows);
+void wrh_workspace_free(wrh_workspace *ws);
+
+/* Test hook: make the attention call of `layer` fail with WR_ERR_INTERNAL once
+ * (layer < 0 disarms).  The device is not involved: the failure is raised on
+ * the host before the launch, so rollback paths can be exercised safely. */
+void wrh_debug_fail_attention_at(int layer);
+
+#endif /* WR_HOST_H */
