@@ -241,14 +241,23 @@ int decode_locked(uint32_t n, wr_hip_kv* const* kv, uint32_t layer, const uint32
     // key range), never at the rest of the batch: a session's arithmetic is then
     // the same whether it is stepped alone or with others, which is what makes
     // the batched step bit-identical to serial steps (reference contract:
-    // src/core/batch.c:15-19).  2048 keys (64 tiles) per workgroup measured best
-    // for the 16-session workload; the floor keeps the in-kernel merge within
-    // kMaxSplits partials for very long contexts.
+    // src/core/batch.c:15-19).  About 1 MiB of K+V per workgroup (2048 keys at
+    // head_dim 128) measured best for the 16-session workload; the session's
+    // tiles are then spread evenly over that many workgroups, and the floor keeps
+    // the in-kernel merge within kMaxSplits partials for very long contexts.
     (void)tiles_total;
     uint32_t max_splits = 1;
     for (uint32_t i = 0; i < n; i++) {
-        uint32_t tpw = g.tune_keys_per_wg ? g.tune_keys_per_wg / kTileKeys : kDefaultTilesPerWg;
-        if (tpw == 0) tpw = 1;
+        uint32_t tpw;
+        if (g.tune_keys_per_wg) {
+            tpw = g.tune_keys_per_wg / kTileKeys;
+            if (tpw == 0) tpw = 1;
+        } else {
+            uint32_t cap = kDefaultTilesPerWg * 128u / (hd < 32 ? 32 : hd);
+            if (cap == 0) cap = 1;
+            const uint32_t want = (tiles[i] + cap - 1) / cap;          // workgroups
+            tpw = (tiles[i] + want - 1) / want;                        // even share
+        }
         const uint32_t floor_tiles = (tiles[i] + kMaxSplits - 1) / kMaxSplits;
         if (tpw < floor_tiles) tpw = floor_tiles;
         a.s[i].tiles_per_wg = tpw;
