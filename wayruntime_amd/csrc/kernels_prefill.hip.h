@@ -18,6 +18,9 @@ struct PrefillArgs {
     float* out;              // [T][nq][hd]
     uint32_t p0, T, nq, nkv, group, hd, ctx_pad, window;
     float qscale;            // softmax scale * log2(e)
+#ifdef WR_PREFILL_PROF
+    unsigned long long* prof;
+#endif
 };
 
 // Any head_dim / group: one workgroup per (row, head), vector ALU only.
@@ -63,6 +66,7 @@ __global__ __launch_bounds__(kDecodeThreads) void prefill_generic_kernel(const P
 // the only operand that is not F16 already); P is rounded to F16 per tile.
 
 constexpr int kPrefillThreads = 256;
+constexpr float kLazyLog2 = 8.0f;    // softmax reference point moves only on jumps above 2^8
 
 __device__ __forceinline__ int prefill_key_perm(int m)
 {
@@ -70,24 +74,195 @@ __device__ __forceinline__ int prefill_key_perm(int m)
     return 16 * (a >> 1) + 8 * g + 4 * (a & 1) + b;
 }
 
-template <int HD>
-__global__ __launch_bounds__(kPrefillThreads, 2) void prefill_mfma_kernel(const PrefillArgs a)
+// Workgroup barrier that waits for this wave's LDS traffic only.  __syncthreads()
+// also drains outstanding global loads, which would pull the tiles being
+// prefetched for later iterations back onto the critical path.
+__device__ __forceinline__ void lds_barrier()
 {
-    constexpr int KSTR = HD + 8;              // halves per K row in LDS (16-byte pad: conflict-free b128 reads)
-    constexpr int VSTR = kVBlock + 8;         // halves per Vt row in LDS
-    constexpr int KCH = HD / 8;               // 16-byte chunks per K row
-    __shared__ __attribute__((aligned(16))) _Float16 lds_k[2][kTileKeys][KSTR];
-    __shared__ __attribute__((aligned(16))) _Float16 lds_v[2][HD][VSTR];
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
 
+template <int HD>
+struct PrefillSmem {
+    // 16-byte row pads make the 128-bit LDS reads of the MFMA operands conflict free
+    _Float16 k[2][kTileKeys][HD + 8];
+    _Float16 v[2][HD][kVBlock + 8];
+};
+
+// One 16-byte chunk per thread and slot: a tile is HD/64 chunks of K and of Vt per thread.
+template <int HD>
+struct PrefillStage {
+    u32x4 k[HD / 64], v[HD / 64];
+};
+
+template <int HD>
+__device__ __forceinline__ void prefill_fetch(PrefillStage<HD>& st, const uint16_t* kbase,
+                                              const uint16_t* vtbase, uint32_t tile, int tid)
+{
+    const u32x4* ksrc = reinterpret_cast<const u32x4*>(kbase + (size_t)tile * kTileKeys * HD);
+    const u32x4* vsrc = reinterpret_cast<const u32x4*>(vtbase + (size_t)tile * HD * kVBlock);
+#pragma unroll
+    for (int c = 0; c < HD / 64; c++) {
+        st.k[c] = ksrc[tid + c * kPrefillThreads];
+        st.v[c] = vsrc[tid + c * kPrefillThreads];
+    }
+}
+
+template <int HD>
+__device__ __forceinline__ void prefill_stash(PrefillSmem<HD>& sm, int buf,
+                                              const PrefillStage<HD>& st, uint32_t tile,
+                                              uint32_t kv_valid, int tid)
+{
+    constexpr int KCH = HD / 8;                           // 16-byte chunks per K row
+    const bool tail = (tile + 1) * kTileKeys > kv_valid;  // tile reaches past the appended rows
+#pragma unroll
+    for (int c = 0; c < HD / 64; c++) {
+        const int ch = tid + c * kPrefillThreads;
+        *reinterpret_cast<u32x4*>(&sm.k[buf][ch / KCH][(ch % KCH) * 8]) = st.k[c];
+        u32x4 v = st.v[c];
+        if (tail) {
+            // rows that were never appended may hold anything: zero them so
+            // 0 * garbage cannot reach the accumulator
+            const uint32_t key0 = tile * kTileKeys + (ch & 3) * 8;
+            uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                if (key0 + 2 * e >= kv_valid) w[e] &= 0xFFFF0000u;
+                if (key0 + 2 * e + 1 >= kv_valid) w[e] &= 0x0000FFFFu;
+            }
+            v = u32x4{w[0], w[1], w[2], w[3]};
+        }
+        *reinterpret_cast<u32x4*>(&sm.v[buf][ch >> 2][(ch & 3) * 8]) = v;
+    }
+}
+
+// Per-wave state of one block of 32 query rows.
+template <int HD>
+struct PrefillRows {
+    half8 qop[HD / 16];      // Q^T operand: column = this lane's row
+    f32x16 o[HD / 32];       // O^T accumulators: dim = dt*32 + 8*(r/4) + 4g + r%4
+    float m_run, l_run;
+    uint32_t pos, row_lo;            // this lane's absolute position and window floor
+    uint32_t w_first_pos, w_hi_lo;   // wave-wide: first row's position, last row's window floor
+    uint32_t wt_first, wt_last;      // tiles this wave takes part in
+    bool wave_ok;
+#ifdef WR_PREFILL_PROF
+    unsigned long long t_qk = 0, t_sm = 0, t_pv = 0, n_tiles = 0;
+#endif
+};
+
+template <int HD>
+__device__ __forceinline__ void prefill_compute(PrefillRows<HD>& R, const PrefillSmem<HD>& sm,
+                                                int buf, uint32_t tile, int n, int g, int krow)
+{
+    if (!R.wave_ok || tile < R.wt_first || tile > R.wt_last) return;
+    const uint32_t kb = tile * kTileKeys;
+#ifdef WR_PREFILL_PROF
+    const unsigned long long c0 = clock64();
+#endif
+    // two independent accumulator chains keep the matrix pipe from waiting on
+    // its own previous result
+    f32x16 c, c_odd;
+#pragma unroll
+    for (int r = 0; r < 16; r++) c[r] = c_odd[r] = 0.f;
+    // all K fragments of the tile are requested before the first MFMA, so the
+    // LDS latency is paid once, not once per contraction step
+    half8 kf[HD / 16];
+#pragma unroll
+    for (int s = 0; s < HD / 16; s++)
+        kf[s] = *reinterpret_cast<const half8*>(&sm.k[buf][krow][s * 16 + g * 8]);
+#pragma unroll
+    for (int s = 0; s < HD / 16; s += 2) {
+        c = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[s], R.qop[s], c, 0, 0, 0);
+        c_odd = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[s + 1], R.qop[s + 1], c_odd, 0, 0, 0);
+    }
+#pragma unroll
+    for (int r = 0; r < 16; r++) c[r] += c_odd[r];
+    // register r of this lane: key kb + 16*(r/8) + 8*g + r%8, row n.
+    // Some (row, key) pair of the tile is invisible: above the diagonal of the
+    // wave's first row, or below the window of its last row.
+    const bool edge = (kb + kTileKeys - 1 > R.w_first_pos) || (kb < R.w_hi_lo);
+    if (edge) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const uint32_t key = kb + 16 * (r >> 3) + 8 * g + (r & 7);
+            if (key > R.pos || key < R.row_lo) c[r] = -INFINITY;
+        }
+    }
+#ifdef WR_PREFILL_PROF
+    asm volatile("s_nop 0" :: "v"(c[0]), "v"(c[15]));
+    const unsigned long long c1 = clock64();
+#endif
+    float tmax = c[0];
+#pragma unroll
+    for (int r = 1; r < 16; r++) tmax = fmaxf(tmax, c[r]);
+    tmax = fmaxf(tmax, wave_xor_f32(tmax, 32));
+    // Lazy reference point: m_run only moves when a row's maximum exceeds it by
+    // more than kLazyLog2 (log2 units).  Until then later tiles' probabilities
+    // are taken relative to the stale reference (at most 2^kLazyLog2, far inside
+    // F16 range) and the accumulators need no rescale; O / l is unchanged, only
+    // the common factor differs.  With 32 independent rows per wave an eager
+    // maximum moves in most tiles, so this takes the 64-register rescale out of
+    // the steady state.
+    const bool jump = tmax > R.m_run + kLazyLog2;          // false for tmax = -inf
+    const float m_new = jump ? tmax : R.m_run;
+    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;   // row with nothing visible yet
+
+    half8 pop[2];
+    float psum = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        const float p = fast_exp2(c[r] - m_safe);
+        psum += p;
+        pop[r >> 3][r & 7] = (_Float16)p;
+    }
+    if (__builtin_amdgcn_ballot_w64(jump) != 0) {
+        const float alpha = jump ? fast_exp2(R.m_run - m_safe) : 1.0f;
+        R.l_run *= alpha;
+#pragma unroll
+        for (int dt = 0; dt < HD / 32; dt++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) R.o[dt][r] *= alpha;
+    }
+    R.m_run = m_new;
+    R.l_run += psum;
+#ifdef WR_PREFILL_PROF
+    asm volatile("s_nop 0" :: "v"(pop[0][0]), "v"(pop[1][7]), "v"(R.o[0][0]));
+    const unsigned long long c2 = clock64();
+#endif
+    // contraction step outermost: consecutive MFMAs hit different accumulators
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+#pragma unroll
+        for (int dt = 0; dt < HD / 32; dt++) {
+            const half8 vf =
+                *reinterpret_cast<const half8*>(&sm.v[buf][dt * 32 + n][16 * t + 8 * g]);
+            R.o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pop[t], R.o[dt], 0, 0, 0);
+        }
+    }
+#ifdef WR_PREFILL_PROF
+    asm volatile("s_nop 0" :: "v"(R.o[0][0]), "v"(R.o[HD / 32 - 1][15]));
+    const unsigned long long c3 = clock64();
+    R.t_qk += c1 - c0; R.t_sm += c2 - c1; R.t_pv += c3 - c2; R.n_tiles++;
+#endif
+}
+
+// One position block of one workgroup: loads Q, streams the visible K / Vt
+// tiles (two tiles of global loads in flight ahead of the one being computed),
+// writes the rows.
+template <int HD>
+__device__ __forceinline__ void prefill_block(const PrefillArgs& a, PrefillSmem<HD>& sm,
+                                              uint32_t pb, uint32_t kvh, uint32_t hc)
+{
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int n = lane & 31, g = lane >> 5;
+#ifdef WR_PREFILL_PROF
+    const unsigned long long t_block0 = clock64();
+#endif
     const uint32_t G = a.group;
     const uint32_t Gw = G < 4 ? G : 4;
-    const uint32_t chunks = G / Gw;                       // head chunks per KV head (1, or 2 for G = 8)
-    const uint32_t kvh = blockIdx.y / chunks, hc = blockIdx.y % chunks;
-    const uint32_t BP = 32 * (4 / Gw);                    // positions per workgroup
-    const uint32_t pb = gridDim.x - 1 - blockIdx.x;       // heaviest block first
+    const uint32_t BP = 32 * (4 / Gw);                    // positions per block
     const uint32_t head = kvh * G + hc * Gw + (wave % Gw);
     const uint32_t row0 = pb * BP + (wave / Gw) * 32;     // first chunk row of this wave
     const uint32_t T = a.T, p0 = a.p0;
@@ -95,156 +270,91 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_mfma_kernel(const 
 
     const uint32_t my_row = row0 + n;
     const bool row_ok = my_row < T;
-    const uint32_t pos = p0 + (row_ok ? my_row : T - 1);  // absolute position (clamped for idle rows)
-    const uint32_t row_lo = (a.window > 0 && pos + 1 > a.window) ? pos + 1 - a.window : 0;
+    PrefillRows<HD> R;
+    R.pos = p0 + (row_ok ? my_row : T - 1);               // clamped for idle rows
+    R.row_lo = (a.window > 0 && R.pos + 1 > a.window) ? R.pos + 1 - a.window : 0;
 
-    // workgroup-wide tile range
+    // block-wide tile range
     const uint32_t wg_last_row = min(T, (pb + 1) * BP) - 1;
     const uint32_t wg_first_pos = p0 + pb * BP;
-    const uint32_t wg_lo = (a.window > 0 && wg_first_pos + 1 > a.window) ? wg_first_pos + 1 - a.window : 0;
+    const uint32_t wg_lo =
+        (a.window > 0 && wg_first_pos + 1 > a.window) ? wg_first_pos + 1 - a.window : 0;
     const uint32_t t_first = wg_lo / kTileKeys;
     const uint32_t t_last = (p0 + wg_last_row) / kTileKeys;          // inclusive
     // this wave's own range (a wave with no valid row computes nothing)
-    const bool wave_ok = row0 < T;
+    R.wave_ok = row0 < T;
     const uint32_t w_last_pos = p0 + min(T - 1, row0 + 31);
-    const uint32_t w_first_pos = p0 + row0;
-    const uint32_t w_lo = (a.window > 0 && w_first_pos + 1 > a.window) ? w_first_pos + 1 - a.window : 0;
-    const uint32_t wt_first = w_lo / kTileKeys;
-    const uint32_t wt_last = w_last_pos / kTileKeys;
+    R.w_first_pos = p0 + row0;
+    const uint32_t w_lo =
+        (a.window > 0 && R.w_first_pos + 1 > a.window) ? R.w_first_pos + 1 - a.window : 0;
+    R.w_hi_lo = (a.window > 0 && w_last_pos + 1 > a.window) ? w_last_pos + 1 - a.window : 0;
+    R.wt_first = w_lo / kTileKeys;
+    R.wt_last = w_last_pos / kTileKeys;
 
-    // Q^T operand: column n = this lane's row, contraction slots (g, j) = dims s*16 + g*8 + j
-    half8 qop[HD / 16];
+    const uint16_t* kbase = a.k + (size_t)kvh * a.ctx_pad * HD;
+    const uint16_t* vtbase = a.vt + (size_t)kvh * (a.ctx_pad / kVBlock) * HD * kVBlock;
+    PrefillStage<HD> s0, s1;
+    uint32_t tile = t_first;
+    prefill_fetch<HD>(s0, kbase, vtbase, tile, tid);
+    if constexpr (HD < 256)
+        if (tile + 1 <= t_last) prefill_fetch<HD>(s1, kbase, vtbase, tile + 1, tid);
+
+    // Q^T operand: contraction slots (g, j) = dims s*16 + g*8 + j, pre-scaled
     {
         const float* qrow = a.q + ((size_t)(row_ok ? my_row : T - 1) * a.nq + head) * HD;
 #pragma unroll
         for (int s = 0; s < HD / 16; s++) {
             const float4 x0 = *reinterpret_cast<const float4*>(qrow + s * 16 + g * 8);
             const float4 x1 = *reinterpret_cast<const float4*>(qrow + s * 16 + g * 8 + 4);
-            qop[s][0] = (_Float16)(x0.x * a.qscale);
-            qop[s][1] = (_Float16)(x0.y * a.qscale);
-            qop[s][2] = (_Float16)(x0.z * a.qscale);
-            qop[s][3] = (_Float16)(x0.w * a.qscale);
-            qop[s][4] = (_Float16)(x1.x * a.qscale);
-            qop[s][5] = (_Float16)(x1.y * a.qscale);
-            qop[s][6] = (_Float16)(x1.z * a.qscale);
-            qop[s][7] = (_Float16)(x1.w * a.qscale);
+            R.qop[s][0] = (_Float16)(x0.x * a.qscale);
+            R.qop[s][1] = (_Float16)(x0.y * a.qscale);
+            R.qop[s][2] = (_Float16)(x0.z * a.qscale);
+            R.qop[s][3] = (_Float16)(x0.w * a.qscale);
+            R.qop[s][4] = (_Float16)(x1.x * a.qscale);
+            R.qop[s][5] = (_Float16)(x1.y * a.qscale);
+            R.qop[s][6] = (_Float16)(x1.z * a.qscale);
+            R.qop[s][7] = (_Float16)(x1.w * a.qscale);
         }
     }
-
-    f32x16 o[HD / 32];
 #pragma unroll
     for (int dt = 0; dt < HD / 32; dt++)
 #pragma unroll
-        for (int r = 0; r < 16; r++) o[dt][r] = 0.f;
-    float m_run = -INFINITY, l_run = 0.f;
-
-    const uint16_t* kbase = a.k + (size_t)kvh * a.ctx_pad * HD;
-    const uint16_t* vtbase = a.vt + (size_t)kvh * (a.ctx_pad / kVBlock) * HD * kVBlock;
+        for (int r = 0; r < 16; r++) R.o[dt][r] = 0.f;
+    R.m_run = -INFINITY;
+    R.l_run = 0.f;
     const int krow = prefill_key_perm(n);                 // LDS row this lane feeds to MFMA row n
 
-    // staging registers: each thread moves HD/64 16-byte chunks of K and of Vt per tile
-    constexpr int NCH = HD / 64;
-    u32x4 stage_k[NCH], stage_v[NCH];
-    auto fetch = [&](uint32_t tile) {
-        const u32x4* ksrc = reinterpret_cast<const u32x4*>(kbase + (size_t)tile * kTileKeys * HD);
-        const u32x4* vsrc = reinterpret_cast<const u32x4*>(vtbase + (size_t)tile * HD * kVBlock);
-#pragma unroll
-        for (int c = 0; c < NCH; c++) {
-            stage_k[c] = ksrc[tid + c * kPrefillThreads];
-            stage_v[c] = vsrc[tid + c * kPrefillThreads];
+    if constexpr (HD >= 256) {
+        // wide heads: one staging set (the second would not fit the register file)
+        for (int buf = 0;; buf ^= 1) {
+            prefill_stash<HD>(sm, buf, s0, tile, kv_valid, tid);
+            lds_barrier();
+            if (tile + 1 <= t_last) prefill_fetch<HD>(s0, kbase, vtbase, tile + 1, tid);
+            prefill_compute<HD>(R, sm, buf, tile, n, g, krow);
+            if (++tile > t_last) break;
         }
-    };
-    auto stash = [&](int buf, uint32_t tile) {
-        const bool tail = (tile + 1) * kTileKeys > kv_valid;    // tile reaches past the appended rows
-#pragma unroll
-        for (int c = 0; c < NCH; c++) {
-            const int ch = tid + c * kPrefillThreads;
-            *reinterpret_cast<u32x4*>(&lds_k[buf][ch / KCH][(ch % KCH) * 8]) = stage_k[c];
-            u32x4 v = stage_v[c];
-            if (tail) {
-                // rows that were never appended may hold anything: zero them so
-                // 0 * garbage cannot reach the accumulator
-                const uint32_t key0 = tile * kTileKeys + (ch & 3) * 8;
-                uint32_t w[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    if (key0 + 2 * e >= kv_valid) w[e] &= 0xFFFF0000u;
-                    if (key0 + 2 * e + 1 >= kv_valid) w[e] &= 0x0000FFFFu;
-                }
-                v = u32x4{w[0], w[1], w[2], w[3]};
-            }
-            *reinterpret_cast<u32x4*>(&lds_v[buf][ch >> 2][(ch & 3) * 8]) = v;
-        }
-    };
-
-    fetch(t_first);
-    int buf = 0;
-    for (uint32_t tile = t_first; tile <= t_last; tile++, buf ^= 1) {
-        stash(buf, tile);
-        __syncthreads();
-        if (tile < t_last) fetch(tile + 1);
-        if (!wave_ok || tile < wt_first || tile > wt_last) continue;
-
-        const uint32_t kb = tile * kTileKeys;
-        f32x16 c;
-#pragma unroll
-        for (int r = 0; r < 16; r++) c[r] = 0.f;
-#pragma unroll
-        for (int s = 0; s < HD / 16; s++) {
-            const half8 kf = *reinterpret_cast<const half8*>(&lds_k[buf][krow][s * 16 + g * 8]);
-            c = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qop[s], c, 0, 0, 0);
-        }
-        // register r of this lane: key kb + 16*(r/8) + 8*g + r%8, row n
-        // some (row, key) pair of this tile is invisible: above the diagonal of
-        // the wave's first row, or below the window of its last row
-        const uint32_t w_hi_lo =
-            (a.window > 0 && w_last_pos + 1 > a.window) ? w_last_pos + 1 - a.window : 0;
-        const bool edge = (kb + kTileKeys - 1 > w_first_pos) || (kb < w_hi_lo);
-        if (edge) {
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const uint32_t key = kb + 16 * (r >> 3) + 8 * g + (r & 7);
-                if (key > pos || key < row_lo) c[r] = -INFINITY;
-            }
-        }
-        float tmax = c[0];
-#pragma unroll
-        for (int r = 1; r < 16; r++) tmax = fmaxf(tmax, c[r]);
-        tmax = fmaxf(tmax, wave_xor_f32(tmax, 32));
-        const float m_new = fmaxf(m_run, tmax);
-        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;   // row with nothing visible yet
-        const float alpha = fast_exp2(m_run - m_safe);
-        m_run = m_new;
-
-        half8 pop[2];
-        float psum = 0.f;
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-            const float p = fast_exp2(c[r] - m_safe);
-            psum += p;
-            pop[r >> 3][r & 7] = (_Float16)p;
-        }
-        l_run = l_run * alpha + psum;
-
-        // rescale only when some row's maximum moved (wave-uniform test)
-        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
-#pragma unroll
-            for (int dt = 0; dt < HD / 32; dt++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) o[dt][r] *= alpha;
-        }
-#pragma unroll
-        for (int dt = 0; dt < HD / 32; dt++) {
-#pragma unroll
-            for (int t = 0; t < 2; t++) {
-                const half8 vf =
-                    *reinterpret_cast<const half8*>(&lds_v[buf][dt * 32 + n][16 * t + 8 * g]);
-                o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pop[t], o[dt], 0, 0, 0);
-            }
+    } else {
+        for (;;) {
+            prefill_stash<HD>(sm, 0, s0, tile, kv_valid, tid);
+            lds_barrier();
+            if (tile + 2 <= t_last) prefill_fetch<HD>(s0, kbase, vtbase, tile + 2, tid);
+            prefill_compute<HD>(R, sm, 0, tile, n, g, krow);
+            if (++tile > t_last) break;
+            prefill_stash<HD>(sm, 1, s1, tile, kv_valid, tid);
+            lds_barrier();
+            if (tile + 2 <= t_last) prefill_fetch<HD>(s1, kbase, vtbase, tile + 2, tid);
+            prefill_compute<HD>(R, sm, 1, tile, n, g, krow);
+            if (++tile > t_last) break;
         }
     }
 
-    const float l_tot = l_run + wave_xor_f32(l_run, 32);
+#ifdef WR_PREFILL_PROF
+    if (a.prof && blockIdx.x == 0 && blockIdx.y == 0 && lane == 0 && wave == 0) {
+        a.prof[0] += R.t_qk; a.prof[1] += R.t_sm; a.prof[2] += R.t_pv; a.prof[3] += R.n_tiles;
+        a.prof[4] += clock64() - t_block0;
+    }
+#endif
+    const float l_tot = R.l_run + wave_xor_f32(R.l_run, 32);
     const float inv = (l_tot > 0.f) ? 1.0f / l_tot : 0.f;
     if (row_ok) {
         float* orow = a.out + ((size_t)my_row * a.nq + head) * HD;
@@ -253,13 +363,34 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_mfma_kernel(const 
 #pragma unroll
             for (int q4 = 0; q4 < 4; q4++) {
                 float4 v;
-                v.x = o[dt][4 * q4 + 0] * inv;
-                v.y = o[dt][4 * q4 + 1] * inv;
-                v.z = o[dt][4 * q4 + 2] * inv;
-                v.w = o[dt][4 * q4 + 3] * inv;
+                v.x = R.o[dt][4 * q4 + 0] * inv;
+                v.y = R.o[dt][4 * q4 + 1] * inv;
+                v.z = R.o[dt][4 * q4 + 2] * inv;
+                v.w = R.o[dt][4 * q4 + 3] * inv;
                 *reinterpret_cast<float4*>(orow + dt * 32 + 8 * q4 + 4 * g) = v;
             }
         }
+    }
+}
+
+// grid = (ceil(blocks / 2), KV heads x head chunks).  Workgroup x takes position
+// block (blocks-1-x) and then block x: a long block and a short one, so every
+// workgroup streams the same number of tiles despite the causal triangle.
+template <int HD>
+__global__ __launch_bounds__(kPrefillThreads, 2) void prefill_mfma_kernel(const PrefillArgs a)
+{
+    __shared__ __attribute__((aligned(16))) PrefillSmem<HD> sm;
+    const uint32_t G = a.group;
+    const uint32_t Gw = G < 4 ? G : 4;
+    const uint32_t chunks = G / Gw;                       // head chunks per KV head (1, or 2 for G = 8)
+    const uint32_t kvh = blockIdx.y / chunks, hc = blockIdx.y % chunks;
+    const uint32_t BP = 32 * (4 / Gw);
+    const uint32_t nblk = (a.T + BP - 1) / BP;
+    const uint32_t lo = blockIdx.x, hi = nblk - 1 - blockIdx.x;
+    prefill_block<HD>(a, sm, hi, kvh, hc);
+    if (hi != lo) {
+        __syncthreads();                                  // LDS buffers change hands
+        prefill_block<HD>(a, sm, lo, kvh, hc);
     }
 }
 

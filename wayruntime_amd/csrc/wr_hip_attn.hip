@@ -344,13 +344,20 @@ int prefill_locked(wr_hip_kv* kv, uint32_t layer, uint32_t p0, uint32_t T, const
     a.window = window;
     const float scale = (scale_override > 0.0f) ? scale_override : 1.0f / sqrtf((float)hd);
     a.qscale = scale * kLog2e;
+#ifdef WR_PREFILL_PROF
+    static unsigned long long* prof = nullptr;
+    if (!prof) { (void)hipMalloc((void**)&prof, 64); }
+    (void)hipMemsetAsync(prof, 0, 64, g.stream);
+    a.prof = prof;
+#endif
     const uint32_t G = a.group;
     const bool mfma = !g.force_generic && (hd == 64 || hd == 128 || hd == 256) &&
                       (G == 1 || G == 2 || G == 4 || G == 8);
     if (mfma) {
         const uint32_t Gw = G < 4 ? G : 4;
         const uint32_t BP = 32 * (4 / Gw);
-        const dim3 grid((T + BP - 1) / BP, kv->nkv * (G / Gw)), block(kPrefillThreads);
+        const uint32_t nblk = (T + BP - 1) / BP;
+        const dim3 grid((nblk + 1) / 2, kv->nkv * (G / Gw)), block(kPrefillThreads);
         if (hd == 64)
             launch_main(prefill_mfma_kernel<64>, grid, block, a);
         else if (hd == 128)
@@ -361,6 +368,15 @@ int prefill_locked(wr_hip_kv* kv, uint32_t layer, uint32_t p0, uint32_t T, const
         launch_main(prefill_generic_kernel, dim3(T, nq), dim3(kDecodeThreads), a);
     }
     HIP_TRY(hipGetLastError(), "prefill launch", layer);
+#ifdef WR_PREFILL_PROF
+    {
+        unsigned long long h[8];
+        (void)hipMemcpyAsync(h, a.prof, 64, hipMemcpyDeviceToHost, g.stream);
+        (void)hipStreamSynchronize(g.stream);
+        fprintf(stderr, "prof: tiles %llu  qk %.0f  softmax %.0f  pv %.0f  block total/tile %.0f clk\n", h[3],
+                (double)h[0] / h[3], (double)h[1] / h[3], (double)h[2] / h[3], (double)h[4] / h[3]);
+    }
+#endif
     g.calls.fetch_add(T, std::memory_order_relaxed);
     return WR_HIP_OK;
 }
