@@ -31,6 +31,15 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0           # MI355X HBM3E
 MFMA_F16_PEAK_TFLOPS = 2500.0   # MI355X dense f16
 
+# HBM bytes one launch of decode_mfma_kernel<128> moves on the default workload
+# (16 sessions x 4096 ctx): rocprofv3 FETCH_SIZE + WRITE_SIZE per dispatch, each
+# scaled by what the same counter reads for a plain 256 MiB copy kernel
+# (FETCH_SIZE x 1.9998 KiB, WRITE_SIZE x 1.0000 KiB).  Counters cannot be read
+# from inside this process, so the figure is carried here from the committed
+# counter summary (profiles/decode_prefill_traffic_pmc.txt) and reported only
+# for the workload it was measured on.
+PMC_TRAFFIC_BYTES = {(16, 4096): 270288670 + 863119}
+
 
 def pooled16(pool16: np.ndarray, salt: int, n: int) -> np.ndarray:
     """n F16 bit patterns drawn from a pool of truncated N(0,1) samples at a
@@ -141,7 +150,7 @@ def main() -> None:
     achieved = bytes_per_step / (kern_avg_ms * 1e-3) / 1e9
     roofline = {"bound": "hbm", "kernel": "decode_mfma_kernel<128>", "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                "traffic": None, "kernel_avg_us": round(kern_avg_ms * 1e3, 2),
+                "traffic": PMC_TRAFFIC_BYTES.get((S, ctx)), "kernel_avg_us": round(kern_avg_ms * 1e3, 2),
                 "bytes_per_launch": bytes_per_step}
 
     # ---- causal prefill (secondary figure of the metric)

@@ -61,9 +61,23 @@ def build_host() -> str:
     return HOST_SO
 
 
+CALIB_BIN = os.path.join(PKG, "calib_copy")
+
+
+def build_calib() -> str:
+    """Counter-calibration copy program (measurement aid, see csrc/calib_copy.hip)."""
+    res = subprocess.run(["hipcc", "-O3", "--offload-arch=gfx950", "-o", CALIB_BIN,
+                          os.path.join(PKG, "csrc", "calib_copy.hip")], capture_output=True, text=True)
+    if res.returncode != 0:
+        sys.stderr.write(res.stderr)
+        raise RuntimeError("hipcc failed building " + CALIB_BIN)
+    return CALIB_BIN
+
+
 def build_all(keep_temps: bool = False) -> None:
     build_hip(keep_temps)
     build_host()
+    build_calib()
 
 
 if __name__ == "__main__":
