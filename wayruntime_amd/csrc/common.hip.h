@@ -66,4 +66,32 @@ __device__ __forceinline__ float wave_xor_f32(float v, int mask)
     return __shfl_xor(v, mask, 64);
 }
 
+// The value lane ^ 32 holds, without going through LDS: v_permlane32_swap
+// exchanges the upper half of its first operand with the lower half of its
+// second, so with the same value in both the two results together hold, in
+// every lane, this lane's value and its partner's.
+__device__ __forceinline__ float wave_partner32(float v)
+{
+    const uint32_t u = __float_as_uint(v);
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    const bool upper = (__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)) & 32u) != 0;
+    return __uint_as_float(upper ? r[0] : r[1]);
+}
+
+// max / sum of this lane's value and lane ^ 32's (order-insensitive, so no
+// select is needed)
+__device__ __forceinline__ float wave_pair32_max(float v)
+{
+    const uint32_t u = __float_as_uint(v);
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+
+__device__ __forceinline__ float wave_pair32_sum(float v)
+{
+    const uint32_t u = __float_as_uint(v);
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 }  // namespace wr

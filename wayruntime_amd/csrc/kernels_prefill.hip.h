@@ -18,9 +18,6 @@ struct PrefillArgs {
     float* out;              // [T][nq][hd]
     uint32_t p0, T, nq, nkv, group, hd, ctx_pad, window;
     float qscale;            // softmax scale * log2(e)
-#ifdef WR_PREFILL_PROF
-    unsigned long long* prof;
-#endif
 };
 
 // Any head_dim / group: one workgroup per (row, head), vector ALU only.
@@ -146,38 +143,47 @@ struct PrefillRows {
     uint32_t w_first_pos, w_hi_lo;   // wave-wide: first row's position, last row's window floor
     uint32_t wt_first, wt_last;      // tiles this wave takes part in
     bool wave_ok;
-#ifdef WR_PREFILL_PROF
-    unsigned long long t_qk = 0, t_sm = 0, t_pv = 0, n_tiles = 0;
-#endif
 };
 
-template <int HD>
-__device__ __forceinline__ void prefill_compute(PrefillRows<HD>& R, const PrefillSmem<HD>& sm,
-                                                int buf, uint32_t tile, int n, int g, int krow)
+// ktile: the tile's 32 K rows, vtile: its Vt block, both with padded rows.
+// DUAL splits the score contraction over two accumulator chains (for kernels
+// that run one wave per SIMD and cannot hide the matrix pipe's latency behind
+// another wave).
+template <int HD, bool DUAL>
+__device__ __forceinline__ void prefill_compute(PrefillRows<HD>& R,
+                                                const _Float16 (*ktile)[HD + 8],
+                                                const _Float16 (*vtile)[kVBlock + 8],
+                                                uint32_t tile, int n, int g, int krow)
 {
     if (!R.wave_ok || tile < R.wt_first || tile > R.wt_last) return;
     const uint32_t kb = tile * kTileKeys;
-#ifdef WR_PREFILL_PROF
-    const unsigned long long c0 = clock64();
-#endif
-    // two independent accumulator chains keep the matrix pipe from waiting on
-    // its own previous result
-    f32x16 c, c_odd;
+    f32x16 c;
 #pragma unroll
-    for (int r = 0; r < 16; r++) c[r] = c_odd[r] = 0.f;
+    for (int r = 0; r < 16; r++) c[r] = 0.f;
     // all K fragments of the tile are requested before the first MFMA, so the
     // LDS latency is paid once, not once per contraction step
     half8 kf[HD / 16];
 #pragma unroll
     for (int s = 0; s < HD / 16; s++)
-        kf[s] = *reinterpret_cast<const half8*>(&sm.k[buf][krow][s * 16 + g * 8]);
+        kf[s] = *reinterpret_cast<const half8*>(&ktile[krow][s * 16 + g * 8]);
+    if constexpr (DUAL) {
+        // two independent accumulator chains keep the matrix pipe from waiting
+        // on its own previous result
+        f32x16 c_odd;
 #pragma unroll
-    for (int s = 0; s < HD / 16; s += 2) {
-        c = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[s], R.qop[s], c, 0, 0, 0);
-        c_odd = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[s + 1], R.qop[s + 1], c_odd, 0, 0, 0);
+        for (int r = 0; r < 16; r++) c_odd[r] = 0.f;
+#pragma unroll
+        for (int s = 0; s < HD / 16; s += 2) {
+            c = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[s], R.qop[s], c, 0, 0, 0);
+            c_odd = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[s + 1], R.qop[s + 1], c_odd, 0, 0, 0);
+        }
+#pragma unroll
+        for (int r = 0; r < 16; r++) c[r] += c_odd[r];
+    } else {
+#pragma unroll
+        for (int s = 0; s < HD / 16; s++)
+            c = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[s], R.qop[s], c, 0, 0, 0);
     }
-#pragma unroll
-    for (int r = 0; r < 16; r++) c[r] += c_odd[r];
     // register r of this lane: key kb + 16*(r/8) + 8*g + r%8, row n.
     // Some (row, key) pair of the tile is invisible: above the diagonal of the
     // wave's first row, or below the window of its last row.
@@ -189,14 +195,10 @@ __device__ __forceinline__ void prefill_compute(PrefillRows<HD>& R, const Prefil
             if (key > R.pos || key < R.row_lo) c[r] = -INFINITY;
         }
     }
-#ifdef WR_PREFILL_PROF
-    asm volatile("s_nop 0" :: "v"(c[0]), "v"(c[15]));
-    const unsigned long long c1 = clock64();
-#endif
     float tmax = c[0];
 #pragma unroll
     for (int r = 1; r < 16; r++) tmax = fmaxf(tmax, c[r]);
-    tmax = fmaxf(tmax, wave_xor_f32(tmax, 32));
+    tmax = wave_pair32_max(tmax);
     // Lazy reference point: m_run only moves when a row's maximum exceeds it by
     // more than kLazyLog2 (log2 units).  Until then later tiles' probabilities
     // are taken relative to the stale reference (at most 2^kLazyLog2, far inside
@@ -226,62 +228,31 @@ __device__ __forceinline__ void prefill_compute(PrefillRows<HD>& R, const Prefil
     }
     R.m_run = m_new;
     R.l_run += psum;
-#ifdef WR_PREFILL_PROF
-    asm volatile("s_nop 0" :: "v"(pop[0][0]), "v"(pop[1][7]), "v"(R.o[0][0]));
-    const unsigned long long c2 = clock64();
-#endif
     // contraction step outermost: consecutive MFMAs hit different accumulators
 #pragma unroll
     for (int t = 0; t < 2; t++) {
 #pragma unroll
         for (int dt = 0; dt < HD / 32; dt++) {
             const half8 vf =
-                *reinterpret_cast<const half8*>(&sm.v[buf][dt * 32 + n][16 * t + 8 * g]);
+                *reinterpret_cast<const half8*>(&vtile[dt * 32 + n][16 * t + 8 * g]);
             R.o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pop[t], R.o[dt], 0, 0, 0);
         }
     }
-#ifdef WR_PREFILL_PROF
-    asm volatile("s_nop 0" :: "v"(R.o[0][0]), "v"(R.o[HD / 32 - 1][15]));
-    const unsigned long long c3 = clock64();
-    R.t_qk += c1 - c0; R.t_sm += c2 - c1; R.t_pv += c3 - c2; R.n_tiles++;
-#endif
 }
 
-// One position block of one workgroup: loads Q, streams the visible K / Vt
-// tiles (two tiles of global loads in flight ahead of the one being computed),
-// writes the rows.
-template <int HD>
-__device__ __forceinline__ void prefill_block(const PrefillArgs& a, PrefillSmem<HD>& sm,
-                                              uint32_t pb, uint32_t kvh, uint32_t hc)
+// Sets up a wave's 32 rows starting at chunk row `row0` for `head`: positions,
+// window floors, tile range, empty accumulators and (LOADQ) the Q^T operand,
+// read straight from global memory, each lane its own row.
+template <int HD, bool LOADQ = true>
+__device__ __forceinline__ void prefill_rows_init(PrefillRows<HD>& R, const PrefillArgs& a,
+                                                  uint32_t row0, uint32_t head, int n, int g)
 {
-    const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
-    const int n = lane & 31, g = lane >> 5;
-#ifdef WR_PREFILL_PROF
-    const unsigned long long t_block0 = clock64();
-#endif
-    const uint32_t G = a.group;
-    const uint32_t Gw = G < 4 ? G : 4;
-    const uint32_t BP = 32 * (4 / Gw);                    // positions per block
-    const uint32_t head = kvh * G + hc * Gw + (wave % Gw);
-    const uint32_t row0 = pb * BP + (wave / Gw) * 32;     // first chunk row of this wave
     const uint32_t T = a.T, p0 = a.p0;
-    const uint32_t kv_valid = p0 + T;                     // rows of the cache that hold data
-
     const uint32_t my_row = row0 + n;
     const bool row_ok = my_row < T;
-    PrefillRows<HD> R;
     R.pos = p0 + (row_ok ? my_row : T - 1);               // clamped for idle rows
     R.row_lo = (a.window > 0 && R.pos + 1 > a.window) ? R.pos + 1 - a.window : 0;
-
-    // block-wide tile range
-    const uint32_t wg_last_row = min(T, (pb + 1) * BP) - 1;
-    const uint32_t wg_first_pos = p0 + pb * BP;
-    const uint32_t wg_lo =
-        (a.window > 0 && wg_first_pos + 1 > a.window) ? wg_first_pos + 1 - a.window : 0;
-    const uint32_t t_first = wg_lo / kTileKeys;
-    const uint32_t t_last = (p0 + wg_last_row) / kTileKeys;          // inclusive
-    // this wave's own range (a wave with no valid row computes nothing)
+    // this wave's own tile range (a wave with no valid row computes nothing)
     R.wave_ok = row0 < T;
     const uint32_t w_last_pos = p0 + min(T - 1, row0 + 31);
     R.w_first_pos = p0 + row0;
@@ -291,17 +262,9 @@ __device__ __forceinline__ void prefill_block(const PrefillArgs& a, PrefillSmem<
     R.wt_first = w_lo / kTileKeys;
     R.wt_last = w_last_pos / kTileKeys;
 
-    const uint16_t* kbase = a.k + (size_t)kvh * a.ctx_pad * HD;
-    const uint16_t* vtbase = a.vt + (size_t)kvh * (a.ctx_pad / kVBlock) * HD * kVBlock;
-    PrefillStage<HD> s0, s1;
-    uint32_t tile = t_first;
-    prefill_fetch<HD>(s0, kbase, vtbase, tile, tid);
-    if constexpr (HD < 256)
-        if (tile + 1 <= t_last) prefill_fetch<HD>(s1, kbase, vtbase, tile + 1, tid);
-
     // Q^T operand: contraction slots (g, j) = dims s*16 + g*8 + j, pre-scaled
-    {
-        const float* qrow = a.q + ((size_t)(row_ok ? my_row : T - 1) * a.nq + head) * HD;
+    const float* qrow = a.q + ((size_t)(row_ok ? my_row : T - 1) * a.nq + head) * HD;
+    if constexpr (LOADQ) {
 #pragma unroll
         for (int s = 0; s < HD / 16; s++) {
             const float4 x0 = *reinterpret_cast<const float4*>(qrow + s * 16 + g * 8);
@@ -322,41 +285,17 @@ __device__ __forceinline__ void prefill_block(const PrefillArgs& a, PrefillSmem<
         for (int r = 0; r < 16; r++) R.o[dt][r] = 0.f;
     R.m_run = -INFINITY;
     R.l_run = 0.f;
-    const int krow = prefill_key_perm(n);                 // LDS row this lane feeds to MFMA row n
+}
 
-    if constexpr (HD >= 256) {
-        // wide heads: one staging set (the second would not fit the register file)
-        for (int buf = 0;; buf ^= 1) {
-            prefill_stash<HD>(sm, buf, s0, tile, kv_valid, tid);
-            lds_barrier();
-            if (tile + 1 <= t_last) prefill_fetch<HD>(s0, kbase, vtbase, tile + 1, tid);
-            prefill_compute<HD>(R, sm, buf, tile, n, g, krow);
-            if (++tile > t_last) break;
-        }
-    } else {
-        for (;;) {
-            prefill_stash<HD>(sm, 0, s0, tile, kv_valid, tid);
-            lds_barrier();
-            if (tile + 2 <= t_last) prefill_fetch<HD>(s0, kbase, vtbase, tile + 2, tid);
-            prefill_compute<HD>(R, sm, 0, tile, n, g, krow);
-            if (++tile > t_last) break;
-            prefill_stash<HD>(sm, 1, s1, tile, kv_valid, tid);
-            lds_barrier();
-            if (tile + 2 <= t_last) prefill_fetch<HD>(s1, kbase, vtbase, tile + 2, tid);
-            prefill_compute<HD>(R, sm, 1, tile, n, g, krow);
-            if (++tile > t_last) break;
-        }
-    }
-
-#ifdef WR_PREFILL_PROF
-    if (a.prof && blockIdx.x == 0 && blockIdx.y == 0 && lane == 0 && wave == 0) {
-        a.prof[0] += R.t_qk; a.prof[1] += R.t_sm; a.prof[2] += R.t_pv; a.prof[3] += R.n_tiles;
-        a.prof[4] += clock64() - t_block0;
-    }
-#endif
-    const float l_tot = R.l_run + wave_xor_f32(R.l_run, 32);
+// Normalises and writes a wave's rows.
+template <int HD>
+__device__ __forceinline__ void prefill_rows_store(const PrefillRows<HD>& R, const PrefillArgs& a,
+                                                   uint32_t row0, uint32_t head, int n, int g)
+{
+    const float l_tot = wave_pair32_sum(R.l_run);
     const float inv = (l_tot > 0.f) ? 1.0f / l_tot : 0.f;
-    if (row_ok) {
+    const uint32_t my_row = row0 + n;
+    if (my_row < a.T) {
         float* orow = a.out + ((size_t)my_row * a.nq + head) * HD;
 #pragma unroll
         for (int dt = 0; dt < HD / 32; dt++) {
@@ -371,6 +310,75 @@ __device__ __forceinline__ void prefill_block(const PrefillArgs& a, PrefillSmem<
             }
         }
     }
+}
+
+// Tile range a block of positions [pb*BP, (pb+1)*BP) streams.
+__device__ __forceinline__ void prefill_block_tiles(const PrefillArgs& a, uint32_t pb, uint32_t BP,
+                                                    uint32_t& t_first, uint32_t& t_last)
+{
+    const uint32_t wg_last_row = min(a.T, (pb + 1) * BP) - 1;
+    const uint32_t wg_first_pos = a.p0 + pb * BP;
+    const uint32_t wg_lo =
+        (a.window > 0 && wg_first_pos + 1 > a.window) ? wg_first_pos + 1 - a.window : 0;
+    t_first = wg_lo / kTileKeys;
+    t_last = (a.p0 + wg_last_row) / kTileKeys;            // inclusive
+}
+
+// One position block of one workgroup: loads Q, streams the visible K / Vt
+// tiles (two tiles of global loads in flight ahead of the one being computed),
+// writes the rows.
+template <int HD>
+__device__ __forceinline__ void prefill_block(const PrefillArgs& a, PrefillSmem<HD>& sm,
+                                              uint32_t pb, uint32_t kvh, uint32_t hc)
+{
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int n = lane & 31, g = lane >> 5;
+    const uint32_t G = a.group;
+    const uint32_t Gw = G < 4 ? G : 4;
+    const uint32_t BP = 32 * (4 / Gw);                    // positions per block
+    const uint32_t head = kvh * G + hc * Gw + (wave % Gw);
+    const uint32_t row0 = pb * BP + (wave / Gw) * 32;     // first chunk row of this wave
+    const uint32_t kv_valid = a.p0 + a.T;                 // rows of the cache that hold data
+    uint32_t t_first, t_last;
+    prefill_block_tiles(a, pb, BP, t_first, t_last);
+
+    const uint16_t* kbase = a.k + (size_t)kvh * a.ctx_pad * HD;
+    const uint16_t* vtbase = a.vt + (size_t)kvh * (a.ctx_pad / kVBlock) * HD * kVBlock;
+    PrefillStage<HD> s0, s1;
+    uint32_t tile = t_first;
+    prefill_fetch<HD>(s0, kbase, vtbase, tile, tid);
+    if constexpr (HD < 256)
+        if (tile + 1 <= t_last) prefill_fetch<HD>(s1, kbase, vtbase, tile + 1, tid);
+
+    PrefillRows<HD> R;
+    prefill_rows_init<HD>(R, a, row0, head, n, g);
+    const int krow = prefill_key_perm(n);                 // LDS row this lane feeds to MFMA row n
+
+    if constexpr (HD >= 256) {
+        // wide heads: one staging set (the second would not fit the register file)
+        for (int buf = 0;; buf ^= 1) {
+            prefill_stash<HD>(sm, buf, s0, tile, kv_valid, tid);
+            lds_barrier();
+            if (tile + 1 <= t_last) prefill_fetch<HD>(s0, kbase, vtbase, tile + 1, tid);
+            prefill_compute<HD, true>(R, sm.k[buf], sm.v[buf], tile, n, g, krow);
+            if (++tile > t_last) break;
+        }
+    } else {
+        for (;;) {
+            prefill_stash<HD>(sm, 0, s0, tile, kv_valid, tid);
+            lds_barrier();
+            if (tile + 2 <= t_last) prefill_fetch<HD>(s0, kbase, vtbase, tile + 2, tid);
+            prefill_compute<HD, true>(R, sm.k[0], sm.v[0], tile, n, g, krow);
+            if (++tile > t_last) break;
+            prefill_stash<HD>(sm, 1, s1, tile, kv_valid, tid);
+            lds_barrier();
+            if (tile + 2 <= t_last) prefill_fetch<HD>(s1, kbase, vtbase, tile + 2, tid);
+            prefill_compute<HD, true>(R, sm.k[1], sm.v[1], tile, n, g, krow);
+            if (++tile > t_last) break;
+        }
+    }
+    prefill_rows_store<HD>(R, a, row0, head, n, g);
 }
 
 // grid = (ceil(blocks / 2), KV heads x head chunks).  Workgroup x takes position
@@ -391,6 +399,522 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_mfma_kernel(const 
     if (hi != lo) {
         __syncthreads();                                  // LDS buffers change hands
         prefill_block<HD>(a, sm, lo, kvh, hc);
+    }
+}
+
+
+// ------------------------------------------------- MFMA, two waves per SIMD --
+// Same arithmetic per wave and tile as above, restructured so that the matrix
+// pipe, the vector ALU, LDS and the global-load path work at the same time:
+//
+//  * The keys of a block are split over two wave sets: waves 0-3 take the even
+//    tiles of the block's range, waves 4-7 the odd ones; the two partial
+//    (m, l, O) triples are merged through LDS at the end.  Eight waves put two
+//    on every SIMD.
+//  * Each wave is software-pipelined across its tiles: while the exponentials
+//    of tile j run on the vector ALU, the score MFMAs of tile j+1 (a dependent
+//    chain with idle slots) and the first half of tile j's P.V MFMAs run on the
+//    matrix pipe.  To have tile j+1's K next to tile j's Vt, K is staged one
+//    step ahead of V.
+//  * The workgroup stages a PAIR of tiles per step (64 keys: contiguous in both
+//    K and the block-transposed V) with one barrier per step.  The stores that
+//    stage step i+1's tiles and the global loads for step i+3 are issued from
+//    inside step i's arithmetic, spread between its MFMAs, instead of in a phase
+//    of their own in which every wave would queue on the same unit.
+//  * Loads and stores are issued unconditionally (indices clamped to the block's
+//    last pair) so the number in flight is the same on every path and the waits
+//    on them stay partial.
+//  * Instruction order inside a step is requested from the scheduler with
+//    scheduling-group barriers: one MFMA, then the few vector / LDS / memory
+//    instructions its execution time covers.
+//
+// Head dims up to 128 only: beyond that a wave needs more than the 256 registers
+// two waves per SIMD leave it.
+
+constexpr int kSplitThreads = 512;
+
+template <int HD>
+struct SplitSmem {
+    _Float16 k[2][2 * kTileKeys][HD + 8];      // [buffer][tile of the pair * 32 + key][dim]
+    _Float16 v[2][2][HD][kVBlock + 8];         // [buffer][tile of the pair][dim][key]
+};
+
+// merge scratch laid over the staging buffers: per sub-wave HD/2 accumulator
+// registers + m + l, one float per lane each
+template <int HD>
+constexpr size_t split_smem_bytes()
+{
+    const size_t stage = sizeof(SplitSmem<HD>);
+    const size_t merge = (size_t)4 * (HD / 2 + 2) * 64 * sizeof(float);
+    return stage > merge ? stage : merge;
+}
+
+// What a block streams (tile pairs 0 .. npairs-1 starting at tile t_first) and
+// from where.
+struct SplitRange {
+    const uint16_t* kbase;
+    const uint16_t* vtbase;
+    uint32_t t_first, t_last, npairs, kv_valid;
+};
+
+// This thread's share of one pair: 16-byte chunks of K and of Vt on their way
+// from global memory to LDS.
+template <int HD>
+struct SplitFeed {
+    u32x4 k[HD / 64], v[HD / 64];
+};
+
+// Loads one pair's K (or Vt) chunks.  When the pair's second tile lies past the
+// block's range (and possibly past the slab) its threads re-read the first tile.
+template <int HD>
+__device__ __forceinline__ void split_fetch(u32x4 (&dst)[HD / 64], const uint16_t* base,
+                                            const SplitRange& rg, uint32_t pair, int tid)
+{
+    constexpr int PER_TILE = 4 * HD;                      // 16-byte chunks per tile
+    pair = min(pair, rg.npairs - 1);
+    const uint32_t tile = rg.t_first + 2 * pair;
+    const bool both = tile + 1 <= rg.t_last;
+    const u32x4* src = reinterpret_cast<const u32x4*>(base + (size_t)tile * kTileKeys * HD);
+#pragma unroll
+    for (int c = 0; c < HD / 64; c++) {
+        const int ch = tid + c * kSplitThreads;
+        dst[c] = src[(ch < PER_TILE || both) ? ch : ch - PER_TILE];
+    }
+}
+
+template <int HD>
+__device__ __forceinline__ void split_stash_k(SplitSmem<HD>& sm, int buf,
+                                              const u32x4 (&st)[HD / 64], int tid)
+{
+    constexpr int KCH = HD / 8;                           // 16-byte chunks per K row
+#pragma unroll
+    for (int c = 0; c < HD / 64; c++) {
+        const int ch = tid + c * kSplitThreads;
+        *reinterpret_cast<u32x4*>(&sm.k[buf][ch / KCH][(ch % KCH) * 8]) = st[c];
+    }
+}
+
+template <int HD>
+__device__ __forceinline__ void split_stash_v(SplitSmem<HD>& sm, int buf,
+                                              const u32x4 (&st)[HD / 64], int tid)
+{
+    constexpr int PER_TILE = 4 * HD;
+#pragma unroll
+    for (int c = 0; c < HD / 64; c++) {
+        const int ch = tid + c * kSplitThreads;
+        const int tp = ch / PER_TILE, cv = ch % PER_TILE;
+        *reinterpret_cast<u32x4*>(&sm.v[buf][tp][cv >> 2][(cv & 3) * 8]) = st[c];
+    }
+}
+
+// Rows that were never appended may hold anything: zero them in the Vt chunks of
+// pair `pair` so 0 * garbage cannot reach the accumulator.  Only the pair that
+// holds the end of the appended rows is affected.
+template <int HD>
+__device__ __forceinline__ void split_mask_tail(u32x4 (&st)[HD / 64], const SplitRange& rg,
+                                                uint32_t pair, int tid)
+{
+    constexpr int PER_TILE = 4 * HD;
+    const uint32_t tile = rg.t_first + 2 * min(pair, rg.npairs - 1);
+    if ((tile + 2) * kTileKeys <= rg.kv_valid) return;
+#pragma unroll
+    for (int c = 0; c < HD / 64; c++) {
+        const int ch = tid + c * kSplitThreads;
+        const int tp = ch / PER_TILE, cv = ch % PER_TILE;
+        const uint32_t key0 = (tile + tp) * kTileKeys + (cv & 3) * 8;
+        uint32_t w[4] = {st[c].x, st[c].y, st[c].z, st[c].w};
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            if (key0 + 2 * e >= rg.kv_valid) w[e] &= 0xFFFF0000u;
+            if (key0 + 2 * e + 1 >= rg.kv_valid) w[e] &= 0x0000FFFFu;
+        }
+        st[c] = u32x4{w[0], w[1], w[2], w[3]};
+    }
+}
+
+// The data movement of step i: the set loaded two steps ago goes to LDS (K of
+// pair i+2, Vt of pair i+1: what step i+1 reads) and is refilled with K of pair
+// i+4 and Vt of pair i+3.
+template <int HD>
+__device__ __forceinline__ void split_move(SplitSmem<HD>& sm, SplitFeed<HD>& f,
+                                           const SplitRange& rg, uint32_t i, int tid)
+{
+    split_stash_k<HD>(sm, i & 1, f.k, tid);
+    split_stash_v<HD>(sm, (i + 1) & 1, f.v, tid);
+    split_fetch<HD>(f.k, rg.kbase, rg, i + 4, tid);
+    split_fetch<HD>(f.v, rg.vtbase, rg, i + 3, tid);
+}
+
+// First part of a tile's softmax: masks, row maximum, reference point (moving
+// it rescales the accumulators).  Returns the value to subtract from the scores.
+template <int HD>
+__device__ __forceinline__ float split_softmax_begin(PrefillRows<HD>& R, f32x16& c, uint32_t tile,
+                                                     int g)
+{
+    const uint32_t kb = tile * kTileKeys;
+    // register r of this lane: key kb + 16*(r/8) + 8*g + r%8, row n.
+    // Some (row, key) pair of the tile is invisible: above the diagonal of the
+    // wave's first row, or below the window of its last row.
+    const bool edge = (kb + kTileKeys - 1 > R.w_first_pos) || (kb < R.w_hi_lo);
+    if (edge) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const uint32_t key = kb + 16 * (r >> 3) + 8 * g + (r & 7);
+            if (key > R.pos || key < R.row_lo) c[r] = -INFINITY;
+        }
+    }
+    float tmax = c[0];
+#pragma unroll
+    for (int r = 1; r < 16; r++) tmax = fmaxf(tmax, c[r]);
+    tmax = wave_pair32_max(tmax);
+    const bool jump = tmax > R.m_run + kLazyLog2;          // false for tmax = -inf
+    const float m_new = jump ? tmax : R.m_run;
+    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;   // row with nothing visible yet
+    if (__builtin_amdgcn_ballot_w64(jump) != 0) {
+        const float alpha = jump ? fast_exp2(R.m_run - m_safe) : 1.0f;
+        R.l_run *= alpha;
+#pragma unroll
+        for (int dt = 0; dt < HD / 32; dt++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) R.o[dt][r] *= alpha;
+    }
+    R.m_run = m_new;
+    return m_safe;
+}
+
+// Scores of one tile only (a wave's first tile).
+template <int HD>
+__device__ __forceinline__ void split_scores(const PrefillRows<HD>& R, f32x16& sn,
+                                             const _Float16 (*ktile)[HD + 8], int g, int krow)
+{
+    half8 kf[HD / 16];
+#pragma unroll
+    for (int s = 0; s < HD / 16; s++)
+        kf[s] = *reinterpret_cast<const half8*>(&ktile[krow][s * 16 + g * 8]);
+    f32x16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0.f;
+#pragma unroll
+    for (int s = 0; s < HD / 16; s++)
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[s], R.qop[s], acc, 0, 0, 0);
+    sn = acc;
+}
+
+// Softmax and P.V of one tile only (a wave's last tile).
+template <int HD>
+__device__ __forceinline__ void split_finish(PrefillRows<HD>& R, f32x16& c,
+                                             const _Float16 (*vtile)[kVBlock + 8], uint32_t tile,
+                                             int n, int g)
+{
+    half8 vf[2][HD / 32];
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int dt = 0; dt < HD / 32; dt++)
+            vf[t][dt] = *reinterpret_cast<const half8*>(&vtile[dt * 32 + n][16 * t + 8 * g]);
+    const float m = split_softmax_begin<HD>(R, c, tile, g);
+    half8 pop[2];
+    float psum = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        const float p = fast_exp2(c[r] - m);
+        psum += p;
+        pop[r >> 3][r & 7] = (_Float16)p;
+    }
+    R.l_run += psum;
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int dt = 0; dt < HD / 32; dt++)
+            R.o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[t][dt], pop[t], R.o[dt], 0, 0, 0);
+}
+
+// Instruction order of the steady-state step, as a request to the scheduler
+// (the counts must be literals, hence the recursion).  Every score MFMA, joined
+// in the second half by one P.V MFMA, is followed by VPS vector instructions;
+// LDS reads go behind the MFMA that frees their registers; the NW staging
+// stores and NW global loads go one at a time behind MFMAs 1.. and 2..
+// Masks: 0x8 MFMA, 0x2 vector ALU, 0x100 LDS read, 0x200 LDS write, 0x20 memory read.
+template <int S, int NS, int VPS, int NW>
+__device__ __forceinline__ void split_step_order()
+{
+    if constexpr (S < NS) {
+        if constexpr (S >= NS / 2)
+            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+        else
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        if constexpr (S == 0 || S == NS / 2) __builtin_amdgcn_sched_group_barrier(0x100, NS / 2, 0);
+        if constexpr (S >= 1 && S <= NW) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+        if constexpr (S >= 2 && S <= NW + 1) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, VPS, 0);
+        split_step_order<S + 1, NS, VPS, NW>();
+    }
+}
+
+// Steady state: softmax and P.V of the tile whose scores are in `c`, interleaved
+// with the score MFMAs of the wave's next tile (result in `sn`) and with the
+// step's data movement.
+template <int HD>
+__device__ __forceinline__ void split_step(PrefillRows<HD>& R, f32x16& c, f32x16& sn,
+                                           SplitSmem<HD>& sm, SplitFeed<HD>& f, const SplitRange& rg,
+                                           uint32_t i, int tid,
+                                           const _Float16 (*ktile_next)[HD + 8],
+                                           const _Float16 (*vtile)[kVBlock + 8], uint32_t tile,
+                                           int n, int g, int krow)
+{
+    constexpr int NS = HD / 16;           // score MFMAs per tile
+    constexpr int EPS = 16 / NS;          // exponentials placed behind each of them
+    constexpr int ND = HD / 32;           // accumulators of O^T (== NS / 2)
+    half8 kf0[NS / 2], kf1[NS / 2], vf0[ND], vf1[ND];
+#pragma unroll
+    for (int s = 0; s < NS / 2; s++)
+        kf0[s] = *reinterpret_cast<const half8*>(&ktile_next[krow][s * 16 + g * 8]);
+#pragma unroll
+    for (int dt = 0; dt < ND; dt++)
+        vf0[dt] = *reinterpret_cast<const half8*>(&vtile[dt * 32 + n][8 * g]);
+    const float m = split_softmax_begin<HD>(R, c, tile, g);
+    __builtin_amdgcn_sched_barrier(0);
+
+    half8 pop[2];
+    float psum = 0.f;
+    f32x16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0.f;
+#pragma unroll
+    for (int s = 0; s < NS; s++) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(s < NS / 2 ? kf0[s % (NS / 2)] : kf1[s % (NS / 2)],
+                                                     R.qop[s], acc, 0, 0, 0);
+        if (s == 0) {
+#pragma unroll
+            for (int s2 = 0; s2 < NS / 2; s2++)
+                kf1[s2] = *reinterpret_cast<const half8*>(
+                    &ktile_next[krow][(NS / 2 + s2) * 16 + g * 8]);
+            split_move<HD>(sm, f, rg, i, tid);
+        }
+        if (s == NS / 2) {
+#pragma unroll
+            for (int dt = 0; dt < ND; dt++)
+                vf1[dt] = *reinterpret_cast<const half8*>(&vtile[dt * 32 + n][16 + 8 * g]);
+        }
+        if (s >= NS / 2) {
+            // the first eight probabilities are complete: their half of P.V fills
+            // the idle slots of the score chain
+            const int dt = s - NS / 2;
+            R.o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf0[dt], pop[0], R.o[dt], 0, 0, 0);
+        }
+#pragma unroll
+        for (int e = 0; e < EPS; e++) {
+            const int r = s * EPS + e;
+            const float p = fast_exp2(c[r] - m);
+            psum += p;
+            pop[r >> 3][r & 7] = (_Float16)p;
+        }
+    }
+    R.l_run += psum;
+#pragma unroll
+    for (int dt = 0; dt < ND; dt++)
+        R.o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf1[dt], pop[1], R.o[dt], 0, 0, 0);
+    // vector work of one probability: subtract, exp2, add, half a pack; plus the
+    // address arithmetic of the data movement
+    split_step_order<0, NS, (7 * EPS + 1) / 2 + 2, 2 * (HD / 64)>();
+    __builtin_amdgcn_sched_group_barrier(0x008, ND, 0);
+    sn = acc;
+}
+
+// Work of one wave in pipeline step i: the tile t_first + 2*i + kg is finished
+// (scores in `c`), the scores of the tile two further go to `sn`, and the
+// wave's share of the step's data movement is issued.
+template <int HD>
+__device__ __forceinline__ void split_wave_step(PrefillRows<HD>& R, f32x16& c, f32x16& sn,
+                                                SplitSmem<HD>& sm, SplitFeed<HD>& f,
+                                                const SplitRange& rg, uint32_t i, int tid, int kg,
+                                                int n, int g, int krow)
+{
+    const uint32_t tile = rg.t_first + 2 * i + kg;
+    const bool has_cur = R.wave_ok && tile >= R.wt_first && tile <= R.wt_last;
+    const bool has_next = R.wave_ok && tile + 2 >= R.wt_first && tile + 2 <= R.wt_last;
+    const int kb = (i + 1) & 1, vb = i & 1;               // K is staged one step ahead of V
+    split_mask_tail<HD>(f.v, rg, i + 1, tid);
+    if (has_cur && has_next) {
+        split_step<HD>(R, c, sn, sm, f, rg, i, tid, &sm.k[kb][kg * kTileKeys], sm.v[vb][kg], tile,
+                       n, g, krow);
+    } else {
+        split_move<HD>(sm, f, rg, i, tid);
+        if (has_next)
+            split_scores<HD>(R, sn, &sm.k[kb][kg * kTileKeys], g, krow);
+        else if (has_cur)
+            split_finish<HD>(R, c, sm.v[vb][kg], tile, n, g);
+    }
+}
+
+template <int HD>
+__device__ __forceinline__ void split_block(const PrefillArgs& a, unsigned char* smem_raw,
+                                            uint32_t pb, uint32_t kvh, uint32_t hc)
+{
+    SplitSmem<HD>& sm = *reinterpret_cast<SplitSmem<HD>*>(smem_raw);
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int n = lane & 31, g = lane >> 5;
+    const int kg = wave >> 2, sub = wave & 3;             // key set (tile parity), rows served
+    const uint32_t G = a.group;
+    const uint32_t Gw = G < 4 ? G : 4;
+    const uint32_t BP = 32 * (4 / Gw);                    // positions per block
+    const uint32_t head = kvh * G + hc * Gw + (sub % Gw);
+    const uint32_t row0 = pb * BP + (sub / Gw) * 32;      // first chunk row of this wave
+    SplitRange rg;
+    prefill_block_tiles(a, pb, BP, rg.t_first, rg.t_last);
+    rg.npairs = (rg.t_last - rg.t_first) / 2 + 1;
+    rg.kv_valid = a.p0 + a.T;                             // rows of the cache that hold data
+    rg.kbase = a.k + (size_t)kvh * a.ctx_pad * HD;
+    rg.vtbase = a.vt + (size_t)kvh * (a.ctx_pad / kVBlock) * HD * kVBlock;
+
+    // Register sets: f1 is stored by odd steps (and by the prologue, "step -1"),
+    // f0 by even steps.  Step i stores K of pair i+2 and Vt of pair i+1.
+    SplitFeed<HD> f0, f1;
+    u32x4 kfirst[HD / 64];
+    split_fetch<HD>(kfirst, rg.kbase, rg, 0, tid);
+    split_fetch<HD>(f1.k, rg.kbase, rg, 1, tid);
+    split_fetch<HD>(f1.v, rg.vtbase, rg, 0, tid);
+    split_fetch<HD>(f0.k, rg.kbase, rg, 2, tid);
+    split_fetch<HD>(f0.v, rg.vtbase, rg, 1, tid);
+
+    PrefillRows<HD> R;
+    prefill_rows_init<HD, false>(R, a, row0, head, n, g);
+    const int krow = prefill_key_perm(n);                 // LDS row this lane feeds to MFMA row n
+
+    // Q: every row is 4*HD contiguous bytes in global memory, so it is read with
+    // whole-row coalesced loads (the two waves serving a sub-block take 16 rows
+    // each), converted to pre-scaled F16 and turned into the per-lane operand
+    // layout through LDS (the Vt staging area, not in use yet).
+    _Float16 (*qs)[32][HD + 8] = reinterpret_cast<_Float16 (*)[32][HD + 8]>(&sm.v[0][0][0][0]);
+    static_assert(sizeof(sm.v) >= (size_t)4 * 32 * (HD + 8) * sizeof(_Float16), "Q staging fits");
+    {
+        constexpr int LPR = HD / 4;                       // lanes per row (one float4 each)
+        constexpr int RPI = 64 / LPR;                     // rows per load instruction
+#pragma unroll
+        for (int j = 0; j < 16 / RPI; j++) {
+            const int r = kg * 16 + j * RPI + lane / LPR;
+            const uint32_t row = min(row0 + r, a.T - 1);  // idle rows re-read the last one
+            const float4 x = *reinterpret_cast<const float4*>(
+                a.q + ((size_t)row * a.nq + head) * HD + (lane % LPR) * 4);
+            half4 h;
+            h[0] = (_Float16)(x.x * a.qscale);
+            h[1] = (_Float16)(x.y * a.qscale);
+            h[2] = (_Float16)(x.z * a.qscale);
+            h[3] = (_Float16)(x.w * a.qscale);
+            *reinterpret_cast<half4*>(&qs[sub][r][(lane % LPR) * 4]) = h;
+        }
+    }
+
+    // prologue: K of pair 0 and Q become visible, then the first scores, then
+    // (Q staging read by everyone) what step 0 reads
+    f32x16 s0, s1;
+#pragma unroll
+    for (int r = 0; r < 16; r++) s0[r] = s1[r] = 0.f;
+    split_stash_k<HD>(sm, 0, kfirst, tid);
+    lds_barrier();
+#pragma unroll
+    for (int s = 0; s < HD / 16; s++)
+        R.qop[s] = *reinterpret_cast<const half8*>(&qs[sub][n][s * 16 + g * 8]);
+    {
+        const uint32_t tile = rg.t_first + kg;
+        if (R.wave_ok && tile >= R.wt_first && tile <= R.wt_last)
+            split_scores<HD>(R, s0, &sm.k[0][kg * kTileKeys], g, krow);
+    }
+    lds_barrier();
+    split_mask_tail<HD>(f1.v, rg, 0, tid);
+    split_move<HD>(sm, f1, rg, 0xFFFFFFFFu, tid);         // step -1: K of pair 1, Vt of pair 0
+
+    for (uint32_t i = 0;; i += 2) {
+        lds_barrier();
+        split_wave_step<HD>(R, s0, s1, sm, f0, rg, i, tid, kg, n, g, krow);
+        if (i + 1 >= rg.npairs) break;
+        lds_barrier();
+        split_wave_step<HD>(R, s1, s0, sm, f1, rg, i + 1, tid, kg, n, g, krow);
+        if (i + 2 >= rg.npairs) break;
+    }
+
+    // merge the odd-tile partials into the even-tile waves
+    constexpr int NREG = HD / 2;
+    float* mg = reinterpret_cast<float*>(smem_raw) + (size_t)sub * (NREG + 2) * 64;
+    __syncthreads();                                      // staging buffers are free
+    if (kg == 1) {
+#pragma unroll
+        for (int dt = 0; dt < HD / 32; dt++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) mg[(dt * 16 + r) * 64 + lane] = R.o[dt][r];
+        mg[NREG * 64 + lane] = R.m_run;
+        mg[(NREG + 1) * 64 + lane] = R.l_run;
+    }
+    __syncthreads();
+    // rows leave through LDS as well: the merged tile is written row-major into
+    // the sub-block's own scratch, then both of its waves store whole rows
+    float (*os)[HD + 4] = reinterpret_cast<float (*)[HD + 4]>(mg);
+    static_assert((size_t)32 * (HD + 4) <= (size_t)(NREG + 2) * 64, "row-major tile fits the merge scratch");
+    if (kg == 0) {
+        const float m1 = mg[NREG * 64 + lane], l1 = mg[(NREG + 1) * 64 + lane];
+        const float m = fmaxf(R.m_run, m1);
+        const float f0m = (R.m_run == -INFINITY) ? 0.f : fast_exp2(R.m_run - m);
+        const float f1m = (m1 == -INFINITY) ? 0.f : fast_exp2(m1 - m);
+        const float l_tot = wave_pair32_sum(R.l_run * f0m + l1 * f1m);
+        const float inv = (l_tot > 0.f) ? 1.0f / l_tot : 0.f;
+        const float w0 = f0m * inv, w1 = f1m * inv;
+#pragma unroll
+        for (int dt = 0; dt < HD / 32; dt++)
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+                R.o[dt][r] = R.o[dt][r] * w0 + mg[(dt * 16 + r) * 64 + lane] * w1;
+        // the scratch has been read into registers; the same wave now reuses it
+#pragma unroll
+        for (int dt = 0; dt < HD / 32; dt++)
+#pragma unroll
+            for (int q4 = 0; q4 < 4; q4++) {
+                float4 v;
+                v.x = R.o[dt][4 * q4 + 0];
+                v.y = R.o[dt][4 * q4 + 1];
+                v.z = R.o[dt][4 * q4 + 2];
+                v.w = R.o[dt][4 * q4 + 3];
+                *reinterpret_cast<float4*>(&os[n][dt * 32 + 8 * q4 + 4 * g]) = v;
+            }
+    }
+    __syncthreads();
+    {
+        constexpr int LPR = HD / 4;                       // lanes per row (one float4 each)
+        constexpr int RPI = 64 / LPR;                     // rows per store instruction
+#pragma unroll
+        for (int j = 0; j < 16 / RPI; j++) {
+            const int r = kg * 16 + j * RPI + lane / LPR;
+            const float4 v = *reinterpret_cast<const float4*>(&os[r][(lane % LPR) * 4]);
+            if (row0 + r < a.T)
+                *reinterpret_cast<float4*>(a.out + ((size_t)(row0 + r) * a.nq + head) * HD +
+                                           (lane % LPR) * 4) = v;
+        }
+    }
+}
+
+// grid = (KV heads x head chunks, ceil(blocks / 2)): consecutive workgroups (which
+// the dispatcher deals round-robin to the XCDs) differ in KV head, so one XCD's
+// L2 keeps seeing the same few heads' K / Vt.  Workgroup y takes position block
+// (blocks-1-y) and then block y: a long block and a short one, so every
+// workgroup streams the same number of tiles despite the causal triangle.
+template <int HD>
+__global__ __launch_bounds__(kSplitThreads, 1) void prefill_split_kernel(const PrefillArgs a)
+{
+    extern __shared__ __attribute__((aligned(16))) unsigned char prefill_smem_raw[];
+    const uint32_t G = a.group;
+    const uint32_t Gw = G < 4 ? G : 4;
+    const uint32_t chunks = G / Gw;
+    const uint32_t kvh = blockIdx.x / chunks, hc = blockIdx.x % chunks;
+    const uint32_t BP = 32 * (4 / Gw);
+    const uint32_t nblk = (a.T + BP - 1) / BP;
+    const uint32_t lo = blockIdx.y, hi = nblk - 1 - blockIdx.y;
+#pragma unroll 1
+    for (int pass = 0; pass < 2; pass++) {
+        if (pass) {
+            if (hi == lo) break;
+            __syncthreads();                              // LDS changes hands
+        }
+        split_block<HD>(a, prefill_smem_raw, pass ? lo : hi, kvh, hc);
     }
 }
 

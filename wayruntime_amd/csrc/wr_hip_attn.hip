@@ -153,14 +153,14 @@ int copy_down_sync(void* dst_host, const void* src_dev, size_t bytes)
 }
 
 template <typename Kern, typename Args>
-void launch_main(Kern kernel, dim3 grid, dim3 block, const Args& args)
+void launch_main(Kern kernel, dim3 grid, dim3 block, const Args& args, size_t lds_bytes = 0)
 {
     if (g.profiling && g.ev_used + 2 <= g.ev.size()) {
-        hipExtLaunchKernelGGL(kernel, grid, block, 0, g.stream, g.ev[g.ev_used],
+        hipExtLaunchKernelGGL(kernel, grid, block, lds_bytes, g.stream, g.ev[g.ev_used],
                               g.ev[g.ev_used + 1], 0, args);
         g.ev_used += 2;
     } else {
-        hipLaunchKernelGGL(kernel, grid, block, 0, g.stream, args);
+        hipLaunchKernelGGL(kernel, grid, block, lds_bytes, g.stream, args);
     }
 }
 
@@ -344,12 +344,6 @@ int prefill_locked(wr_hip_kv* kv, uint32_t layer, uint32_t p0, uint32_t T, const
     a.window = window;
     const float scale = (scale_override > 0.0f) ? scale_override : 1.0f / sqrtf((float)hd);
     a.qscale = scale * kLog2e;
-#ifdef WR_PREFILL_PROF
-    static unsigned long long* prof = nullptr;
-    if (!prof) { (void)hipMalloc((void**)&prof, 64); }
-    (void)hipMemsetAsync(prof, 0, 64, g.stream);
-    a.prof = prof;
-#endif
     const uint32_t G = a.group;
     const bool mfma = !g.force_generic && (hd == 64 || hd == 128 || hd == 256) &&
                       (G == 1 || G == 2 || G == 4 || G == 8);
@@ -357,26 +351,27 @@ int prefill_locked(wr_hip_kv* kv, uint32_t layer, uint32_t p0, uint32_t T, const
         const uint32_t Gw = G < 4 ? G : 4;
         const uint32_t BP = 32 * (4 / Gw);
         const uint32_t nblk = (T + BP - 1) / BP;
-        const dim3 grid((nblk + 1) / 2, kv->nkv * (G / Gw)), block(kPrefillThreads);
+        const uint32_t npairs = (nblk + 1) / 2, ny = kv->nkv * (G / Gw);
+#ifndef WR_PREFILL_ONE_WAVE_PER_SIMD
         if (hd == 64)
-            launch_main(prefill_mfma_kernel<64>, grid, block, a);
+            launch_main(prefill_split_kernel<64>, dim3(ny, npairs), dim3(kSplitThreads), a,
+                        split_smem_bytes<64>());
         else if (hd == 128)
-            launch_main(prefill_mfma_kernel<128>, grid, block, a);
+            launch_main(prefill_split_kernel<128>, dim3(ny, npairs), dim3(kSplitThreads), a,
+                        split_smem_bytes<128>());
         else
-            launch_main(prefill_mfma_kernel<256>, grid, block, a);
+#else
+        if (hd == 64)
+            launch_main(prefill_mfma_kernel<64>, dim3(npairs, ny), dim3(kPrefillThreads), a);
+        else if (hd == 128)
+            launch_main(prefill_mfma_kernel<128>, dim3(npairs, ny), dim3(kPrefillThreads), a);
+        else
+#endif
+            launch_main(prefill_mfma_kernel<256>, dim3(npairs, ny), dim3(kPrefillThreads), a);
     } else {
         launch_main(prefill_generic_kernel, dim3(T, nq), dim3(kDecodeThreads), a);
     }
     HIP_TRY(hipGetLastError(), "prefill launch", layer);
-#ifdef WR_PREFILL_PROF
-    {
-        unsigned long long h[8];
-        (void)hipMemcpyAsync(h, a.prof, 64, hipMemcpyDeviceToHost, g.stream);
-        (void)hipStreamSynchronize(g.stream);
-        fprintf(stderr, "prof: tiles %llu  qk %.0f  softmax %.0f  pv %.0f  block total/tile %.0f clk\n", h[3],
-                (double)h[0] / h[3], (double)h[1] / h[3], (double)h[2] / h[3], (double)h[4] / h[3]);
-    }
-#endif
     g.calls.fetch_add(T, std::memory_order_relaxed);
     return WR_HIP_OK;
 }
@@ -441,6 +436,18 @@ int wr_hip_attn_init(int device)
         if (e == hipSuccess) e = hipMemsetAsync(g.d_counters, 0, cb, g.stream);
         if (e == hipSuccess) e = hipStreamSynchronize(g.stream);
         if (e != hipSuccess) rc = hip_fail(e, "ticket array", 0);
+    }
+    if (rc == WR_HIP_OK) {
+        // the two-waves-per-SIMD prefill kernels stage more than the 64 KiB a
+        // kernel may use without asking
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(prefill_split_kernel<64>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           (int)split_smem_bytes<64>());
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute(reinterpret_cast<const void*>(prefill_split_kernel<128>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)split_smem_bytes<128>());
+        if (e != hipSuccess) rc = hip_fail(e, "prefill LDS size", 0);
     }
     if (rc != WR_HIP_OK) {
         g.inited = false;
