@@ -413,136 +413,175 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_mfma_kernel(const 
 //    on every SIMD.
 //  * Each wave is software-pipelined across its tiles: while the exponentials
 //    of tile j run on the vector ALU, the score MFMAs of tile j+1 (a dependent
-//    chain with idle slots) and the first half of tile j's P.V MFMAs run on the
-//    matrix pipe.  To have tile j+1's K next to tile j's Vt, K is staged one
-//    step ahead of V.
+//    chain) and the first half of tile j's P.V MFMAs run on the matrix pipe.
+//    To have tile j+1's K next to tile j's Vt, K is staged one step ahead of V.
 //  * The workgroup stages a PAIR of tiles per step (64 keys: contiguous in both
-//    K and the block-transposed V) with one barrier per step.  The stores that
-//    stage step i+1's tiles and the global loads for step i+3 are issued from
-//    inside step i's arithmetic, spread between its MFMAs, instead of in a phase
-//    of their own in which every wave would queue on the same unit.
-//  * Loads and stores are issued unconditionally (indices clamped to the block's
-//    last pair) so the number in flight is the same on every path and the waits
-//    on them stay partial.
+//    K and the block-transposed V) with one barrier per step, in a ring of three
+//    pair buffers.  Tiles travel from global memory straight into LDS
+//    (global_load_lds_dwordx4: no staging registers, no LDS store instructions),
+//    issued from inside the step's arithmetic three steps (K) / two steps (Vt)
+//    before their first use.
+//  * Such a load writes the wave's 64 x 16 bytes to consecutive LDS addresses, so
+//    rows cannot be padded; the 16-byte chunks of a row are permuted instead
+//    (chunk c of row r sits at slot c ^ f(r)), on the global side where any
+//    permutation inside a row keeps the access coalesced.  f is chosen so that
+//    the sixteen rows a 128-bit LDS read touches per cycle fall into sixteen
+//    different slots of the 256-byte bank row.
+//  * Loads are issued unconditionally (pair indices clamped to the block's last
+//    pair; duplicates land in ring slots nobody reads) so the number in flight
+//    is the same at every barrier and "all but the newest N" is a fixed wait.
 //  * Instruction order inside a step is requested from the scheduler with
-//    scheduling-group barriers: one MFMA, then the few vector / LDS / memory
+//    scheduling-group barriers: one MFMA, then the few vector / LDS
 //    instructions its execution time covers.
 //
 // Head dims up to 128 only: beyond that a wave needs more than the 256 registers
 // two waves per SIMD leave it.
 
 constexpr int kSplitThreads = 512;
+constexpr int kRing = 3;
 
 template <int HD>
-struct SplitSmem {
-    _Float16 k[2][2 * kTileKeys][HD + 8];      // [buffer][tile of the pair * 32 + key][dim]
-    _Float16 v[2][2][HD][kVBlock + 8];         // [buffer][tile of the pair][dim][key]
+struct SplitLds {
+    static constexpr int RB = 2 * HD;                     // bytes per K row
+    static constexpr int CPR = HD / 8;                    // 16-byte chunks per K row
+    static constexpr int RPB = 256 / RB > 0 ? 256 / RB : 1;   // K rows per 256-byte bank row
+    static constexpr int KPAIR = 2 * kTileKeys * RB;      // bytes of one pair's K
+    static constexpr int VPAIR = 2 * HD * kVBlock * 2;    // bytes of one pair's Vt (two blocks)
+    static constexpr int NL = KPAIR / 1024 / 8;           // loads per wave and pair, each of K and Vt
+    static constexpr int K_OFF = 0;
+    static constexpr int V_OFF = kRing * KPAIR;
+    static constexpr int Q_OFF = V_OFF + kRing * VPAIR;   // Q staging, [4][32][HD + 8] halves
+    static constexpr int Q_BYTES = 4 * 32 * (HD + 8) * 2;
+    static constexpr int MERGE_BYTES = 4 * (HD / 2 + 2) * 64 * 4;   // laid over the ring
+    static constexpr int TOTAL = Q_OFF + Q_BYTES;
+    static_assert(MERGE_BYTES <= Q_OFF, "merge scratch fits the ring");
+    static_assert(KPAIR == VPAIR && NL >= 1, "one chunk schedule serves K and Vt");
+    // slot permutation of K rows / Vt rows
+    __device__ static constexpr int fk(int row) { return (row / RPB) & (CPR - 1); }
+    __device__ static constexpr int fv(int row) { return (row >> 2) & 3; }
 };
 
-// merge scratch laid over the staging buffers: per sub-wave HD/2 accumulator
-// registers + m + l, one float per lane each
 template <int HD>
 constexpr size_t split_smem_bytes()
 {
-    const size_t stage = sizeof(SplitSmem<HD>);
-    const size_t merge = (size_t)4 * (HD / 2 + 2) * 64 * sizeof(float);
-    return stage > merge ? stage : merge;
+    return SplitLds<HD>::TOTAL;
 }
 
-// What a block streams (tile pairs 0 .. npairs-1 starting at tile t_first) and
-// from where.
-struct SplitRange {
-    const uint16_t* kbase;
-    const uint16_t* vtbase;
+// What a block streams (tile pairs 0 .. npairs-1 starting at tile t_first), from
+// where, and this lane's invariant addresses.
+template <int HD>
+struct SplitCtx {
+    const unsigned char* kbase;       // this KV head's K / Vt, bytes
+    const unsigned char* vtbase;
+    uint32_t lds0;                    // LDS byte address of the staging area
     uint32_t t_first, t_last, npairs, kv_valid;
+    uint32_t gk_off[SplitLds<HD>::NL];    // lane's byte offset inside a pair's K, per load
+    uint32_t gv_off[SplitLds<HD>::NL];    // ... inside a pair's Vt
+    uint32_t kread[HD / 16];          // LDS offsets of the K operand reads (ring slot 0)
+    uint32_t vread[2];                // ... of the Vt operand reads, dt = 0
 };
 
-// This thread's share of one pair: 16-byte chunks of K and of Vt on their way
-// from global memory to LDS.
-template <int HD>
-struct SplitFeed {
-    u32x4 k[HD / 64], v[HD / 64];
-};
-
-// Loads one pair's K (or Vt) chunks.  When the pair's second tile lies past the
-// block's range (and possibly past the slab) its threads re-read the first tile.
-template <int HD>
-__device__ __forceinline__ void split_fetch(u32x4 (&dst)[HD / 64], const uint16_t* base,
-                                            const SplitRange& rg, uint32_t pair, int tid)
+// Tells the compiler that a pointer is the same in every lane (keeps the
+// arithmetic on it in scalar registers).
+__device__ __forceinline__ const unsigned char* uniform_ptr(const unsigned char* p)
 {
-    constexpr int PER_TILE = 4 * HD;                      // 16-byte chunks per tile
-    pair = min(pair, rg.npairs - 1);
-    const uint32_t tile = rg.t_first + 2 * pair;
-    const bool both = tile + 1 <= rg.t_last;
-    const u32x4* src = reinterpret_cast<const u32x4*>(base + (size_t)tile * kTileKeys * HD);
+    const uint64_t b = reinterpret_cast<uint64_t>(p);
+    // the builtin returns a signed int: widen through uint32_t, or a low half
+    // with its top bit set would smear ones over the high half
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)b);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(b >> 32));
+    return reinterpret_cast<const unsigned char*>((uint64_t)lo | ((uint64_t)hi << 32));
+}
+
+// One 64 x 16-byte load from global memory straight into LDS.  The LDS address
+// (wave-uniform, in M0) receives lane 0's 16 bytes, lane i's go 16*i further.
+__device__ __forceinline__ void lds_direct_load(uint32_t lds_addr, const unsigned char* base,
+                                                uint32_t lane_off)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(lds_addr), "v"(lane_off), "s"(base)
+                 : "memory");
+}
+
+// Loads of one pair's K into ring slot `slot`.  Chunk q = wave + 8u of the
+// pair: 1024 consecutive bytes.  When the pair's second tile lies past the
+// block's range (and possibly past the slab) its loads re-read the first tile.
+template <int HD>
+__device__ __forceinline__ void split_issue_k(const SplitCtx<HD>& cx, uint32_t pair, int slot,
+                                              int wave)
+{
+    using L = SplitLds<HD>;
+    pair = min(pair, cx.npairs - 1);
+    const uint32_t tile = cx.t_first + 2 * pair;
+    const bool both = tile + 1 <= cx.t_last;
+    const unsigned char* src = cx.kbase + (size_t)tile * kTileKeys * L::RB;
 #pragma unroll
-    for (int c = 0; c < HD / 64; c++) {
-        const int ch = tid + c * kSplitThreads;
-        dst[c] = src[(ch < PER_TILE || both) ? ch : ch - PER_TILE];
+    for (int u = 0; u < L::NL; u++) {
+        const int q = wave + 8 * u;
+        const bool second = q * 1024 >= L::KPAIR / 2;     // chunk belongs to the pair's second tile
+        const unsigned char* b = (second && !both) ? src - L::KPAIR / 2 : src;
+        lds_direct_load(cx.lds0 + L::K_OFF + slot * L::KPAIR + q * 1024, b, cx.gk_off[u]);
     }
 }
 
 template <int HD>
-__device__ __forceinline__ void split_stash_k(SplitSmem<HD>& sm, int buf,
-                                              const u32x4 (&st)[HD / 64], int tid)
+__device__ __forceinline__ void split_issue_v(const SplitCtx<HD>& cx, uint32_t pair, int slot,
+                                              int wave)
 {
-    constexpr int KCH = HD / 8;                           // 16-byte chunks per K row
+    using L = SplitLds<HD>;
+    pair = min(pair, cx.npairs - 1);
+    const uint32_t tile = cx.t_first + 2 * pair;
+    const bool both = tile + 1 <= cx.t_last;
+    const unsigned char* src = cx.vtbase + (size_t)tile * HD * kVBlock * 2;
 #pragma unroll
-    for (int c = 0; c < HD / 64; c++) {
-        const int ch = tid + c * kSplitThreads;
-        *reinterpret_cast<u32x4*>(&sm.k[buf][ch / KCH][(ch % KCH) * 8]) = st[c];
+    for (int u = 0; u < L::NL; u++) {
+        const int q = wave + 8 * u;
+        const bool second = q * 1024 >= L::VPAIR / 2;
+        const unsigned char* b = (second && !both) ? src - L::VPAIR / 2 : src;
+        lds_direct_load(cx.lds0 + L::V_OFF + slot * L::VPAIR + q * 1024, b, cx.gv_off[u]);
     }
 }
 
+// Rows that were never appended may hold anything: zero them in the staged Vt
+// of pair `pair` so 0 * garbage cannot reach the accumulator.  Only the pair
+// holding the end of the appended rows is affected.  Every lane patches the
+// chunks its own loads delivered, so the caller only has to have waited for
+// this wave's loads.
 template <int HD>
-__device__ __forceinline__ void split_stash_v(SplitSmem<HD>& sm, int buf,
-                                              const u32x4 (&st)[HD / 64], int tid)
+__device__ __forceinline__ void split_patch_tail(unsigned char* smem, const SplitCtx<HD>& cx,
+                                                 uint32_t pair, int wave, int lane)
 {
-    constexpr int PER_TILE = 4 * HD;
+    using L = SplitLds<HD>;
+    if (pair >= cx.npairs) return;
+    const uint32_t tile = cx.t_first + 2 * pair;
+    if ((tile + 2) * kTileKeys <= cx.kv_valid) return;
+    const int slot = pair % kRing;
 #pragma unroll
-    for (int c = 0; c < HD / 64; c++) {
-        const int ch = tid + c * kSplitThreads;
-        const int tp = ch / PER_TILE, cv = ch % PER_TILE;
-        *reinterpret_cast<u32x4*>(&sm.v[buf][tp][cv >> 2][(cv & 3) * 8]) = st[c];
-    }
-}
-
-// Rows that were never appended may hold anything: zero them in the Vt chunks of
-// pair `pair` so 0 * garbage cannot reach the accumulator.  Only the pair that
-// holds the end of the appended rows is affected.
-template <int HD>
-__device__ __forceinline__ void split_mask_tail(u32x4 (&st)[HD / 64], const SplitRange& rg,
-                                                uint32_t pair, int tid)
-{
-    constexpr int PER_TILE = 4 * HD;
-    const uint32_t tile = rg.t_first + 2 * min(pair, rg.npairs - 1);
-    if ((tile + 2) * kTileKeys <= rg.kv_valid) return;
-#pragma unroll
-    for (int c = 0; c < HD / 64; c++) {
-        const int ch = tid + c * kSplitThreads;
-        const int tp = ch / PER_TILE, cv = ch % PER_TILE;
-        const uint32_t key0 = (tile + tp) * kTileKeys + (cv & 3) * 8;
-        uint32_t w[4] = {st[c].x, st[c].y, st[c].z, st[c].w};
+    for (int u = 0; u < L::NL; u++) {
+        const int q = wave + 8 * u;
+        const int row = q * 16 + lane / 4;                // row of the pair's 2*HD Vt rows
+        const int c = (lane & 3) ^ L::fv(row);            // key chunk this slot holds
+        const uint32_t key0 = (tile + row / HD) * kTileKeys + c * 8;
+        u32x4* at = reinterpret_cast<u32x4*>(smem + L::V_OFF + slot * L::VPAIR + q * 1024 + lane * 16);
+        u32x4 v = *at;
+        uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-            if (key0 + 2 * e >= rg.kv_valid) w[e] &= 0xFFFF0000u;
-            if (key0 + 2 * e + 1 >= rg.kv_valid) w[e] &= 0x0000FFFFu;
+            if (key0 + 2 * e >= cx.kv_valid) w[e] &= 0xFFFF0000u;
+            if (key0 + 2 * e + 1 >= cx.kv_valid) w[e] &= 0x0000FFFFu;
         }
-        st[c] = u32x4{w[0], w[1], w[2], w[3]};
+        *at = u32x4{w[0], w[1], w[2], w[3]};
     }
 }
 
-// The data movement of step i: the set loaded two steps ago goes to LDS (K of
-// pair i+2, Vt of pair i+1: what step i+1 reads) and is refilled with K of pair
-// i+4 and Vt of pair i+3.
+// The data movement of step i: K of pair i+3 and Vt of pair i+2 replace K of
+// pair i and Vt of pair i-1, both read for the last time in step i-1.
 template <int HD>
-__device__ __forceinline__ void split_move(SplitSmem<HD>& sm, SplitFeed<HD>& f,
-                                           const SplitRange& rg, uint32_t i, int tid)
+__device__ __forceinline__ void split_move(const SplitCtx<HD>& cx, uint32_t i, int wave)
 {
-    split_stash_k<HD>(sm, i & 1, f.k, tid);
-    split_stash_v<HD>(sm, (i + 1) & 1, f.v, tid);
-    split_fetch<HD>(f.k, rg.kbase, rg, i + 4, tid);
-    split_fetch<HD>(f.v, rg.vtbase, rg, i + 3, tid);
+    split_issue_k<HD>(cx, i + 3, i % kRing, wave);
+    split_issue_v<HD>(cx, i + 2, (i + 2) % kRing, wave);
 }
 
 // First part of a tile's softmax: masks, row maximum, reference point (moving
@@ -582,15 +621,17 @@ __device__ __forceinline__ float split_softmax_begin(PrefillRows<HD>& R, f32x16&
     return m_safe;
 }
 
-// Scores of one tile only (a wave's first tile).
+// Scores of one tile only (a wave's first tile).  kslot: byte offset of the ring
+// slot holding the tile's pair.
 template <int HD>
 __device__ __forceinline__ void split_scores(const PrefillRows<HD>& R, f32x16& sn,
-                                             const _Float16 (*ktile)[HD + 8], int g, int krow)
+                                             const unsigned char* smem, const SplitCtx<HD>& cx,
+                                             uint32_t kslot)
 {
     half8 kf[HD / 16];
 #pragma unroll
     for (int s = 0; s < HD / 16; s++)
-        kf[s] = *reinterpret_cast<const half8*>(&ktile[krow][s * 16 + g * 8]);
+        kf[s] = *reinterpret_cast<const half8*>(smem + kslot + cx.kread[s]);
     f32x16 acc;
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[r] = 0.f;
@@ -600,42 +641,12 @@ __device__ __forceinline__ void split_scores(const PrefillRows<HD>& R, f32x16& s
     sn = acc;
 }
 
-// Softmax and P.V of one tile only (a wave's last tile).
-template <int HD>
-__device__ __forceinline__ void split_finish(PrefillRows<HD>& R, f32x16& c,
-                                             const _Float16 (*vtile)[kVBlock + 8], uint32_t tile,
-                                             int n, int g)
-{
-    half8 vf[2][HD / 32];
-#pragma unroll
-    for (int t = 0; t < 2; t++)
-#pragma unroll
-        for (int dt = 0; dt < HD / 32; dt++)
-            vf[t][dt] = *reinterpret_cast<const half8*>(&vtile[dt * 32 + n][16 * t + 8 * g]);
-    const float m = split_softmax_begin<HD>(R, c, tile, g);
-    half8 pop[2];
-    float psum = 0.f;
-#pragma unroll
-    for (int r = 0; r < 16; r++) {
-        const float p = fast_exp2(c[r] - m);
-        psum += p;
-        pop[r >> 3][r & 7] = (_Float16)p;
-    }
-    R.l_run += psum;
-#pragma unroll
-    for (int t = 0; t < 2; t++)
-#pragma unroll
-        for (int dt = 0; dt < HD / 32; dt++)
-            R.o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[t][dt], pop[t], R.o[dt], 0, 0, 0);
-}
-
 // Instruction order of the steady-state step, as a request to the scheduler
 // (the counts must be literals, hence the recursion).  Every score MFMA, joined
 // in the second half by one P.V MFMA, is followed by VPS vector instructions;
-// LDS reads go behind the MFMA that frees their registers; the NW staging
-// stores and NW global loads go one at a time behind MFMAs 1.. and 2..
-// Masks: 0x8 MFMA, 0x2 vector ALU, 0x100 LDS read, 0x200 LDS write, 0x20 memory read.
-template <int S, int NS, int VPS, int NW>
+// LDS reads go behind the MFMA that frees their registers.
+// Masks: 0x8 MFMA, 0x2 vector ALU, 0x100 LDS read.
+template <int S, int NS, int VPS>
 __device__ __forceinline__ void split_step_order()
 {
     if constexpr (S < NS) {
@@ -644,10 +655,8 @@ __device__ __forceinline__ void split_step_order()
         else
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         if constexpr (S == 0 || S == NS / 2) __builtin_amdgcn_sched_group_barrier(0x100, NS / 2, 0);
-        if constexpr (S >= 1 && S <= NW) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-        if constexpr (S >= 2 && S <= NW + 1) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
         __builtin_amdgcn_sched_group_barrier(0x002, VPS, 0);
-        split_step_order<S + 1, NS, VPS, NW>();
+        split_step_order<S + 1, NS, VPS>();
     }
 }
 
@@ -656,11 +665,9 @@ __device__ __forceinline__ void split_step_order()
 // step's data movement.
 template <int HD>
 __device__ __forceinline__ void split_step(PrefillRows<HD>& R, f32x16& c, f32x16& sn,
-                                           SplitSmem<HD>& sm, SplitFeed<HD>& f, const SplitRange& rg,
-                                           uint32_t i, int tid,
-                                           const _Float16 (*ktile_next)[HD + 8],
-                                           const _Float16 (*vtile)[kVBlock + 8], uint32_t tile,
-                                           int n, int g, int krow)
+                                           const unsigned char* smem, const SplitCtx<HD>& cx,
+                                           uint32_t i, int wave, uint32_t kslot, uint32_t vslot,
+                                           uint32_t tile, int g)
 {
     constexpr int NS = HD / 16;           // score MFMAs per tile
     constexpr int EPS = 16 / NS;          // exponentials placed behind each of them
@@ -668,10 +675,10 @@ __device__ __forceinline__ void split_step(PrefillRows<HD>& R, f32x16& c, f32x16
     half8 kf0[NS / 2], kf1[NS / 2], vf0[ND], vf1[ND];
 #pragma unroll
     for (int s = 0; s < NS / 2; s++)
-        kf0[s] = *reinterpret_cast<const half8*>(&ktile_next[krow][s * 16 + g * 8]);
+        kf0[s] = *reinterpret_cast<const half8*>(smem + kslot + cx.kread[s]);
 #pragma unroll
     for (int dt = 0; dt < ND; dt++)
-        vf0[dt] = *reinterpret_cast<const half8*>(&vtile[dt * 32 + n][8 * g]);
+        vf0[dt] = *reinterpret_cast<const half8*>(smem + vslot + cx.vread[0] + dt * 2048);
     const float m = split_softmax_begin<HD>(R, c, tile, g);
     __builtin_amdgcn_sched_barrier(0);
 
@@ -687,14 +694,12 @@ __device__ __forceinline__ void split_step(PrefillRows<HD>& R, f32x16& c, f32x16
         if (s == 0) {
 #pragma unroll
             for (int s2 = 0; s2 < NS / 2; s2++)
-                kf1[s2] = *reinterpret_cast<const half8*>(
-                    &ktile_next[krow][(NS / 2 + s2) * 16 + g * 8]);
-            split_move<HD>(sm, f, rg, i, tid);
+                kf1[s2] = *reinterpret_cast<const half8*>(smem + kslot + cx.kread[NS / 2 + s2]);
         }
         if (s == NS / 2) {
 #pragma unroll
             for (int dt = 0; dt < ND; dt++)
-                vf1[dt] = *reinterpret_cast<const half8*>(&vtile[dt * 32 + n][16 + 8 * g]);
+                vf1[dt] = *reinterpret_cast<const half8*>(smem + vslot + cx.vread[1] + dt * 2048);
         }
         if (s >= NS / 2) {
             // the first eight probabilities are complete: their half of P.V fills
@@ -714,46 +719,47 @@ __device__ __forceinline__ void split_step(PrefillRows<HD>& R, f32x16& c, f32x16
 #pragma unroll
     for (int dt = 0; dt < ND; dt++)
         R.o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf1[dt], pop[1], R.o[dt], 0, 0, 0);
-    // vector work of one probability: subtract, exp2, add, half a pack; plus the
-    // address arithmetic of the data movement
-    split_step_order<0, NS, (7 * EPS + 1) / 2 + 2, 2 * (HD / 64)>();
+    // vector work of one probability: subtract, exp2, add, half a pack
+    split_step_order<0, NS, (7 * EPS + 1) / 2 + 1>();
     __builtin_amdgcn_sched_group_barrier(0x008, ND, 0);
     sn = acc;
+    // the loads for later steps leave once the operand reads are in the queue
+    split_move<HD>(cx, i, wave);
 }
 
 // Work of one wave in pipeline step i: the tile t_first + 2*i + kg is finished
 // (scores in `c`), the scores of the tile two further go to `sn`, and the
-// wave's share of the step's data movement is issued.
+// wave's share of the step's loads is issued.  Every wave runs the same code in
+// every step: a wave whose range does not hold the step's tile works on scores
+// of -inf (probabilities 0; the staged Vt it multiplies them with is real data
+// of the block), and scores computed for a tile past its range are never used.
+// One path keeps the accumulators in the same registers throughout the loop.
 template <int HD>
 __device__ __forceinline__ void split_wave_step(PrefillRows<HD>& R, f32x16& c, f32x16& sn,
-                                                SplitSmem<HD>& sm, SplitFeed<HD>& f,
-                                                const SplitRange& rg, uint32_t i, int tid, int kg,
-                                                int n, int g, int krow)
+                                                const unsigned char* smem, const SplitCtx<HD>& cx,
+                                                uint32_t i, int wave, int g)
 {
-    const uint32_t tile = rg.t_first + 2 * i + kg;
+    using L = SplitLds<HD>;
+    const int kg = wave >> 2;
+    const uint32_t tile = cx.t_first + 2 * i + kg;
     const bool has_cur = R.wave_ok && tile >= R.wt_first && tile <= R.wt_last;
-    const bool has_next = R.wave_ok && tile + 2 >= R.wt_first && tile + 2 <= R.wt_last;
-    const int kb = (i + 1) & 1, vb = i & 1;               // K is staged one step ahead of V
-    split_mask_tail<HD>(f.v, rg, i + 1, tid);
-    if (has_cur && has_next) {
-        split_step<HD>(R, c, sn, sm, f, rg, i, tid, &sm.k[kb][kg * kTileKeys], sm.v[vb][kg], tile,
-                       n, g, krow);
-    } else {
-        split_move<HD>(sm, f, rg, i, tid);
-        if (has_next)
-            split_scores<HD>(R, sn, &sm.k[kb][kg * kTileKeys], g, krow);
-        else if (has_cur)
-            split_finish<HD>(R, c, sm.v[vb][kg], tile, n, g);
+    if (!has_cur) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) c[r] = -INFINITY;
     }
+    const uint32_t kslot = L::K_OFF + ((i + 1) % kRing) * L::KPAIR;   // K is one step ahead of Vt
+    const uint32_t vslot = L::V_OFF + (i % kRing) * L::VPAIR;
+    split_step<HD>(R, c, sn, smem, cx, i, wave, kslot, vslot, tile, g);
 }
 
 template <int HD>
-__device__ __forceinline__ void split_block(const PrefillArgs& a, unsigned char* smem_raw,
+__device__ __forceinline__ void split_block(const PrefillArgs& a, unsigned char* smem,
                                             uint32_t pb, uint32_t kvh, uint32_t hc)
 {
-    SplitSmem<HD>& sm = *reinterpret_cast<SplitSmem<HD>*>(smem_raw);
+    using L = SplitLds<HD>;
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // in a scalar register
     const int n = lane & 31, g = lane >> 5;
     const int kg = wave >> 2, sub = wave & 3;             // key set (tile parity), rows served
     const uint32_t G = a.group;
@@ -761,33 +767,54 @@ __device__ __forceinline__ void split_block(const PrefillArgs& a, unsigned char*
     const uint32_t BP = 32 * (4 / Gw);                    // positions per block
     const uint32_t head = kvh * G + hc * Gw + (sub % Gw);
     const uint32_t row0 = pb * BP + (sub / Gw) * 32;      // first chunk row of this wave
-    SplitRange rg;
-    prefill_block_tiles(a, pb, BP, rg.t_first, rg.t_last);
-    rg.npairs = (rg.t_last - rg.t_first) / 2 + 1;
-    rg.kv_valid = a.p0 + a.T;                             // rows of the cache that hold data
-    rg.kbase = a.k + (size_t)kvh * a.ctx_pad * HD;
-    rg.vtbase = a.vt + (size_t)kvh * (a.ctx_pad / kVBlock) * HD * kVBlock;
+    SplitCtx<HD> cx;
+    prefill_block_tiles(a, pb, BP, cx.t_first, cx.t_last);
+    cx.npairs = (cx.t_last - cx.t_first) / 2 + 1;
+    cx.kv_valid = a.p0 + a.T;                             // rows of the cache that hold data
+    cx.kbase = uniform_ptr(reinterpret_cast<const unsigned char*>(a.k + (size_t)kvh * a.ctx_pad * HD));
+    cx.vtbase = uniform_ptr(reinterpret_cast<const unsigned char*>(
+        a.vt + (size_t)kvh * (a.ctx_pad / kVBlock) * HD * kVBlock));
+    // low half of a generic LDS pointer = LDS byte address
+    cx.lds0 = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)smem);
+#pragma unroll
+    for (int u = 0; u < L::NL; u++) {
+        const int q = wave + 8 * u;
+        {   // K: lane -> (row of the pair, slot); fetch the chunk that belongs in that slot
+            const int row = q * (1024 / L::RB) + lane / L::CPR;
+            const int c = (lane % L::CPR) ^ L::fk(row);
+            cx.gk_off[u] = row * L::RB + c * 16;
+        }
+        {   // Vt: rows of 64 bytes, four slots each
+            const int row = q * 16 + lane / 4;
+            const int c = (lane & 3) ^ L::fv(row);
+            cx.gv_off[u] = row * 64 + c * 16;
+        }
+    }
+    {
+        const int krow = kg * kTileKeys + prefill_key_perm(n);   // pair row this lane feeds to MFMA row n
+#pragma unroll
+        for (int s = 0; s < HD / 16; s++)
+            cx.kread[s] = krow * L::RB + (((2 * s + g) ^ L::fk(krow)) * 16);
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+            cx.vread[t] = kg * (L::VPAIR / 2) + n * 64 + (((2 * t + g) ^ L::fv(n)) * 16);
+    }
 
-    // Register sets: f1 is stored by odd steps (and by the prologue, "step -1"),
-    // f0 by even steps.  Step i stores K of pair i+2 and Vt of pair i+1.
-    SplitFeed<HD> f0, f1;
-    u32x4 kfirst[HD / 64];
-    split_fetch<HD>(kfirst, rg.kbase, rg, 0, tid);
-    split_fetch<HD>(f1.k, rg.kbase, rg, 1, tid);
-    split_fetch<HD>(f1.v, rg.vtbase, rg, 0, tid);
-    split_fetch<HD>(f0.k, rg.kbase, rg, 2, tid);
-    split_fetch<HD>(f0.v, rg.vtbase, rg, 1, tid);
+    // Everything step 0 and step 1 read, in order of need.
+    split_issue_k<HD>(cx, 0, 0, wave);
+    split_issue_k<HD>(cx, 1, 1, wave);
+    split_issue_v<HD>(cx, 0, 0, wave);
+    split_issue_k<HD>(cx, 2, 2, wave);
+    split_issue_v<HD>(cx, 1, 1, wave);
 
     PrefillRows<HD> R;
     prefill_rows_init<HD, false>(R, a, row0, head, n, g);
-    const int krow = prefill_key_perm(n);                 // LDS row this lane feeds to MFMA row n
 
     // Q: every row is 4*HD contiguous bytes in global memory, so it is read with
     // whole-row coalesced loads (the two waves serving a sub-block take 16 rows
     // each), converted to pre-scaled F16 and turned into the per-lane operand
-    // layout through LDS (the Vt staging area, not in use yet).
-    _Float16 (*qs)[32][HD + 8] = reinterpret_cast<_Float16 (*)[32][HD + 8]>(&sm.v[0][0][0][0]);
-    static_assert(sizeof(sm.v) >= (size_t)4 * 32 * (HD + 8) * sizeof(_Float16), "Q staging fits");
+    // layout through LDS.
+    _Float16 (*qs)[32][HD + 8] = reinterpret_cast<_Float16 (*)[32][HD + 8]>(smem + L::Q_OFF);
     {
         constexpr int LPR = HD / 4;                       // lanes per row (one float4 each)
         constexpr int RPI = 64 / LPR;                     // rows per load instruction
@@ -806,38 +833,42 @@ __device__ __forceinline__ void split_block(const PrefillArgs& a, unsigned char*
         }
     }
 
-    // prologue: K of pair 0 and Q become visible, then the first scores, then
-    // (Q staging read by everyone) what step 0 reads
+    // prologue: the first pairs and Q become visible, then the first scores
     f32x16 s0, s1;
 #pragma unroll
     for (int r = 0; r < 16; r++) s0[r] = s1[r] = 0.f;
-    split_stash_k<HD>(sm, 0, kfirst, tid);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     lds_barrier();
 #pragma unroll
     for (int s = 0; s < HD / 16; s++)
         R.qop[s] = *reinterpret_cast<const half8*>(&qs[sub][n][s * 16 + g * 8]);
     {
-        const uint32_t tile = rg.t_first + kg;
+        const uint32_t tile = cx.t_first + kg;
         if (R.wave_ok && tile >= R.wt_first && tile <= R.wt_last)
-            split_scores<HD>(R, s0, &sm.k[0][kg * kTileKeys], g, krow);
+            split_scores<HD>(R, s0, smem, cx, L::K_OFF);
     }
-    lds_barrier();
-    split_mask_tail<HD>(f1.v, rg, 0, tid);
-    split_move<HD>(sm, f1, rg, 0xFFFFFFFFu, tid);         // step -1: K of pair 1, Vt of pair 0
 
+    // Before barrier i every load but the ones step i-1 issued has landed: K of
+    // pair i+1 and Vt of pair i, which step i reads, left in step i-2.
     for (uint32_t i = 0;; i += 2) {
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * L::NL) : "memory");
+        split_patch_tail<HD>(smem, cx, i, wave, lane);
         lds_barrier();
-        split_wave_step<HD>(R, s0, s1, sm, f0, rg, i, tid, kg, n, g, krow);
-        if (i + 1 >= rg.npairs) break;
+        split_wave_step<HD>(R, s0, s1, smem, cx, i, wave, g);
+        if (i + 1 >= cx.npairs) break;
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * L::NL) : "memory");
+        split_patch_tail<HD>(smem, cx, i + 1, wave, lane);
         lds_barrier();
-        split_wave_step<HD>(R, s1, s0, sm, f1, rg, i + 1, tid, kg, n, g, krow);
-        if (i + 2 >= rg.npairs) break;
+        split_wave_step<HD>(R, s1, s0, smem, cx, i + 1, wave, g);
+        if (i + 2 >= cx.npairs) break;
     }
 
-    // merge the odd-tile partials into the even-tile waves
+    // merge the odd-tile partials into the even-tile waves; the ring must be
+    // quiet first (the last steps' loads still target it)
     constexpr int NREG = HD / 2;
-    float* mg = reinterpret_cast<float*>(smem_raw) + (size_t)sub * (NREG + 2) * 64;
-    __syncthreads();                                      // staging buffers are free
+    float* mg = reinterpret_cast<float*>(smem) + (size_t)sub * (NREG + 2) * 64;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
     if (kg == 1) {
 #pragma unroll
         for (int dt = 0; dt < HD / 32; dt++)
