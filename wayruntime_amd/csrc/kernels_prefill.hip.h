@@ -415,9 +415,14 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_mfma_kernel(const 
 //    of tile j run on the vector ALU, the score MFMAs of tile j+1 (a dependent
 //    chain) and the first half of tile j's P.V MFMAs run on the matrix pipe.
 //    To have tile j+1's K next to tile j's Vt, K is staged one step ahead of V.
-//  * The workgroup stages a PAIR of tiles per step (64 keys: contiguous in both
-//    K and the block-transposed V) with one barrier per step, in a ring of three
-//    pair buffers.  Tiles travel from global memory straight into LDS
+//  * The two wave sets run independently of each other until the merge: each
+//    stages its own tiles in its own ring of three tile buffers and synchronises
+//    its four waves with a counter in LDS instead of the workgroup barrier.
+//    The two waves that share a SIMD belong to different sets, so they drift
+//    apart and one's barrier wait or LDS latency is covered by the other's
+//    arithmetic; a workgroup-wide barrier per step would keep them in lock-step,
+//    both waiting at the same time.
+//  * Tiles travel from global memory straight into LDS
 //    (global_load_lds_dwordx4: no staging registers, no LDS store instructions),
 //    issued from inside the step's arithmetic three steps (K) / two steps (Vt)
 //    before their first use.
@@ -427,8 +432,8 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_mfma_kernel(const 
 //    permutation inside a row keeps the access coalesced.  f is chosen so that
 //    the sixteen rows a 128-bit LDS read touches per cycle fall into sixteen
 //    different slots of the 256-byte bank row.
-//  * Loads are issued unconditionally (pair indices clamped to the block's last
-//    pair; duplicates land in ring slots nobody reads) so the number in flight
+//  * Loads are issued unconditionally (tile indices clamped to the set's last
+//    tile; duplicates land in ring slots nobody reads) so the number in flight
 //    is the same at every barrier and "all but the newest N" is a fixed wait.
 //  * Instruction order inside a step is requested from the scheduler with
 //    scheduling-group barriers: one MFMA, then the few vector / LDS
@@ -445,17 +450,18 @@ struct SplitLds {
     static constexpr int RB = 2 * HD;                     // bytes per K row
     static constexpr int CPR = HD / 8;                    // 16-byte chunks per K row
     static constexpr int RPB = 256 / RB > 0 ? 256 / RB : 1;   // K rows per 256-byte bank row
-    static constexpr int KPAIR = 2 * kTileKeys * RB;      // bytes of one pair's K
-    static constexpr int VPAIR = 2 * HD * kVBlock * 2;    // bytes of one pair's Vt (two blocks)
-    static constexpr int NL = KPAIR / 1024 / 8;           // loads per wave and pair, each of K and Vt
-    static constexpr int K_OFF = 0;
-    static constexpr int V_OFF = kRing * KPAIR;
-    static constexpr int Q_OFF = V_OFF + kRing * VPAIR;   // Q staging, [4][32][HD + 8] halves
+    static constexpr int KTILE = kTileKeys * RB;          // bytes of one tile's K
+    static constexpr int VTILE = HD * kVBlock * 2;        // bytes of one tile's Vt block
+    static constexpr int NL = KTILE / 1024 / 4;           // loads per wave and tile, each of K and Vt
+    static constexpr int SET_BYTES = kRing * (KTILE + VTILE);   // one wave set's ring
+    static constexpr int V_IN_SET = kRing * KTILE;        // Vt slots follow the K slots
+    static constexpr int Q_OFF = 2 * SET_BYTES;           // Q staging, [4][32][HD + 8] halves
     static constexpr int Q_BYTES = 4 * 32 * (HD + 8) * 2;
-    static constexpr int MERGE_BYTES = 4 * (HD / 2 + 2) * 64 * 4;   // laid over the ring
-    static constexpr int TOTAL = Q_OFF + Q_BYTES;
-    static_assert(MERGE_BYTES <= Q_OFF, "merge scratch fits the ring");
-    static_assert(KPAIR == VPAIR && NL >= 1, "one chunk schedule serves K and Vt");
+    static constexpr int CNT_OFF = Q_OFF + Q_BYTES;       // the two sets' arrival counters
+    static constexpr int MERGE_BYTES = 4 * (HD / 2 + 2) * 64 * 4;   // laid over the rings
+    static constexpr int TOTAL = CNT_OFF + 16;
+    static_assert(MERGE_BYTES <= Q_OFF, "merge scratch fits the rings");
+    static_assert(KTILE == VTILE && NL >= 1, "one chunk schedule serves K and Vt");
     // slot permutation of K rows / Vt rows
     __device__ static constexpr int fk(int row) { return (row / RPB) & (CPR - 1); }
     __device__ static constexpr int fv(int row) { return (row >> 2) & 3; }
@@ -467,18 +473,25 @@ constexpr size_t split_smem_bytes()
     return SplitLds<HD>::TOTAL;
 }
 
-// What a block streams (tile pairs 0 .. npairs-1 starting at tile t_first), from
-// where, and this lane's invariant addresses.
+// What one wave set streams (tiles t0, t0+2, ... : nt of them), from where, and
+// this lane's invariant addresses.
 template <int HD>
 struct SplitCtx {
     const unsigned char* kbase;       // this KV head's K / Vt, bytes
     const unsigned char* vtbase;
-    uint32_t lds0;                    // LDS byte address of the staging area
-    uint32_t t_first, t_last, npairs, kv_valid;
-    uint32_t gk_off[SplitLds<HD>::NL];    // lane's byte offset inside a pair's K, per load
-    uint32_t gv_off[SplitLds<HD>::NL];    // ... inside a pair's Vt
-    uint32_t kread[HD / 16];          // LDS offsets of the K operand reads (ring slot 0)
-    uint32_t vread[2];                // ... of the Vt operand reads, dt = 0
+    uint32_t lds0;                    // LDS byte address of the kernel's dynamic LDS
+    uint32_t ring;                    // byte offset of this set's ring in it
+    uint32_t cnt;                     // byte offset of this set's arrival counter
+    uint32_t t0, nt, t_last, kv_valid;   // nt may be 0 (the odd set of a one-tile block)
+    // Lane-invariant addresses, one register each; the others follow from them:
+    // a wave's second load of a tile is the first one 4 KiB further (same slot
+    // permutation), and the operand read of contraction step s / half t is the
+    // first one with address bits 5-7 / bit 5 flipped (the permutation is an
+    // XOR of the chunk index, the step is the chunk index's upper bits).
+    uint32_t gk_off;                  // lane's byte offset inside a K tile, first load
+    uint32_t gv_off;                  // ... inside a Vt block
+    uint32_t kread;                   // LDS offset of the K operand read of step 0 (ring slot 0)
+    uint32_t vread;                   // ... of the Vt operand read of t = 0, dt = 0
 };
 
 // Tells the compiler that a pointer is the same in every lane (keeps the
@@ -504,66 +517,53 @@ __device__ __forceinline__ void lds_direct_load(uint32_t lds_addr, const unsigne
                  : "memory");
 }
 
-// Loads of one pair's K into ring slot `slot`.  Chunk q = wave + 8u of the
-// pair: 1024 consecutive bytes.  When the pair's second tile lies past the
-// block's range (and possibly past the slab) its loads re-read the first tile.
+// Loads of the set's j-th K tile into ring slot `slot`.  Chunk q = sub + 4u of
+// the tile: 1024 consecutive bytes.
 template <int HD>
-__device__ __forceinline__ void split_issue_k(const SplitCtx<HD>& cx, uint32_t pair, int slot,
-                                              int wave)
+__device__ __forceinline__ void split_issue_k(const SplitCtx<HD>& cx, uint32_t j, int slot, int sub)
 {
     using L = SplitLds<HD>;
-    pair = min(pair, cx.npairs - 1);
-    const uint32_t tile = cx.t_first + 2 * pair;
-    const bool both = tile + 1 <= cx.t_last;
-    const unsigned char* src = cx.kbase + (size_t)tile * kTileKeys * L::RB;
+    const uint32_t tile = min(cx.t0 + 2 * j, cx.t_last);  // past the range: a duplicate nobody reads
+    const unsigned char* src = cx.kbase + (size_t)tile * L::KTILE;
 #pragma unroll
-    for (int u = 0; u < L::NL; u++) {
-        const int q = wave + 8 * u;
-        const bool second = q * 1024 >= L::KPAIR / 2;     // chunk belongs to the pair's second tile
-        const unsigned char* b = (second && !both) ? src - L::KPAIR / 2 : src;
-        lds_direct_load(cx.lds0 + L::K_OFF + slot * L::KPAIR + q * 1024, b, cx.gk_off[u]);
-    }
+    for (int u = 0; u < L::NL; u++)
+        lds_direct_load(cx.lds0 + cx.ring + slot * L::KTILE + (sub + 4 * u) * 1024, src + u * 4096,
+                        cx.gk_off);
 }
 
 template <int HD>
-__device__ __forceinline__ void split_issue_v(const SplitCtx<HD>& cx, uint32_t pair, int slot,
-                                              int wave)
+__device__ __forceinline__ void split_issue_v(const SplitCtx<HD>& cx, uint32_t j, int slot, int sub)
 {
     using L = SplitLds<HD>;
-    pair = min(pair, cx.npairs - 1);
-    const uint32_t tile = cx.t_first + 2 * pair;
-    const bool both = tile + 1 <= cx.t_last;
-    const unsigned char* src = cx.vtbase + (size_t)tile * HD * kVBlock * 2;
+    const uint32_t tile = min(cx.t0 + 2 * j, cx.t_last);
+    const unsigned char* src = cx.vtbase + (size_t)tile * L::VTILE;
 #pragma unroll
-    for (int u = 0; u < L::NL; u++) {
-        const int q = wave + 8 * u;
-        const bool second = q * 1024 >= L::VPAIR / 2;
-        const unsigned char* b = (second && !both) ? src - L::VPAIR / 2 : src;
-        lds_direct_load(cx.lds0 + L::V_OFF + slot * L::VPAIR + q * 1024, b, cx.gv_off[u]);
-    }
+    for (int u = 0; u < L::NL; u++)
+        lds_direct_load(cx.lds0 + cx.ring + L::V_IN_SET + slot * L::VTILE + (sub + 4 * u) * 1024,
+                        src + u * 4096, cx.gv_off);
 }
 
 // Rows that were never appended may hold anything: zero them in the staged Vt
-// of pair `pair` so 0 * garbage cannot reach the accumulator.  Only the pair
-// holding the end of the appended rows is affected.  Every lane patches the
-// chunks its own loads delivered, so the caller only has to have waited for
+// of the set's j-th tile so 0 * garbage cannot reach the accumulator.  Only the
+// tile holding the end of the appended rows is affected.  Every lane patches
+// the chunks its own loads delivered, so the caller only has to have waited for
 // this wave's loads.
 template <int HD>
 __device__ __forceinline__ void split_patch_tail(unsigned char* smem, const SplitCtx<HD>& cx,
-                                                 uint32_t pair, int wave, int lane)
+                                                 uint32_t j, int sub, int lane)
 {
     using L = SplitLds<HD>;
-    if (pair >= cx.npairs) return;
-    const uint32_t tile = cx.t_first + 2 * pair;
-    if ((tile + 2) * kTileKeys <= cx.kv_valid) return;
-    const int slot = pair % kRing;
+    const uint32_t tile = min(cx.t0 + 2 * j, cx.t_last);  // as loaded (an idle set holds a duplicate)
+    if ((tile + 1) * kTileKeys <= cx.kv_valid) return;
+    const int slot = j % kRing;
 #pragma unroll
     for (int u = 0; u < L::NL; u++) {
-        const int q = wave + 8 * u;
-        const int row = q * 16 + lane / 4;                // row of the pair's 2*HD Vt rows
+        const int q = sub + 4 * u;
+        const int row = q * 16 + lane / 4;                // Vt row (dimension)
         const int c = (lane & 3) ^ L::fv(row);            // key chunk this slot holds
-        const uint32_t key0 = (tile + row / HD) * kTileKeys + c * 8;
-        u32x4* at = reinterpret_cast<u32x4*>(smem + L::V_OFF + slot * L::VPAIR + q * 1024 + lane * 16);
+        const uint32_t key0 = tile * kTileKeys + c * 8;
+        u32x4* at = reinterpret_cast<u32x4*>(smem + cx.ring + L::V_IN_SET + slot * L::VTILE +
+                                             q * 1024 + lane * 16);
         u32x4 v = *at;
         uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
@@ -575,13 +575,33 @@ __device__ __forceinline__ void split_patch_tail(unsigned char* smem, const Spli
     }
 }
 
-// The data movement of step i: K of pair i+3 and Vt of pair i+2 replace K of
-// pair i and Vt of pair i-1, both read for the last time in step i-1.
+// The data movement of step j: K of the set's tile j+3 and Vt of tile j+2
+// replace K of tile j and Vt of tile j-1, both read for the last time in step j-1.
 template <int HD>
-__device__ __forceinline__ void split_move(const SplitCtx<HD>& cx, uint32_t i, int wave)
+__device__ __forceinline__ void split_move(const SplitCtx<HD>& cx, uint32_t j, int sub)
 {
-    split_issue_k<HD>(cx, i + 3, i % kRing, wave);
-    split_issue_v<HD>(cx, i + 2, (i + 2) % kRing, wave);
+    split_issue_k<HD>(cx, j + 3, j % kRing, sub);
+    split_issue_v<HD>(cx, j + 2, (j + 2) % kRing, sub);
+}
+
+// Barrier among the four waves of one set: every wave adds one to the set's
+// counter in LDS and waits until it has reached `target` (4 x the number of
+// barriers so far; the counter is never reset inside a block).  The wait is
+// bounded: should a wave never arrive, the others go on (with wrong data)
+// instead of hanging the device.
+__device__ __forceinline__ void set_barrier(unsigned char* smem, uint32_t cnt_off, uint32_t target,
+                                            int lane)
+{
+    uint32_t* cnt = reinterpret_cast<uint32_t*>(smem + cnt_off);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    if (lane == 0) __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    for (uint32_t spins = 0; spins < (1u << 22); spins++) {
+        const uint32_t seen = (uint32_t)__builtin_amdgcn_readfirstlane(
+            __hip_atomic_load(cnt, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP));
+        if ((int32_t)(seen - target) >= 0) break;
+        __builtin_amdgcn_s_sleep(1);
+    }
+    asm volatile("" ::: "memory");
 }
 
 // First part of a tile's softmax: masks, row maximum, reference point (moving
@@ -622,7 +642,7 @@ __device__ __forceinline__ float split_softmax_begin(PrefillRows<HD>& R, f32x16&
 }
 
 // Scores of one tile only (a wave's first tile).  kslot: byte offset of the ring
-// slot holding the tile's pair.
+// slot holding the tile's K.
 template <int HD>
 __device__ __forceinline__ void split_scores(const PrefillRows<HD>& R, f32x16& sn,
                                              const unsigned char* smem, const SplitCtx<HD>& cx,
@@ -631,7 +651,7 @@ __device__ __forceinline__ void split_scores(const PrefillRows<HD>& R, f32x16& s
     half8 kf[HD / 16];
 #pragma unroll
     for (int s = 0; s < HD / 16; s++)
-        kf[s] = *reinterpret_cast<const half8*>(smem + kslot + cx.kread[s]);
+        kf[s] = *reinterpret_cast<const half8*>(smem + ((kslot + cx.kread) ^ (s * 32)));
     f32x16 acc;
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[r] = 0.f;
@@ -675,10 +695,10 @@ __device__ __forceinline__ void split_step(PrefillRows<HD>& R, f32x16& c, f32x16
     half8 kf0[NS / 2], kf1[NS / 2], vf0[ND], vf1[ND];
 #pragma unroll
     for (int s = 0; s < NS / 2; s++)
-        kf0[s] = *reinterpret_cast<const half8*>(smem + kslot + cx.kread[s]);
+        kf0[s] = *reinterpret_cast<const half8*>(smem + ((kslot + cx.kread) ^ (s * 32)));
 #pragma unroll
     for (int dt = 0; dt < ND; dt++)
-        vf0[dt] = *reinterpret_cast<const half8*>(smem + vslot + cx.vread[0] + dt * 2048);
+        vf0[dt] = *reinterpret_cast<const half8*>(smem + (vslot + cx.vread) + dt * 2048);
     const float m = split_softmax_begin<HD>(R, c, tile, g);
     __builtin_amdgcn_sched_barrier(0);
 
@@ -694,12 +714,12 @@ __device__ __forceinline__ void split_step(PrefillRows<HD>& R, f32x16& c, f32x16
         if (s == 0) {
 #pragma unroll
             for (int s2 = 0; s2 < NS / 2; s2++)
-                kf1[s2] = *reinterpret_cast<const half8*>(smem + kslot + cx.kread[NS / 2 + s2]);
+                kf1[s2] = *reinterpret_cast<const half8*>(smem + ((kslot + cx.kread) ^ ((NS / 2 + s2) * 32)));
         }
         if (s == NS / 2) {
 #pragma unroll
             for (int dt = 0; dt < ND; dt++)
-                vf1[dt] = *reinterpret_cast<const half8*>(smem + vslot + cx.vread[1] + dt * 2048);
+                vf1[dt] = *reinterpret_cast<const half8*>(smem + ((vslot + cx.vread) ^ 32) + dt * 2048);
         }
         if (s >= NS / 2) {
             // the first eight probabilities are complete: their half of P.V fills
@@ -724,32 +744,31 @@ __device__ __forceinline__ void split_step(PrefillRows<HD>& R, f32x16& c, f32x16
     __builtin_amdgcn_sched_group_barrier(0x008, ND, 0);
     sn = acc;
     // the loads for later steps leave once the operand reads are in the queue
-    split_move<HD>(cx, i, wave);
+    split_move<HD>(cx, i, wave & 3);
 }
 
-// Work of one wave in pipeline step i: the tile t_first + 2*i + kg is finished
-// (scores in `c`), the scores of the tile two further go to `sn`, and the
-// wave's share of the step's loads is issued.  Every wave runs the same code in
-// every step: a wave whose range does not hold the step's tile works on scores
-// of -inf (probabilities 0; the staged Vt it multiplies them with is real data
-// of the block), and scores computed for a tile past its range are never used.
-// One path keeps the accumulators in the same registers throughout the loop.
+// Work of one wave in its set's step j: the set's j-th tile is finished (scores
+// in `c`), the scores of tile j+1 go to `sn`, and the wave's share of the step's
+// loads is issued.  Every wave runs the same code in every step: a wave whose
+// range does not hold the step's tile works on scores of -inf (probabilities 0;
+// the staged Vt it multiplies them with is real data of the block), and scores
+// computed for a tile past its range are never used.  One path keeps the
+// accumulators in the same registers throughout the loop.
 template <int HD>
 __device__ __forceinline__ void split_wave_step(PrefillRows<HD>& R, f32x16& c, f32x16& sn,
                                                 const unsigned char* smem, const SplitCtx<HD>& cx,
-                                                uint32_t i, int wave, int g)
+                                                uint32_t j, int wave, int g)
 {
     using L = SplitLds<HD>;
-    const int kg = wave >> 2;
-    const uint32_t tile = cx.t_first + 2 * i + kg;
+    const uint32_t tile = cx.t0 + 2 * j;
     const bool has_cur = R.wave_ok && tile >= R.wt_first && tile <= R.wt_last;
     if (!has_cur) {
 #pragma unroll
         for (int r = 0; r < 16; r++) c[r] = -INFINITY;
     }
-    const uint32_t kslot = L::K_OFF + ((i + 1) % kRing) * L::KPAIR;   // K is one step ahead of Vt
-    const uint32_t vslot = L::V_OFF + (i % kRing) * L::VPAIR;
-    split_step<HD>(R, c, sn, smem, cx, i, wave, kslot, vslot, tile, g);
+    const uint32_t kslot = cx.ring + ((j + 1) % kRing) * L::KTILE;   // K is one step ahead of Vt
+    const uint32_t vslot = cx.ring + L::V_IN_SET + (j % kRing) * L::VTILE;
+    split_step<HD>(R, c, sn, smem, cx, j, wave, kslot, vslot, tile, g);
 }
 
 template <int HD>
@@ -767,45 +786,45 @@ __device__ __forceinline__ void split_block(const PrefillArgs& a, unsigned char*
     const uint32_t BP = 32 * (4 / Gw);                    // positions per block
     const uint32_t head = kvh * G + hc * Gw + (sub % Gw);
     const uint32_t row0 = pb * BP + (sub / Gw) * 32;      // first chunk row of this wave
+    uint32_t t_first, t_last;
+    prefill_block_tiles(a, pb, BP, t_first, t_last);
     SplitCtx<HD> cx;
-    prefill_block_tiles(a, pb, BP, cx.t_first, cx.t_last);
-    cx.npairs = (cx.t_last - cx.t_first) / 2 + 1;
+    cx.t0 = t_first + kg;                                 // this set's tiles: t0, t0 + 2, ...
+    cx.nt = (cx.t0 <= t_last) ? (t_last - cx.t0) / 2 + 1 : 0;
+    cx.t_last = t_last;
     cx.kv_valid = a.p0 + a.T;                             // rows of the cache that hold data
     cx.kbase = uniform_ptr(reinterpret_cast<const unsigned char*>(a.k + (size_t)kvh * a.ctx_pad * HD));
     cx.vtbase = uniform_ptr(reinterpret_cast<const unsigned char*>(
         a.vt + (size_t)kvh * (a.ctx_pad / kVBlock) * HD * kVBlock));
     // low half of a generic LDS pointer = LDS byte address
     cx.lds0 = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)smem);
-#pragma unroll
-    for (int u = 0; u < L::NL; u++) {
-        const int q = wave + 8 * u;
-        {   // K: lane -> (row of the pair, slot); fetch the chunk that belongs in that slot
-            const int row = q * (1024 / L::RB) + lane / L::CPR;
-            const int c = (lane % L::CPR) ^ L::fk(row);
-            cx.gk_off[u] = row * L::RB + c * 16;
-        }
-        {   // Vt: rows of 64 bytes, four slots each
-            const int row = q * 16 + lane / 4;
-            const int c = (lane & 3) ^ L::fv(row);
-            cx.gv_off[u] = row * 64 + c * 16;
-        }
-    }
+    cx.ring = kg * L::SET_BYTES;
+    cx.cnt = L::CNT_OFF + kg * 4;
     {
-        const int krow = kg * kTileKeys + prefill_key_perm(n);   // pair row this lane feeds to MFMA row n
-#pragma unroll
-        for (int s = 0; s < HD / 16; s++)
-            cx.kread[s] = krow * L::RB + (((2 * s + g) ^ L::fk(krow)) * 16);
-#pragma unroll
-        for (int t = 0; t < 2; t++)
-            cx.vread[t] = kg * (L::VPAIR / 2) + n * 64 + (((2 * t + g) ^ L::fv(n)) * 16);
+        // K: lane -> (row of the tile, slot); fetch the chunk that belongs in that slot
+        const int row = sub * (1024 / L::RB) + lane / L::CPR;
+        cx.gk_off = row * L::RB + ((lane % L::CPR) ^ L::fk(row)) * 16;
+        // Vt: rows of 64 bytes, four slots each
+        const int vrow = sub * 16 + lane / 4;
+        cx.gv_off = vrow * 64 + ((lane & 3) ^ L::fv(vrow)) * 16;
+        static_assert(L::NL == 1 || (L::fk(4 * (1024 / L::RB)) == L::fk(0) && L::fv(64) == L::fv(0) &&
+                                     4 * (1024 / L::RB) * L::RB == 4096),
+                      "the second load is the first one 4 KiB further");
+        const int krow = prefill_key_perm(n);             // tile row this lane feeds to MFMA row n
+        cx.kread = krow * L::RB + ((g ^ L::fk(krow)) * 16);
+        cx.vread = n * 64 + ((g ^ L::fv(n)) * 16);
     }
 
-    // Everything step 0 and step 1 read, in order of need.
-    split_issue_k<HD>(cx, 0, 0, wave);
-    split_issue_k<HD>(cx, 1, 1, wave);
-    split_issue_v<HD>(cx, 0, 0, wave);
-    split_issue_k<HD>(cx, 2, 2, wave);
-    split_issue_v<HD>(cx, 1, 1, wave);
+    // Everything steps 0 and 1 of this set read, in order of need.  (A set
+    // without a tile, the odd set of a one-tile block, goes through one step
+    // all the same, on duplicates of the block's last tile and scores of -inf:
+    // a path around the loop would cost the loop its register allocation.)
+    split_issue_k<HD>(cx, 0, 0, sub);
+    split_issue_k<HD>(cx, 1, 1, sub);
+    split_issue_v<HD>(cx, 0, 0, sub);
+    split_issue_k<HD>(cx, 2, 2, sub);
+    split_issue_v<HD>(cx, 1, 1, sub);
+    if (tid < 2) reinterpret_cast<uint32_t*>(smem + L::CNT_OFF)[tid] = 0;
 
     PrefillRows<HD> R;
     prefill_rows_init<HD, false>(R, a, row0, head, n, g);
@@ -833,7 +852,8 @@ __device__ __forceinline__ void split_block(const PrefillArgs& a, unsigned char*
         }
     }
 
-    // prologue: the first pairs and Q become visible, then the first scores
+    // prologue: the first tiles, Q and the zeroed counters become visible to
+    // the whole workgroup, then every set computes its first scores
     f32x16 s0, s1;
 #pragma unroll
     for (int r = 0; r < 16; r++) s0[r] = s1[r] = 0.f;
@@ -842,25 +862,26 @@ __device__ __forceinline__ void split_block(const PrefillArgs& a, unsigned char*
 #pragma unroll
     for (int s = 0; s < HD / 16; s++)
         R.qop[s] = *reinterpret_cast<const half8*>(&qs[sub][n][s * 16 + g * 8]);
-    {
-        const uint32_t tile = cx.t_first + kg;
-        if (R.wave_ok && tile >= R.wt_first && tile <= R.wt_last)
-            split_scores<HD>(R, s0, smem, cx, L::K_OFF);
-    }
+    if (R.wave_ok && cx.t0 >= R.wt_first && cx.t0 <= R.wt_last)
+        split_scores<HD>(R, s0, smem, cx, cx.ring);
 
-    // Before barrier i every load but the ones step i-1 issued has landed: K of
-    // pair i+1 and Vt of pair i, which step i reads, left in step i-2.
-    for (uint32_t i = 0;; i += 2) {
+    // Before the barrier of step j every load of this wave but the ones step
+    // j-1 issued has landed: K of tile j+1 and Vt of tile j, which step j
+    // reads, left in step j-2.  The barrier is the set's own: it publishes the
+    // four waves' loads to each other and tells them that the slots step j
+    // overwrites are no longer being read.
+    const uint32_t nsteps = max(cx.nt, 1u);
+    for (uint32_t j = 0;; j += 2) {
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * L::NL) : "memory");
-        split_patch_tail<HD>(smem, cx, i, wave, lane);
-        lds_barrier();
-        split_wave_step<HD>(R, s0, s1, smem, cx, i, wave, g);
-        if (i + 1 >= cx.npairs) break;
+        split_patch_tail<HD>(smem, cx, j, sub, lane);
+        set_barrier(smem, cx.cnt, 4 * (j + 1), lane);
+        split_wave_step<HD>(R, s0, s1, smem, cx, j, wave, g);
+        if (j + 1 >= nsteps) break;
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * L::NL) : "memory");
-        split_patch_tail<HD>(smem, cx, i + 1, wave, lane);
-        lds_barrier();
-        split_wave_step<HD>(R, s1, s0, smem, cx, i + 1, wave, g);
-        if (i + 2 >= cx.npairs) break;
+        split_patch_tail<HD>(smem, cx, j + 1, sub, lane);
+        set_barrier(smem, cx.cnt, 4 * (j + 2), lane);
+        split_wave_step<HD>(R, s1, s0, smem, cx, j + 1, wave, g);
+        if (j + 2 >= nsteps) break;
     }
 
     // merge the odd-tile partials into the even-tile waves; the ring must be
