@@ -763,6 +763,9 @@ __device__ __forceinline__ void split_wave_step(PrefillRows<HD>& R, f32x16& c, f
     const uint32_t tile = cx.t0 + 2 * j;
     const bool has_cur = R.wave_ok && tile >= R.wt_first && tile <= R.wt_last;
     if (!has_cur) {
+        // rare and wave-uniform: keep it a branch (the empty statement stops the
+        // compiler from turning it into sixteen selects executed in every step)
+        asm volatile("" ::: "memory");
 #pragma unroll
         for (int r = 0; r < 16; r++) c[r] = -INFINITY;
     }
