@@ -604,11 +604,29 @@ __device__ __forceinline__ void set_barrier(unsigned char* smem, uint32_t cnt_of
     asm volatile("" ::: "memory");
 }
 
-// First part of a tile's softmax: masks, row maximum, reference point (moving
-// it rescales the accumulators).  Returns the value to subtract from the scores.
+// max of three without the canonicalising self-maximum the compiler puts in
+// front of every fmaxf operand (the operands here are never signalling NaNs
+// that anyone would want quieted)
+__device__ __forceinline__ float max3_raw(float a, float b, float c)
+{
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
+// First part of a tile's softmax: masks, row maximum, reference point.
+//
+// The scores arrive with the row's reference point already subtracted: the
+// score chain starts from the accumulator block `negm` (-m_run in all sixteen
+// registers; 0 while the row has no reference yet), so in the steady state the
+// probabilities are exp2 of the scores as they are, with no subtraction.  The
+// reference moves only when a row's maximum exceeds it by more than kLazyLog2
+// (or is the row's first finite score): then the scores of this tile are
+// shifted, the accumulators rescaled and `negm` rewritten.  With 32 independent
+// rows per wave an eager maximum would move in most tiles.
 template <int HD>
-__device__ __forceinline__ float split_softmax_begin(PrefillRows<HD>& R, f32x16& c, uint32_t tile,
-                                                     int g)
+__device__ __forceinline__ void split_softmax_begin(PrefillRows<HD>& R, f32x16& negm, f32x16& c,
+                                                    uint32_t tile, int g)
 {
     const uint32_t kb = tile * kTileKeys;
     // register r of this lane: key kb + 16*(r/8) + 8*g + r%8, row n.
@@ -622,43 +640,55 @@ __device__ __forceinline__ float split_softmax_begin(PrefillRows<HD>& R, f32x16&
             if (key > R.pos || key < R.row_lo) c[r] = -INFINITY;
         }
     }
-    float tmax = c[0];
+    float tmax = max3_raw(c[0], c[1], c[2]);
 #pragma unroll
-    for (int r = 1; r < 16; r++) tmax = fmaxf(tmax, c[r]);
-    tmax = wave_pair32_max(tmax);
-    const bool jump = tmax > R.m_run + kLazyLog2;          // false for tmax = -inf
-    const float m_new = jump ? tmax : R.m_run;
-    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;   // row with nothing visible yet
+    for (int r = 3; r < 15; r += 2) tmax = max3_raw(tmax, c[r], c[r + 1]);
+    tmax = max3_raw(tmax, c[15], c[15]);
+    {
+        const uint32_t u = __float_as_uint(tmax);
+        const auto sw = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+        tmax = max3_raw(__uint_as_float(sw[0]), __uint_as_float(sw[1]), tmax);   // same in both lanes of a row
+    }
+    const bool unset = (R.m_run == -INFINITY);
+    const bool jump = unset ? (tmax > -INFINITY) : (tmax > kLazyLog2);
     if (__builtin_amdgcn_ballot_w64(jump) != 0) {
-        const float alpha = jump ? fast_exp2(R.m_run - m_safe) : 1.0f;
+        const float delta = jump ? tmax : 0.f;
+        const float alpha = jump ? (unset ? 0.f : fast_exp2(-delta)) : 1.0f;
         R.l_run *= alpha;
 #pragma unroll
         for (int dt = 0; dt < HD / 32; dt++)
 #pragma unroll
             for (int r = 0; r < 16; r++) R.o[dt][r] *= alpha;
+        // The two blocks are updated in place, with the instructions spelled
+        // out: left to itself the compiler gives the updated values new
+        // registers and pays for it with 32 copies on the path that skips this
+        // branch, which is the one that matters.
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+            asm volatile("v_sub_f32 %0, %0, %1" : "+v"(c[r]) : "v"(delta));
+        if (jump) R.m_run = (unset ? 0.f : R.m_run) + delta;
+        const float nm = (R.m_run == -INFINITY) ? 0.f : -R.m_run;
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+            asm volatile("v_mov_b32 %0, %1" : "+v"(negm[r]) : "v"(nm));
     }
-    R.m_run = m_new;
-    return m_safe;
 }
 
 // Scores of one tile only (a wave's first tile).  kslot: byte offset of the ring
 // slot holding the tile's K.
 template <int HD>
-__device__ __forceinline__ void split_scores(const PrefillRows<HD>& R, f32x16& sn,
-                                             const unsigned char* smem, const SplitCtx<HD>& cx,
-                                             uint32_t kslot)
+__device__ __forceinline__ void split_scores(const PrefillRows<HD>& R, const f32x16& negm,
+                                             f32x16& sn, const unsigned char* smem,
+                                             const SplitCtx<HD>& cx, uint32_t kslot)
 {
     half8 kf[HD / 16];
 #pragma unroll
     for (int s = 0; s < HD / 16; s++)
         kf[s] = *reinterpret_cast<const half8*>(smem + ((kslot + cx.kread) ^ (s * 32)));
-    f32x16 acc;
+    sn = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[0], R.qop[0], negm, 0, 0, 0);
 #pragma unroll
-    for (int r = 0; r < 16; r++) acc[r] = 0.f;
-#pragma unroll
-    for (int s = 0; s < HD / 16; s++)
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[s], R.qop[s], acc, 0, 0, 0);
-    sn = acc;
+    for (int s = 1; s < HD / 16; s++)
+        sn = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[s], R.qop[s], sn, 0, 0, 0);
 }
 
 // Instruction order of the steady-state step, as a request to the scheduler
@@ -684,7 +714,7 @@ __device__ __forceinline__ void split_step_order()
 // with the score MFMAs of the wave's next tile (result in `sn`) and with the
 // step's data movement.
 template <int HD>
-__device__ __forceinline__ void split_step(PrefillRows<HD>& R, f32x16& c, f32x16& sn,
+__device__ __forceinline__ void split_step(PrefillRows<HD>& R, f32x16& negm, f32x16& c, f32x16& sn,
                                            const unsigned char* smem, const SplitCtx<HD>& cx,
                                            uint32_t i, int wave, uint32_t kslot, uint32_t vslot,
                                            uint32_t tile, int g)
@@ -699,18 +729,21 @@ __device__ __forceinline__ void split_step(PrefillRows<HD>& R, f32x16& c, f32x16
 #pragma unroll
     for (int dt = 0; dt < ND; dt++)
         vf0[dt] = *reinterpret_cast<const half8*>(smem + (vslot + cx.vread) + dt * 2048);
-    const float m = split_softmax_begin<HD>(R, c, tile, g);
+    split_softmax_begin<HD>(R, negm, c, tile, g);
     __builtin_amdgcn_sched_barrier(0);
 
     half8 pop[2];
     float psum = 0.f;
-    f32x16 acc;
-#pragma unroll
-    for (int r = 0; r < 16; r++) acc[r] = 0.f;
+    const half2v ones = {(_Float16)1.0f, (_Float16)1.0f};
 #pragma unroll
     for (int s = 0; s < NS; s++) {
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(s < NS / 2 ? kf0[s % (NS / 2)] : kf1[s % (NS / 2)],
-                                                     R.qop[s], acc, 0, 0, 0);
+        // the chain starts from the reference block and writes the next scores
+        // directly (no copy of either)
+        if (s == 0)
+            sn = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf0[0], R.qop[0], negm, 0, 0, 0);
+        else
+            sn = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                s < NS / 2 ? kf0[s % (NS / 2)] : kf1[s % (NS / 2)], R.qop[s], sn, 0, 0, 0);
         if (s == 0) {
 #pragma unroll
             for (int s2 = 0; s2 < NS / 2; s2++)
@@ -727,22 +760,25 @@ __device__ __forceinline__ void split_step(PrefillRows<HD>& R, f32x16& c, f32x16
             const int dt = s - NS / 2;
             R.o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf0[dt], pop[0], R.o[dt], 0, 0, 0);
         }
+        // probabilities in pairs: two exp2, one pack to F16, one dot product with
+        // (1, 1) that adds the two ROUNDED values to the row sum, so the
+        // normaliser is the sum of exactly what P.V multiplies
 #pragma unroll
-        for (int e = 0; e < EPS; e++) {
+        for (int e = 0; e < EPS; e += 2) {
             const int r = s * EPS + e;
-            const float p = fast_exp2(c[r] - m);
-            psum += p;
-            pop[r >> 3][r & 7] = (_Float16)p;
+            const half2v ph = {(_Float16)fast_exp2(c[r]), (_Float16)fast_exp2(c[r + 1])};
+            psum = __builtin_amdgcn_fdot2(ph, ones, psum, false);
+            pop[r >> 3][r & 7] = ph[0];
+            pop[r >> 3][(r & 7) + 1] = ph[1];
         }
     }
     R.l_run += psum;
 #pragma unroll
     for (int dt = 0; dt < ND; dt++)
         R.o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf1[dt], pop[1], R.o[dt], 0, 0, 0);
-    // vector work of one probability: subtract, exp2, add, half a pack
-    split_step_order<0, NS, (7 * EPS + 1) / 2 + 1>();
+    // vector work of one probability: exp2, half a pack, half a dot product
+    split_step_order<0, NS, 2 * EPS + 1>();
     __builtin_amdgcn_sched_group_barrier(0x008, ND, 0);
-    sn = acc;
     // the loads for later steps leave once the operand reads are in the queue
     split_move<HD>(cx, i, wave & 3);
 }
@@ -755,7 +791,8 @@ __device__ __forceinline__ void split_step(PrefillRows<HD>& R, f32x16& c, f32x16
 // computed for a tile past its range are never used.  One path keeps the
 // accumulators in the same registers throughout the loop.
 template <int HD>
-__device__ __forceinline__ void split_wave_step(PrefillRows<HD>& R, f32x16& c, f32x16& sn,
+__device__ __forceinline__ void split_wave_step(PrefillRows<HD>& R, f32x16& negm, f32x16& c,
+                                                f32x16& sn,
                                                 const unsigned char* smem, const SplitCtx<HD>& cx,
                                                 uint32_t j, int wave, int g)
 {
@@ -771,7 +808,7 @@ __device__ __forceinline__ void split_wave_step(PrefillRows<HD>& R, f32x16& c, f
     }
     const uint32_t kslot = cx.ring + ((j + 1) % kRing) * L::KTILE;   // K is one step ahead of Vt
     const uint32_t vslot = cx.ring + L::V_IN_SET + (j % kRing) * L::VTILE;
-    split_step<HD>(R, c, sn, smem, cx, j, wave, kslot, vslot, tile, g);
+    split_step<HD>(R, negm, c, sn, smem, cx, j, wave, kslot, vslot, tile, g);
 }
 
 template <int HD>
@@ -857,16 +894,16 @@ __device__ __forceinline__ void split_block(const PrefillArgs& a, unsigned char*
 
     // prologue: the first tiles, Q and the zeroed counters become visible to
     // the whole workgroup, then every set computes its first scores
-    f32x16 s0, s1;
+    f32x16 s0, s1, negm;
 #pragma unroll
-    for (int r = 0; r < 16; r++) s0[r] = s1[r] = 0.f;
+    for (int r = 0; r < 16; r++) s0[r] = s1[r] = negm[r] = 0.f;
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     lds_barrier();
 #pragma unroll
     for (int s = 0; s < HD / 16; s++)
         R.qop[s] = *reinterpret_cast<const half8*>(&qs[sub][n][s * 16 + g * 8]);
     if (R.wave_ok && cx.t0 >= R.wt_first && cx.t0 <= R.wt_last)
-        split_scores<HD>(R, s0, smem, cx, cx.ring);
+        split_scores<HD>(R, negm, s0, smem, cx, cx.ring);
 
     // Before the barrier of step j every load of this wave but the ones step
     // j-1 issued has landed: K of tile j+1 and Vt of tile j, which step j
@@ -878,12 +915,12 @@ __device__ __forceinline__ void split_block(const PrefillArgs& a, unsigned char*
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * L::NL) : "memory");
         split_patch_tail<HD>(smem, cx, j, sub, lane);
         set_barrier(smem, cx.cnt, 4 * (j + 1), lane);
-        split_wave_step<HD>(R, s0, s1, smem, cx, j, wave, g);
+        split_wave_step<HD>(R, negm, s0, s1, smem, cx, j, wave, g);
         if (j + 1 >= nsteps) break;
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * L::NL) : "memory");
         split_patch_tail<HD>(smem, cx, j + 1, sub, lane);
         set_barrier(smem, cx.cnt, 4 * (j + 2), lane);
-        split_wave_step<HD>(R, s1, s0, smem, cx, j + 1, wave, g);
+        split_wave_step<HD>(R, negm, s1, s0, smem, cx, j + 1, wave, g);
         if (j + 2 >= nsteps) break;
     }
 
