@@ -179,12 +179,15 @@ def main() -> None:
         qp_dev.free()
         op_dev.free()
 
-    # ---- CPU baseline: the oracle on the same data, one core, bounded sample
+    # ---- CPU baseline: the oracle on the same data, bounded sample.  The
+    # reference runs one attention call on one core, so one core is the faithful
+    # figure; sessions are independent, so one thread per session is the best a
+    # caller of the reference could do, and is reported beside it.
     cpu = None
     if args.cpu_seconds > 0:
         done_bytes, t_cpu, n_calls = 0, 0.0, 0
         s = 0
-        while t_cpu < args.cpu_seconds:
+        while t_cpu < args.cpu_seconds * 0.6:
             k16, v16 = host_kv[s % S]
             tc = time.perf_counter()
             oracle.attention(q_host[0, s % S][None], k16, v16)
@@ -192,9 +195,37 @@ def main() -> None:
             done_bytes += 2 * 2 * nkv * hd * ctx
             n_calls += 1
             s += 1
+        per_call = t_cpu / n_calls
+        # session-parallel: the foreign calls release the interpreter lock
+        from concurrent.futures import ThreadPoolExecutor
+        n_thr = min(S, os.cpu_count() or 1)
+        rounds = max(1, int(args.cpu_seconds * 0.4 / per_call))
+
+        def worker(i):
+            k16, v16 = host_kv[i % S]
+            for _ in range(rounds):
+                oracle.attention(q_host[0, i % S][None], k16, v16)
+
+        tp = time.perf_counter()
+        with ThreadPoolExecutor(n_thr) as ex:
+            list(ex.map(worker, range(n_thr)))
+        t_par = time.perf_counter() - tp
+        par_gbs = n_thr * rounds * 2 * 2 * nkv * hd * ctx / t_par / 1e9
+        cpu_model = ""
+        try:
+            with open("/proc/cpuinfo") as f:
+                for ln in f:
+                    if ln.startswith("model name"):
+                        cpu_model = ln.split(":", 1)[1].strip()
+                        break
+        except OSError:
+            pass
         cpu = {"value": round(done_bytes / t_cpu / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
                "sample": "%d single-session calls of the same workload (32/8/128, ctx %d), "
-                         "%.1f s of CPU time, host has %d cpus" % (n_calls, ctx, t_cpu, os.cpu_count())}
+                         "%.1f s of CPU time" % (n_calls, ctx, t_cpu),
+               "session_parallel": {"value": round(par_gbs, 4), "unit": "GB/s", "cores": n_thr,
+                                    "sample": "%d threads x %d calls, %.1f s" % (n_thr, rounds, t_par)},
+               "host": "%s, %d cpus visible" % (cpu_model, os.cpu_count() or 0)}
 
     line = {
         "metric": "decode-attn HBM GB/s (% peak) at 16 sess x 4K ctx; prefill attn TFLOP/s",

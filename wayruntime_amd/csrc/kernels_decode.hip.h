@@ -324,9 +324,7 @@ void decode_mfma_kernel(const DecodeArgs a)
     // then overlaps the staging of Q.
     DecodeFrag<HD> fa, fb;
     uint32_t t = tr.t_begin + wave;
-#ifndef WR_EXP_NOHOIST
     if (t < tr.t_end) load_frag<HD>(fa, kbase, vtbase, t, lane);
-#endif
 
     // Q^T operand through LDS: row c of lds_q is MFMA column c.  Columns
     // 0..G-1 hold the hi terms of the group's heads, G..2G-1 the lo terms,
@@ -361,9 +359,6 @@ void decode_mfma_kernel(const DecodeArgs a)
     st.l = 0.f;
 
     if (t < tr.t_end) {
-#ifdef WR_EXP_NOHOIST
-        load_frag<HD>(fa, kbase, vtbase, t, lane);
-#endif
         for (;;) {
             const uint32_t t1 = t + kDecodeWaves;
             if (t1 < tr.t_end) load_frag<HD>(fb, kbase, vtbase, t1, lane);

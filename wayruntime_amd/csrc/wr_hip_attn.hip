@@ -352,21 +352,13 @@ int prefill_locked(wr_hip_kv* kv, uint32_t layer, uint32_t p0, uint32_t T, const
         const uint32_t BP = 32 * (4 / Gw);
         const uint32_t nblk = (T + BP - 1) / BP;
         const uint32_t npairs = (nblk + 1) / 2, ny = kv->nkv * (G / Gw);
-#ifndef WR_PREFILL_ONE_WAVE_PER_SIMD
         if (hd == 64)
             launch_main(prefill_split_kernel<64>, dim3(ny, npairs), dim3(kSplitThreads), a,
                         split_smem_bytes<64>());
         else if (hd == 128)
             launch_main(prefill_split_kernel<128>, dim3(ny, npairs), dim3(kSplitThreads), a,
                         split_smem_bytes<128>());
-        else
-#else
-        if (hd == 64)
-            launch_main(prefill_mfma_kernel<64>, dim3(npairs, ny), dim3(kPrefillThreads), a);
-        else if (hd == 128)
-            launch_main(prefill_mfma_kernel<128>, dim3(npairs, ny), dim3(kPrefillThreads), a);
-        else
-#endif
+        else   // 256: one wave per SIMD (the accumulators alone need 256 registers)
             launch_main(prefill_mfma_kernel<256>, dim3(npairs, ny), dim3(kPrefillThreads), a);
     } else {
         launch_main(prefill_generic_kernel, dim3(T, nq), dim3(kDecodeThreads), a);
