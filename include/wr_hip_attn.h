@@ -98,6 +98,18 @@ int wr_hip_attn_append(wr_hip_kv *kv, uint32_t layer, uint32_t pos,
                        uint32_t n_rows, const float *k_f32,
                        const float *v_f32);
 
+/* Append with the rotary embedding of the K rows done on the device (the step
+ * the reference performs on the host right before kv_append_row:
+ * wri_op_rope, src/core/kernels.c:1356-1412, called at session.c:477-478).
+ * k_f32 holds the rows BEFORE rotation; cos_sin is host F32
+ * [n_rows, n_rot, 2] = (cos, sin) of each row's angles, n_rot <= hd/2 pairs
+ * rotated (element j with element j + hd/2).  The rotated rows are bit
+ * identical to the reference's, so the cache is too.  v_f32 as in append. */
+int wr_hip_attn_append_rope(wr_hip_kv *kv, uint32_t layer, uint32_t pos,
+                            uint32_t n_rows, const float *k_f32,
+                            const float *v_f32, const float *cos_sin,
+                            uint32_t n_rot);
+
 /* Test / tooling access to the cache in the reference's layout: F16 bit
  * patterns, position-major [n_rows, nkv, hd_layer] (the layout of the
  * reference's kv_k / kv_v tensors, src/core/internal.h:492-497).
@@ -155,6 +167,13 @@ void *wr_hip_attn_stream(void);          /* hipStream_t of the library */
 int wr_hip_attn_append_dev(wr_hip_kv *kv, uint32_t layer, uint32_t pos,
                            uint32_t n_rows, const float *k_f32_dev,
                            const float *v_f32_dev);
+
+/* The same rotation alone, in place on device F32 rows [rows, heads, hd]
+ * (wri_op_rope, src/core/kernels.c:1356-1412, for callers that keep Q or K on
+ * the device); cos_sin_dev is device F32 [rows, n_rot, 2].  Asynchronous on
+ * the library's stream like the other *_dev calls. */
+int wr_hip_attn_rope_dev(void *x_dev, const void *cos_sin_dev, uint32_t rows,
+                         uint32_t heads, uint32_t hd, uint32_t n_rot);
 int wr_hip_attn_decode_batched_dev(uint32_t n, wr_hip_kv *const *kv,
                                    uint32_t layer, const uint32_t *seq_k,
                                    const float *q_dev, float *out_dev,

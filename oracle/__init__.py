@@ -98,6 +98,8 @@ def _load_oracle() -> C.CDLL:
     lib.wro_causal_prefill_rows.argtypes = [_f32p, _u16p, _u16p, _f32p] + [C.c_uint32] * 6 + [
         C.c_float, C.c_uint32]
     lib.wro_rope.argtypes = [_f32p] + [C.c_uint32] * 4 + [C.c_float, C.c_uint32]
+    lib.wro_rope_table.argtypes = [_f32p] + [C.c_uint32] * 3 + [C.c_float, C.c_uint32]
+    lib.wro_rope_table.restype = C.c_int
     return lib
 
 
@@ -194,6 +196,15 @@ def rope(x: np.ndarray, pos: int, theta: float, n_rot_pairs: int = 0) -> np.ndar
     if rc != 0:
         raise ValueError(rc)
     return y
+
+
+def rope_table(seq: int, hd: int, pos: int, theta: float, n_rot_pairs: int = 0) -> np.ndarray:
+    """(cos, sin) of the angles wro_rope uses: float32 [seq, n_rot, 2]."""
+    buf = np.zeros((seq, hd // 2, 2), dtype=np.float32)
+    n_rot = lib().wro_rope_table(buf, seq, hd, pos, theta, n_rot_pairs)
+    if n_rot < 0:
+        raise ValueError(n_rot)
+    return np.ascontiguousarray(buf.reshape(-1)[: seq * n_rot * 2].reshape(seq, n_rot, 2))
 
 
 # --------------------------------------------------------------- reference --

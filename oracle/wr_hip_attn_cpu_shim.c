@@ -101,6 +101,35 @@ int wr_hip_attn_append(wr_hip_kv *kv, uint32_t layer, uint32_t pos, uint32_t n_r
     return WR_HIP_OK;
 }
 
+int wr_hip_attn_append_rope(wr_hip_kv *kv, uint32_t layer, uint32_t pos, uint32_t n_rows,
+                            const float *k, const float *v, const float *cos_sin, uint32_t n_rot)
+{
+    if (!g_inited) return WR_HIP_ERR_STATE;
+    if (!layer_ok(kv, layer)) return WR_HIP_ERR_INVAL;
+    if (n_rows == 0) return WR_HIP_OK;
+    if (!k || !v || (!cos_sin && n_rot > 0)) return WR_HIP_ERR_INVAL;
+    if ((uint64_t)pos + n_rows > kv->max_ctx) return WR_HIP_ERR_CTX_FULL;
+    const uint32_t hd = kv->hd[layer], half = hd / 2;
+    if (n_rot > half) return WR_HIP_ERR_INVAL;
+    const size_t row = (size_t)kv->nkv * hd;
+    for (uint32_t r = 0; r < n_rows; r++)
+        for (uint32_t h = 0; h < kv->nkv; h++) {
+            const float *x = k + (size_t)r * row + (size_t)h * hd;
+            uint16_t *dst = kv->k[layer] + ((size_t)pos + r) * row + (size_t)h * hd;
+            for (uint32_t j = 0; j < hd; j++) dst[j] = wro_f32_to_f16(x[j]);
+            for (uint32_t j = 0; j < n_rot; j++) {
+                const float c = cos_sin[((size_t)r * n_rot + j) * 2];
+                const float sn = cos_sin[((size_t)r * n_rot + j) * 2 + 1];
+                const float x0 = x[j], x1 = x[j + half];
+                dst[j] = wro_f32_to_f16(x0 * c - x1 * sn);
+                dst[j + half] = wro_f32_to_f16(x0 * sn + x1 * c);
+            }
+        }
+    for (size_t i = 0; i < (size_t)n_rows * row; i++)
+        kv->v[layer][(size_t)pos * row + i] = wro_f32_to_f16(v[i]);
+    return WR_HIP_OK;
+}
+
 int wr_hip_attn_kv_read(wr_hip_kv *kv, uint32_t layer, uint32_t pos, uint32_t n_rows,
                         uint16_t *k, uint16_t *v)
 {

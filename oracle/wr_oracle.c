@@ -435,6 +435,33 @@ void wro_batched_decode(uint32_t n, const float *const *q,
 
 /* ------------------------------------------------------------------ RoPE -- */
 
+/* The (cos, sin) pairs wro_rope uses for `seq` rows starting at `pos`
+ * (kernels.c:1384-1404, the angle arithmetic lifted out of the rotation):
+ * out[s][j] = {cos, sin} for j < n_rot, n_rot as resolved by wro_rope.  Returns
+ * n_rot, or a negative status. */
+int wro_rope_table(float *out, uint32_t seq, uint32_t hd, uint32_t pos,
+                   float theta_base, uint32_t n_rot_pairs)
+{
+    if (!out || seq == 0) return WRO_ERR_INVAL;
+    if (hd < 2 || (hd & 1)) return WRO_ERR_INVAL;
+    const uint64_t half = hd / 2;
+    if (theta_base < 1.0f) theta_base = 10000.0f;
+    const float lnb = wro_log(theta_base);
+    uint64_t n_rot = half;
+    if (n_rot_pairs >= 1 && (uint64_t)n_rot_pairs < half) n_rot = n_rot_pairs;
+    for (uint64_t s = 0; s < seq; s++) {
+        const uint64_t p = (uint64_t)pos + s;
+        for (uint64_t j = 0; j < n_rot; j++) {
+            const float exponent = (float)(2 * j) / (float)hd;
+            const float powv = wro_exp(exponent * lnb);
+            const float angle = (float)p / powv;
+            out[(s * n_rot + j) * 2] = wro_cos(angle);
+            out[(s * n_rot + j) * 2 + 1] = wro_sin(angle);
+        }
+    }
+    return (int)n_rot;
+}
+
 /* kernels.c:1356-1412 */
 int wro_rope(float *x, uint32_t seq, uint32_t heads, uint32_t hd,
              uint32_t pos, float theta_base, uint32_t n_rot_pairs)

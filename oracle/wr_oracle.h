@@ -136,6 +136,8 @@ void wro_batched_decode(uint32_t n, const float *const *q,
  * x is [seq, heads, hd] F32, rotated in place; first row is at `pos`.
  * pinned by: bit-compare against the compiled reference; ops_test_rope
  * known answers (kernels.c:2160-2183). */
+int wro_rope_table(float *out, uint32_t seq, uint32_t hd, uint32_t pos,
+                   float theta_base, uint32_t n_rot_pairs);
 int wro_rope(float *x, uint32_t seq, uint32_t heads, uint32_t hd,
              uint32_t pos, float theta_base, uint32_t n_rot_pairs);
 

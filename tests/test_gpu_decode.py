@@ -73,6 +73,55 @@ def test_append_matches_oracle_append_row():
     kv.close()
 
 
+
+@pytest.mark.parametrize("nkv,hd,theta,n_rot_pairs,pos0,chunks", [
+    (8, 128, 1e6, 0, 0, [1, 1, 31, 40, 1]),          # Qwen3-like, block boundaries
+    (8, 128, 5e5, 0, 32760, [1, 7]),                 # long positions: thousands of range-reduction steps
+    (4, 256, 1e6, 0, 5, [33]),
+    (2, 64, 1e4, 10, 0, [3, 30]),                    # partial rotary: only 10 of 32 pairs rotate
+])
+def test_append_rope_cache_bits_equal_rotate_then_truncate(nkv, hd, theta, n_rot_pairs, pos0, chunks):
+    """K rotated on the device inside the append must leave the same cache bits
+    as the reference order of operations: wri_op_rope on the host, then the
+    truncating append.  V is untouched by the rotation."""
+    total = sum(chunks)
+    kv = hipattn.KVCache(1, hd, nkv, pos0 + total)
+    k32 = synth.normal(300 + hd, (total, nkv, hd), std=2.0)
+    v32 = synth.normal(301 + hd, (total, nkv, hd), std=2.0)
+    at = 0
+    for n in chunks:
+        print("append_rope", nkv, hd, "pos", pos0 + at, "n", n, flush=True)
+        tab = oracle.rope_table(n, hd, pos0 + at, theta, n_rot_pairs)
+        assert kv.append_rope(0, pos0 + at, k32[at:at + n], v32[at:at + n], tab) == hipattn.OK
+        at += n
+    want_k = synth.f32_to_f16_trunc(oracle.rope(k32, pos0, theta, n_rot_pairs))
+    want_v = synth.f32_to_f16_trunc(v32)
+    got_k, got_v = kv.read_f16(0, pos0, total)
+    assert got_k.tobytes() == want_k.tobytes()
+    assert got_v.tobytes() == want_v.tobytes()
+    kv.close()
+
+
+def test_rope_dev_equals_reference_rotation_and_error_contract():
+    rows, heads, hd = 5, 16, 128
+    x = synth.normal(310, (rows, heads, hd))
+    tab = oracle.rope_table(rows, hd, 1000, 1e6)
+    xd = hipattn.DeviceBuffer.from_host(x)
+    td = hipattn.DeviceBuffer.from_host(tab)
+    hipattn.rope_dev(xd, td, rows, heads, hd, tab.shape[1])
+    hipattn.sync()
+    got = xd.to_host((rows, heads, hd))
+    assert got.tobytes() == oracle.rope(x, 1000, 1e6).tobytes()
+    lib = hipattn.lib()
+    assert lib.wr_hip_attn_rope_dev(None, td.p, rows, heads, hd, 64) == hipattn.ERR_INVAL
+    assert lib.wr_hip_attn_rope_dev(xd.p, td.p, rows, heads, hd, 65) == hipattn.ERR_INVAL
+    assert lib.wr_hip_attn_rope_dev(xd.p, td.p, rows, heads, 127, 10) == hipattn.ERR_INVAL
+    kv = hipattn.KVCache(1, hd, 2, 4)
+    k = synth.normal(311, (2, 2, hd))
+    assert kv.append_rope(0, 3, k, k, tab[:2]) == hipattn.ERR_CTX_FULL      # writes nothing
+    assert lib.wr_hip_attn_append_rope(kv.h, 0, 0, 1, k.ctypes.data, k.ctypes.data, None, 4) == hipattn.ERR_INVAL
+    kv.close(); xd.free(); td.free()
+
 # ------------------------------------------------------------------ decode --
 
 def _run_decode(nq, nkv, hd, ctx, sc=0.0, win=0, seed=1, rows=None, generic=False, keys_per_wg=0):

@@ -395,3 +395,29 @@ def test_oracle_equals_compiled_reference_on_normal_inputs(nq, nkv, hd, ctx, sc,
     assert rc == 0
     got = oracle.attention(q, k, v, scale_override=sc, window=win)
     assert got.tobytes() == want.tobytes()
+
+
+@pytest.mark.parametrize("hd,pos,theta,n_rot_pairs", [
+    (128, 0, 1e6, 0), (128, 4095, 5e5, 0), (64, 77, 1e4, 0), (256, 32775, 1e6, 0), (128, 300, 1e6, 20),
+    (20, 9, 0.5, 0),                                    # theta < 1 falls back to 10000
+])
+def test_rope_table_is_the_rotation_s_own_angles(hd, pos, theta, n_rot_pairs):
+    """The (cos, sin) table handed to the device append must be exactly what
+    wro_rope uses: rotating by hand with the table (separately rounded float32
+    products) reproduces wro_rope bit for bit, rows at consecutive positions."""
+    seq, heads = 3, 2
+    x = synth.normal(900 + hd, (seq, heads, hd))
+    want = oracle.rope(x, pos, theta, n_rot_pairs)
+    tab = oracle.rope_table(seq, hd, pos, theta, n_rot_pairs)
+    half = hd // 2
+    n_rot = tab.shape[1]
+    assert n_rot == (n_rot_pairs if 1 <= n_rot_pairs < half else half)
+    got = x.copy()
+    c = tab[:, None, :, 0]
+    s_ = tab[:, None, :, 1]
+    x0 = x[:, :, :n_rot]
+    x1 = x[:, :, half:half + n_rot]
+    got[:, :, :n_rot] = (x0 * c).astype(np.float32) - (x1 * s_).astype(np.float32)
+    got[:, :, half:half + n_rot] = (x0 * s_).astype(np.float32) + (x1 * c).astype(np.float32)
+    assert got.tobytes() == want.tobytes()
+

@@ -75,6 +75,40 @@ __global__ __launch_bounds__(256) void append_v_kernel(const Src* __restrict__ s
     }
 }
 
+// Rotary position embedding in place on F32 rows [rows][heads][hd], split-half
+// pairing (element j with element j + hd/2, j < n_rot), as the reference
+// applies it before the append (reference: src/core/kernels.c:1356-1412):
+//   r[j] = x0*c - x1*s,  r[j + hd/2] = x0*s + x1*c
+// with c = cs[row][j][0], s = cs[row][j][1].  The angles come from the caller:
+// the reference reduces them with a loop of single subtractions of 2*pi whose
+// rounding only the same loop reproduces, thousands of dependent steps at long
+// positions, which one CPU core runs faster than one GPU lane.  The products
+// and the sum are rounded separately (no fused multiply-add), so the rotated
+// values, and with them the cache bits, equal the reference's bit for bit.
+__global__ __launch_bounds__(256) void rope_rows_kernel(float* __restrict__ x,
+                                                        const float* __restrict__ cs,
+                                                        uint32_t rows, uint32_t heads,
+                                                        uint32_t hd, uint32_t n_rot)
+{
+// The products and their sum must round one by one.  The pragma covers the
+// operators written in this function; the __fmul_rn / __fadd_rn intrinsics do
+// not help, they are plain operators defined under the default contraction.
+#pragma clang fp contract(off)
+    const size_t total = (size_t)rows * heads * n_rot;
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const uint32_t j = (uint32_t)(idx % n_rot);
+    const uint32_t h = (uint32_t)((idx / n_rot) % heads);
+    const uint32_t r = (uint32_t)(idx / ((size_t)n_rot * heads));
+    const uint32_t half = hd / 2;
+    float* row = x + ((size_t)r * heads + h) * hd;
+    const float c = cs[((size_t)r * n_rot + j) * 2], sn = cs[((size_t)r * n_rot + j) * 2 + 1];
+    const float x0 = row[j], x1 = row[j + half];
+    const float a0 = x0 * c, b0 = x1 * sn, a1 = x0 * sn, b1 = x1 * c;
+    row[j] = a0 - b0;
+    row[j + half] = a1 + b1;
+}
+
 // Export rows back in position-major order [n_rows][nkv][hd] (tests, tooling).
 __global__ __launch_bounds__(256) void export_kv_kernel(const uint16_t* __restrict__ k,
                                                         const uint16_t* __restrict__ vt,

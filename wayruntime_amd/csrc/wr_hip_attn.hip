@@ -572,6 +572,55 @@ int wr_hip_attn_append_dev(wr_hip_kv* kv, uint32_t layer, uint32_t pos, uint32_t
     return append_rows_locked<float>(kv, layer, pos, n_rows, k_f32_dev, v_f32_dev);
 }
 
+int wr_hip_attn_rope_dev(void* x_dev, const void* cos_sin_dev, uint32_t rows, uint32_t heads,
+                         uint32_t hd, uint32_t n_rot)
+{
+    if (!g.inited) return WR_HIP_ERR_STATE;
+    if (!x_dev || !cos_sin_dev) return WR_HIP_ERR_INVAL;
+    if (hd < 2 || (hd & 1) || heads == 0 || n_rot > hd / 2) return WR_HIP_ERR_INVAL;
+    if (rows == 0 || n_rot == 0) return WR_HIP_OK;
+    Locked lk;
+    const size_t total = (size_t)rows * heads * n_rot;
+    hipLaunchKernelGGL(rope_rows_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
+                       g.stream, reinterpret_cast<float*>(x_dev),
+                       reinterpret_cast<const float*>(cos_sin_dev), rows, heads, hd, n_rot);
+    HIP_TRY(hipGetLastError(), "rope launch", 0);
+    return WR_HIP_OK;
+}
+
+int wr_hip_attn_append_rope(wr_hip_kv* kv, uint32_t layer, uint32_t pos, uint32_t n_rows,
+                            const float* k_f32, const float* v_f32, const float* cos_sin,
+                            uint32_t n_rot)
+{
+    int rc = check_append(kv, layer, pos, n_rows, k_f32, v_f32);
+    if (rc) return rc;
+    if (!cos_sin && n_rot > 0) return WR_HIP_ERR_INVAL;
+    if (n_rot > kv->hd[layer] / 2) return WR_HIP_ERR_INVAL;
+    if (n_rows == 0) return WR_HIP_OK;
+    const uint32_t hd = kv->hd[layer], nkv = kv->nkv;
+    const size_t bytes = (size_t)n_rows * nkv * hd * sizeof(float);
+    const size_t tbytes = (size_t)n_rows * n_rot * 2 * sizeof(float);
+    Locked lk;
+    rc = ensure_device(g.d_stage, 2 * bytes + tbytes);
+    if (rc) return rc;
+    float* dk = reinterpret_cast<float*>(g.d_stage.p);
+    float* dv = reinterpret_cast<float*>((uint8_t*)g.d_stage.p + bytes);
+    float* dt = reinterpret_cast<float*>((uint8_t*)g.d_stage.p + 2 * bytes);
+    rc = copy_up(dk, k_f32, bytes, 0);
+    if (rc == WR_HIP_OK) rc = copy_up(dv, v_f32, bytes, bytes);
+    if (rc == WR_HIP_OK) rc = copy_up(dt, cos_sin, tbytes, 2 * bytes);
+    if (rc == WR_HIP_OK && n_rot > 0) {
+        const size_t total = (size_t)n_rows * nkv * n_rot;
+        hipLaunchKernelGGL(rope_rows_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
+                           g.stream, dk, dt, n_rows, nkv, hd, n_rot);
+        HIP_TRY(hipGetLastError(), "rope launch", layer);
+    }
+    if (rc == WR_HIP_OK) rc = append_rows_locked<float>(kv, layer, pos, n_rows, dk, dv);
+    // the staging buffers are reused by the next call: wait for the kernels
+    if (rc == WR_HIP_OK) HIP_TRY(hipStreamSynchronize(g.stream), "append sync", layer);
+    return rc;
+}
+
 int wr_hip_attn_append(wr_hip_kv* kv, uint32_t layer, uint32_t pos, uint32_t n_rows,
                        const float* k_f32, const float* v_f32)
 {

@@ -58,6 +58,8 @@ def load() -> C.CDLL:
         "wr_hip_attn_sync": (C.c_int, []),
         "wr_hip_attn_stream": (_vp, []),
         "wr_hip_attn_append_dev": (C.c_int, [_vp, _u32, _u32, _u32, _vp, _vp]),
+        "wr_hip_attn_append_rope": (C.c_int, [_vp, _u32, _u32, _u32, _vp, _vp, _vp, _u32]),
+        "wr_hip_attn_rope_dev": (C.c_int, [_vp, _vp, _u32, _u32, _u32, _u32]),
         "wr_hip_attn_decode_batched_dev": (C.c_int, [_u32, C.POINTER(_vp), _u32, C.POINTER(_u32),
                                                      _vp, _vp, _u32, C.c_float, _u32]),
         "wr_hip_attn_prefill_dev": (C.c_int, [_vp, _u32, _u32, _u32, _vp, _vp, _u32, C.c_float,
@@ -147,6 +149,17 @@ class KVCache:
         v = np.ascontiguousarray(v, dtype=np.float32)
         assert k.shape == v.shape
         return lib().wr_hip_attn_append(self.h, layer, pos, k.shape[0], _ptr(k), _ptr(v))
+
+    def append_rope(self, layer: int, pos: int, k: np.ndarray, v: np.ndarray,
+                    cos_sin: np.ndarray) -> int:
+        """k (before rotation), v float32 [n_rows, nkv, hd]; cos_sin float32
+        [n_rows, n_rot, 2]; returns the wr_status."""
+        k = np.ascontiguousarray(k, dtype=np.float32)
+        v = np.ascontiguousarray(v, dtype=np.float32)
+        cs = np.ascontiguousarray(cos_sin, dtype=np.float32)
+        assert k.shape == v.shape and cs.shape[0] == k.shape[0] and cs.shape[2] == 2
+        return lib().wr_hip_attn_append_rope(self.h, layer, pos, k.shape[0], _ptr(k), _ptr(v),
+                                             _ptr(cs), cs.shape[1])
 
     def write_f16(self, layer: int, pos: int, k16: np.ndarray, v16: np.ndarray,
                   chunk_rows: int = 8192) -> None:
@@ -252,6 +265,11 @@ def append_dev(cache: KVCache, layer: int, pos: int, n_rows: int, k_dev: DeviceB
                v_dev: DeviceBuffer) -> None:
     _check(lib().wr_hip_attn_append_dev(cache.h, layer, pos, n_rows, k_dev.p, v_dev.p),
            "append_dev")
+
+
+def rope_dev(x_dev: DeviceBuffer, cos_sin_dev: DeviceBuffer, rows: int, heads: int, hd: int,
+             n_rot: int) -> None:
+    _check(lib().wr_hip_attn_rope_dev(x_dev.p, cos_sin_dev.p, rows, heads, hd, n_rot), "rope_dev")
 
 
 def sync() -> None:

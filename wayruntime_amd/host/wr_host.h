@@ -79,6 +79,7 @@ typedef struct wrh_workspace {
     float *k, *v;                        /* [R][n_kv*hd] */
     float *gate, *up;                    /* [R][ffn]     */
     float *proj;                         /* [R][hidden]  */
+    float *rope;                         /* [R][hd/2][2] (cos, sin) of the rows' angles */
     void  *block;
 } wrh_workspace;
 
@@ -105,6 +106,9 @@ void wrh_matmul(wr_engine *e, const float *A, uint32_t R, uint32_t lda, const wr
                 float *C, uint32_t ldc);
 void wrh_rope(float *x, uint32_t heads, uint32_t hd, uint32_t pos, float theta,
               uint32_t n_rot_pairs);
+uint32_t wrh_rope_table(float *cos_sin, uint32_t hd, uint32_t pos, float theta,
+                        uint32_t n_rot_pairs);
+void wrh_rope_apply(float *x, uint32_t heads, uint32_t hd, const float *cos_sin, uint32_t n_rot);
 void wrh_swiglu(wr_engine *e, float *gate, const float *up, uint64_t n);
 void wrh_add(float *acc, const float *x, uint64_t n);
 

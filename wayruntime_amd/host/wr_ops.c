@@ -180,6 +180,40 @@ void wrh_rope(float *x, uint32_t heads, uint32_t hd, uint32_t pos, float theta,
     }
 }
 
+/* The (cos, sin) pairs wrh_rope uses at position pos: cos_sin[j] = {cos, sin}
+ * for j < n_rot (returned; n_rot <= hd/2). */
+uint32_t wrh_rope_table(float *cos_sin, uint32_t hd, uint32_t pos, float theta,
+                        uint32_t n_rot_pairs)
+{
+    const uint32_t half = hd / 2;
+    if (theta < 1.0f) theta = 10000.0f;
+    const float lnb = wrh_log(theta);
+    uint32_t n_rot = half;
+    if (n_rot_pairs >= 1 && n_rot_pairs < half) n_rot = n_rot_pairs;
+    for (uint32_t j = 0; j < n_rot; j++) {
+        const float exponent = (float)(2 * j) / (float)hd;
+        const float powv = wrh_exp(exponent * lnb);
+        const float angle = (float)pos / powv;
+        cos_sin[2 * j] = wrh_cos(angle);
+        cos_sin[2 * j + 1] = wrh_sin(angle);
+    }
+    return n_rot;
+}
+
+void wrh_rope_apply(float *x, uint32_t heads, uint32_t hd, const float *cos_sin, uint32_t n_rot)
+{
+    const uint32_t half = hd / 2;
+    for (uint32_t j = 0; j < n_rot; j++) {
+        const float cs = cos_sin[2 * j], sn = cos_sin[2 * j + 1];
+        for (uint32_t h = 0; h < heads; h++) {
+            float *r = x + (size_t)h * hd;
+            const float x0 = r[j], x1 = r[j + half];
+            r[j] = x0 * cs - x1 * sn;
+            r[j + half] = x0 * sn + x1 * cs;
+        }
+    }
+}
+
 void wrh_swiglu(wr_engine *e, float *gate, const float *up, uint64_t n)
 {
     if (e) __atomic_fetch_add(&e->ctr[WR_CTR_FUSED_CALLS], 1, __ATOMIC_RELAXED);

@@ -45,7 +45,8 @@ int wrh_workspace_init(wrh_workspace *ws, const wr_model *m, uint32_t rows)
     const size_t qd = round64((size_t)rows * m->n_q * m->head_dim);
     const size_t kd = round64((size_t)rows * m->n_kv * m->head_dim);
     const size_t fd = round64((size_t)rows * m->ffn);
-    const size_t total = 3 * h + 2 * qd + 2 * kd + 2 * fd;
+    const size_t rd = round64((size_t)rows * m->head_dim);
+    const size_t total = 3 * h + 2 * qd + 2 * kd + 2 * fd + rd;
     float *b = NULL;
     if (posix_memalign((void **)&b, 64, total * sizeof(float)) != 0 || !b) return WR_ERR_NOMEM;
     ws->block = b;
@@ -58,7 +59,8 @@ int wrh_workspace_init(wrh_workspace *ws, const wr_model *m, uint32_t rows)
     ws->k = b;         b += kd;
     ws->v = b;         b += kd;
     ws->gate = b;      b += fd;
-    ws->up = b;
+    ws->up = b;        b += fd;
+    ws->rope = b;
     return WR_OK;
 }
 
@@ -108,10 +110,16 @@ static wr_status forward_rows(wr_model *m, wrh_workspace *ws, uint32_t R, wr_ses
             wrh_rmsnorm(ws->q, m->q_norm[L].data, m->q_norm[L].n, ws->q, R * nq, hd, m->rms_eps);
             wrh_rmsnorm(ws->k, m->k_norm[L].data, m->k_norm[L].n, ws->k, R * nkv, hd, m->rms_eps);
         }
+        /* RoPE (reference: session.c:475-478): the rows' angles are worked out
+         * once here; Q is rotated on the host, K on the device inside the
+         * append (same arithmetic, same bits), so K goes up as projected. */
+        const uint32_t n_rot =
+            (m->n_rot_pairs >= 1 && m->n_rot_pairs < hd / 2) ? m->n_rot_pairs : hd / 2;
+        const size_t ts = (size_t)2 * n_rot;              /* table row: n_rot (cos, sin) pairs */
         for (uint32_t r = 0; r < R; r++) {
             const uint32_t p = (mode == FWD_BATCH) ? ss[r]->pos : pos0 + r;
-            wrh_rope(ws->q + (size_t)r * qd, nq, hd, p, m->rope_base, m->n_rot_pairs);
-            wrh_rope(ws->k + (size_t)r * kd, nkv, hd, p, m->rope_base, m->n_rot_pairs);
+            (void)wrh_rope_table(ws->rope + r * ts, hd, p, m->rope_base, m->n_rot_pairs);
+            wrh_rope_apply(ws->q + (size_t)r * qd, nq, hd, ws->rope + r * ts, n_rot);
         }
 
         /* Append after RoPE, then attend: the new token attends to itself. */
@@ -125,8 +133,8 @@ static wr_status forward_rows(wr_model *m, wrh_workspace *ws, uint32_t R, wr_ses
             const float *qp[WR_BATCH_MAX];
             float *op[WR_BATCH_MAX];
             for (uint32_t r = 0; r < R; r++) {
-                rc = wr_hip_attn_append(ss[r]->kv, L, ss[r]->pos, 1, ws->k + (size_t)r * kd,
-                                        ws->v + (size_t)r * kd);
+                rc = wr_hip_attn_append_rope(ss[r]->kv, L, ss[r]->pos, 1, ws->k + (size_t)r * kd,
+                                             ws->v + (size_t)r * kd, ws->rope + r * ts, n_rot);
                 if (rc != WR_HIP_OK) return (rc == WR_HIP_ERR_CTX_FULL) ? WR_ERR_CTX_FULL
                                                                          : op_fail(e, "kv append", L, rc);
                 ss[r]->kv_rows[L] = ss[r]->pos + 1;
@@ -138,7 +146,7 @@ static wr_status forward_rows(wr_model *m, wrh_workspace *ws, uint32_t R, wr_ses
             rc = wr_hip_attn_decode_batched(R, kvs, L, seq_k, qp, op, nq, 0.0f, 0);
         } else {
             wr_session *s = ss[0];
-            rc = wr_hip_attn_append(s->kv, L, pos0, R, ws->k, ws->v);
+            rc = wr_hip_attn_append_rope(s->kv, L, pos0, R, ws->k, ws->v, ws->rope, n_rot);
             if (rc != WR_HIP_OK) return (rc == WR_HIP_ERR_CTX_FULL) ? WR_ERR_CTX_FULL
                                                                      : op_fail(e, "kv append", L, rc);
             s->kv_rows[L] = pos0 + R;
