@@ -2,17 +2,31 @@
 //
 // Layout of one layer of one session (all F16 bit patterns):
 //
-//   K   [nkv][ctx_pad][hd]            head-major, one row per cached position
-//   Vt  [nkv][ctx_pad/32][hd][32]     head-major, transposed in blocks of 32
-//                                     positions: the 32 values of one
-//                                     dimension are contiguous (64 bytes)
+//   K   [nkv][ctx_pad/32][2][hdp/8][16][8]   head-major, in tiles of 32 positions
+//   Vt  [nkv][ctx_pad/32][hd][32]            head-major, transposed in blocks of
+//                                            32 positions: the 32 values of one
+//                                            dimension are contiguous (64 bytes)
 //
-// ctx_pad is max_ctx rounded up to 32.  Head-major K makes the stream one
-// (session, kv head) workgroup reads fully contiguous.  The blocked transpose
-// of V puts the contraction index of P.V (positions) innermost, which is what
-// an MFMA operand wants, so neither kernel has to transpose V on the fly.
-// The slab is zero-filled at creation; rows above the caller's cursor are
-// never trusted (kernels mask them), only required to be addressable.
+// ctx_pad is max_ctx rounded up to 32; hdp is head_dim rounded up to 8.
+//
+// A K tile is stored in the order the decode kernel's matrix instruction eats
+// it.  Position p of a tile belongs to half t = (p >> 2) & 1 and slot
+// m = (p >> 3) * 4 + (p & 3) of that half; inside a half, the 16-byte chunk
+// c = d / 8 of all 16 slots is contiguous: unit (t, c, m) sits at
+// ((t * hdp/8 + c) * 16 + m) * 16 bytes.  One MFMA operand load (row m of 16,
+// lane group g reads chunk 4s + g) is then 64 lanes x 16 bytes = one contiguous
+// KiB.  With position-major rows the same load touches sixteen rows for 64
+// bytes each, and a compute unit streams that pattern at a third of the rate
+// (33 against 80-90 GB/s measured for one workgroup), which is what a ragged
+// batch's longest workgroups and a single session's few workgroups run at.
+// The halves and slots are the permutation that leaves each lane group's
+// scores on eight consecutive positions, the order Vt is read in.
+//
+// The blocked transpose of V puts the contraction index of P.V (positions)
+// innermost, which is what an MFMA operand wants, so neither kernel has to
+// transpose V on the fly.  The slab is zero-filled at creation; rows above the
+// caller's cursor are never trusted (kernels mask them), only required to be
+// addressable.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -45,10 +59,26 @@ __device__ __forceinline__ uint16_t f32_to_f16_trunc(float f)
     return (uint16_t)r;
 }
 
-__device__ __forceinline__ size_t k_row_offset(uint32_t kvh, uint32_t ctx_pad, uint32_t pos,
-                                               uint32_t hd)
+constexpr int kKTile = 32;            // positions per K tile
+
+__host__ __device__ __forceinline__ uint32_t k_padded_hd(uint32_t hd) { return (hd + 7u) & ~7u; }
+
+// half and slot of a position inside its K tile, and back
+__device__ __forceinline__ uint32_t k_tile_half(uint32_t p) { return (p >> 2) & 1u; }
+__device__ __forceinline__ uint32_t k_tile_slot(uint32_t p) { return ((p >> 3) << 2) | (p & 3u); }
+__device__ __forceinline__ uint32_t k_tile_pos(uint32_t half, uint32_t slot)
 {
-    return ((size_t)kvh * ctx_pad + pos) * hd;
+    return ((slot >> 2) << 3) | (half << 2) | (slot & 3u);
+}
+
+// element offset of (kvh, pos, d) inside K
+__device__ __forceinline__ size_t k_offset(uint32_t kvh, uint32_t ctx_pad, uint32_t pos, uint32_t d,
+                                           uint32_t hd)
+{
+    const uint32_t hdp = k_padded_hd(hd);
+    const uint32_t p = pos % kKTile;
+    const uint32_t unit = (k_tile_half(p) * (hdp / 8) + d / 8) * 16 + k_tile_slot(p);
+    return ((size_t)kvh * ctx_pad + (pos - p)) * hdp + (size_t)unit * 8 + (d & 7u);
 }
 
 // element offset of (kvh, pos, d) inside Vt

@@ -19,7 +19,8 @@ __device__ __forceinline__ uint16_t to_cache_bits<float>(float v) { return f32_t
 template <>
 __device__ __forceinline__ uint16_t to_cache_bits<uint16_t>(uint16_t v) { return v; }
 
-// K side: one thread per element; reads and writes are both unit-stride in d.
+// K side: one thread per element; reads are unit-stride in d, writes go out in
+// 16-byte chunks (eight consecutive d of one position).
 template <typename Src>
 __global__ __launch_bounds__(256) void append_k_kernel(const Src* __restrict__ src,
                                                        uint16_t* __restrict__ k, uint32_t pos,
@@ -32,7 +33,7 @@ __global__ __launch_bounds__(256) void append_k_kernel(const Src* __restrict__ s
     const uint32_t d = (uint32_t)(idx % hd);
     const uint32_t kvh = (uint32_t)((idx / hd) % nkv);
     const uint32_t r = (uint32_t)(idx / ((size_t)hd * nkv));
-    k[k_row_offset(kvh, ctx_pad, pos + r, hd) + d] = to_cache_bits<Src>(src[idx]);
+    k[k_offset(kvh, ctx_pad, pos + r, d, hd)] = to_cache_bits<Src>(src[idx]);
 }
 
 // V side: a workgroup owns a 32-position x 64-dimension tile of one KV head.
@@ -123,7 +124,7 @@ __global__ __launch_bounds__(256) void export_kv_kernel(const uint16_t* __restri
     const uint32_t d = (uint32_t)(idx % hd);
     const uint32_t kvh = (uint32_t)((idx / hd) % nkv);
     const uint32_t r = (uint32_t)(idx / ((size_t)hd * nkv));
-    k_out[idx] = k[k_row_offset(kvh, ctx_pad, pos + r, hd) + d];
+    k_out[idx] = k[k_offset(kvh, ctx_pad, pos + r, d, hd)];
     v_out[idx] = vt[vt_offset(kvh, ctx_pad, pos + r, d, hd)];
 }
 

@@ -7,7 +7,8 @@
 // workgroups and merged by log-sum-exp), so results agree to rounding, not
 // bit for bit.
 //
-// Work decomposition: grid = (key splits, KV heads, sessions).  One workgroup
+// Work decomposition: grid = (KV heads, work-list entries), one entry per
+// (session, key split).  One workgroup
 // owns ONE KV head of one session over a contiguous run of 32-key tiles and
 // serves the whole GQA group from it, so every K and V byte is fetched from
 // HBM exactly once.  Its four waves take tiles round-robin and keep private
@@ -71,6 +72,13 @@ struct DecodeArgs {
     uint32_t nq, nkv, group, hd;
     uint32_t max_splits;
     float qscale;            // softmax scale * log2(e)
+    // Work list: one entry per (session, key split) that exists, longest first;
+    // entry = session << 8 | split.  The grid is (heads, entries) with the head
+    // index fastest, so that with 8 KV heads each XCD (workgroups go to XCDs
+    // round-robin by linear id) serves one KV head of every session and gets
+    // the same share of a ragged batch.
+    uint32_t n_items;
+    uint16_t items[kBatchMax * 64];
 };
 
 struct TileRange {
@@ -94,6 +102,8 @@ __device__ __forceinline__ TileRange split_tiles(const DecodeSession& S, uint32_
 // heads (log-sum-exp over the split maxima, one normalisation), writes the
 // final rows and puts the counter back to zero for the next launch.
 constexpr int kMaxSplits = 64;        // key splits per session (host picks tiles_per_wg to respect it)
+static_assert(kTileKeys == kKTile, "decode tiles are the cache's K tiles");
+static_assert(sizeof(DecodeArgs::items) == kBatchMax * kMaxSplits * sizeof(uint16_t), "work list size");
 
 // Partial rows cross workgroups (and XCDs, each with its own L2) inside one
 // launch.  They are written and read with agent-scope relaxed atomics: on
@@ -193,25 +203,41 @@ struct DecodeFrag {
 __device__ __forceinline__ half8 stream_load(const half8* p) { return __builtin_nontemporal_load(p); }
 
 template <int HD>
+__device__ __forceinline__ void load_frag_k(DecodeFrag<HD>& f, const uint16_t* __restrict__ kbase,
+                                            uint32_t tile, int lane)
+{
+    // Half t of the tile feeds sub-tile t: MFMA row m is slot m of the half, and
+    // lane group g reads chunk 4s + g of it for contraction step s.  In the
+    // cache's K layout that is one contiguous KiB per load.  Slot m of half t is
+    // position 8*(m/4) + 4t + m%4 of the tile, so the accumulator of lane group
+    // g ends up holding keys 8g .. 8g+7 in order: exactly the eight consecutive
+    // positions that group reads from Vt.
+    const half8* base = reinterpret_cast<const half8*>(kbase + (size_t)tile * kTileKeys * HD) + lane;
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+#pragma unroll
+        for (int s = 0; s < HD / 32; s++)
+            f.k[t][s] = stream_load(&base[(t * (HD / 8) + s * 4) * 16]);
+    }
+}
+
+template <int HD>
+__device__ __forceinline__ void load_frag_v(DecodeFrag<HD>& f, const uint16_t* __restrict__ vtbase,
+                                            uint32_t tile, int lane)
+{
+    const int m = lane & 15, g = lane >> 4;
+    const half8* vb = reinterpret_cast<const half8*>(vtbase + (size_t)tile * HD * kVBlock);
+#pragma unroll
+    for (int dt = 0; dt < HD / 16; dt++) f.v[dt] = stream_load(&vb[(dt * 16 + m) * 4 + g]);
+}
+
+template <int HD>
 __device__ __forceinline__ void load_frag(DecodeFrag<HD>& f, const uint16_t* __restrict__ kbase,
                                           const uint16_t* __restrict__ vtbase, uint32_t tile,
                                           int lane)
 {
-    const int m = lane & 15, g = lane >> 4;
-    const uint32_t kb = tile * kTileKeys;
-    // Sub-tile t feeds MFMA row m with key kb + 8*(m/4) + 4t + m%4, so that the
-    // accumulator of lane group g ends up holding keys kb+8g .. kb+8g+7 in
-    // order: exactly the eight consecutive positions that group reads from Vt.
-#pragma unroll
-    for (int t = 0; t < 2; t++) {
-        const uint32_t key = kb + 8 * (m >> 2) + 4 * t + (m & 3);
-        const half8* row = reinterpret_cast<const half8*>(kbase + (size_t)key * HD);
-#pragma unroll
-        for (int s = 0; s < HD / 32; s++) f.k[t][s] = stream_load(&row[s * 4 + g]);
-    }
-    const half8* vb = reinterpret_cast<const half8*>(vtbase + (size_t)tile * HD * kVBlock);
-#pragma unroll
-    for (int dt = 0; dt < HD / 16; dt++) f.v[dt] = stream_load(&vb[(dt * 16 + m) * 4 + g]);
+    load_frag_k<HD>(f, kbase, tile, lane);
+    load_frag_v<HD>(f, vtbase, tile, lane);
 }
 
 template <int HD>
@@ -221,17 +247,11 @@ struct DecodeState {
     float l;                 // this lane group's share of the denominator
 };
 
-// col_kind: 0 = hi column of a head, 1 = lo column, 2 = unused column.
+// Scores of one tile, S^T[key][column], before the hi and lo columns are added.
 template <int HD>
-__device__ __forceinline__ void process_tile(DecodeState<HD>& st, DecodeFrag<HD>& f,
-                                             const half8 (&qop)[HD / 32], uint32_t tile,
-                                             uint32_t key_lo, uint32_t seq_k, int lane,
-                                             int partner_addr, int col_kind)
+__device__ __forceinline__ void tile_scores(f32x4 (&c)[2], const DecodeFrag<HD>& f,
+                                            const half8 (&qop)[HD / 32])
 {
-    const int g = lane >> 4;
-    const uint32_t kb = tile * kTileKeys;
-
-    f32x4 c[2];
 #pragma unroll
     for (int t = 0; t < 2; t++) {
         c[t] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -239,6 +259,35 @@ __device__ __forceinline__ void process_tile(DecodeState<HD>& st, DecodeFrag<HD>
         for (int s = 0; s < HD / 32; s++)
             c[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(f.k[t][s], qop[s], c[t], 0, 0, 0);
     }
+}
+
+// Same, with the Q^T operand read from LDS row by row instead of being held in
+// registers (the 256-wide head has no registers to spare for it).
+template <int HD>
+__device__ __forceinline__ void tile_scores_lds(f32x4 (&c)[2], const DecodeFrag<HD>& f,
+                                                const _Float16* __restrict__ qrow)
+{
+    c[0] = f32x4{0.f, 0.f, 0.f, 0.f};
+    c[1] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < HD / 32; s++) {
+        const half8 qs = *reinterpret_cast<const half8*>(qrow + s * 32);
+        c[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(f.k[0][s], qs, c[0], 0, 0, 0);
+        c[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(f.k[1][s], qs, c[1], 0, 0, 0);
+    }
+}
+
+// Online-softmax update of one tile from its raw scores, and the P.V product.
+// col_kind: 0 = hi column of a head, 1 = lo column, 2 = unused column.
+template <int HD>
+__device__ __forceinline__ void tile_update(DecodeState<HD>& st, DecodeFrag<HD>& f,
+                                            const f32x4 (&c)[2], uint32_t tile, uint32_t key_lo,
+                                            uint32_t seq_k, int lane, int partner_addr,
+                                            int col_kind)
+{
+    const int g = lane >> 4;
+    const uint32_t kb = tile * kTileKeys;
+
     // score = hi column + lo column; both columns of a head end up with the sum
     float sc[8];
 #pragma unroll
@@ -298,19 +347,35 @@ __device__ __forceinline__ void process_tile(DecodeState<HD>& st, DecodeFrag<HD>
     }
 }
 
-// Waves per SIMD the register budget is sized for: two double-buffered tiles of
-// a 256-wide head need more than 256 registers, so that shape runs one wave
-// per SIMD with the full 512-register file (32 KB of loads in flight per wave).
 template <int HD>
-constexpr int decode_waves_per_simd() { return HD >= 256 ? 1 : 2; }
+__device__ __forceinline__ void process_tile(DecodeState<HD>& st, DecodeFrag<HD>& f,
+                                             const half8 (&qop)[HD / 32], uint32_t tile,
+                                             uint32_t key_lo, uint32_t seq_k, int lane,
+                                             int partner_addr, int col_kind)
+{
+    f32x4 c[2];
+    tile_scores<HD>(c, f, qop);
+    tile_update<HD>(st, f, c, tile, key_lo, seq_k, lane, partner_addr, col_kind);
+}
+
+// Two waves per SIMD for every shape.  Up to head_dim 128 a wave double-buffers
+// whole tiles in registers.  One tile of a 256-wide head is already 128
+// registers, so that shape keeps a single tile and asks for the next tile's K
+// as soon as the scores are out and for its V as soon as P.V is done; the
+// other wave of the SIMD computes while those loads are in flight.  (Double
+// buffering it with one wave per SIMD and 512 registers spilled addresses, and
+// a spill reload waits for every load in flight.)
+template <int HD>
+constexpr bool decode_single_buffered() { return HD >= 256; }
 
 template <int HD>
-__global__ __launch_bounds__(kDecodeThreads, decode_waves_per_simd<HD>())
+__global__ __launch_bounds__(kDecodeThreads, 2)
 void decode_mfma_kernel(const DecodeArgs a)
 {
-    const uint32_t split = blockIdx.x, kvh = blockIdx.y, sess = blockIdx.z;
+    const uint32_t kvh = blockIdx.x;
+    const uint32_t item = a.items[blockIdx.y];
+    const uint32_t sess = item >> 8, split = item & 0xFFu;
     const DecodeSession S = a.s[sess];
-    if (split >= S.n_splits) return;
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n = lane & 15, g = lane >> 4;
@@ -343,10 +408,13 @@ void decode_mfma_kernel(const DecodeArgs a)
             lds_q[2 * G + idx / HD][idx % HD] = (_Float16)0.0f;
     }
     __syncthreads();
-    half8 qop[HD / 32];
+    constexpr bool kSingle = decode_single_buffered<HD>();
+    half8 qop[kSingle ? 1 : HD / 32];
+    if constexpr (!kSingle) {
 #pragma unroll
-    for (int s = 0; s < HD / 32; s++)
-        qop[s] = *reinterpret_cast<const half8*>(&lds_q[n][s * 32 + g * 8]);
+        for (int s = 0; s < HD / 32; s++)
+            qop[s] = *reinterpret_cast<const half8*>(&lds_q[n][s * 32 + g * 8]);
+    }
 
     const int col_kind = (n < G) ? 0 : ((n < 2 * G) ? 1 : 2);
     const int partner = (n < G) ? lane + G : ((n < 2 * G) ? lane - G : lane);
@@ -358,17 +426,44 @@ void decode_mfma_kernel(const DecodeArgs a)
     st.m = -INFINITY;
     st.l = 0.f;
 
-    if (t < tr.t_end) {
-        for (;;) {
-            const uint32_t t1 = t + kDecodeWaves;
-            if (t1 < tr.t_end) load_frag<HD>(fb, kbase, vtbase, t1, lane);
+    // Loads inside the loops below are unconditional, and the last one or two
+    // tiles are peeled off: the compiler places its waits by counting loads
+    // issued since the one it needs, and a load that is only sometimes issued
+    // makes it assume the smaller count, which turns "wait for this tile" into
+    // "wait for the prefetched tile as well".
+    if constexpr (kSingle) {
+        const _Float16* qrow = &lds_q[n][g * 8];
+        if (t < tr.t_end) {
+            f32x4 c[2];
+            while (t + kDecodeWaves < tr.t_end) {
+                // keeps the Q^T reads inside the loop: hoisted, they would cost
+                // the registers this path does not have
+                asm volatile("" ::: "memory");
+                tile_scores_lds<HD>(c, fa, qrow);
+                load_frag_k<HD>(fa, kbase, t + kDecodeWaves, lane);
+                tile_update<HD>(st, fa, c, t, S.key_lo, S.seq_k, lane, partner_addr, col_kind);
+                load_frag_v<HD>(fa, vtbase, t + kDecodeWaves, lane);
+                t += kDecodeWaves;
+            }
+            tile_scores_lds<HD>(c, fa, qrow);
+            tile_update<HD>(st, fa, c, t, S.key_lo, S.seq_k, lane, partner_addr, col_kind);
+        }
+    } else if (t < tr.t_end) {
+        while (t + 2 * kDecodeWaves < tr.t_end) {
+            load_frag<HD>(fb, kbase, vtbase, t + kDecodeWaves, lane);
             process_tile<HD>(st, fa, qop, t, S.key_lo, S.seq_k, lane, partner_addr, col_kind);
-            if (t1 >= tr.t_end) break;
-            const uint32_t t2 = t1 + kDecodeWaves;
-            if (t2 < tr.t_end) load_frag<HD>(fa, kbase, vtbase, t2, lane);
-            process_tile<HD>(st, fb, qop, t1, S.key_lo, S.seq_k, lane, partner_addr, col_kind);
-            if (t2 >= tr.t_end) break;
-            t = t2;
+            load_frag<HD>(fa, kbase, vtbase, t + 2 * kDecodeWaves, lane);
+            process_tile<HD>(st, fb, qop, t + kDecodeWaves, S.key_lo, S.seq_k, lane, partner_addr,
+                             col_kind);
+            t += 2 * kDecodeWaves;
+        }
+        if (t + kDecodeWaves < tr.t_end) {
+            load_frag<HD>(fb, kbase, vtbase, t + kDecodeWaves, lane);
+            process_tile<HD>(st, fa, qop, t, S.key_lo, S.seq_k, lane, partner_addr, col_kind);
+            process_tile<HD>(st, fb, qop, t + kDecodeWaves, S.key_lo, S.seq_k, lane, partner_addr,
+                             col_kind);
+        } else {
+            process_tile<HD>(st, fa, qop, t, S.key_lo, S.seq_k, lane, partner_addr, col_kind);
         }
     }
     // denominator: add the four lane groups' shares
@@ -463,12 +558,13 @@ __device__ __forceinline__ void generic_attend_wg(GenericShared& sh, const uint1
     float m = -INFINITY, l = 0.f;
 
     for (uint32_t key = key_begin + wave; key < key_end; key += kDecodeWaves) {
-        const uint16_t* krow = k + k_row_offset(kvh, ctx_pad, key, hd);
         float dot = 0.f;
 #pragma unroll
         for (int i = 0; i < kGenericMaxPerLane; i++) {
             const uint32_t d = lane + 64 * i;
-            if (d < hd) dot += qv[i] * (float)(*reinterpret_cast<const _Float16*>(krow + d));
+            if (d < hd)
+                dot += qv[i] * (float)(*reinterpret_cast<const _Float16*>(
+                                   k + k_offset(kvh, ctx_pad, key, d, hd)));
         }
 #pragma unroll
         for (int off = 32; off >= 1; off >>= 1) dot += wave_xor_f32(dot, off);
@@ -520,9 +616,10 @@ __device__ __forceinline__ GenericMerge merge_generic(const GenericShared& sh)
 
 __global__ __launch_bounds__(kDecodeThreads) void decode_generic_kernel(const DecodeArgs a)
 {
-    const uint32_t split = blockIdx.x, head = blockIdx.y, sess = blockIdx.z;
+    const uint32_t head = blockIdx.x;
+    const uint32_t item = a.items[blockIdx.y];
+    const uint32_t sess = item >> 8, split = item & 0xFFu;
     const DecodeSession S = a.s[sess];
-    if (split >= S.n_splits) return;
     const uint32_t hd = a.hd;
     const uint32_t kvh = head / a.group;
     const TileRange tr = split_tiles(S, split);

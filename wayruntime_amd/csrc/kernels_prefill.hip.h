@@ -115,7 +115,9 @@ __device__ __forceinline__ void prefill_stash(PrefillSmem<HD>& sm, int buf,
 #pragma unroll
     for (int c = 0; c < HD / 64; c++) {
         const int ch = tid + c * kPrefillThreads;
-        *reinterpret_cast<u32x4*>(&sm.k[buf][ch / KCH][(ch % KCH) * 8]) = st.k[c];
+        // unit ch of the cache's K tile is (half, chunk, slot); LDS keeps rows by position
+        const int krow = (int)k_tile_pos(ch / (KCH * 16), ch % 16);
+        *reinterpret_cast<u32x4*>(&sm.k[buf][krow][((ch / 16) % KCH) * 8]) = st.k[c];
         u32x4 v = st.v[c];
         if (tail) {
             // rows that were never appended may hold anything: zero them so
@@ -484,8 +486,8 @@ struct SplitCtx {
     uint32_t cnt;                     // byte offset of this set's arrival counter
     uint32_t t0, nt, t_last, kv_valid;   // nt may be 0 (the odd set of a one-tile block)
     // Lane-invariant addresses, one register each; the others follow from them:
-    // a wave's second load of a tile is the first one 4 KiB further (same slot
-    // permutation), and the operand read of contraction step s / half t is the
+    // a wave's second load of a tile is the first one kKStep / 4 KiB further (same
+    // slot permutation), and the operand read of contraction step s / half t is the
     // first one with address bits 5-7 / bit 5 flipped (the permutation is an
     // XOR of the chunk index, the step is the chunk index's upper bits).
     uint32_t gk_off;                  // lane's byte offset inside a K tile, first load
@@ -517,8 +519,10 @@ __device__ __forceinline__ void lds_direct_load(uint32_t lds_addr, const unsigne
                  : "memory");
 }
 
-// Loads of the set's j-th K tile into ring slot `slot`.  Chunk q = sub + 4u of
-// the tile: 1024 consecutive bytes.
+// Loads of the set's j-th K tile into ring slot `slot`.  KiB q = sub + 4u of the
+// LDS image (tile rows by position, 1024 / RB rows per KiB) is gathered from the
+// cache's K tile, 16 bytes per lane: rows 16 apart share half and chunk and sit
+// eight slots = 128 bytes apart there.
 template <int HD>
 __device__ __forceinline__ void split_issue_k(const SplitCtx<HD>& cx, uint32_t j, int slot, int sub)
 {
@@ -527,7 +531,7 @@ __device__ __forceinline__ void split_issue_k(const SplitCtx<HD>& cx, uint32_t j
     const unsigned char* src = cx.kbase + (size_t)tile * L::KTILE;
 #pragma unroll
     for (int u = 0; u < L::NL; u++)
-        lds_direct_load(cx.lds0 + cx.ring + slot * L::KTILE + (sub + 4 * u) * 1024, src + u * 4096,
+        lds_direct_load(cx.lds0 + cx.ring + slot * L::KTILE + (sub + 4 * u) * 1024, src + u * 128,
                         cx.gk_off);
 }
 
@@ -843,13 +847,14 @@ __device__ __forceinline__ void split_block(const PrefillArgs& a, unsigned char*
     {
         // K: lane -> (row of the tile, slot); fetch the chunk that belongs in that slot
         const int row = sub * (1024 / L::RB) + lane / L::CPR;
-        cx.gk_off = row * L::RB + ((lane % L::CPR) ^ L::fk(row)) * 16;
+        const int chunk = (lane % L::CPR) ^ L::fk(row);
+        cx.gk_off = ((k_tile_half(row) * L::CPR + chunk) * 16 + k_tile_slot(row)) * 16;
         // Vt: rows of 64 bytes, four slots each
         const int vrow = sub * 16 + lane / 4;
         cx.gv_off = vrow * 64 + ((lane & 3) ^ L::fv(vrow)) * 16;
-        static_assert(L::NL == 1 || (L::fk(4 * (1024 / L::RB)) == L::fk(0) && L::fv(64) == L::fv(0) &&
-                                     4 * (1024 / L::RB) * L::RB == 4096),
-                      "the second load is the first one 4 KiB further");
+        static_assert(L::NL == 1 || (L::NL == 2 && 4 * (1024 / L::RB) == 16 && L::fk(16) == L::fk(0) &&
+                                     L::fv(64) == L::fv(0)),
+                      "the second load is 16 K rows (128 bytes in the cache) / 64 Vt rows (4 KiB) further");
         const int krow = prefill_key_perm(n);             // tile row this lane feeds to MFMA row n
         cx.kread = krow * L::RB + ((g ^ L::fk(krow)) * 16);
         cx.vread = n * 64 + ((g ^ L::fv(n)) * 16);

@@ -242,9 +242,13 @@ int decode_locked(uint32_t n, wr_hip_kv* const* kv, uint32_t layer, const uint32
     // the same whether it is stepped alone or with others, which is what makes
     // the batched step bit-identical to serial steps (reference contract:
     // src/core/batch.c:15-19).  About 1 MiB of K+V per workgroup (2048 keys at
-    // head_dim 128) measured best for the 16-session workload; the session's
-    // tiles are then spread evenly over that many workgroups, and the floor keeps
-    // the in-kernel merge within kMaxSplits partials for very long contexts.
+    // head_dim 128, 1024 at 256) measured best for 16 sessions of 4096; from
+    // 16K keys up an eighth of the session per workgroup measured better
+    // (fewer partials and workgroup turnovers: 82 % -> 86 % of HBM peak at
+    // 16 x 32768).  The session's tiles are spread evenly over the workgroups,
+    // and the floor keeps the in-kernel merge within kMaxSplits partials.
+    // A single long session gets few workgroups this way; a caller that serves
+    // one session at a time can lower the figure with wr_hip_attn_set_tuning.
     (void)tiles_total;
     uint32_t max_splits = 1;
     for (uint32_t i = 0; i < n; i++) {
@@ -255,6 +259,7 @@ int decode_locked(uint32_t n, wr_hip_kv* const* kv, uint32_t layer, const uint32
         } else {
             uint32_t cap = kDefaultTilesPerWg * 128u / (hd < 32 ? 32 : hd);
             if (cap == 0) cap = 1;
+            if (cap < tiles[i] / 8) cap = tiles[i] / 8;
             const uint32_t want = (tiles[i] + cap - 1) / cap;          // workgroups
             tpw = (tiles[i] + want - 1) / want;                        // even share
         }
@@ -263,6 +268,32 @@ int decode_locked(uint32_t n, wr_hip_kv* const* kv, uint32_t layer, const uint32
         a.s[i].tiles_per_wg = tpw;
         a.s[i].n_splits = (tiles[i] + tpw - 1) / tpw;
         if (a.s[i].n_splits > max_splits) max_splits = a.s[i].n_splits;
+    }
+    // work list, longest entries first (ties keep session, split order)
+    {
+        uint32_t len[kBatchMax * kMaxSplits];
+        uint32_t cnt = 0;
+        for (uint32_t i = 0; i < n; i++) {
+            for (uint32_t sp = 0; sp < a.s[i].n_splits; sp++) {
+                const uint32_t begin = sp * a.s[i].tiles_per_wg;
+                const uint32_t left = tiles[i] - begin;
+                len[cnt] = left < a.s[i].tiles_per_wg ? left : a.s[i].tiles_per_wg;
+                a.items[cnt++] = (uint16_t)((i << 8) | sp);
+            }
+        }
+        for (uint32_t i = 1; i < cnt; i++) {           // insertion sort: at most 1024 entries
+            const uint32_t l = len[i];
+            const uint16_t it = a.items[i];
+            uint32_t j = i;
+            while (j > 0 && len[j - 1] < l) {
+                len[j] = len[j - 1];
+                a.items[j] = a.items[j - 1];
+                j--;
+            }
+            len[j] = l;
+            a.items[j] = it;
+        }
+        a.n_items = cnt;
     }
     a.q = q_dev;
     a.out = out_dev;
@@ -285,7 +316,7 @@ int decode_locked(uint32_t n, wr_hip_kv* const* kv, uint32_t layer, const uint32
     }
 
     if (use_mfma) {
-        const dim3 grid(max_splits, nkv, n), block(kDecodeThreads);
+        const dim3 grid(nkv, a.n_items), block(kDecodeThreads);
         if (hd == 64)
             launch_main(decode_mfma_kernel<64>, grid, block, a);
         else if (hd == 128)
@@ -293,7 +324,7 @@ int decode_locked(uint32_t n, wr_hip_kv* const* kv, uint32_t layer, const uint32
         else
             launch_main(decode_mfma_kernel<256>, grid, block, a);
     } else {
-        launch_main(decode_generic_kernel, dim3(max_splits, nq, n), dim3(kDecodeThreads), a);
+        launch_main(decode_generic_kernel, dim3(nq, a.n_items), dim3(kDecodeThreads), a);
     }
     HIP_TRY(hipGetLastError(), "decode launch", layer);
     g.calls.fetch_add(n, std::memory_order_relaxed);
@@ -518,11 +549,13 @@ int wr_hip_attn_kv_create(uint32_t n_layers, const uint32_t* hd_per_layer, uint3
         kv->hd[L] = hd_per_layer[L];
         if (kv->hd[L] == 0) continue;
         any = true;
-        const size_t side = ((size_t)nkv * kv->ctx_pad * kv->hd[L] * 2 + 255) & ~(size_t)255;
+        // K rows are padded to whole 16-byte chunks (common.hip.h); Vt is not
+        const size_t k_side = ((size_t)nkv * kv->ctx_pad * k_padded_hd(kv->hd[L]) * 2 + 255) & ~(size_t)255;
+        const size_t v_side = ((size_t)nkv * kv->ctx_pad * kv->hd[L] * 2 + 255) & ~(size_t)255;
         kv->k_off[L] = cur;
-        cur += side;
+        cur += k_side;
         kv->vt_off[L] = cur;
-        cur += side;
+        cur += v_side;
     }
     if (!any) {
         delete kv;
