@@ -184,6 +184,39 @@ int wr_hip_attn_prefill_dev(wr_hip_kv *kv, uint32_t layer, uint32_t p0,
                             uint32_t nq, float scale_override,
                             uint32_t window);
 
+/* ---- projections ---------------------------------------------------------
+ * The matrix products either side of the attention path, for callers that want
+ * Q/K/V made and the output projected where the cache lives: replaces
+ * wri_op_matmul at src/core/session.c:446-457 (wq, wk, wv) and :499-506 (wo)
+ * for F16 weights (the reference widens them to F32 at load,
+ * src/core/loader.c:164-190, and multiplies in F32, src/core/kernels.c:124-137;
+ * here the F16 values are multiplied with F32 activations split into two
+ * half-precision terms and summed in F32: results agree to F32 rounding, not
+ * bit for bit, because the order of the sum differs).
+ *
+ * A weight is W[n_out][n_in], `n_in` contiguous (src/core/internal.h:113-118),
+ * given as n_parts row blocks that are stacked in order (wq, wk, wv become one
+ * product); n_in must be a multiple of 32 and the total n_out of 16, else
+ * WR_HIP_ERR_INVAL.  The device copy is private to the library. */
+typedef struct wr_hip_weight wr_hip_weight;
+int  wr_hip_proj_weight_create(uint32_t n_parts, const uint16_t *const *parts_f16,
+                               const uint32_t *rows_per_part, uint32_t n_in,
+                               wr_hip_weight **out);
+void wr_hip_proj_weight_destroy(wr_hip_weight *w);
+uint32_t wr_hip_proj_weight_rows(const wr_hip_weight *w);
+uint32_t wr_hip_proj_weight_cols(const wr_hip_weight *w);
+
+/* y[rows][n_out] = x[rows][n_in] . W^T, host F32 in and out, synchronous. */
+int wr_hip_proj_rows(const wr_hip_weight *w, uint32_t rows, const float *x,
+                     float *y);
+/* Device-resident form, asynchronous on the library stream: row strides ldx >=
+ * n_in and ldy >= n_out (ldy a multiple of 4, y_dev 16-byte aligned);
+ * add_dev, if not NULL, is [rows][ldy] and is added to the product (the
+ * residual add that follows wo, src/core/session.c:505-506). */
+int wr_hip_proj_rows_dev(const wr_hip_weight *w, uint32_t rows,
+                         const float *x_dev, uint32_t ldx,
+                         const float *add_dev, float *y_dev, uint32_t ldy);
+
 /* Tuning knobs for measurement (0 = automatic): keys handled per workgroup in
  * the split-K decode kernel, and a switch forcing the generic (non-MFMA)
  * kernels.  Not needed by a normal caller. */

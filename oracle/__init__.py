@@ -100,6 +100,9 @@ def _load_oracle() -> C.CDLL:
     lib.wro_rope.argtypes = [_f32p] + [C.c_uint32] * 4 + [C.c_float, C.c_uint32]
     lib.wro_rope_table.argtypes = [_f32p] + [C.c_uint32] * 3 + [C.c_float, C.c_uint32]
     lib.wro_rope_table.restype = C.c_int
+    lib.wro_matmul_w16.argtypes = [_f32p, _u16p, _f32p] + [C.c_uint32] * 3
+    lib.wro_rmsnorm.argtypes = [_f32p, C.c_void_p, C.c_uint32, _f32p, C.c_uint32, C.c_uint32,
+                                C.c_float]
     return lib
 
 
@@ -205,6 +208,34 @@ def rope_table(seq: int, hd: int, pos: int, theta: float, n_rot_pairs: int = 0) 
     if n_rot < 0:
         raise ValueError(n_rot)
     return np.ascontiguousarray(buf.reshape(-1)[: seq * n_rot * 2].reshape(seq, n_rot, 2))
+
+
+def matmul_w16(x: np.ndarray, w16: np.ndarray) -> np.ndarray:
+    """x [M, K] float32, w16 [N, K] F16 bit patterns -> x . W^T, float32 [M, N]."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    w16 = np.ascontiguousarray(w16, dtype=np.uint16)
+    y = np.empty((x.shape[0], w16.shape[0]), dtype=np.float32)
+    rc = lib().wro_matmul_w16(x, w16, y, x.shape[0], x.shape[1], w16.shape[0])
+    if rc != 0:
+        raise ValueError(rc)
+    return y
+
+
+def rmsnorm(x: np.ndarray, w, eps: float) -> np.ndarray:
+    """Rows of x (last axis = dim) normalised; w float32 [wn] or None."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    dim = x.shape[-1]
+    rows = x.size // dim
+    out = np.empty_like(x)
+    if w is None:
+        wp, wn = None, 0
+    else:
+        w = np.ascontiguousarray(w, dtype=np.float32)
+        wp, wn = w.ctypes.data, w.size
+    rc = lib().wro_rmsnorm(x.reshape(-1), wp, wn, out.reshape(-1), rows, dim, eps)
+    if rc != 0:
+        raise ValueError(rc)
+    return out
 
 
 # --------------------------------------------------------------- reference --

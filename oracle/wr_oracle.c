@@ -495,3 +495,55 @@ int wro_rope(float *x, uint32_t seq, uint32_t heads, uint32_t hd,
     }
     return WRO_OK;
 }
+
+/* ------------------------------------------------------------------------
+ * Projections.  The reference widens F16 weights to F32 when it loads them
+ * (src/core/loader.c:164-190) and multiplies activation rows with the
+ * GGML-layout weight W[out][in] in F32 (wri_op_matmul, src/core/kernels.c,
+ * GGML branch).  Its inner loop is chosen at run time from a scalar, an AVX2
+ * and an AVX-512 variant that sum in different orders (kernels.c:124-137,
+ * 273-340), so its own results differ in the last bits from host to host; the
+ * restatement follows the scalar variant (kernels.c:124-137): one running F32
+ * sum per output, inputs in ascending order, product and sum rounded
+ * separately.
+ * ---------------------------------------------------------------------- */
+int wro_matmul_w16(const float *a, const uint16_t *w_f16, float *c, uint32_t M,
+                   uint32_t K, uint32_t N)
+{
+    if (!a || !w_f16 || !c || M == 0 || K == 0 || N == 0) return WRO_ERR_INVAL;
+    for (uint32_t i = 0; i < M; i++) {
+        const float *arow = a + (size_t)i * K;
+        for (uint32_t j = 0; j < N; j++) {
+            const uint16_t *wrow = w_f16 + (size_t)j * K;
+            float sum = 0;
+            for (uint32_t k = 0; k < K; k++)
+                sum += arow[k] * wro_f16_to_f32(wrow[k]);
+            c[(size_t)i * N + j] = sum;
+        }
+    }
+    return WRO_OK;
+}
+
+/* Weighted RMS normalisation of `rows` rows of `dim` values, w indexed modulo
+ * wn (wn == 0: no weight).  src/core/kernels.c:1276-1316. */
+int wro_rmsnorm(const float *x, const float *w, uint32_t wn, float *out,
+                uint32_t rows, uint32_t dim, float eps)
+{
+    if (!x || !out || dim == 0) return WRO_ERR_INVAL;
+    if (wn > 0 && !w) return WRO_ERR_INVAL;
+    for (uint32_t r = 0; r < rows; r++) {
+        const float *xr = x + (size_t)r * dim;
+        float sumsq = 0;
+        for (uint32_t j = 0; j < dim; j++) {
+            const float v = xr[j];
+            sumsq += v * v;
+        }
+        const float inv_rms = 1.0f / wro_sqrt(sumsq / (float)dim + eps);
+        for (uint32_t j = 0; j < dim; j++) {
+            const float v = xr[j];
+            const float ww = (wn > 0) ? w[j % wn] : 1.0f;
+            out[(size_t)r * dim + j] = v * inv_rms * ww;
+        }
+    }
+    return WRO_OK;
+}

@@ -141,6 +141,15 @@ int wro_rope_table(float *out, uint32_t seq, uint32_t hd, uint32_t pos,
 int wro_rope(float *x, uint32_t seq, uint32_t heads, uint32_t hd,
              uint32_t pos, float theta_base, uint32_t n_rot_pairs);
 
+/* y[M][N] = a[M][K] . W[N][K]^T, W given as F16 bit patterns and widened to
+ * F32 first; scalar summation order (src/core/kernels.c:124-137). */
+int wro_matmul_w16(const float *a, const uint16_t *w_f16, float *c, uint32_t M,
+                   uint32_t K, uint32_t N);
+
+/* src/core/kernels.c:1276-1316 */
+int wro_rmsnorm(const float *x, const float *w, uint32_t wn, float *out,
+                uint32_t rows, uint32_t dim, float eps);
+
 #ifdef __cplusplus
 }
 #endif

@@ -100,3 +100,38 @@ def f16_encode_bits() -> np.ndarray:
                       0x7F800001, 0x00000001, 0x007FFFFF, 0xC0000000, 0x3F7FFFFF],
                      dtype=np.uint32)
     return np.concatenate([edges, h])
+
+
+# ---- RMS normalisation: name, rows, dim, weight length (0 = none), eps
+NORM_CASES = [
+    ("hidden_1024", 3, 1024, 1024, 1e-6),
+    ("per_head_128", 16, 128, 128, 1e-6),          # Qwen3 Q/K norm: [heads, head_dim] rows
+    ("per_head_256_eps5", 8, 256, 256, 1e-5),
+    ("weightless_64", 4, 64, 0, 1e-6),             # the V-norm shape
+    ("weight_wraps", 2, 12, 4, 1e-5),              # weight indexed modulo its length
+]
+
+
+def norm_inputs(case):
+    name, rows, dim, wn, _eps = case
+    base = (sum(ord(c) * (i + 3) for i, c in enumerate(name)) * 2654435761) & 0xFFFFFFFF
+    x = synth.hash_bell(base + 1, (rows, dim)) * np.float32(2.5)
+    w = (synth.hash_bell(base + 2, (wn,)) * np.float32(0.25) + np.float32(1.0)) if wn else None
+    return x, w
+
+
+# ---- projections  y = x . W^T, F16 weights: name, rows, n_in, n_out, weight std
+MATMUL_CASES = [
+    ("qkv_like", 2, 1024, 96, 0.02),
+    ("wo_like", 1, 2048, 64, 0.02),
+    ("rows9_k96", 9, 96, 48, 0.5),
+    ("k32_n16", 3, 32, 16, 1.0),
+]
+
+
+def matmul_inputs(case):
+    name, rows, n_in, n_out, wstd = case
+    base = (sum(ord(c) * (i + 5) for i, c in enumerate(name)) * 2654435761) & 0xFFFFFFFF
+    x = synth.hash_bell(base + 1, (rows, n_in))
+    w16 = synth.f32_to_f16_trunc(synth.hash_bell(base + 2, (n_out, n_in)) * np.float32(wstd))
+    return x, w16

@@ -14,6 +14,9 @@ bit-for-bit by the tests), so the files hold expected outputs only:
     mathx_golden.npz  exp/log/sqrt/sin/cos on fixed grids
     f16_golden.npz    truncating encode of fixed float32 bit patterns,
                       decode of all 65536 binary16 patterns (as uint32 bits)
+    ops_golden.npz    RMS normalisation and GGML-layout matmul outputs (the
+                      matmul through whichever SIMD variant this host selects;
+                      its variant number is stored beside the outputs)
 """
 from __future__ import annotations
 
@@ -70,6 +73,35 @@ def main() -> None:
                     for b in bits], dtype=np.uint16)
     dec = np.array([ref.wri_f16_to_f32(h) for h in range(65536)], dtype=np.float32).view(np.uint32)
     np.savez_compressed(os.path.join(HERE, "f16_golden.npz"), encode=enc, decode_bits=dec)
+
+    ops = {}
+    ref.wri_op_rmsnorm.argtypes = [C.POINTER(oracle.Tensor)] * 3 + [C.c_float]
+    ref.wri_op_matmul.argtypes = [C.POINTER(oracle.Tensor)] * 3
+    ref.wri_simd_matmul_variant.restype = C.c_int
+    for case in cases.NORM_CASES:
+        name, _rows, _dim, wn, eps = case
+        x, w = cases.norm_inputs(case)
+        y = np.empty_like(x)
+        tx, ty = oracle.wrap(x), oracle.wrap(y)
+        tw = oracle.wrap(w) if wn else None
+        rc = ref.wri_op_rmsnorm(C.byref(tx), C.byref(tw) if wn else None, C.byref(ty), eps)
+        assert rc == 0, (name, rc)
+        ops["norm_" + name] = y
+    GGML_WEIGHT = 1 << 3                               # src/core/internal.h:113-118
+    for case in cases.MATMUL_CASES:
+        name, rows, n_in, n_out, _std = case
+        x, w16 = cases.matmul_inputs(case)
+        # the loader widens F16 weights to F32 before any multiply (loader.c:164-190)
+        w32 = np.array([ref.wri_f16_to_f32(int(h)) for h in w16.reshape(-1)],
+                       dtype=np.float32).reshape(n_out, n_in)
+        y = np.empty((rows, n_out), dtype=np.float32)
+        ta, tc = oracle.wrap(x), oracle.wrap(y)
+        tb = oracle.wrap(w32, shape=(n_in, n_out), flags=GGML_WEIGHT)
+        rc = ref.wri_op_matmul(C.byref(ta), C.byref(tb), C.byref(tc))
+        assert rc == 0, (name, rc)
+        ops["matmul_" + name] = y
+    ops["matmul_variant"] = np.array([ref.wri_simd_matmul_variant()], dtype=np.int32)
+    np.savez(os.path.join(HERE, "ops_golden.npz"), **ops)
 
     for f in sorted(os.listdir(HERE)):
         if f.endswith(".npz"):

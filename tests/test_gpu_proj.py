@@ -1,0 +1,158 @@
+"""Row projections on the device (y = x . W^T, F16 weights, F32 rows) against
+the CPU oracle's restatement of the reference matmul, through the C ABI.
+
+The device sums in a different order (matrix-core tiles of 32 inputs, F32
+accumulation) and feeds each activation as two half-precision terms, so the
+results agree to F32 rounding, not bit for bit.  Tolerance, per output: 3e-7 *
+sqrt(n_in) * sum_k |x_k w_k| (a few F32 ulps of the magnitudes summed, growing
+like a random walk with the length of the sum), which is also what separates
+the reference's own SIMD variants from its scalar loop."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import oracle
+from wayruntime_amd import hipattn, synth
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _device():
+    hipattn.init()
+    yield
+
+
+def _w16(seed, n_out, n_in, std):
+    return synth.f32_to_f16_trunc(synth.normal(seed, (n_out, n_in), std=std))
+
+
+def _widen(w16):
+    # IEEE binary16 -> float64, the same values the reference's decoder yields
+    return np.ascontiguousarray(w16).view(np.float16).astype(np.float64)
+
+
+def _check(got, x, w16, what):
+    want = oracle.matmul_w16(x, w16)
+    mag = np.abs(x.astype(np.float64)) @ np.abs(_widen(w16)).T
+    tol = 3e-7 * np.sqrt(x.shape[1]) * mag + 1e-37
+    err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    assert not np.isnan(got).any(), what
+    assert np.all(err <= tol), f"{what}: worst err/tol = {np.max(err / tol):.3f}"
+
+
+@pytest.mark.parametrize("rows,n_in,n_out,std", [
+    (1, 1024, 4096, 0.02),        # Qwen3-0.6B: wq, wk, wv stacked
+    (1, 2048, 1024, 0.02),        # wo
+    (16, 1024, 3072, 0.02),       # a full batch through an FFN-sized weight
+    (9, 96, 48, 0.5),             # three input tiles: no full batch of eight, tail loop only
+    (3, 320, 16, 1.0),            # ten input tiles: one batch and a tail; a single output tile
+    (8, 32, 64, 1.0),             # one input tile
+    (17, 512, 80, 0.1),           # rows pad to four groups of eight; outputs not a multiple of 64
+    (300, 256, 128, 0.1),         # more rows than one launch takes
+])
+def test_projection_shapes_vs_oracle(rows, n_in, n_out, std):
+    print("proj", rows, n_in, n_out, flush=True)
+    x = synth.normal(rows * 7 + n_in, (rows, n_in))
+    w16 = _w16(n_out + 3, n_out, n_in, std)
+    w = hipattn.Weight([w16])
+    _check(w.rows(x), x, w16, f"{rows}x{n_in}x{n_out}")
+    w.close()
+
+
+def test_stacked_parts_equal_separate_weights():
+    n_in = 1024
+    parts = [_w16(11, 2048, n_in, 0.02), _w16(12, 1024, n_in, 0.02), _w16(13, 1024, n_in, 0.02)]
+    x = synth.normal(14, (2, n_in))
+    stacked = hipattn.Weight(parts)
+    y = stacked.rows(x)
+    assert y.shape == (2, 4096)
+    off = 0
+    for p in parts:
+        single = hipattn.Weight([p])
+        assert np.array_equal(single.rows(x), y[:, off:off + p.shape[0]])
+        off += p.shape[0]
+        single.close()
+    stacked.close()
+
+
+def test_small_integers_are_exact():
+    # every product and partial sum is exact in F32 and the half-precision split
+    # of a small integer has no low term: any correct implementation gives the
+    # integer result bit for bit, a wrong tile or lane mapping cannot
+    rng = np.random.default_rng(9)
+    rows, n_in, n_out = 5, 160, 48
+    xi = rng.integers(-8, 9, size=(rows, n_in))
+    wi = rng.integers(-8, 9, size=(n_out, n_in))
+    w16 = np.array([oracle.f32_to_f16(float(v)) for v in range(-8, 9)], dtype=np.uint16)[wi + 8]
+    w = hipattn.Weight([w16])
+    got = w.rows(xi.astype(np.float32))
+    assert np.array_equal(got, (xi @ wi.T).astype(np.float32))
+    w.close()
+
+
+def test_row_magnitudes_do_not_matter():
+    # rows of very different scale in one call, and one row whose entries span
+    # fourteen orders of magnitude: the per-row power-of-two scaling and the
+    # scaled low term keep F32-level accuracy (reference: float64)
+    n_in, n_out = 256, 32
+    x = synth.normal(21, (5, n_in))
+    x[0] *= np.float32(1e-20)
+    x[1] *= np.float32(1e20)
+    x[2, 1:] *= np.float32(5e-5)         # one entry of order 1, the rest tiny
+    x[3] = 0.0
+    x[4, ::2] *= np.float32(1e-14)
+    w16 = _w16(22, n_out, n_in, 0.5)
+    w = hipattn.Weight([w16])
+    got = w.rows(x).astype(np.float64)
+    wf = _widen(w16)
+    want = x.astype(np.float64) @ wf.T
+    mag = np.abs(x.astype(np.float64)) @ np.abs(wf).T
+    assert np.all(got[3] == 0.0)
+    assert np.all(np.abs(got - want) <= 3e-7 * np.sqrt(n_in) * mag + 1e-37)
+    w.close()
+
+
+def test_device_form_with_strides_and_residual_add():
+    rows, n_in, n_out = 6, 128, 64
+    ldx, ldy = n_in + 32, n_out + 8
+    x = synth.normal(31, (rows, ldx))
+    add = synth.normal(32, (rows, ldy))
+    w16 = _w16(33, n_out, n_in, 0.2)
+    w = hipattn.Weight([w16])
+    xd = hipattn.DeviceBuffer.from_host(x)
+    ad = hipattn.DeviceBuffer.from_host(add)
+    yd = hipattn.DeviceBuffer.from_host(np.full((rows, ldy), 7.0, dtype=np.float32))
+    w.rows_dev(rows, xd, ldx, yd, ldy, add_dev=ad)
+    hipattn.sync()
+    y = yd.to_host((rows, ldy))
+    plain = w.rows(np.ascontiguousarray(x[:, :n_in]))
+    assert np.array_equal(y[:, :n_out], plain + add[:, :n_out])
+    assert np.all(y[:, n_out:] == 7.0)              # padding columns are not touched
+    for b in (xd, ad, yd):
+        b.free()
+    w.close()
+
+
+def test_error_contract():
+    lib = hipattn.lib()
+    h = C.c_void_p()
+    good = _w16(41, 16, 32, 1.0)
+    ptrs = (C.c_void_p * 1)(good.ctypes.data)
+
+    def create(rows, n_in):
+        return lib.wr_hip_proj_weight_create(1, ptrs, (C.c_uint32 * 1)(rows), n_in, C.byref(h))
+
+    assert create(16, 31) == hipattn.ERR_INVAL           # inputs not a multiple of 32
+    assert create(8, 32) == hipattn.ERR_INVAL            # outputs not a multiple of 16
+    assert create(0, 32) == hipattn.ERR_INVAL
+    assert lib.wr_hip_proj_weight_create(0, ptrs, (C.c_uint32 * 1)(16), 32, C.byref(h)) == hipattn.ERR_INVAL
+    assert lib.wr_hip_proj_weight_create(1, None, (C.c_uint32 * 1)(16), 32, C.byref(h)) == hipattn.ERR_INVAL
+    assert create(16, 32) == hipattn.OK
+    x = np.zeros((1, 32), dtype=np.float32)
+    y = np.zeros((1, 16), dtype=np.float32)
+    assert lib.wr_hip_proj_rows(h, 1, None, y.ctypes.data) == hipattn.ERR_INVAL
+    assert lib.wr_hip_proj_rows(None, 1, x.ctypes.data, y.ctypes.data) == hipattn.ERR_INVAL
+    assert lib.wr_hip_proj_rows(h, 0, x.ctypes.data, y.ctypes.data) == hipattn.OK     # nothing to do
+    lib.wr_hip_proj_weight_destroy(h)

@@ -421,3 +421,69 @@ def test_rope_table_is_the_rotation_s_own_angles(hd, pos, theta, n_rot_pairs):
     got[:, :, half:half + n_rot] = (x0 * s_).astype(np.float32) + (x1 * c).astype(np.float32)
     assert got.tobytes() == want.tobytes()
 
+
+
+# ---------------------------------------------- RMS normalisation, matmul ----
+
+@pytest.mark.parametrize("case", cases.NORM_CASES, ids=[c[0] for c in cases.NORM_CASES])
+def test_rmsnorm_bit_exact_vs_reference_fixture(case):
+    name, _rows, _dim, _wn, eps = case
+    x, w = cases.norm_inputs(case)
+    got = oracle.rmsnorm(x, w, eps)
+    want = _npz("ops_golden.npz")["norm_" + name]
+    assert got.tobytes() == want.tobytes(), name
+
+
+def test_rmsnorm_reference_self_test_and_closed_form():
+    # src/core/kernels.c:2116-2139: row [1,2,3,4], mean square 7.5
+    x = np.array([[1, 2, 3, 4]], dtype=np.float32)
+    y = oracle.rmsnorm(x, np.ones(4, dtype=np.float32), 1e-5)
+    assert abs(y[0, 0] - 1.0 / 2.7386) < 0.01 and abs(y[0, 3] - 4.0 / 2.7386) < 0.02
+    y2 = oracle.rmsnorm(x, None, 1e-6)
+    assert np.all(np.abs(y2[0] - x[0] / 2.7386) < 0.02)
+    # closed form in float64, the weight applied modulo its length
+    xs = synth.normal(71, (5, 96), std=3.0)
+    w = synth.normal(72, (8,)) + np.float32(1.0)
+    want = xs.astype(np.float64) / np.sqrt((xs.astype(np.float64) ** 2).mean(-1, keepdims=True) + 1e-6)
+    want = want * np.tile(w.astype(np.float64), 12)
+    got = oracle.rmsnorm(xs, w, 1e-6)
+    assert np.max(np.abs(got - want)) < 2e-5 * np.max(np.abs(want))
+    # a row scaled by a power of two normalises to the same values (eps aside)
+    a = oracle.rmsnorm(xs, None, 0.0)
+    b = oracle.rmsnorm(xs * np.float32(8.0), None, 0.0)
+    assert np.max(np.abs(a - b)) < 1e-6
+
+
+@pytest.mark.parametrize("case", cases.MATMUL_CASES, ids=[c[0] for c in cases.MATMUL_CASES])
+def test_matmul_w16_vs_reference_fixture(case):
+    # The fixture was written by whichever SIMD variant the fixture host
+    # selected; the variants differ from the scalar order the oracle follows by
+    # rounding only.  Bound: a few ulp of the sum of magnitudes.
+    name, _rows, n_in, _n_out, _std = case
+    x, w16 = cases.matmul_inputs(case)
+    got = oracle.matmul_w16(x, w16)
+    want = _npz("ops_golden.npz")["matmul_" + name]
+    w = np.array([oracle.f16_to_f32(int(h)) for h in w16.reshape(-1)], dtype=np.float64).reshape(w16.shape)
+    mag = np.abs(x.astype(np.float64)) @ np.abs(w).T
+    assert np.all(np.abs(got.astype(np.float64) - want) <= 1.5e-7 * np.sqrt(n_in) * mag + 1e-30), name
+
+
+def test_matmul_w16_exact_on_integers_and_not_transposed():
+    # small integers: every partial sum is exact in F32, so any summation order
+    # gives the same bits; the shapes are all different, so a swapped or
+    # transposed operand cannot produce the right answer
+    rng = np.random.default_rng(5)
+    M, K, N = 3, 40, 7
+    xi = rng.integers(-8, 9, size=(M, K))
+    wi = rng.integers(-8, 9, size=(N, K))
+    x = xi.astype(np.float32)
+    w16 = np.array([oracle.f32_to_f16(float(v)) for v in wi.reshape(-1)], dtype=np.uint16).reshape(N, K)
+    got = oracle.matmul_w16(x, w16)
+    assert got.shape == (M, N)
+    assert np.array_equal(got, (xi @ wi.T).astype(np.float32))
+    # float64 on random data
+    xs = synth.normal(81, (2, 300))
+    ws = synth.f32_to_f16_trunc(synth.normal(82, (5, 300), std=0.1))
+    wf = np.array([oracle.f16_to_f32(int(h)) for h in ws.reshape(-1)], dtype=np.float64).reshape(5, 300)
+    want = xs.astype(np.float64) @ wf.T
+    assert np.max(np.abs(oracle.matmul_w16(xs, ws) - want)) < 2e-6 * np.max(np.abs(want)) + 1e-6

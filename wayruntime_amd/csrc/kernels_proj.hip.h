@@ -1,0 +1,221 @@
+// Row projections  Y[R][N] = X[R][K] . W[N][K]^T  with F16 weights and F32
+// activations: the Q/K/V/output projections either side of the attention
+// path (reference: wri_op_matmul at src/core/session.c:446-457 and :499-506,
+// inner loops src/core/kernels.c:124-137; weights are W[out][in] with `in`
+// contiguous, src/core/internal.h:113-118, and F16 tensors are widened to F32
+// before the multiply, src/core/loader.c:164-190).
+//
+// Decode sends 1..16 rows through a projection, so the work is reading W once:
+// HBM-bound, algorithmic bytes per launch = 2 * N * K.  The multiply-adds run
+// on v_mfma_f32_16x16x32_f16 to keep them off the vector ALUs, as in the decode
+// kernel, and F32 accuracy is kept the same way: each row is scaled by a power
+// of two into [1, 2) (by its largest magnitude), split into two half-precision
+// terms x = hi + lo * 2^-11, and the two terms take two COLUMNS of the same MFMA
+// (column c = hi of row c, column c + 8 = lo of row c, eight rows per MFMA).
+// The columns are combined and the scale undone at the end; sums are F32.
+//
+// Layouts on the device (both private to the library):
+//
+//   W   [N/16][K/32][64][8] halves: tile (nt, kt) is the MFMA A operand of
+//       outputs 16nt..16nt+15 and inputs 32kt..32kt+31 in lane order (lane =
+//       16g + m holds W[16nt + m][32kt + 8g .. +8]), one contiguous KiB per
+//       operand load; a wave streams the K/32 consecutive KiBs of its outputs.
+//   X   fragments [ceil(R/8)][K/32][64][8] halves, the matching B operands
+//       (lane 16g + c: column c, inputs 32kt + 8g .. +8), written by
+//       proj_prep_kernel, read by every wave (L2 / L1 hits), plus one F32
+//       scale per row (proj_scale_kernel).
+//
+// One wave owns 16 outputs for all rows; a workgroup is four waves = 64
+// outputs.  N must be a multiple of 16 and K a multiple of 32.
+#pragma once
+
+#include "common.hip.h"
+
+namespace wr {
+
+constexpr int kProjThreads = 256;
+constexpr int kProjMaxRows = 256;                 // rows per launch (32 row groups)
+constexpr int kProjKBatch = 8;                    // k-steps (KiBs of W) a wave keeps in flight per buffer
+
+// Row-major F16 W[N][K] -> tile order.  One thread per 16-byte unit.
+__global__ __launch_bounds__(256) void proj_pack_weights_kernel(const uint16_t* __restrict__ w,
+                                                                u32x4* __restrict__ tiles,
+                                                                uint32_t N, uint32_t K)
+{
+    const size_t unit = (size_t)blockIdx.x * blockDim.x + threadIdx.x;     // destination unit
+    const size_t total = (size_t)N * K / 8;
+    if (unit >= total) return;
+    const uint32_t lane = (uint32_t)(unit & 63);
+    const size_t tile = unit >> 6;
+    const uint32_t kt = (uint32_t)(tile % (K / 32));
+    const uint32_t nt = (uint32_t)(tile / (K / 32));
+    const uint32_t m = lane & 15, g = lane >> 4;
+    const u32x4* src = reinterpret_cast<const u32x4*>(w + ((size_t)(nt * 16 + m) * K + kt * 32 + g * 8));
+    tiles[unit] = *src;
+}
+
+// Per-row scale: scales[row] = 2^e with 2^e <= max|x[row]| < 2^(e+1) (1 for a
+// row of zeros).  One wave per row.
+__global__ __launch_bounds__(256) void proj_scale_kernel(const float* __restrict__ x, uint32_t ldx,
+                                                         float* __restrict__ scales, uint32_t R,
+                                                         uint32_t K)
+{
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= R) return;
+    float mx = 0.f;
+    for (uint32_t k = lane; k < K; k += 64) mx = fmaxf(mx, fabsf(x[(size_t)row * ldx + k]));
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) mx = fmaxf(mx, wave_xor_f32(mx, off));
+    if (lane == 0) {
+        uint32_t ex = (__float_as_uint(mx) >> 23) & 0xFFu;
+        if (ex == 0 || ex == 0xFF) ex = 127;              // zeros, subnormals, inf / NaN rows: no scaling
+        if (ex > 253) ex = 253;                           // keeps the inverse 2^-e a normal number
+        scales[row] = __uint_as_float(ex << 23);
+    }
+}
+
+// X[R][K] F32 -> B-operand fragments.  Row r is divided by its scale (exact: a
+// power of two), so its largest magnitude lies in [1, 2), and split into
+//   hi = binary16(v), flushed to zero below the normal range, and
+//   lo = binary16((v - hi) * 2^11),
+// i.e. v = hi + lo * 2^-11 to about 2^-22 |v| (2^-25 of the row's largest value
+// for elements so small that hi is flushed).  Keeping lo scaled up keeps both
+// terms in the normal binary16 range, so the result does not depend on how the
+// matrix cores treat subnormal inputs.  grid = (ceil(K/128), row groups): each
+// wave writes one k tile of one row group.
+constexpr float kProjLoScale = 2048.0f;
+
+__global__ __launch_bounds__(256) void proj_prep_kernel(const float* __restrict__ x, uint32_t ldx,
+                                                        half8* __restrict__ frag,
+                                                        const float* __restrict__ scales, uint32_t R,
+                                                        uint32_t K)
+{
+    const uint32_t grp = blockIdx.y;
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t kt = blockIdx.x * 4 + wave;
+    if (kt >= K / 32) return;
+    const uint32_t c = lane & 15, g = lane >> 4;
+    const uint32_t row = grp * 8 + (c & 7);
+    half8 out;
+#pragma unroll
+    for (int j = 0; j < 8; j++) out[j] = (_Float16)0.0f;
+    if (row < R) {
+        // 1 / 2^e: exponent field 254 - field(2^e)
+        const float inv = __uint_as_float((254u << 23) - __float_as_uint(scales[row]));
+        const float* src = x + (size_t)row * ldx + kt * 32 + g * 8;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const float v = src[j] * inv;
+            _Float16 hi = (_Float16)v;
+            if (fabsf((float)hi) < 6.103515625e-05f) hi = (_Float16)0.0f;      // 2^-14
+            out[j] = (c < 8) ? hi : (_Float16)((v - (float)hi) * kProjLoScale);
+        }
+    }
+    frag[((size_t)grp * (K / 32) + kt) * 64 + lane] = out;
+}
+
+struct ProjArgs {
+    const half8* w;          // tile order
+    const half8* xfrag;      // [groups][K/32][64]
+    const float* scales;     // [R]
+    const float* bias_rows;  // optional [R][N] added to the result (residual), or nullptr
+    float* y;                // [R][ldy]
+    uint32_t N, K, R, ldy;
+    uint32_t groups;         // ceil(R / 8)
+};
+
+// GROUPS = row groups of eight handled per launch (template so the accumulators
+// stay in registers): 1, 2, 4, ... 32.
+template <int GROUPS>
+__global__ __launch_bounds__(kProjThreads) void proj_rows_kernel(const ProjArgs a)
+{
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t nt = blockIdx.x * 4 + wave;                  // this wave's 16 outputs
+    if (nt * 16 >= a.N) return;
+    const uint32_t ktiles = a.K / 32;
+    const half8* wp = a.w + (size_t)nt * ktiles * 64 + lane;
+    const half8* xp = a.xfrag + lane;
+
+    f32x4 acc[GROUPS];
+#pragma unroll
+    for (int gi = 0; gi < GROUPS; gi++) acc[gi] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    // W is read exactly once per launch (non-temporal); X fragments are shared
+    // by every wave of the grid and stay cached.
+    half8 wa[kProjKBatch], wb[kProjKBatch];
+    uint32_t kt = 0;
+    const uint32_t full = ktiles / kProjKBatch * kProjKBatch;
+    if (full > 0) {
+#pragma unroll
+        for (int u = 0; u < kProjKBatch; u++) wa[u] = __builtin_nontemporal_load(&wp[(size_t)u * 64]);
+    }
+    // Loads in the loop are unconditional and the last batch is peeled, so the
+    // compiler's load counting keeps the prefetched batch in flight.
+    while (kt + 2 * kProjKBatch <= full) {
+#pragma unroll
+        for (int u = 0; u < kProjKBatch; u++)
+            wb[u] = __builtin_nontemporal_load(&wp[(size_t)(kt + kProjKBatch + u) * 64]);
+#pragma unroll
+        for (int u = 0; u < kProjKBatch; u++) {
+#pragma unroll
+            for (int gi = 0; gi < GROUPS; gi++) {
+                const half8 xb = xp[((size_t)gi * ktiles + kt + u) * 64];
+                acc[gi] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wa[u], xb, acc[gi], 0, 0, 0);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kProjKBatch; u++) wa[u] = wb[u];
+        kt += kProjKBatch;
+    }
+    if (kt + kProjKBatch <= full) {
+#pragma unroll
+        for (int u = 0; u < kProjKBatch; u++) {
+#pragma unroll
+            for (int gi = 0; gi < GROUPS; gi++) {
+                const half8 xb = xp[((size_t)gi * ktiles + kt + u) * 64];
+                acc[gi] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wa[u], xb, acc[gi], 0, 0, 0);
+            }
+        }
+        kt += kProjKBatch;
+    }
+    for (; kt < ktiles; kt++) {                              // K/32 not a multiple of the batch
+        const half8 wv = __builtin_nontemporal_load(&wp[(size_t)kt * 64]);
+#pragma unroll
+        for (int gi = 0; gi < GROUPS; gi++) {
+            const half8 xb = xp[((size_t)gi * ktiles + kt) * 64];
+            acc[gi] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wv, xb, acc[gi], 0, 0, 0);
+        }
+    }
+
+    // Accumulator layout: lane 16g + c holds outputs 16nt + 4g .. +3 of column c.
+    // Column c (< 8) is the hi term of row c, column c + 8 its lo term.
+    const int c = lane & 15, g = lane >> 4;
+    const int partner_addr = (lane ^ 8) * 4;
+#pragma unroll
+    for (int gi = 0; gi < GROUPS; gi++) {
+        f32x4 v = acc[gi];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const float other =
+                __int_as_float(__builtin_amdgcn_ds_bpermute(partner_addr, __float_as_int(v[i])));
+            v[i] += other * (1.0f / kProjLoScale);      // meaningful in the hi columns only
+        }
+        const uint32_t row = gi * 8 + (c & 7);
+        if (c < 8 && row < a.R) {
+            const float sc = a.scales[row];
+            const size_t o = (size_t)row * a.ldy + nt * 16 + g * 4;
+            f32x4 r;
+#pragma unroll
+            for (int i = 0; i < 4; i++) r[i] = v[i] * sc;
+            if (a.bias_rows) {
+                const f32x4 b = *reinterpret_cast<const f32x4*>(a.bias_rows + o);
+#pragma unroll
+                for (int i = 0; i < 4; i++) r[i] += b[i];
+            }
+            *reinterpret_cast<f32x4*>(a.y + o) = r;
+        }
+    }
+}
+
+}  // namespace wr

@@ -22,8 +22,15 @@
 #include "kernels_append.hip.h"
 #include "kernels_decode.hip.h"
 #include "kernels_prefill.hip.h"
+#include "kernels_proj.hip.h"
 
 using namespace wr;
+
+struct wr_hip_weight {
+    uint32_t n_out, n_in;
+    void* tiles;                 // F16, tile order (kernels_proj.hip.h)
+    size_t bytes;
+};
 
 struct wr_hip_kv {
     uint32_t n_layers, nkv, max_ctx, ctx_pad;
@@ -49,6 +56,7 @@ struct Lib {
     char name[320] = "uninitialised";
     Buffer d_stage;              // device staging for host-pointer entry points
     Buffer d_part;               // split-K partials
+    Buffer d_proj;               // projection operand fragments and row scales
     uint32_t* d_counters = nullptr;   // split-K tickets, zero whenever no launch is in flight
     Buffer h_pin;                // pinned host staging
     std::atomic<uint64_t> calls{0};
@@ -423,6 +431,70 @@ struct Locked {
 
 }  // namespace
 
+// projections: launch helpers (caller holds g.mu)
+namespace {
+
+template <int GROUPS>
+void launch_proj(const ProjArgs& a)
+{
+    launch_main(proj_rows_kernel<GROUPS>, dim3((a.N / 16 + 3) / 4), dim3(kProjThreads), a);
+}
+
+// y_dev[rows][ldy] = x_dev[rows][ldx] . W^T (+ add_dev), rows <= kProjMaxRows.
+// Caller holds g.mu.
+int proj_chunk_locked(const wr_hip_weight* w, uint32_t rows, const float* x_dev, uint32_t ldx,
+                      const float* add_dev, float* y_dev, uint32_t ldy)
+{
+    uint32_t groups = 1;
+    while (groups * 8 < rows) groups *= 2;
+    const uint32_t ktiles = w->n_in / 32;
+    const size_t frag_bytes = (size_t)groups * ktiles * 1024;
+    int rc = ensure_device(g.d_proj, frag_bytes + kProjMaxRows * sizeof(float));
+    if (rc) return rc;
+    half8* frag = reinterpret_cast<half8*>(g.d_proj.p);
+    float* scales = reinterpret_cast<float*>((uint8_t*)g.d_proj.p + frag_bytes);
+    hipLaunchKernelGGL(proj_scale_kernel, dim3((rows + 3) / 4), dim3(256), 0, g.stream, x_dev, ldx,
+                       scales, rows, w->n_in);
+    hipLaunchKernelGGL(proj_prep_kernel, dim3((ktiles + 3) / 4, groups), dim3(256), 0, g.stream, x_dev,
+                       ldx, frag, scales, rows, w->n_in);
+    ProjArgs a;
+    a.w = reinterpret_cast<const half8*>(w->tiles);
+    a.xfrag = frag;
+    a.scales = scales;
+    a.bias_rows = add_dev;
+    a.y = y_dev;
+    a.N = w->n_out;
+    a.K = w->n_in;
+    a.R = rows;
+    a.ldy = ldy;
+    a.groups = groups;
+    switch (groups) {
+    case 1: launch_proj<1>(a); break;
+    case 2: launch_proj<2>(a); break;
+    case 4: launch_proj<4>(a); break;
+    case 8: launch_proj<8>(a); break;
+    case 16: launch_proj<16>(a); break;
+    default: launch_proj<32>(a); break;
+    }
+    HIP_TRY(hipGetLastError(), "projection launch", 0);
+    return WR_HIP_OK;
+}
+
+int proj_locked(const wr_hip_weight* w, uint32_t rows, const float* x_dev, uint32_t ldx,
+                const float* add_dev, float* y_dev, uint32_t ldy)
+{
+    for (uint32_t done = 0; done < rows; done += kProjMaxRows) {
+        const uint32_t n = rows - done < (uint32_t)kProjMaxRows ? rows - done : (uint32_t)kProjMaxRows;
+        int rc = proj_chunk_locked(w, n, x_dev + (size_t)done * ldx, ldx,
+                                   add_dev ? add_dev + (size_t)done * ldy : nullptr,
+                                   y_dev + (size_t)done * ldy, ldy);
+        if (rc) return rc;
+    }
+    return WR_HIP_OK;
+}
+
+}  // namespace
+
 // ======================================================================= ABI
 
 extern "C" {
@@ -495,6 +567,8 @@ void wr_hip_attn_shutdown(void)
     if (g.d_counters) (void)hipFree(g.d_counters);
     g.d_counters = nullptr;
     if (g.h_pin.p) (void)hipHostFree(g.h_pin.p);
+    if (g.d_proj.p) (void)hipFree(g.d_proj.p);
+    g.d_proj = Buffer();
     g.d_stage = Buffer();
     g.d_part = Buffer();
     g.h_pin = Buffer();
@@ -847,6 +921,117 @@ int wr_hip_attn_sync(void)
 }
 
 void* wr_hip_attn_stream(void) { return g.inited ? (void*)g.stream : nullptr; }
+
+// ------------------------------------------------------------ projections --
+
+int wr_hip_proj_weight_create(uint32_t n_parts, const uint16_t* const* parts_f16,
+                              const uint32_t* rows_per_part, uint32_t n_in, wr_hip_weight** out)
+{
+    if (!out) return WR_HIP_ERR_INVAL;
+    *out = nullptr;
+    if (!g.inited) return WR_HIP_ERR_STATE;
+    if (n_parts == 0 || !parts_f16 || !rows_per_part || n_in == 0 || n_in % 32 != 0)
+        return WR_HIP_ERR_INVAL;
+    uint64_t n_out = 0;
+    for (uint32_t i = 0; i < n_parts; i++) {
+        if (!parts_f16[i] || rows_per_part[i] == 0) return WR_HIP_ERR_INVAL;
+        n_out += rows_per_part[i];
+    }
+    if (n_out % 16 != 0 || n_out > 0x7FFFFFFFu) return WR_HIP_ERR_INVAL;
+    wr_hip_weight* w = new (std::nothrow) wr_hip_weight();
+    if (!w) return WR_HIP_ERR_NOMEM;
+    w->n_out = (uint32_t)n_out;
+    w->n_in = n_in;
+    w->bytes = (size_t)n_out * n_in * 2;
+    w->tiles = nullptr;
+
+    Locked lk;
+    void* rowmajor = nullptr;
+    hipError_t e = hipMalloc(&w->tiles, w->bytes);
+    if (e == hipSuccess) e = hipMalloc(&rowmajor, w->bytes);
+    if (e != hipSuccess) {
+        logmsg(0, "projection: device weight alloc failed (%zu bytes): %s", w->bytes,
+               hipGetErrorString(e));
+        if (w->tiles) (void)hipFree(w->tiles);
+        delete w;
+        return WR_HIP_ERR_NOMEM;
+    }
+    size_t off = 0;
+    for (uint32_t i = 0; i < n_parts && e == hipSuccess; i++) {
+        const size_t nb = (size_t)rows_per_part[i] * n_in * 2;
+        e = hipMemcpyAsync((uint8_t*)rowmajor + off, parts_f16[i], nb, hipMemcpyHostToDevice, g.stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(g.stream);     // pageable source
+        off += nb;
+    }
+    if (e == hipSuccess) {
+        const size_t units = w->bytes / 16;
+        hipLaunchKernelGGL(proj_pack_weights_kernel, dim3((uint32_t)((units + 255) / 256)), dim3(256),
+                           0, g.stream, reinterpret_cast<const uint16_t*>(rowmajor),
+                           reinterpret_cast<u32x4*>(w->tiles), w->n_out, w->n_in);
+        e = hipGetLastError();
+        if (e == hipSuccess) e = hipStreamSynchronize(g.stream);
+    }
+    (void)hipFree(rowmajor);
+    if (e != hipSuccess) {
+        (void)hipFree(w->tiles);
+        delete w;
+        return hip_fail(e, "weight upload", 0);
+    }
+    *out = w;
+    return WR_HIP_OK;
+}
+
+void wr_hip_proj_weight_destroy(wr_hip_weight* w)
+{
+    if (!w) return;
+    if (g.inited) {
+        Locked lk;
+        (void)hipStreamSynchronize(g.stream);
+        (void)hipFree(w->tiles);
+    }
+    delete w;
+}
+
+static int check_proj(const wr_hip_weight* w, uint32_t rows, const void* x, uint32_t ldx,
+                      const void* y, uint32_t ldy)
+{
+    if (!g.inited) return WR_HIP_ERR_STATE;
+    if (!w || !x || !y) return WR_HIP_ERR_INVAL;
+    if (rows == 0) return WR_HIP_OK;
+    if (ldx < w->n_in || ldy < w->n_out || ldy % 4 != 0) return WR_HIP_ERR_INVAL;
+    return WR_HIP_OK;
+}
+
+int wr_hip_proj_rows_dev(const wr_hip_weight* w, uint32_t rows, const float* x_dev, uint32_t ldx,
+                         const float* add_dev, float* y_dev, uint32_t ldy)
+{
+    int rc = check_proj(w, rows, x_dev, ldx, y_dev, ldy);
+    if (rc || rows == 0) return rc;
+    if (((uintptr_t)y_dev & 15) || (add_dev && ((uintptr_t)add_dev & 15))) return WR_HIP_ERR_INVAL;
+    Locked lk;
+    return proj_locked(w, rows, x_dev, ldx, add_dev, y_dev, ldy);
+}
+
+int wr_hip_proj_rows(const wr_hip_weight* w, uint32_t rows, const float* x, float* y)
+{
+    if (w && (w->n_out % 4 != 0)) return WR_HIP_ERR_INVAL;
+    int rc = check_proj(w, rows, x, w ? w->n_in : 0, y, w ? w->n_out : 0);
+    if (rc || rows == 0) return rc;
+    const size_t xb = ((size_t)rows * w->n_in * sizeof(float) + 255) & ~(size_t)255;
+    const size_t yb = (size_t)rows * w->n_out * sizeof(float);
+    Locked lk;
+    rc = ensure_device(g.d_stage, xb + yb);
+    if (rc) return rc;
+    float* dx = reinterpret_cast<float*>(g.d_stage.p);
+    float* dy = reinterpret_cast<float*>((uint8_t*)g.d_stage.p + xb);
+    rc = copy_up(dx, x, (size_t)rows * w->n_in * sizeof(float), 0);
+    if (rc == WR_HIP_OK) rc = proj_locked(w, rows, dx, w->n_in, nullptr, dy, w->n_out);
+    if (rc == WR_HIP_OK) rc = copy_down_sync(y, dy, yb);
+    return rc;
+}
+
+uint32_t wr_hip_proj_weight_rows(const wr_hip_weight* w) { return w ? w->n_out : 0; }
+uint32_t wr_hip_proj_weight_cols(const wr_hip_weight* w) { return w ? w->n_in : 0; }
 
 int wr_hip_attn_profile_begin(uint32_t max_launches)
 {

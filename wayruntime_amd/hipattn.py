@@ -64,6 +64,13 @@ def load() -> C.CDLL:
                                                      _vp, _vp, _u32, C.c_float, _u32]),
         "wr_hip_attn_prefill_dev": (C.c_int, [_vp, _u32, _u32, _u32, _vp, _vp, _u32, C.c_float,
                                               _u32]),
+        "wr_hip_proj_weight_create": (C.c_int, [_u32, C.POINTER(_vp), C.POINTER(_u32), _u32,
+                                                C.POINTER(_vp)]),
+        "wr_hip_proj_weight_destroy": (None, [_vp]),
+        "wr_hip_proj_weight_rows": (_u32, [_vp]),
+        "wr_hip_proj_weight_cols": (_u32, [_vp]),
+        "wr_hip_proj_rows": (C.c_int, [_vp, _u32, _vp, _vp]),
+        "wr_hip_proj_rows_dev": (C.c_int, [_vp, _u32, _vp, _u32, _vp, _vp, _u32]),
         "wr_hip_attn_set_tuning": (None, [_u32, C.c_int]),
         "wr_hip_attn_profile_begin": (C.c_int, [_u32]),
         "wr_hip_attn_profile_end": (C.c_int, [C.POINTER(C.c_double), C.POINTER(_u32)]),
@@ -270,6 +277,41 @@ def append_dev(cache: KVCache, layer: int, pos: int, n_rows: int, k_dev: DeviceB
 def rope_dev(x_dev: DeviceBuffer, cos_sin_dev: DeviceBuffer, rows: int, heads: int, hd: int,
              n_rot: int) -> None:
     _check(lib().wr_hip_attn_rope_dev(x_dev.p, cos_sin_dev.p, rows, heads, hd, n_rot), "rope_dev")
+
+
+class Weight:
+    """A projection weight on the device (wr_hip_weight): row blocks of F16 bit
+    patterns [rows_i, n_in], stacked in order."""
+
+    def __init__(self, parts):
+        init()
+        parts = [np.ascontiguousarray(p, dtype=np.uint16) for p in parts]
+        n_in = parts[0].shape[1]
+        assert all(p.ndim == 2 and p.shape[1] == n_in for p in parts)
+        ptrs = (_vp * len(parts))(*[_ptr(p) for p in parts])
+        rows = (_u32 * len(parts))(*[p.shape[0] for p in parts])
+        self.h = _vp()
+        _check(lib().wr_hip_proj_weight_create(len(parts), ptrs, rows, n_in, C.byref(self.h)),
+               "proj_weight_create")
+        self.n_out = int(lib().wr_hip_proj_weight_rows(self.h))
+        self.n_in = int(lib().wr_hip_proj_weight_cols(self.h))
+
+    def rows(self, x: np.ndarray) -> np.ndarray:
+        """y = x . W^T for host F32 rows [R, n_in]."""
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        y = np.empty((x.shape[0], self.n_out), dtype=np.float32)
+        _check(lib().wr_hip_proj_rows(self.h, x.shape[0], _ptr(x), _ptr(y)), "proj_rows")
+        return y
+
+    def rows_dev(self, rows: int, x_dev, ldx: int, y_dev, ldy: int, add_dev=None) -> None:
+        _check(lib().wr_hip_proj_rows_dev(self.h, rows, x_dev.p, ldx,
+                                          add_dev.p if add_dev is not None else None, y_dev.p, ldy),
+               "proj_rows_dev")
+
+    def close(self) -> None:
+        if self.h:
+            lib().wr_hip_proj_weight_destroy(self.h)
+            self.h = _vp()
 
 
 def sync() -> None:
