@@ -119,101 +119,162 @@ struct ProjArgs {
     const half8* w;          // tile order
     const half8* xfrag;      // [groups][K/32][64]
     const float* scales;     // [R]
-    const float* bias_rows;  // optional [R][N] added to the result (residual), or nullptr
+    const float* bias_rows;  // optional [R][ldy] added to the result (residual), or nullptr
     float* y;                // [R][ldy]
     uint32_t N, K, R, ldy;
-    uint32_t groups;         // ceil(R / 8)
+    uint32_t ksplit;         // waves of a workgroup that share one run of outputs: 1, 2 or 4
 };
 
-// GROUPS = row groups of eight handled per launch (template so the accumulators
-// stay in registers): 1, 2, 4, ... 32.
-template <int GROUPS>
+// One wave-step: NT weight tiles against GROUPS operand fragments.
+template <int GROUPS, int NT>
+__device__ __forceinline__ void proj_step(f32x4 (&acc)[NT][GROUPS], const half8 (&wv)[NT],
+                                          const half8* __restrict__ xp, uint32_t ktiles, uint32_t kt)
+{
+#pragma unroll
+    for (int gi = 0; gi < GROUPS; gi++) {
+        const half8 xb = xp[((size_t)gi * ktiles + kt) * 64];
+#pragma unroll
+        for (int t = 0; t < NT; t++)
+            acc[t][gi] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wv[t], xb, acc[t][gi], 0, 0, 0);
+    }
+}
+
+// GROUPS = row groups of eight handled per launch, NT = 16-output tiles per
+// wave (templates, so the accumulators stay in registers).  A workgroup is four
+// waves.  With ksplit = 1 they own four consecutive runs of 16*NT outputs; with
+// ksplit = 2 or 4 that many waves share a run and take contiguous parts of the
+// input range (a narrow weight then still puts a thousand waves on the chip),
+// and their sums are added through LDS in part order, so the result does not
+// depend on timing.  Every X fragment a wave loads serves NT weight tiles:
+// with two row groups (9..16 rows) NT = 2 keeps the operand traffic through
+// the vector cache at the two bytes per weight byte of the one-group case.
+template <int GROUPS, int NT>
 __global__ __launch_bounds__(kProjThreads) void proj_rows_kernel(const ProjArgs a)
 {
+    constexpr int KB = (NT == 1) ? kProjKBatch : kProjKBatch / 2;      // k-steps per register batch
+    // partial sums of the waves with part > 0: (4 / S) runs x (S - 1) parts <= 3 entries
+    __shared__ f32x4 s_part[(GROUPS <= 2) ? 3 * NT * GROUPS * 64 : 1];
+
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const uint32_t nt = blockIdx.x * 4 + wave;                  // this wave's 16 outputs
-    if (nt * 16 >= a.N) return;
+    const uint32_t S = a.ksplit;
+    const uint32_t slot = wave / S, part = wave % S;
+    const uint32_t run = blockIdx.x * (4 / S) + slot;            // this wave's run of 16*NT outputs
+    const uint32_t nt0 = run * NT;
+    const uint32_t ntiles = a.N / 16;
+    const bool live = nt0 < ntiles;                              // N/16 need not be a multiple of the runs per block
     const uint32_t ktiles = a.K / 32;
-    const half8* wp = a.w + (size_t)nt * ktiles * 64 + lane;
+    const uint32_t kper = ktiles / S;                            // host guarantees divisibility
+    const uint32_t k_begin = part * kper, k_end = k_begin + kper;
     const half8* xp = a.xfrag + lane;
 
-    f32x4 acc[GROUPS];
+    f32x4 acc[NT][GROUPS];
 #pragma unroll
-    for (int gi = 0; gi < GROUPS; gi++) acc[gi] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < NT; t++)
+#pragma unroll
+        for (int gi = 0; gi < GROUPS; gi++) acc[t][gi] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    // W is read exactly once per launch (non-temporal); X fragments are shared
-    // by every wave of the grid and stay cached.
-    half8 wa[kProjKBatch], wb[kProjKBatch];
-    uint32_t kt = 0;
-    const uint32_t full = ktiles / kProjKBatch * kProjKBatch;
-    if (full > 0) {
+    if (live) {
+        // tile t of this wave; a run that sticks out past N re-reads the last tile and drops the result
+        const half8* wp[NT];
 #pragma unroll
-        for (int u = 0; u < kProjKBatch; u++) wa[u] = __builtin_nontemporal_load(&wp[(size_t)u * 64]);
+        for (int t = 0; t < NT; t++) {
+            const uint32_t nt = (nt0 + t < ntiles) ? nt0 + t : ntiles - 1;
+            wp[t] = a.w + (size_t)nt * ktiles * 64 + lane;
+        }
+        // W is read exactly once per launch (non-temporal); X fragments are
+        // shared by every wave of the grid and stay cached.  Loads inside the
+        // loop are unconditional and the last batch is peeled, so the
+        // compiler's load counting keeps the prefetched batch in flight.
+        half8 wa[KB][NT], wb[KB][NT];
+        uint32_t kt = k_begin;
+        const uint32_t full_end = k_begin + kper / KB * KB;
+        if (kt < full_end) {
+#pragma unroll
+            for (int u = 0; u < KB; u++)
+#pragma unroll
+                for (int t = 0; t < NT; t++)
+                    wa[u][t] = __builtin_nontemporal_load(&wp[t][(size_t)(kt + u) * 64]);
+            while (kt + 2 * KB <= full_end) {
+#pragma unroll
+                for (int u = 0; u < KB; u++)
+#pragma unroll
+                    for (int t = 0; t < NT; t++)
+                        wb[u][t] = __builtin_nontemporal_load(&wp[t][(size_t)(kt + KB + u) * 64]);
+#pragma unroll
+                for (int u = 0; u < KB; u++) proj_step<GROUPS, NT>(acc, wa[u], xp, ktiles, kt + u);
+#pragma unroll
+                for (int u = 0; u < KB; u++)
+#pragma unroll
+                    for (int t = 0; t < NT; t++) wa[u][t] = wb[u][t];
+                kt += KB;
+            }
+#pragma unroll
+            for (int u = 0; u < KB; u++) proj_step<GROUPS, NT>(acc, wa[u], xp, ktiles, kt + u);
+            kt += KB;
+        }
+        for (; kt < k_end; kt++) {                               // part not a multiple of the batch
+            half8 wv[NT];
+#pragma unroll
+            for (int t = 0; t < NT; t++) wv[t] = __builtin_nontemporal_load(&wp[t][(size_t)kt * 64]);
+            proj_step<GROUPS, NT>(acc, wv, xp, ktiles, kt);
+        }
     }
-    // Loads in the loop are unconditional and the last batch is peeled, so the
-    // compiler's load counting keeps the prefetched batch in flight.
-    while (kt + 2 * kProjKBatch <= full) {
+
+    if constexpr (GROUPS <= 2) {
+        if (S > 1) {                                             // uniform over the workgroup
+            if (part > 0) {
 #pragma unroll
-        for (int u = 0; u < kProjKBatch; u++)
-            wb[u] = __builtin_nontemporal_load(&wp[(size_t)(kt + kProjKBatch + u) * 64]);
+                for (int t = 0; t < NT; t++)
 #pragma unroll
-        for (int u = 0; u < kProjKBatch; u++) {
+                    for (int gi = 0; gi < GROUPS; gi++)
+                        s_part[(((slot * (S - 1) + (part - 1)) * NT + t) * GROUPS + gi) * 64 + lane] = acc[t][gi];
+            }
+            __syncthreads();
+            if (part > 0) return;
+            for (uint32_t p = 1; p < S; p++) {
 #pragma unroll
-            for (int gi = 0; gi < GROUPS; gi++) {
-                const half8 xb = xp[((size_t)gi * ktiles + kt + u) * 64];
-                acc[gi] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wa[u], xb, acc[gi], 0, 0, 0);
+                for (int t = 0; t < NT; t++)
+#pragma unroll
+                    for (int gi = 0; gi < GROUPS; gi++) {
+                        const f32x4 o = s_part[(((slot * (S - 1) + (p - 1)) * NT + t) * GROUPS + gi) * 64 + lane];
+#pragma unroll
+                        for (int i = 0; i < 4; i++) acc[t][gi][i] += o[i];
+                    }
             }
         }
-#pragma unroll
-        for (int u = 0; u < kProjKBatch; u++) wa[u] = wb[u];
-        kt += kProjKBatch;
     }
-    if (kt + kProjKBatch <= full) {
-#pragma unroll
-        for (int u = 0; u < kProjKBatch; u++) {
-#pragma unroll
-            for (int gi = 0; gi < GROUPS; gi++) {
-                const half8 xb = xp[((size_t)gi * ktiles + kt + u) * 64];
-                acc[gi] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wa[u], xb, acc[gi], 0, 0, 0);
-            }
-        }
-        kt += kProjKBatch;
-    }
-    for (; kt < ktiles; kt++) {                              // K/32 not a multiple of the batch
-        const half8 wv = __builtin_nontemporal_load(&wp[(size_t)kt * 64]);
-#pragma unroll
-        for (int gi = 0; gi < GROUPS; gi++) {
-            const half8 xb = xp[((size_t)gi * ktiles + kt) * 64];
-            acc[gi] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wv, xb, acc[gi], 0, 0, 0);
-        }
-    }
+    if (!live) return;
 
     // Accumulator layout: lane 16g + c holds outputs 16nt + 4g .. +3 of column c.
     // Column c (< 8) is the hi term of row c, column c + 8 its lo term.
     const int c = lane & 15, g = lane >> 4;
     const int partner_addr = (lane ^ 8) * 4;
 #pragma unroll
-    for (int gi = 0; gi < GROUPS; gi++) {
-        f32x4 v = acc[gi];
+    for (int t = 0; t < NT; t++) {
+        const uint32_t nt = nt0 + t;
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const float other =
-                __int_as_float(__builtin_amdgcn_ds_bpermute(partner_addr, __float_as_int(v[i])));
-            v[i] += other * (1.0f / kProjLoScale);      // meaningful in the hi columns only
-        }
-        const uint32_t row = gi * 8 + (c & 7);
-        if (c < 8 && row < a.R) {
-            const float sc = a.scales[row];
-            const size_t o = (size_t)row * a.ldy + nt * 16 + g * 4;
-            f32x4 r;
+        for (int gi = 0; gi < GROUPS; gi++) {
+            f32x4 v = acc[t][gi];
 #pragma unroll
-            for (int i = 0; i < 4; i++) r[i] = v[i] * sc;
-            if (a.bias_rows) {
-                const f32x4 b = *reinterpret_cast<const f32x4*>(a.bias_rows + o);
-#pragma unroll
-                for (int i = 0; i < 4; i++) r[i] += b[i];
+            for (int i = 0; i < 4; i++) {
+                const float other =
+                    __int_as_float(__builtin_amdgcn_ds_bpermute(partner_addr, __float_as_int(v[i])));
+                v[i] += other * (1.0f / kProjLoScale);      // meaningful in the hi columns only
             }
-            *reinterpret_cast<f32x4*>(a.y + o) = r;
+            const uint32_t row = gi * 8 + (c & 7);
+            if (c < 8 && row < a.R && nt < ntiles) {
+                const float sc = a.scales[row];
+                const size_t o = (size_t)row * a.ldy + nt * 16 + g * 4;
+                f32x4 r;
+#pragma unroll
+                for (int i = 0; i < 4; i++) r[i] = v[i] * sc;
+                if (a.bias_rows) {
+                    const f32x4 b = *reinterpret_cast<const f32x4*>(a.bias_rows + o);
+#pragma unroll
+                    for (int i = 0; i < 4; i++) r[i] += b[i];
+                }
+                *reinterpret_cast<f32x4*>(a.y + o) = r;
+            }
         }
     }
 }

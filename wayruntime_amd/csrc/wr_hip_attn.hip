@@ -434,10 +434,13 @@ struct Locked {
 // projections: launch helpers (caller holds g.mu)
 namespace {
 
-template <int GROUPS>
+template <int GROUPS, int NT>
 void launch_proj(const ProjArgs& a)
 {
-    launch_main(proj_rows_kernel<GROUPS>, dim3((a.N / 16 + 3) / 4), dim3(kProjThreads), a);
+    const uint32_t runs = (a.N / 16 + NT - 1) / NT;              // runs of 16*NT outputs
+    const uint32_t per_block = 4 / a.ksplit;
+    launch_main(proj_rows_kernel<GROUPS, NT>, dim3((runs + per_block - 1) / per_block),
+                dim3(kProjThreads), a);
 }
 
 // y_dev[rows][ldy] = x_dev[rows][ldx] . W^T (+ add_dev), rows <= kProjMaxRows.
@@ -467,14 +470,27 @@ int proj_chunk_locked(const wr_hip_weight* w, uint32_t rows, const float* x_dev,
     a.K = w->n_in;
     a.R = rows;
     a.ldy = ldy;
-    a.groups = groups;
+    // Waves that share a run of outputs (contiguous parts of the inputs, summed
+    // through LDS in a fixed order): enough that a narrow weight still gives
+    // about a thousand waves.  A function of the weight's shape and the row
+    // group count only, so a projection's arithmetic never depends on what
+    // else is in flight.
+    const uint32_t nt_per_wave = (groups == 2) ? 2 : 1;
+    const uint32_t runs = (w->n_out / 16 + nt_per_wave - 1) / nt_per_wave;
+    uint32_t ksplit = 1;
+    if (groups <= 2) {
+        while (ksplit < 4 && runs * ksplit < 1024 && ktiles % (ksplit * 2) == 0 &&
+               ktiles / (ksplit * 2) >= 4)
+            ksplit *= 2;
+    }
+    a.ksplit = ksplit;
     switch (groups) {
-    case 1: launch_proj<1>(a); break;
-    case 2: launch_proj<2>(a); break;
-    case 4: launch_proj<4>(a); break;
-    case 8: launch_proj<8>(a); break;
-    case 16: launch_proj<16>(a); break;
-    default: launch_proj<32>(a); break;
+    case 1: launch_proj<1, 1>(a); break;
+    case 2: launch_proj<2, 2>(a); break;
+    case 4: launch_proj<4, 1>(a); break;
+    case 8: launch_proj<8, 1>(a); break;
+    case 16: launch_proj<16, 1>(a); break;
+    default: launch_proj<32, 1>(a); break;
     }
     HIP_TRY(hipGetLastError(), "projection launch", 0);
     return WR_HIP_OK;
