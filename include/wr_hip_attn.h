@@ -217,6 +217,38 @@ int wr_hip_proj_rows_dev(const wr_hip_weight *w, uint32_t rows,
                          const float *x_dev, uint32_t ldx,
                          const float *add_dev, float *y_dev, uint32_t ldy);
 
+/* ---- row steps between the projections and the attention path --------------
+ * For callers that keep a layer's activations on the device.  All arguments
+ * are device pointers (wr_hip_attn_dev_alloc), all calls are asynchronous on
+ * the library stream.  Sums over a row are tree reductions here and
+ * sequential loops in the reference, so results agree to F32 rounding.
+ *
+ * rmsnorm: out[r][j] = x[r][j] / sqrt(mean_j x[r][j]^2 + eps) * w[j % wn], or
+ * without weight when wn == 0 (wri_op_rmsnorm, src/core/kernels.c:1276-1316;
+ * called at src/core/session.c:443, 509, 538). */
+int wr_hip_rows_rmsnorm_dev(const float *x_dev, uint32_t ldx, const float *w_dev,
+                            uint32_t wn, float *out_dev, uint32_t ldo,
+                            uint32_t rows, uint32_t dim, float eps);
+
+/* qkv_prep: rows of a stacked projection [nq heads | nkv K heads | nkv V heads]
+ * (row stride ld) are split into Q [rows, nq, hd], K and V [rows, nkv, hd].
+ * Q and K heads get the per-head RMSNorm when q_norm_dev / k_norm_dev ([hd],
+ * both or neither) are given (Qwen3, src/core/session.c:459-470), then the
+ * rotary embedding with the caller's table cos_sin_dev [rows, n_rot, 2]
+ * (split-half pairing, src/core/kernels.c:1356-1412, called at
+ * session.c:473-480); V is copied.  hd must be even and <= 1024. */
+int wr_hip_rows_qkv_prep_dev(const float *qkv_dev, uint32_t ld, uint32_t rows,
+                             uint32_t nq, uint32_t nkv, uint32_t hd,
+                             const float *q_norm_dev, const float *k_norm_dev,
+                             float eps, const float *cos_sin_dev, uint32_t n_rot,
+                             float *q_out_dev, float *k_out_dev, float *v_out_dev);
+
+/* swiglu: act[r][j] = silu(gu[r][j]) * gu[r][ffn + j] for rows of a stacked
+ * gate/up projection (wri_op_fused_silu_mul, src/core/kernels.c:1243-1258 with
+ * silu at :963-967; called at session.c:523-526). */
+int wr_hip_rows_swiglu_dev(const float *gate_up_dev, uint32_t ld, float *act_dev,
+                           uint32_t ldo, uint32_t rows, uint32_t ffn);
+
 /* Tuning knobs for measurement (0 = automatic): keys handled per workgroup in
  * the split-K decode kernel, and a switch forcing the generic (non-MFMA)
  * kernels.  Not needed by a normal caller. */

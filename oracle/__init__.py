@@ -101,6 +101,7 @@ def _load_oracle() -> C.CDLL:
     lib.wro_rope_table.argtypes = [_f32p] + [C.c_uint32] * 3 + [C.c_float, C.c_uint32]
     lib.wro_rope_table.restype = C.c_int
     lib.wro_matmul_w16.argtypes = [_f32p, _u16p, _f32p] + [C.c_uint32] * 3
+    lib.wro_silu_mul.argtypes = [_f32p, _f32p, _f32p, C.c_uint64]
     lib.wro_rmsnorm.argtypes = [_f32p, C.c_void_p, C.c_uint32, _f32p, C.c_uint32, C.c_uint32,
                                 C.c_float]
     return lib
@@ -219,6 +220,16 @@ def matmul_w16(x: np.ndarray, w16: np.ndarray) -> np.ndarray:
     if rc != 0:
         raise ValueError(rc)
     return y
+
+
+def silu_mul(g: np.ndarray, u: np.ndarray) -> np.ndarray:
+    g = np.ascontiguousarray(g, dtype=np.float32)
+    u = np.ascontiguousarray(u, dtype=np.float32)
+    out = np.empty_like(g)
+    rc = lib().wro_silu_mul(g.reshape(-1), u.reshape(-1), out.reshape(-1), g.size)
+    if rc != 0:
+        raise ValueError(rc)
+    return out
 
 
 def rmsnorm(x: np.ndarray, w, eps: float) -> np.ndarray:

@@ -547,3 +547,16 @@ int wro_rmsnorm(const float *x, const float *w, uint32_t wn, float *out,
     }
     return WRO_OK;
 }
+
+/* Gated activation, src/core/kernels.c:1243-1258 with silu at :963-967:
+ * out[i] = (g[i] * (1 / (1 + exp(-g[i])))) * u[i], exp being the polynomial. */
+int wro_silu_mul(const float *g, const float *u, float *out, uint64_t n)
+{
+    if (!g || !u || !out) return WRO_ERR_INVAL;
+    for (uint64_t i = 0; i < n; i++) {
+        const float a = g[i];
+        const float sig = 1.0f / (1.0f + wro_exp(-a));
+        out[i] = (a * sig) * u[i];
+    }
+    return WRO_OK;
+}

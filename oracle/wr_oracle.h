@@ -150,6 +150,9 @@ int wro_matmul_w16(const float *a, const uint16_t *w_f16, float *c, uint32_t M,
 int wro_rmsnorm(const float *x, const float *w, uint32_t wn, float *out,
                 uint32_t rows, uint32_t dim, float eps);
 
+/* src/core/kernels.c:1243-1258, 963-967 */
+int wro_silu_mul(const float *g, const float *u, float *out, uint64_t n);
+
 #ifdef __cplusplus
 }
 #endif

@@ -135,3 +135,11 @@ def matmul_inputs(case):
     x = synth.hash_bell(base + 1, (rows, n_in))
     w16 = synth.f32_to_f16_trunc(synth.hash_bell(base + 2, (n_out, n_in)) * np.float32(wstd))
     return x, w16
+
+
+def silu_inputs():
+    """Gate values over the whole useful range (incl. the exp clamp at -88) and up values."""
+    g = np.concatenate([np.linspace(-100.0, 100.0, 2001, dtype=np.float32),
+                        synth.hash_bell(777, (2047,)) * np.float32(4.0)])
+    u = synth.hash_bell(778, (g.size,))
+    return np.ascontiguousarray(g), np.ascontiguousarray(u)

@@ -100,6 +100,12 @@ def main() -> None:
         rc = ref.wri_op_matmul(C.byref(ta), C.byref(tb), C.byref(tc))
         assert rc == 0, (name, rc)
         ops["matmul_" + name] = y
+    ref.wri_op_fused_silu_mul.argtypes = [C.POINTER(oracle.Tensor)] * 3
+    g, u = cases.silu_inputs()
+    y = np.empty_like(g)
+    tg, tu, ty = oracle.wrap(g), oracle.wrap(u), oracle.wrap(y)
+    assert ref.wri_op_fused_silu_mul(C.byref(tg), C.byref(tu), C.byref(ty)) == 0
+    ops["silu_mul"] = y
     ops["matmul_variant"] = np.array([ref.wri_simd_matmul_variant()], dtype=np.int32)
     np.savez(os.path.join(HERE, "ops_golden.npz"), **ops)
 

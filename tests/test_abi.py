@@ -14,7 +14,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 def _declared(header):
     text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(wr_hip_(?:attn|proj)_\w+)\s*\(", text)))
+    return sorted(set(re.findall(r"\b(wr_hip_(?:attn|proj|rows)_\w+)\s*\(", text)))
 
 
 def test_library_exports_every_declared_symbol():

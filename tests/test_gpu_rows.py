@@ -1,0 +1,127 @@
+"""Row steps on the device (RMSNorm, Q/K/V split with per-head norm and rotary
+embedding, gated activation) against the CPU oracle, through the C ABI.
+
+Sums over a row are tree reductions on the device and sequential loops in the
+reference, and the device's exp is not the reference's polynomial, so these
+agree to F32 rounding: |got - want| <= 4e-6 * max|want| per call (the largest
+term is the polynomial exp's own 2e-6).  Where no sum or exp is involved
+(rotation without the norm, the V copy) the bits are equal."""
+import numpy as np
+import pytest
+
+import oracle
+from wayruntime_amd import hipattn, synth
+
+pytestmark = pytest.mark.gpu
+
+TOL = 4e-6
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _device():
+    hipattn.init()
+    yield
+
+
+def _dev(a):
+    return hipattn.DeviceBuffer.from_host(np.ascontiguousarray(a, dtype=np.float32))
+
+
+def _close(got, want):
+    assert not np.isnan(got).any()
+    assert np.max(np.abs(got.astype(np.float64) - want)) <= TOL * np.max(np.abs(want))
+
+
+@pytest.mark.parametrize("rows,dim,wn,eps", [(3, 1024, 1024, 1e-6), (16, 4096, 4096, 1e-5),
+                                             (1, 96, 0, 1e-6), (2, 300, 4, 1e-6)])
+def test_rmsnorm_rows(rows, dim, wn, eps):
+    print("rmsnorm", rows, dim, wn, flush=True)
+    ldx, ldo = dim + 8, dim + 4
+    x = synth.normal(dim + rows, (rows, ldx), std=2.0)
+    w = synth.normal(dim, (wn,)) + np.float32(1.0) if wn else None
+    xd, od = _dev(x), _dev(np.full((rows, ldo), 9.0))
+    wd = _dev(w) if wn else None
+    rc = hipattn.lib().wr_hip_rows_rmsnorm_dev(xd.p, ldx, wd.p if wn else None, wn, od.p, ldo, rows,
+                                               dim, eps)
+    assert rc == hipattn.OK
+    hipattn.sync()
+    got = od.to_host((rows, ldo))
+    _close(got[:, :dim], oracle.rmsnorm(np.ascontiguousarray(x[:, :dim]), w, eps).astype(np.float64))
+    assert np.all(got[:, dim:] == 9.0)
+
+
+@pytest.mark.parametrize("rows,nq,nkv,hd,norm,theta,n_rot_pairs,pos", [
+    (1, 16, 8, 128, True, 1e6, 0, 77),          # Qwen3: per-head norm, full rotation
+    (5, 32, 8, 128, False, 5e5, 0, 4000),       # Llama: no norm
+    (3, 8, 4, 256, True, 1e6, 0, 0),
+    (2, 4, 2, 64, False, 1e4, 10, 9),           # partial rotation, pairs across lanes
+    (2, 2, 1, 32, True, 1e4, 0, 3),
+])
+def test_qkv_prep(rows, nq, nkv, hd, norm, theta, n_rot_pairs, pos):
+    print("qkv_prep", rows, nq, nkv, hd, norm, flush=True)
+    width = (nq + 2 * nkv) * hd
+    ld = width + 16
+    qkv = synth.normal(hd + rows, (rows, ld), std=1.5)
+    qn = synth.normal(1, (hd,)) * np.float32(0.1) + np.float32(1.0)
+    kn = synth.normal(2, (hd,)) * np.float32(0.1) + np.float32(1.0)
+    tab = oracle.rope_table(rows, hd, pos, theta, n_rot_pairs)
+    n_rot = tab.shape[1]
+    qd, kd = nq * hd, nkv * hd
+    bufs = [_dev(qkv), _dev(qn), _dev(kn), _dev(tab), _dev(np.zeros((rows, qd))),
+            _dev(np.zeros((rows, kd))), _dev(np.zeros((rows, kd)))]
+    xd, qnd, knd, td, qo, ko, vo = bufs
+    eps = 1e-6
+    rc = hipattn.lib().wr_hip_rows_qkv_prep_dev(xd.p, ld, rows, nq, nkv, hd,
+                                                qnd.p if norm else None, knd.p if norm else None,
+                                                eps, td.p, n_rot, qo.p, ko.p, vo.p)
+    assert rc == hipattn.OK
+    hipattn.sync()
+    q_in = np.ascontiguousarray(qkv[:, :qd]).reshape(rows, nq, hd)
+    k_in = np.ascontiguousarray(qkv[:, qd:qd + kd]).reshape(rows, nkv, hd)
+    v_in = np.ascontiguousarray(qkv[:, qd + kd:width]).reshape(rows, nkv, hd)
+    if norm:
+        q_in = oracle.rmsnorm(q_in, qn, eps)
+        k_in = oracle.rmsnorm(k_in, kn, eps)
+    want_q = oracle.rope(q_in, pos, theta, n_rot_pairs)
+    want_k = oracle.rope(k_in, pos, theta, n_rot_pairs)
+    got_q, got_k, got_v = qo.to_host((rows, nq, hd)), ko.to_host((rows, nkv, hd)), vo.to_host((rows, nkv, hd))
+    assert np.array_equal(got_v, v_in)
+    if norm:
+        _close(got_q, want_q.astype(np.float64))
+        _close(got_k, want_k.astype(np.float64))
+    else:
+        assert got_q.tobytes() == want_q.tobytes()
+        assert got_k.tobytes() == want_k.tobytes()
+    for b in bufs:
+        b.free()
+
+
+def test_swiglu_rows():
+    rows, ffn = 3, 3072
+    ld, ldo = 2 * ffn + 8, ffn + 4
+    gu = synth.normal(5, (rows, ld), std=3.0)
+    gu[0, :8] = [-100.0, -60.0, -20.0, 0.0, 20.0, 60.0, 80.0, 100.0]
+    gd, ad = _dev(gu), _dev(np.full((rows, ldo), 9.0))
+    assert hipattn.lib().wr_hip_rows_swiglu_dev(gd.p, ld, ad.p, ldo, rows, ffn) == hipattn.OK
+    hipattn.sync()
+    got = ad.to_host((rows, ldo))
+    want = oracle.silu_mul(np.ascontiguousarray(gu[:, :ffn]), np.ascontiguousarray(gu[:, ffn:2 * ffn]))
+    _close(got[:, :ffn], want.astype(np.float64))
+    assert np.all(got[:, ffn:] == 9.0)
+    gd.free()
+    ad.free()
+
+
+def test_error_contract():
+    lib = hipattn.lib()
+    d = _dev(np.zeros(4096))
+    assert lib.wr_hip_rows_rmsnorm_dev(None, 8, None, 0, d.p, 8, 1, 8, 1e-6) == hipattn.ERR_INVAL
+    assert lib.wr_hip_rows_rmsnorm_dev(d.p, 4, None, 0, d.p, 8, 1, 8, 1e-6) == hipattn.ERR_INVAL   # stride < dim
+    assert lib.wr_hip_rows_rmsnorm_dev(d.p, 8, None, 3, d.p, 8, 1, 8, 1e-6) == hipattn.ERR_INVAL   # weight missing
+    # odd head_dim, stride too small, one norm vector without the other, table missing
+    assert lib.wr_hip_rows_qkv_prep_dev(d.p, 64, 1, 1, 1, 7, None, None, 1e-6, d.p, 3, d.p, d.p, d.p) == hipattn.ERR_INVAL
+    assert lib.wr_hip_rows_qkv_prep_dev(d.p, 8, 1, 1, 1, 8, None, None, 1e-6, d.p, 4, d.p, d.p, d.p) == hipattn.ERR_INVAL
+    assert lib.wr_hip_rows_qkv_prep_dev(d.p, 24, 1, 1, 1, 8, d.p, None, 1e-6, d.p, 4, d.p, d.p, d.p) == hipattn.ERR_INVAL
+    assert lib.wr_hip_rows_qkv_prep_dev(d.p, 24, 1, 1, 1, 8, None, None, 1e-6, None, 4, d.p, d.p, d.p) == hipattn.ERR_INVAL
+    assert lib.wr_hip_rows_swiglu_dev(d.p, 8, d.p, 8, 1, 8) == hipattn.ERR_INVAL                    # stride < 2 ffn
+    d.free()

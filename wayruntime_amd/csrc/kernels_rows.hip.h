@@ -1,0 +1,125 @@
+// Row-wise steps around the attention path for callers that keep a layer's
+// activations on the device: RMS normalisation, the split of a stacked Q/K/V
+// projection into rotated Q, rotated K and V (per-head RMSNorm and rotary
+// embedding fused, the steps the reference runs between the projections and
+// the cache append, src/core/session.c:459-486), and the gated activation.
+// All are tiny byte-moving kernels; none is on the timed attention path.
+//
+// Arithmetic follows the reference's formulas (src/core/kernels.c:1276-1316
+// RMSNorm, :1356-1412 rotary, :963-967 SiLU); sums over a row are tree
+// reductions here, sequential there, so results agree to F32 rounding.
+#pragma once
+
+#include "common.hip.h"
+
+namespace wr {
+
+constexpr int kRowsMaxHd = 1024;      // largest head_dim (reference: WR_FLASH_D_MAX)
+
+__device__ __forceinline__ float wave_sum_f32(float v)
+{
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v += wave_xor_f32(v, off);
+    return v;
+}
+
+// out[r][j] = x[r][j] * (1 / sqrt(mean_j x^2 + eps)) * w[j % wn]   (wn == 0: no weight)
+// One workgroup of 256 threads per row.
+__global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const float* __restrict__ x, uint32_t ldx,
+                                                           const float* __restrict__ w, uint32_t wn,
+                                                           float* __restrict__ out, uint32_t ldo,
+                                                           uint32_t dim, float eps)
+{
+    __shared__ float s_sum[4];
+    const uint32_t r = blockIdx.x;
+    const float* xr = x + (size_t)r * ldx;
+    float ss = 0.f;
+    for (uint32_t j = threadIdx.x; j < dim; j += 256) {
+        const float v = xr[j];
+        ss += v * v;
+    }
+    ss = wave_sum_f32(ss);
+    if ((threadIdx.x & 63) == 0) s_sum[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    const float total = (s_sum[0] + s_sum[1]) + (s_sum[2] + s_sum[3]);
+    const float inv_rms = 1.0f / sqrtf(total / (float)dim + eps);
+    float* orow = out + (size_t)r * ldo;
+    for (uint32_t j = threadIdx.x; j < dim; j += 256) {
+        const float ww = wn ? w[j % wn] : 1.0f;
+        orow[j] = xr[j] * inv_rms * ww;
+    }
+}
+
+struct QkvPrepArgs {
+    const float* qkv;        // [rows][ld]: nq query heads, then nkv key heads, then nkv value heads
+    const float* q_norm;     // [hd] per-head RMSNorm weights, or nullptr for no Q/K norm
+    const float* k_norm;
+    const float* cos_sin;    // [rows][n_rot][2]
+    float* q_out;            // [rows][nq][hd]
+    float* k_out;            // [rows][nkv][hd]
+    float* v_out;            // [rows][nkv][hd]
+    uint32_t ld, nq, nkv, hd, n_rot;
+    float eps;
+};
+
+// grid = (rows, nq + 2 nkv), one wave per (row, head).  Q and K heads: optional
+// RMSNorm over the head, then the rotary embedding (split-half pairing, element
+// j with j + hd/2 for j < n_rot, products and sums rounded one by one as in
+// rope_rows_kernel); V heads are copied.
+__global__ __launch_bounds__(64) void qkv_prep_kernel(const QkvPrepArgs a)
+{
+#pragma clang fp contract(off)
+    __shared__ float s[kRowsMaxHd];
+    const uint32_t r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const uint32_t hd = a.hd, half = hd / 2;
+    const float* src = a.qkv + (size_t)r * a.ld + (size_t)h * hd;
+    if (h >= a.nq + a.nkv) {
+        float* dst = a.v_out + ((size_t)r * a.nkv + (h - a.nq - a.nkv)) * hd;
+        for (uint32_t j = lane; j < hd; j += 64) dst[j] = src[j];
+        return;
+    }
+    const bool is_q = h < a.nq;
+    const float* nw = is_q ? a.q_norm : a.k_norm;
+    float* dst = is_q ? a.q_out + ((size_t)r * a.nq + h) * hd
+                      : a.k_out + ((size_t)r * a.nkv + (h - a.nq)) * hd;
+    float ss = 0.f;
+    for (uint32_t j = lane; j < hd; j += 64) {
+        const float v = src[j];
+        s[j] = v;
+        ss += v * v;
+    }
+    if (nw) {
+        ss = wave_sum_f32(ss);
+        const float inv_rms = 1.0f / sqrtf(ss / (float)hd + a.eps);
+        for (uint32_t j = lane; j < hd; j += 64) s[j] = s[j] * inv_rms * nw[j];
+    }
+    __syncthreads();
+    const float* cs = a.cos_sin + (size_t)r * a.n_rot * 2;
+    for (uint32_t j = lane; j < half; j += 64) {
+        const float x0 = s[j], x1 = s[j + half];
+        if (j < a.n_rot) {
+            const float c = cs[2 * j], sn = cs[2 * j + 1];
+            const float a0 = x0 * c, b0 = x1 * sn, a1 = x0 * sn, b1 = x1 * c;
+            dst[j] = a0 - b0;
+            dst[j + half] = a1 + b1;
+        } else {
+            dst[j] = x0;
+            dst[j + half] = x1;
+        }
+    }
+}
+
+// act[r][j] = silu(gu[r][j]) * gu[r][ffn + j],  silu(x) = x / (1 + exp(-x))
+__global__ __launch_bounds__(256) void swiglu_rows_kernel(const float* __restrict__ gu, uint32_t ld,
+                                                          float* __restrict__ act, uint32_t ldo,
+                                                          uint32_t rows, uint32_t ffn)
+{
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (size_t)rows * ffn) return;
+    const uint32_t r = (uint32_t)(idx / ffn), j = (uint32_t)(idx % ffn);
+    const float g = gu[(size_t)r * ld + j], u = gu[(size_t)r * ld + ffn + j];
+    const float sig = 1.0f / (1.0f + expf(-g));
+    act[(size_t)r * ldo + j] = (g * sig) * u;
+}
+
+}  // namespace wr

@@ -23,6 +23,7 @@
 #include "kernels_decode.hip.h"
 #include "kernels_prefill.hip.h"
 #include "kernels_proj.hip.h"
+#include "kernels_rows.hip.h"
 
 using namespace wr;
 
@@ -1044,6 +1045,69 @@ int wr_hip_proj_rows(const wr_hip_weight* w, uint32_t rows, const float* x, floa
     if (rc == WR_HIP_OK) rc = proj_locked(w, rows, dx, w->n_in, nullptr, dy, w->n_out);
     if (rc == WR_HIP_OK) rc = copy_down_sync(y, dy, yb);
     return rc;
+}
+
+// ------------------------------------------------------------- row steps --
+
+int wr_hip_rows_rmsnorm_dev(const float* x_dev, uint32_t ldx, const float* w_dev, uint32_t wn,
+                            float* out_dev, uint32_t ldo, uint32_t rows, uint32_t dim, float eps)
+{
+    if (!g.inited) return WR_HIP_ERR_STATE;
+    if (!x_dev || !out_dev || dim == 0 || ldx < dim || ldo < dim) return WR_HIP_ERR_INVAL;
+    if (wn > 0 && !w_dev) return WR_HIP_ERR_INVAL;
+    if (rows == 0) return WR_HIP_OK;
+    Locked lk;
+    hipLaunchKernelGGL(rmsnorm_rows_kernel, dim3(rows), dim3(256), 0, g.stream, x_dev, ldx, w_dev, wn,
+                       out_dev, ldo, dim, eps);
+    HIP_TRY(hipGetLastError(), "rmsnorm launch", 0);
+    return WR_HIP_OK;
+}
+
+int wr_hip_rows_qkv_prep_dev(const float* qkv_dev, uint32_t ld, uint32_t rows, uint32_t nq,
+                             uint32_t nkv, uint32_t hd, const float* q_norm_dev,
+                             const float* k_norm_dev, float eps, const float* cos_sin_dev,
+                             uint32_t n_rot, float* q_out_dev, float* k_out_dev, float* v_out_dev)
+{
+    if (!g.inited) return WR_HIP_ERR_STATE;
+    if (!qkv_dev || !q_out_dev || !k_out_dev || !v_out_dev) return WR_HIP_ERR_INVAL;
+    if (nq == 0 || nkv == 0 || hd < 2 || (hd & 1) || hd > (uint32_t)kRowsMaxHd) return WR_HIP_ERR_INVAL;
+    if ((uint64_t)ld < (uint64_t)(nq + 2 * nkv) * hd) return WR_HIP_ERR_INVAL;
+    if (n_rot > hd / 2 || (n_rot > 0 && !cos_sin_dev)) return WR_HIP_ERR_INVAL;
+    if ((q_norm_dev == nullptr) != (k_norm_dev == nullptr)) return WR_HIP_ERR_INVAL;
+    if (rows == 0) return WR_HIP_OK;
+    QkvPrepArgs a;
+    a.qkv = qkv_dev;
+    a.q_norm = q_norm_dev;
+    a.k_norm = k_norm_dev;
+    a.cos_sin = cos_sin_dev;
+    a.q_out = q_out_dev;
+    a.k_out = k_out_dev;
+    a.v_out = v_out_dev;
+    a.ld = ld;
+    a.nq = nq;
+    a.nkv = nkv;
+    a.hd = hd;
+    a.n_rot = n_rot;
+    a.eps = eps;
+    Locked lk;
+    hipLaunchKernelGGL(qkv_prep_kernel, dim3(rows, nq + 2 * nkv), dim3(64), 0, g.stream, a);
+    HIP_TRY(hipGetLastError(), "qkv prep launch", 0);
+    return WR_HIP_OK;
+}
+
+int wr_hip_rows_swiglu_dev(const float* gate_up_dev, uint32_t ld, float* act_dev, uint32_t ldo,
+                           uint32_t rows, uint32_t ffn)
+{
+    if (!g.inited) return WR_HIP_ERR_STATE;
+    if (!gate_up_dev || !act_dev || ffn == 0 || (uint64_t)ld < 2ull * ffn || ldo < ffn)
+        return WR_HIP_ERR_INVAL;
+    if (rows == 0) return WR_HIP_OK;
+    Locked lk;
+    const size_t total = (size_t)rows * ffn;
+    hipLaunchKernelGGL(swiglu_rows_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0,
+                       g.stream, gate_up_dev, ld, act_dev, ldo, rows, ffn);
+    HIP_TRY(hipGetLastError(), "swiglu launch", 0);
+    return WR_HIP_OK;
 }
 
 uint32_t wr_hip_proj_weight_rows(const wr_hip_weight* w) { return w ? w->n_out : 0; }
