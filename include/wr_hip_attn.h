@@ -184,6 +184,12 @@ int wr_hip_attn_prefill_dev(wr_hip_kv *kv, uint32_t layer, uint32_t p0,
                             uint32_t nq, float scale_override,
                             uint32_t window);
 
+/* What this build of the library offers beyond the attention path proper
+ * (bit mask).  A caller that wants the projections and row steps below on the
+ * device checks WR_HIP_CAP_PROJ first and otherwise keeps them on the host. */
+#define WR_HIP_CAP_PROJ 1u
+uint32_t wr_hip_attn_caps(void);
+
 /* ---- projections ---------------------------------------------------------
  * The matrix products either side of the attention path, for callers that want
  * Q/K/V made and the output projected where the cache lives: replaces

@@ -211,3 +211,68 @@ int wr_hip_attn_prefill(wr_hip_kv *kv, uint32_t layer, uint32_t p0, uint32_t T, 
     g_calls += T;
     return WR_HIP_OK;
 }
+
+/* ---- not offered by the test double -----------------------------------------
+ * The host engine asks wr_hip_attn_caps() before it uses any of these and keeps
+ * its own CPU walk when the answer is 0; they exist so the engine links. */
+uint32_t wr_hip_attn_caps(void) { return 0; }
+void *wr_hip_attn_dev_alloc(size_t bytes) { (void)bytes; return NULL; }
+void wr_hip_attn_dev_free(void *p) { (void)p; }
+int wr_hip_attn_h2d(void *d, const void *s, size_t n) { (void)d; (void)s; (void)n; return WR_HIP_ERR_STATE; }
+int wr_hip_attn_d2h(void *d, const void *s, size_t n) { (void)d; (void)s; (void)n; return WR_HIP_ERR_STATE; }
+int wr_hip_attn_sync(void) { return WR_HIP_ERR_STATE; }
+int wr_hip_attn_append_dev(wr_hip_kv *kv, uint32_t layer, uint32_t pos, uint32_t n_rows,
+                           const float *k, const float *v)
+{
+    (void)kv; (void)layer; (void)pos; (void)n_rows; (void)k; (void)v;
+    return WR_HIP_ERR_STATE;
+}
+int wr_hip_attn_decode_batched_dev(uint32_t n, wr_hip_kv *const *kv, uint32_t layer,
+                                   const uint32_t *seq_k, const float *q, float *out, uint32_t nq,
+                                   float scale_override, uint32_t window)
+{
+    (void)n; (void)kv; (void)layer; (void)seq_k; (void)q; (void)out; (void)nq; (void)scale_override;
+    (void)window;
+    return WR_HIP_ERR_STATE;
+}
+int wr_hip_attn_prefill_dev(wr_hip_kv *kv, uint32_t layer, uint32_t p0, uint32_t T, const float *q,
+                            float *out, uint32_t nq, float scale_override, uint32_t window)
+{
+    (void)kv; (void)layer; (void)p0; (void)T; (void)q; (void)out; (void)nq; (void)scale_override;
+    (void)window;
+    return WR_HIP_ERR_STATE;
+}
+int wr_hip_proj_weight_create(uint32_t n_parts, const uint16_t *const *parts, const uint32_t *rows,
+                              uint32_t n_in, wr_hip_weight **out)
+{
+    (void)n_parts; (void)parts; (void)rows; (void)n_in;
+    if (out) *out = NULL;
+    return WR_HIP_ERR_STATE;
+}
+void wr_hip_proj_weight_destroy(wr_hip_weight *w) { (void)w; }
+int wr_hip_proj_rows_dev(const wr_hip_weight *w, uint32_t rows, const float *x, uint32_t ldx,
+                         const float *add, float *y, uint32_t ldy)
+{
+    (void)w; (void)rows; (void)x; (void)ldx; (void)add; (void)y; (void)ldy;
+    return WR_HIP_ERR_STATE;
+}
+int wr_hip_rows_rmsnorm_dev(const float *x, uint32_t ldx, const float *w, uint32_t wn, float *out,
+                            uint32_t ldo, uint32_t rows, uint32_t dim, float eps)
+{
+    (void)x; (void)ldx; (void)w; (void)wn; (void)out; (void)ldo; (void)rows; (void)dim; (void)eps;
+    return WR_HIP_ERR_STATE;
+}
+int wr_hip_rows_qkv_prep_dev(const float *qkv, uint32_t ld, uint32_t rows, uint32_t nq, uint32_t nkv,
+                             uint32_t hd, const float *qn, const float *kn, float eps,
+                             const float *cs, uint32_t n_rot, float *q, float *k, float *v)
+{
+    (void)qkv; (void)ld; (void)rows; (void)nq; (void)nkv; (void)hd; (void)qn; (void)kn; (void)eps;
+    (void)cs; (void)n_rot; (void)q; (void)k; (void)v;
+    return WR_HIP_ERR_STATE;
+}
+int wr_hip_rows_swiglu_dev(const float *gu, uint32_t ld, float *act, uint32_t ldo, uint32_t rows,
+                           uint32_t ffn)
+{
+    (void)gu; (void)ld; (void)act; (void)ldo; (void)rows; (void)ffn;
+    return WR_HIP_ERR_STATE;
+}

@@ -4,14 +4,17 @@
 Qwen3-0.6B-architecture model (28 layers, hidden 1024, 16/8 heads, head_dim 128,
 F16 weights N(0, 0.02) from seed 0x5EED0100).
 
-    python tests/golden/make_e2e_golden.py [--small]
+    python tests/golden/make_e2e_golden.py [--small | --small16]
 
 Workload: 128 prompt token ids uniform in [0, vocab) from splitmix64, prefill of
 the first 127, then 129 greedy steps (the last prompt token plus 128 generated
 tokens).  Stored per step: the greedy token, the top-2 logit gap and eight
 probe logits, plus a CRC of the model file so a test can tell "inputs differ"
 from "results differ".  --small writes the same for a 2-layer toy model
-(e2e_tiny_golden.npz) that the CPU-only tests can run in a second.
+(e2e_tiny_golden.npz) that the CPU-only tests can run in a second; --small16
+for a 3-layer toy model whose every dimension is a multiple of 32 (vocab 320),
+the smallest shape that can run with its weights on the device
+(e2e_small16_golden.npz).
 """
 from __future__ import annotations
 
@@ -33,6 +36,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 
 TINY = gw.ModelShape(n_layers=2, hidden=64, ffn=128, n_q=4, n_kv=2, head_dim=32, vocab=300,
                      context=512)
+SMALL16 = gw.ModelShape(n_layers=3, hidden=128, ffn=256, n_q=4, n_kv=2, head_dim=64, vocab=320,
+                        context=512)
 PROBES = 8
 
 
@@ -98,10 +103,12 @@ def run_reference(path: str, prompt: np.ndarray, n_steps: int, max_ctx: int):
 
 def main() -> None:
     small = "--small" in sys.argv
+    small16 = "--small16" in sys.argv
     oracle.build(ref=True)
-    shape = TINY if small else gw.QWEN3_0_6B
-    n_prompt, n_steps = (12, 20) if small else (128, 129)
-    out = os.path.join(HERE, "e2e_tiny_golden.npz" if small else "e2e_qwen3_golden.npz")
+    shape = TINY if small else (SMALL16 if small16 else gw.QWEN3_0_6B)
+    n_prompt, n_steps = (12, 20) if small else ((40, 40) if small16 else (128, 129))
+    out = os.path.join(HERE, "e2e_tiny_golden.npz" if small else
+                       ("e2e_small16_golden.npz" if small16 else "e2e_qwen3_golden.npz"))
     with tempfile.TemporaryDirectory(dir="/tmp") as d:
         path = os.path.join(d, "model.gguf")
         gw.write_model(path, shape)

@@ -1,13 +1,16 @@
 """End to end on the device: the C11 host engine (wr_engine / wr_model /
-wr_session API) with attention and the KV cache on the GPU, against the greedy
-token stream the compiled reference produced for the same random-init model
-(tests/golden/e2e_*_golden.npz, written by tests/golden/make_e2e_golden.py)."""
+wr_session API) against the greedy token stream the compiled reference produced
+for the same random-init model (tests/golden/e2e_*_golden.npz, written by
+tests/golden/make_e2e_golden.py).  Every test runs twice: with the whole layer
+walk on the device (weights uploaded at load, the default for F16 models) and
+with the host walk that sends only the cache append and attention to the GPU
+(WAYRT_HOST_LAYERS=1 while the model loads)."""
 import os
 
 import numpy as np
 import pytest
 
-from tests.golden.make_e2e_golden import TINY, file_crc, workload
+from tests.golden.make_e2e_golden import SMALL16, TINY, file_crc, workload
 from wayruntime_amd import engine as E, gguf_writer as gw, hipattn
 
 pytestmark = pytest.mark.gpu
@@ -20,6 +23,15 @@ def eng():
     e = E.Engine(E.HOST_SO)
     yield e
     e.close()
+
+
+@pytest.fixture(params=["device_walk", "host_walk"])
+def walk(request, monkeypatch):
+    if request.param == "host_walk":
+        monkeypatch.setenv("WAYRT_HOST_LAYERS", "1")
+    else:
+        monkeypatch.delenv("WAYRT_HOST_LAYERS", raising=False)
+    return request.param
 
 
 def _run_stream(model, g, n_prompt):
@@ -50,18 +62,32 @@ def _run_stream(model, g, n_prompt):
     return np.array(got), forced, worst_probe
 
 
-def test_tiny_model_stream_on_device(eng, tmp_path):
+def test_tiny_model_stream_on_device(eng, tmp_path, walk):
     g = np.load(os.path.join(GOLD, "e2e_tiny_golden.npz"))
     p = str(tmp_path / "tiny.gguf")
     gw.write_model(p, TINY)
     m = eng.load(p)
     got, forced, probe = _run_stream(m, g, len(g["prompt"]))
-    print("tiny: forced", forced, "probe err", probe, flush=True)
+    print("tiny", walk, ": forced", forced, "probe err", probe, flush=True)
     assert forced == len(g["tokens"]) and np.array_equal(got, g["tokens"]) and probe < 1e-4
     m.close()
 
 
-def test_qwen3_0_6b_greedy_stream_matches_reference(eng, tmp_path):
+def test_small16_model_stream_on_device(eng, tmp_path, walk):
+    # the smallest shape the device walk takes (TINY's vocabulary of 300 keeps it on the host walk)
+    g = np.load(os.path.join(GOLD, "e2e_small16_golden.npz"))
+    p = str(tmp_path / "small16.gguf")
+    gw.write_model(p, SMALL16)
+    if file_crc(p) != int(g["model_crc"][0]):
+        pytest.skip("random-init model file differs from the one the golden stream was made with")
+    m = eng.load(p)
+    got, forced, probe = _run_stream(m, g, len(g["prompt"]))
+    print("small16", walk, ": forced", forced, "probe err", probe, flush=True)
+    assert forced == len(g["tokens"]) and np.array_equal(got, g["tokens"]) and probe < 1e-3
+    m.close()
+
+
+def test_qwen3_0_6b_greedy_stream_matches_reference(eng, tmp_path, walk):
     # 28 layers, hidden 1024, 16/8 heads, head_dim 128, F16 weights N(0, 0.02):
     # 127-token prefill, then 129 greedy steps
     g = np.load(os.path.join(GOLD, "e2e_qwen3_golden.npz"))
@@ -75,7 +101,7 @@ def test_qwen3_0_6b_greedy_stream_matches_reference(eng, tmp_path):
     before = eng.counters()[E.WR_CTR_ATTENTION_CALLS]
     got, forced, probe = _run_stream(m, g, 128)
     n = len(g["tokens"])
-    print(f"qwen3: teacher-forced {forced}/{n}, probe logit err {probe:.2e}, "
+    print(f"qwen3 ({walk}): teacher-forced {forced}/{n}, probe logit err {probe:.2e}, "
           f"min reference top-2 gap {float(g['gaps'].min()):.4f}", flush=True)
     assert forced == n                                   # argmax agrees at every step
     assert np.array_equal(got, g["tokens"])              # and the free-running stream is identical
@@ -86,12 +112,12 @@ def test_qwen3_0_6b_greedy_stream_matches_reference(eng, tmp_path):
     os.remove(p)
 
 
-def test_batched_step_equals_serial_on_device(eng, tmp_path):
-    p = str(tmp_path / "tiny.gguf")
-    gw.write_model(p, TINY)
+def test_batched_step_equals_serial_on_device(eng, tmp_path, walk):
+    p = str(tmp_path / "small16.gguf")
+    gw.write_model(p, SMALL16)
     m = eng.load(p)
-    n = 5
-    prompts = [workload(TINY, 4 + 7 * i) for i in range(n)]
+    n = 12                                  # more than eight rows: two row groups in the projections
+    prompts = [workload(SMALL16, 4 + 7 * i) for i in range(n)]
     batch = [m.session(128) for _ in range(n)]
     serial = [m.session(128) for _ in range(n)]
     for i in range(n):

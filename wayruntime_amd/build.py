@@ -45,7 +45,7 @@ def build_hip(keep_temps: bool = False) -> str:
 
 HOST_SO = os.path.join(PKG, "libwayruntime_amd.so")
 HOST_DIR = os.path.join(PKG, "host")
-HOST_SRCS = ["wr_math.c", "wr_ops.c", "wr_model.c", "wr_session.c"]
+HOST_SRCS = ["wr_math.c", "wr_ops.c", "wr_model.c", "wr_session.c", "wr_device.c"]
 # -ffp-contract=off: the scalar ops keep the reference's multiply-then-add
 # rounding; the matmul uses explicit FMA intrinsics and is not affected.
 HOST_CFLAGS = ["-std=c11", "-O3", "-mavx2", "-mfma", "-mf16c", "-ffp-contract=off", "-fopenmp",

@@ -473,14 +473,15 @@ int proj_chunk_locked(const wr_hip_weight* w, uint32_t rows, const float* x_dev,
     a.ldy = ldy;
     // Waves that share a run of outputs (contiguous parts of the inputs, summed
     // through LDS in a fixed order): enough that a narrow weight still gives
-    // about a thousand waves.  A function of the weight's shape and the row
-    // group count only, so a projection's arithmetic never depends on what
-    // else is in flight.
-    const uint32_t nt_per_wave = (groups == 2) ? 2 : 1;
-    const uint32_t runs = (w->n_out / 16 + nt_per_wave - 1) / nt_per_wave;
+    // about a thousand waves.  A function of the weight's shape only: a row's
+    // sums are then split the same way whether it travels alone or with up to
+    // fifteen others, so a batched step's rows equal the serial steps' bit
+    // for bit (reference contract: src/core/batch.c:15-19).  Larger row counts
+    // (prefill chunks) use one wave per run.
+    const uint32_t tiles = w->n_out / 16;
     uint32_t ksplit = 1;
     if (groups <= 2) {
-        while (ksplit < 4 && runs * ksplit < 1024 && ktiles % (ksplit * 2) == 0 &&
+        while (ksplit < 4 && tiles * ksplit < 1024 && ktiles % (ksplit * 2) == 0 &&
                ktiles / (ksplit * 2) >= 4)
             ksplit *= 2;
     }
@@ -606,6 +607,8 @@ void wr_hip_attn_set_log(wr_hip_log_fn fn, void* user)
 uint64_t wr_hip_attn_calls(void) { return g.calls.load(std::memory_order_relaxed); }
 
 const char* wr_hip_attn_device_name(void) { return g.name; }
+
+uint32_t wr_hip_attn_caps(void) { return WR_HIP_CAP_PROJ; }
 
 void wr_hip_attn_set_tuning(uint32_t decode_keys_per_wg, int force_generic)
 {

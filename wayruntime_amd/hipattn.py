@@ -40,6 +40,7 @@ def load() -> C.CDLL:
         "wr_hip_attn_shutdown": (None, []),
         "wr_hip_attn_calls": (C.c_uint64, []),
         "wr_hip_attn_device_name": (C.c_char_p, []),
+        "wr_hip_attn_caps": (_u32, []),
         "wr_hip_attn_kv_create": (C.c_int, [_u32, C.POINTER(_u32), _u32, _u32, C.POINTER(_vp)]),
         "wr_hip_attn_kv_destroy": (None, [_vp]),
         "wr_hip_attn_kv_bytes": (C.c_uint64, [_vp]),

@@ -1,0 +1,267 @@
+/*
+ * wr_device.c — the layer walk with every matrix product and row step on the
+ * device (reference: src/core/session.c:440-538, the same block wr_session.c
+ * walks on the host).  Used when the device library offers projections
+ * (WR_HIP_CAP_PROJ) and every matrix of the model is F16 with dimensions the
+ * projection kernel takes; WAYRT_HOST_LAYERS=1 in the environment keeps the
+ * host walk.  Per call the host embeds the rows and works out the rotary
+ * angles (the reference's polynomial sin / cos and range reduction stay on the
+ * host), sends both up once, runs the layers without coming back, and brings
+ * down the logits (wr_step, wr_batch_step) or nothing (wr_prefill).
+ *
+ * Sums run in a different order than on the host (matrix-core tiles, tree
+ * reductions), so activations agree with the host walk to F32 rounding, not
+ * bit for bit; the greedy token stream is compared with the reference's in
+ * the end-to-end test.
+ */
+#define _POSIX_C_SOURCE 200809L
+#include "wr_host.h"
+
+#include <stdlib.h>
+#include <string.h>
+
+typedef struct dev_layer {
+    wr_hip_weight *wqkv, *wo, *wgu, *wdown;
+    const float *attn_norm, *ffn_norm, *q_norm, *k_norm;      /* device */
+} dev_layer;
+
+struct wrh_dev_model {
+    dev_layer     L[WRH_MAX_LAYERS];
+    wr_hip_weight *lm_head;
+    float         *vecs;                                       /* one device block for all norm vectors */
+    const float   *final_norm;
+};
+
+static int proj_dims_ok(const wrh_weight *w)
+{
+    return w->is_f16 && w->cols % 32 == 0;
+}
+
+void wrh_device_model_free(wr_model *m)
+{
+    struct wrh_dev_model *d = m->dev;
+    if (!d) return;
+    for (uint32_t l = 0; l < m->n_layers; l++) {
+        wr_hip_proj_weight_destroy(d->L[l].wqkv);
+        wr_hip_proj_weight_destroy(d->L[l].wo);
+        wr_hip_proj_weight_destroy(d->L[l].wgu);
+        wr_hip_proj_weight_destroy(d->L[l].wdown);
+    }
+    wr_hip_proj_weight_destroy(d->lm_head);
+    wr_hip_attn_dev_free(d->vecs);
+    free(d);
+    m->dev = NULL;
+}
+
+static int stack(wr_hip_weight **out, const wrh_weight *a, const wrh_weight *b, const wrh_weight *c)
+{
+    const uint16_t *parts[3] = {a->data, b ? b->data : NULL, c ? c->data : NULL};
+    uint32_t rows[3] = {a->rows, b ? b->rows : 0, c ? c->rows : 0};
+    return wr_hip_proj_weight_create(c ? 3 : (b ? 2 : 1), parts, rows, a->cols, out);
+}
+
+/* WR_OK with m->dev set, WR_OK with m->dev NULL when the model stays on the
+ * host walk, or an error when uploading a model that qualifies fails. */
+wr_status wrh_device_model_init(wr_model *m)
+{
+    m->dev = NULL;
+    const char *env = getenv("WAYRT_HOST_LAYERS");
+    if (env && env[0] == '1') return WR_OK;
+    if (!(wr_hip_attn_caps() & WR_HIP_CAP_PROJ)) return WR_OK;
+    const uint32_t qd = m->n_q * m->head_dim, kd = m->n_kv * m->head_dim;
+    int ok = proj_dims_ok(&m->lm_head) && m->vocab % 16 == 0 && (qd + 2 * kd) % 16 == 0 &&
+             m->hidden % 16 == 0 && (2 * m->ffn) % 16 == 0;
+    for (uint32_t l = 0; l < m->n_layers && ok; l++)
+        ok = proj_dims_ok(&m->wq[l]) && proj_dims_ok(&m->wk[l]) && proj_dims_ok(&m->wv[l]) &&
+             proj_dims_ok(&m->wo[l]) && proj_dims_ok(&m->w_gate[l]) && proj_dims_ok(&m->w_up[l]) &&
+             proj_dims_ok(&m->w_down[l]);
+    if (!ok) {
+        wrh_logf(m->engine, 2, "device layers: model keeps the host walk (needs F16 matrices, "
+                              "inputs a multiple of 32, outputs of 16)");
+        return WR_OK;
+    }
+
+    struct wrh_dev_model *d = calloc(1, sizeof *d);
+    if (!d) return WR_ERR_NOMEM;
+    m->dev = d;
+    int rc = WR_HIP_OK;
+    /* norm vectors: [final | per layer: attn, ffn, (q, k)] */
+    const size_t per_layer = 2 * (size_t)m->hidden + (m->has_qk_norm ? 2 * (size_t)m->head_dim : 0);
+    const size_t n_vec = m->hidden + per_layer * m->n_layers;
+    float *host = malloc(n_vec * sizeof(float));
+    d->vecs = wr_hip_attn_dev_alloc(n_vec * sizeof(float));
+    if (!host || !d->vecs) rc = WR_HIP_ERR_NOMEM;
+    if (rc == WR_HIP_OK) {
+        size_t at = 0;
+        memcpy(host + at, m->final_norm.data, m->hidden * sizeof(float));
+        d->final_norm = d->vecs + at;
+        at += m->hidden;
+        for (uint32_t l = 0; l < m->n_layers; l++) {
+            memcpy(host + at, m->attn_norm[l].data, m->hidden * sizeof(float));
+            d->L[l].attn_norm = d->vecs + at;
+            at += m->hidden;
+            memcpy(host + at, m->ffn_norm[l].data, m->hidden * sizeof(float));
+            d->L[l].ffn_norm = d->vecs + at;
+            at += m->hidden;
+            if (m->has_qk_norm) {
+                memcpy(host + at, m->q_norm[l].data, m->head_dim * sizeof(float));
+                d->L[l].q_norm = d->vecs + at;
+                at += m->head_dim;
+                memcpy(host + at, m->k_norm[l].data, m->head_dim * sizeof(float));
+                d->L[l].k_norm = d->vecs + at;
+                at += m->head_dim;
+            }
+        }
+        rc = wr_hip_attn_h2d(d->vecs, host, n_vec * sizeof(float));
+    }
+    free(host);
+    for (uint32_t l = 0; l < m->n_layers && rc == WR_HIP_OK; l++) {
+        rc = stack(&d->L[l].wqkv, &m->wq[l], &m->wk[l], &m->wv[l]);
+        if (rc == WR_HIP_OK) rc = stack(&d->L[l].wo, &m->wo[l], NULL, NULL);
+        if (rc == WR_HIP_OK) rc = stack(&d->L[l].wgu, &m->w_gate[l], &m->w_up[l], NULL);
+        if (rc == WR_HIP_OK) rc = stack(&d->L[l].wdown, &m->w_down[l], NULL, NULL);
+    }
+    if (rc == WR_HIP_OK) rc = stack(&d->lm_head, &m->lm_head, NULL, NULL);
+    if (rc != WR_HIP_OK) {
+        wrh_logf(m->engine, 0, "device layers: weight upload failed (rc=%d)", rc);
+        wrh_device_model_free(m);
+        return (rc == WR_HIP_ERR_NOMEM) ? WR_ERR_NOMEM : WR_ERR_INTERNAL;
+    }
+    wrh_logf(m->engine, 2, "device layers: %u layers and the LM head are on the device", m->n_layers);
+    return WR_OK;
+}
+
+/* ------------------------------------------------------------- workspace -- */
+
+static size_t r64(size_t n) { return (n + 63) & ~(size_t)63; }       /* floats: 256-byte steps */
+
+int wrh_devspace_init(wrh_devspace *ws, const wr_model *m, uint32_t rows, uint32_t logit_rows)
+{
+    memset(ws, 0, sizeof *ws);
+    const size_t hidden = m->hidden, qd = (size_t)m->n_q * m->head_dim, kd = (size_t)m->n_kv * m->head_dim;
+    const size_t ffn = m->ffn, R = rows;
+    const size_t total = 2 * r64(R * hidden) + r64(R * (qd + 2 * kd)) + 2 * r64(R * qd) + 2 * r64(R * kd) +
+                         r64(R * 2 * ffn) + r64(R * ffn) + r64(R * m->head_dim) +
+                         r64((size_t)logit_rows * m->vocab);
+    float *b = wr_hip_attn_dev_alloc(total * sizeof(float));
+    if (!b) return WR_ERR_NOMEM;
+    ws->block = b;
+    ws->rows_cap = rows;
+    ws->logit_rows = logit_rows;
+    ws->resid = b;   b += r64(R * hidden);
+    ws->normed = b;  b += r64(R * hidden);
+    ws->qkv = b;     b += r64(R * (qd + 2 * kd));
+    ws->q = b;       b += r64(R * qd);
+    ws->attn = b;    b += r64(R * qd);
+    ws->k = b;       b += r64(R * kd);
+    ws->v = b;       b += r64(R * kd);
+    ws->gu = b;      b += r64(R * 2 * ffn);
+    ws->act = b;     b += r64(R * ffn);
+    ws->rope = b;    b += r64(R * m->head_dim);
+    ws->logits = b;
+    return WR_OK;
+}
+
+void wrh_devspace_free(wrh_devspace *ws)
+{
+    if (ws->block) wr_hip_attn_dev_free(ws->block);
+    memset(ws, 0, sizeof *ws);
+}
+
+/* --------------------------------------------------------------- forward -- */
+
+static wr_status dev_fail(wr_engine *e, const char *what, uint32_t layer, int rc)
+{
+    wrh_logf(e, 0, "session: %s failed at layer %u (rc=%d)", what, layer, rc);
+    if (rc == WR_HIP_ERR_CTX_FULL) return WR_ERR_CTX_FULL;
+    return (rc < 0) ? (wr_status)rc : WR_ERR_INTERNAL;
+}
+
+#define TRY(call, what)                                        \
+    do {                                                       \
+        rc = (call);                                           \
+        if (rc != WR_HIP_OK) return dev_fail(e, what, L, rc);  \
+    } while (0)
+
+/* Same contract as the host walk's forward_rows (wr_session.c), plus: when
+ * logits_host is not NULL, the LM head runs for the first `logit_rows` rows
+ * and their logits [logit_rows][vocab] are brought down. */
+wr_status wrh_forward_rows_device(wr_model *m, wrh_workspace *hs, wrh_devspace *ds, uint32_t R,
+                                  wr_session *const *ss, const uint32_t *tokens, uint32_t pos0,
+                                  int batch, int prefill, int fail_layer, float *logits_host,
+                                  uint32_t logit_rows)
+{
+    wr_engine *e = m->engine;
+    const struct wrh_dev_model *d = m->dev;
+    const uint32_t hidden = m->hidden, hd = m->head_dim, nq = m->n_q, nkv = m->n_kv;
+    const uint32_t qd = nq * hd, kd = nkv * hd, ffn = m->ffn;
+    const uint32_t n_rot = (m->n_rot_pairs >= 1 && m->n_rot_pairs < hd / 2) ? m->n_rot_pairs : hd / 2;
+    const size_t ts = (size_t)2 * n_rot;
+    uint32_t L = 0;
+    int rc;
+
+    for (uint32_t r = 0; r < R; r++) {
+        rc = wrh_embed(&m->embed, tokens[r], hs->residual + (size_t)r * hidden);
+        if (rc != WR_OK) return dev_fail(e, "embed", 0, rc);
+        const uint32_t p = batch ? ss[r]->pos : pos0 + r;
+        (void)wrh_rope_table(hs->rope + r * ts, hd, p, m->rope_base, m->n_rot_pairs);
+    }
+    TRY(wr_hip_attn_h2d(ds->resid, hs->residual, (size_t)R * hidden * sizeof(float)), "rows up");
+    TRY(wr_hip_attn_h2d(ds->rope, hs->rope, (size_t)R * ts * sizeof(float)), "angles up");
+
+    for (L = 0; L < m->n_layers; L++) {
+        const dev_layer *dl = &d->L[L];
+        TRY(wr_hip_rows_rmsnorm_dev(ds->resid, hidden, dl->attn_norm, hidden, ds->normed, hidden, R,
+                                    hidden, m->rms_eps), "attn norm");
+        TRY(wr_hip_proj_rows_dev(dl->wqkv, R, ds->normed, hidden, NULL, ds->qkv, qd + 2 * kd),
+            "qkv projection");
+        TRY(wr_hip_rows_qkv_prep_dev(ds->qkv, qd + 2 * kd, R, nq, nkv, hd, dl->q_norm, dl->k_norm,
+                                     m->rms_eps, ds->rope, n_rot, ds->q, ds->k, ds->v), "qkv prep");
+
+        if (fail_layer == (int)L) return dev_fail(e, "gqa (injected)", L, WR_ERR_INTERNAL);
+        if (batch) {
+            wr_hip_kv *kvs[WR_BATCH_MAX];
+            uint32_t seq_k[WR_BATCH_MAX];
+            for (uint32_t r = 0; r < R; r++) {
+                TRY(wr_hip_attn_append_dev(ss[r]->kv, L, ss[r]->pos, 1, ds->k + (size_t)r * kd,
+                                           ds->v + (size_t)r * kd), "kv append");
+                ss[r]->kv_rows[L] = ss[r]->pos + 1;
+                kvs[r] = ss[r]->kv;
+                seq_k[r] = ss[r]->pos + 1;
+            }
+            TRY(wr_hip_attn_decode_batched_dev(R, kvs, L, seq_k, ds->q, ds->attn, nq, 0.0f, 0), "gqa");
+        } else {
+            wr_session *s = ss[0];
+            TRY(wr_hip_attn_append_dev(s->kv, L, pos0, R, ds->k, ds->v), "kv append");
+            s->kv_rows[L] = pos0 + R;
+            if (prefill) {
+                TRY(wr_hip_attn_prefill_dev(s->kv, L, pos0, R, ds->q, ds->attn, nq, 0.0f, 0), "gqa");
+            } else {
+                wr_hip_kv *one[1] = {s->kv};
+                const uint32_t sk = pos0 + 1;
+                TRY(wr_hip_attn_decode_batched_dev(1, one, L, &sk, ds->q, ds->attn, nq, 0.0f, 0), "gqa");
+            }
+        }
+        TRY(wr_hip_proj_rows_dev(dl->wo, R, ds->attn, qd, ds->resid, ds->resid, hidden),
+            "output projection");
+        TRY(wr_hip_rows_rmsnorm_dev(ds->resid, hidden, dl->ffn_norm, hidden, ds->normed, hidden, R,
+                                    hidden, m->rms_eps), "ffn norm");
+        TRY(wr_hip_proj_rows_dev(dl->wgu, R, ds->normed, hidden, NULL, ds->gu, 2 * ffn),
+            "gate/up projection");
+        TRY(wr_hip_rows_swiglu_dev(ds->gu, 2 * ffn, ds->act, ffn, R, ffn), "swiglu");
+        TRY(wr_hip_proj_rows_dev(dl->wdown, R, ds->act, ffn, ds->resid, ds->resid, hidden),
+            "down projection");
+    }
+    L = m->n_layers;
+    TRY(wr_hip_rows_rmsnorm_dev(ds->resid, hidden, d->final_norm, hidden, ds->normed, hidden, R,
+                                hidden, m->rms_eps), "final norm");
+    if (logits_host && logit_rows) {
+        TRY(wr_hip_proj_rows_dev(d->lm_head, logit_rows, ds->normed, hidden, NULL, ds->logits,
+                                 m->vocab), "lm head");
+        TRY(wr_hip_attn_d2h(logits_host, ds->logits, (size_t)logit_rows * m->vocab * sizeof(float)),
+            "logits down");
+    } else {
+        TRY(wr_hip_attn_sync(), "sync");
+    }
+    return WR_OK;
+}

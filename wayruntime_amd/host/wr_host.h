@@ -65,6 +65,8 @@ struct wr_model {
     wrh_weight wq[WRH_MAX_LAYERS], wk[WRH_MAX_LAYERS], wv[WRH_MAX_LAYERS], wo[WRH_MAX_LAYERS];
     wrh_weight w_gate[WRH_MAX_LAYERS], w_up[WRH_MAX_LAYERS], w_down[WRH_MAX_LAYERS];
 
+    struct wrh_dev_model *dev;   /* device copies of the weights, NULL on the host walk */
+
     void           *map;         /* mmap of the GGUF file */
     size_t          map_bytes;
     pthread_mutex_t lock;        /* guards session_refs */
@@ -83,6 +85,19 @@ typedef struct wrh_workspace {
     void  *block;
 } wrh_workspace;
 
+/* Device scratch for R rows of the device walk (wr_device.c). */
+typedef struct wrh_devspace {
+    uint32_t rows_cap, logit_rows;
+    float *resid, *normed;               /* [R][hidden] */
+    float *qkv;                          /* [R][(n_q + 2 n_kv) * hd] */
+    float *q, *attn;                     /* [R][n_q*hd] */
+    float *k, *v;                        /* [R][n_kv*hd] */
+    float *gu, *act;                     /* [R][2 ffn], [R][ffn] */
+    float *rope;                         /* [R][hd/2][2] */
+    float *logits;                       /* [logit_rows][vocab] */
+    float *block;
+} wrh_devspace;
+
 struct wr_session {
     wr_model       *model;
     pthread_mutex_t lock;
@@ -93,6 +108,7 @@ struct wr_session {
     uint32_t        kv_rows[WRH_MAX_LAYERS]; /* per-layer cursor (the reference's valid_rows) */
     float          *logits;                  /* [vocab] */
     wrh_workspace   ws1;                     /* one-row scratch for wr_step */
+    wrh_devspace    ds1;                     /* its device counterpart (device walk only) */
 };
 
 /* ---- ops (wr_ops.c) -------------------------------------------------------
@@ -119,6 +135,16 @@ extern wr_engine *wrh_engine;           /* the process engine, NULL when none */
 /* ---- forward (wr_session.c) ------------------------------------------------ */
 int  wrh_workspace_init(wrh_workspace *ws, const wr_model *m, uint32_t rows);
 void wrh_workspace_free(wrh_workspace *ws);
+
+/* ---- device walk (wr_device.c) --------------------------------------------- */
+wr_status wrh_device_model_init(wr_model *m);
+void      wrh_device_model_free(wr_model *m);
+int       wrh_devspace_init(wrh_devspace *ws, const wr_model *m, uint32_t rows, uint32_t logit_rows);
+void      wrh_devspace_free(wrh_devspace *ws);
+wr_status wrh_forward_rows_device(wr_model *m, wrh_workspace *hs, wrh_devspace *ds, uint32_t R,
+                                  wr_session *const *ss, const uint32_t *tokens, uint32_t pos0,
+                                  int batch, int prefill, int fail_layer, float *logits_host,
+                                  uint32_t logit_rows);
 
 /* Test hook: make the attention call of `layer` fail with WR_ERR_INTERNAL once
  * (layer < 0 disarms).  The device is not involved: the failure is raised on

@@ -593,6 +593,13 @@ wr_status wr_model_load(wr_engine *e, const char *path, const wr_model_params *p
         m->all_f16 = (uint8_t)(m->all_f16 && m->wq[l].is_f16);
 #undef NAME
     }
+    /* every matrix F16, not only the first one looked at */
+    for (uint32_t l = 0; l < m->n_layers; l++)
+        m->all_f16 = (uint8_t)(m->all_f16 && m->wk[l].is_f16 && m->wv[l].is_f16 && m->wo[l].is_f16 &&
+                               m->w_gate[l].is_f16 && m->w_up[l].is_f16 && m->w_down[l].is_f16);
+    m->all_f16 = (uint8_t)(m->all_f16 && m->lm_head.is_f16);
+    /* weights and layer walk on the device where the library and the model allow it */
+    if ((rc = wrh_device_model_init(m)) != WR_OK) goto fail;
     free(g.t);
     m->map = map;
     m->map_bytes = (size_t)st.st_size;
@@ -622,6 +629,7 @@ void wr_model_free(wr_model *m)
         return;
     }
     if (m->engine && m->engine->models_live) m->engine->models_live--;
+    wrh_device_model_free(m);
     munmap(m->map, m->map_bytes);
     pthread_mutex_destroy(&m->lock);
     free(m);

@@ -6,8 +6,10 @@
  * src/core/session.c:440-534): RMSNorm, Q/K/V projections, per-head Q/K
  * RMSNorm (Qwen3), RoPE, KV append, attention, output projection, residual,
  * RMSNorm, SwiGLU, down projection, residual; final RMSNorm; LM head.
- * Here it runs over R rows at once (layer-major), and the two steps in the
- * middle go to the device:
+ * Here it runs over R rows at once (layer-major).  When the model's weights
+ * are on the device (wr_device.c) the whole walk runs there; otherwise the
+ * walk below runs on the host and the two steps in the middle go to the
+ * device:
  *
  *   reference kv_append_row (session.c:139-154, called :483-486)
  *                                  -> wr_hip_attn_append
@@ -173,6 +175,14 @@ static wr_status forward_rows(wr_model *m, wrh_workspace *ws, uint32_t R, wr_ses
     return WR_OK;
 }
 
+/* The injected failure, taken once: the layer to fail at, or -1. */
+static int take_fail_layer(const wr_model *m)
+{
+    const int fl = g_fail_attention_layer;
+    if (fl >= 0 && (uint32_t)fl < m->n_layers) g_fail_attention_layer = -1;
+    return fl;
+}
+
 /* Cursors back to the committed position (reference: session.c:160-168).
  * Rows above the cursor stay in device memory and are never read. */
 static void kv_rollback(wr_session *s)
@@ -211,8 +221,10 @@ wr_status wr_session_create(wr_model *m, const wr_session_params *params, wr_ses
         return (wr_status)rc;
     }
     s->logits = malloc((size_t)m->vocab * sizeof(float));
-    if (!s->logits || wrh_workspace_init(&s->ws1, m, 1) != WR_OK) {
+    if (!s->logits || wrh_workspace_init(&s->ws1, m, 1) != WR_OK ||
+        (m->dev && wrh_devspace_init(&s->ds1, m, 1, 1) != WR_OK)) {
         free(s->logits);
+        wrh_workspace_free(&s->ws1);
         wr_hip_attn_kv_destroy(s->kv);
         free(s);
         return WR_ERR_NOMEM;
@@ -234,6 +246,7 @@ void wr_session_destroy(wr_session *s)
     pthread_mutex_unlock(&m->lock);
     wr_hip_attn_kv_destroy(s->kv);
     wrh_workspace_free(&s->ws1);
+    wrh_devspace_free(&s->ds1);
     free(s->logits);
     pthread_mutex_destroy(&s->lock);
     free(s);
@@ -263,9 +276,14 @@ const float *wr_step(wr_session *s, uint32_t token)
         st = WR_ERR_CTX_FULL;                              /* consumed nothing */
     } else {
         wr_session *one[1] = {s};
-        st = forward_rows(m, &s->ws1, 1, one, &token, s->pos, FWD_STEP);
-        if (st == WR_OK)
-            wrh_matmul(m->engine, s->ws1.normed, 1, m->hidden, &m->lm_head, s->logits, m->vocab);
+        if (m->dev) {
+            st = wrh_forward_rows_device(m, &s->ws1, &s->ds1, 1, one, &token, s->pos, 0, 0,
+                                         take_fail_layer(m), s->logits, 1);
+        } else {
+            st = forward_rows(m, &s->ws1, 1, one, &token, s->pos, FWD_STEP);
+            if (st == WR_OK)
+                wrh_matmul(m->engine, s->ws1.normed, 1, m->hidden, &m->lm_head, s->logits, m->vocab);
+        }
         if (st == WR_OK)
             __atomic_store_n(&s->pos, s->pos + 1, __ATOMIC_RELEASE);
         else
@@ -296,15 +314,23 @@ int wr_prefill(wr_session *s, const uint32_t *ids, uint32_t n)
         for (uint32_t i = 0; i < n && st == WR_OK; i++)
             if (ids[i] >= m->vocab) st = WR_ERR_INVAL;
         wrh_workspace ws;
+        wrh_devspace ds;
+        memset(&ds, 0, sizeof ds);
         const uint32_t chunk = n < WRH_PREFILL_CHUNK ? n : WRH_PREFILL_CHUNK;
         if (st == WR_OK && wrh_workspace_init(&ws, m, chunk) != WR_OK) st = WR_ERR_NOMEM;
         if (st == WR_OK) {
+            if (m->dev && wrh_devspace_init(&ds, m, chunk, 0) != WR_OK) st = WR_ERR_NOMEM;
             wr_session *one[1] = {s};
             for (uint32_t done = 0; done < n && st == WR_OK; done += chunk) {
                 const uint32_t rows = (n - done < chunk) ? n - done : chunk;
-                st = forward_rows(m, &ws, rows, one, ids + done, s->pos, FWD_PREFILL);
+                if (m->dev)
+                    st = wrh_forward_rows_device(m, &ws, &ds, rows, one, ids + done, s->pos, 0, 1,
+                                                 take_fail_layer(m), NULL, 0);
+                else
+                    st = forward_rows(m, &ws, rows, one, ids + done, s->pos, FWD_PREFILL);
                 if (st == WR_OK) __atomic_store_n(&s->pos, s->pos + rows, __ATOMIC_RELEASE);
             }
+            wrh_devspace_free(&ds);
             wrh_workspace_free(&ws);
         }
         if (st != WR_OK) {
@@ -361,10 +387,20 @@ int wr_batch_step(wr_session *const *sessions, const uint32_t *tokens, uint32_t 
         big = malloc((size_t)n * m->vocab * sizeof(float));
         if (!big) st = WR_ERR_NOMEM;
     }
-    if (st == WR_OK) st = forward_rows(m, &ws, n, sessions, tokens, 0, FWD_BATCH);
+    wrh_devspace ds;
+    memset(&ds, 0, sizeof ds);
+    if (st == WR_OK && m->dev && wrh_devspace_init(&ds, m, n, n) != WR_OK) st = WR_ERR_NOMEM;
+    if (st == WR_OK) {
+        if (m->dev)
+            st = wrh_forward_rows_device(m, &ws, &ds, n, sessions, tokens, 0, 1, 0,
+                                         take_fail_layer(m), big, n);
+        else
+            st = forward_rows(m, &ws, n, sessions, tokens, 0, FWD_BATCH);
+    }
+    wrh_devspace_free(&ds);
     if (st == WR_OK) {
         /* one LM-head product for all n rows (reference: batch.c:45-104), then demux */
-        wrh_matmul(m->engine, ws.normed, n, m->hidden, &m->lm_head, big, m->vocab);
+        if (!m->dev) wrh_matmul(m->engine, ws.normed, n, m->hidden, &m->lm_head, big, m->vocab);
         for (uint32_t i = 0; i < n; i++)
             memcpy(sessions[i]->logits, big + (size_t)i * m->vocab, (size_t)m->vocab * sizeof(float));
         for (uint32_t i = 0; i < n; i++)
