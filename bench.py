@@ -13,7 +13,9 @@ Prints ONE JSON line.  `value` is algorithmic K/V bytes per step divided by
 wall time per step (whole step: split-K kernel + combine).  `roofline` is for
 the split-K kernel alone, timed with per-launch events.  `cpu_baseline` is the
 CPU oracle (a bit-exact restatement of the reference op) on the same data, one
-core, on a bounded sample.  `prefill` reports causal prefill attention.
+core, on a bounded sample.  `prefill` reports causal prefill attention,
+`projection` the row projections either side of the path (proj_rows_kernel,
+HBM-bound on the F16 weight bytes).
 """
 from __future__ import annotations
 
@@ -64,6 +66,7 @@ def main() -> None:
     ap.add_argument("--cpu-seconds", type=float, default=12.0,
                     help="budget for the CPU baseline sample (0 disables it)")
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--no-proj", action="store_true")
     ap.add_argument("--keys-per-wg", type=int, default=0)
     args = ap.parse_args()
 
@@ -179,6 +182,37 @@ def main() -> None:
         qp_dev.free()
         op_dev.free()
 
+    # ---- row projections either side of the attention path (secondary figure):
+    # 16 rows through Llama-3-8B-sized F16 weights, HBM-bound on the weight
+    # bytes; distinct copies are walked so the weights come from HBM.
+    proj = None
+    if not args.no_proj:
+        proj = {}
+        rng = np.random.default_rng(7)
+        rows = 16
+        for name, n_out, n_in, copies in (("qkv 6144x4096", 6144, 4096, 6),
+                                          ("gate_up 28672x4096", 28672, 4096, 3),
+                                          ("lm_head 128256x4096", 128256, 4096, 2)):
+            ws = [hipattn.Weight([rng.integers(0, 0x3C00, size=(n_out, n_in), dtype=np.uint16)])
+                  for _ in range(copies)]
+            xd = hipattn.DeviceBuffer.from_host(synth.normal(9, (rows, n_in)))
+            yd = hipattn.DeviceBuffer(rows * n_out * 4)
+            reps = 24
+            for i in range(3 * copies):
+                ws[i % copies].rows_dev(rows, xd, n_in, yd, n_out)
+            hipattn.profile_begin(reps)
+            for i in range(reps):
+                ws[i % copies].rows_dev(rows, xd, n_in, yd, n_out)
+            pms, pn = hipattn.profile_end()
+            us = pms / max(pn, 1) * 1e3
+            gbs = 2.0 * n_out * n_in / (us * 1e-6) / 1e9
+            proj[name] = {"rows": rows, "kernel_us": round(us, 2), "GB/s": round(gbs, 1),
+                          "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)}
+            for w in ws:
+                w.close()
+            xd.free()
+            yd.free()
+
     # ---- CPU baseline: the oracle on the same data, bounded sample.  The
     # reference runs one attention call on one core, so one core is the faithful
     # figure; sessions are independent, so one thread per session is the best a
@@ -237,7 +271,7 @@ def main() -> None:
                                "%d sessions x %d ctx, %d cache layers walked" % (S, ctx, L),
                    "sessions": S, "ctx": ctx, "layers": L},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
-        "roofline": roofline, "cpu_baseline": cpu, "prefill": prefill,
+        "roofline": roofline, "cpu_baseline": cpu, "prefill": prefill, "projection": proj,
         "check": {"max_abs": max_abs, "rel_l2": rel_l2},
         "device": hipattn.device_name(), "setup_s": round(setup_s, 1),
     }

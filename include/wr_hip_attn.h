@@ -168,6 +168,16 @@ int wr_hip_attn_append_dev(wr_hip_kv *kv, uint32_t layer, uint32_t pos,
                            uint32_t n_rows, const float *k_f32_dev,
                            const float *v_f32_dev);
 
+/* One new row for each of n <= WR_HIP_BATCH_MAX sessions in one launch: row i
+ * of k_f32_dev / v_f32_dev [n, nkv, hd] goes to position pos[i] of kv[i] (the n
+ * kv_append_row calls of a batched step, src/core/batch.c:152-167 through
+ * session.c:483-486).  Any pos[i] >= max_ctx is WR_HIP_ERR_CTX_FULL and
+ * nothing is written; caches must differ and agree in nkv and head_dim. */
+int wr_hip_attn_append_batched_dev(uint32_t n, wr_hip_kv *const *kv,
+                                   uint32_t layer, const uint32_t *pos,
+                                   const float *k_f32_dev,
+                                   const float *v_f32_dev);
+
 /* The same rotation alone, in place on device F32 rows [rows, heads, hd]
  * (wri_op_rope, src/core/kernels.c:1356-1412, for callers that keep Q or K on
  * the device); cos_sin_dev is device F32 [rows, n_rot, 2].  Asynchronous on

@@ -227,6 +227,12 @@ int wr_hip_attn_append_dev(wr_hip_kv *kv, uint32_t layer, uint32_t pos, uint32_t
     (void)kv; (void)layer; (void)pos; (void)n_rows; (void)k; (void)v;
     return WR_HIP_ERR_STATE;
 }
+int wr_hip_attn_append_batched_dev(uint32_t n, wr_hip_kv *const *kv, uint32_t layer,
+                                   const uint32_t *pos, const float *k, const float *v)
+{
+    (void)n; (void)kv; (void)layer; (void)pos; (void)k; (void)v;
+    return WR_HIP_ERR_STATE;
+}
 int wr_hip_attn_decode_batched_dev(uint32_t n, wr_hip_kv *const *kv, uint32_t layer,
                                    const uint32_t *seq_k, const float *q, float *out, uint32_t nq,
                                    float scale_override, uint32_t window)

@@ -322,3 +322,39 @@ def test_error_contract():
     assert lib.wr_hip_attn_decode_batched(2, kvp, 0, sk, ptrs, outs, 16, 0.0, 0) == hipattn.ERR_INVAL
     assert lib.wr_hip_attn_init(0) == hipattn.ERR_STATE      # single engine per process
     kv.close()
+
+
+def test_batched_append_writes_the_same_bits_as_single_appends():
+    # one row per session in one launch, sessions at different positions and
+    # capacities; the cache must hold what per-session appends put there, and
+    # neighbouring rows must be untouched
+    import ctypes as C
+    nkv, hd, n = 4, 128, 5
+    caps = [40, 64, 33, 100, 70]
+    pos = [0, 31, 32, 63, 69]
+    k = synth.normal(501, (n, nkv, hd), std=3.0)
+    v = synth.normal(502, (n, nkv, hd), std=3.0)
+    batch = [hipattn.KVCache(2, hd, nkv, c) for c in caps]
+    single = [hipattn.KVCache(2, hd, nkv, c) for c in caps]
+    kd, vd = hipattn.DeviceBuffer.from_host(k), hipattn.DeviceBuffer.from_host(v)
+    lib = hipattn.lib()
+    hs = (C.c_void_p * n)(*[c.h for c in batch])
+    ps = (C.c_uint32 * n)(*pos)
+    assert lib.wr_hip_attn_append_batched_dev(n, hs, 1, ps, kd.p, vd.p) == hipattn.OK
+    hipattn.sync()
+    for i in range(n):
+        assert single[i].append(1, pos[i], k[i:i + 1], v[i:i + 1]) == 0
+        gk, gv = batch[i].read_f16(1, 0, caps[i])
+        wk, wv = single[i].read_f16(1, 0, caps[i])
+        assert np.array_equal(gk, wk) and np.array_equal(gv, wv), i
+        assert np.array_equal(gk[pos[i]], synth.f32_to_f16_trunc(k[i]))
+    # a full cache anywhere in the batch refuses the whole call
+    ps_full = (C.c_uint32 * n)(*[0, 31, 33, 63, 69])
+    assert lib.wr_hip_attn_append_batched_dev(n, hs, 1, ps_full, kd.p, vd.p) == hipattn.ERR_CTX_FULL
+    assert lib.wr_hip_attn_append_batched_dev(0, hs, 1, ps, kd.p, vd.p) == hipattn.ERR_LIMIT
+    hs_dup = (C.c_void_p * 2)(batch[0].h, batch[0].h)
+    assert lib.wr_hip_attn_append_batched_dev(2, hs_dup, 1, ps, kd.p, vd.p) == hipattn.ERR_INVAL
+    for c in batch + single:
+        c.close()
+    kd.free()
+    vd.free()

@@ -110,6 +110,30 @@ __global__ __launch_bounds__(256) void rope_rows_kernel(float* __restrict__ x,
     row[j + half] = a1 + b1;
 }
 
+// One new row for each of up to 16 sessions in one launch (the batched decode
+// step appends one position per session and layer).  grid = sessions.
+struct AppendBatchArgs {
+    uint16_t* k[16];
+    uint16_t* vt[16];
+    uint32_t pos[16];
+    uint32_t ctx_pad[16];
+    const float* k_src;      // [n][nkv][hd]
+    const float* v_src;
+    uint32_t nkv, hd;
+};
+
+__global__ __launch_bounds__(256) void append_batch_kernel(const AppendBatchArgs a)
+{
+    const uint32_t i = blockIdx.x;
+    const uint32_t row = a.nkv * a.hd;
+    const uint32_t pos = a.pos[i], ctx_pad = a.ctx_pad[i];
+    for (uint32_t idx = threadIdx.x; idx < row; idx += 256) {
+        const uint32_t kvh = idx / a.hd, d = idx % a.hd;
+        a.k[i][k_offset(kvh, ctx_pad, pos, d, a.hd)] = f32_to_f16_trunc(a.k_src[(size_t)i * row + idx]);
+        a.vt[i][vt_offset(kvh, ctx_pad, pos, d, a.hd)] = f32_to_f16_trunc(a.v_src[(size_t)i * row + idx]);
+    }
+}
+
 // Export rows back in position-major order [n_rows][nkv][hd] (tests, tooling).
 __global__ __launch_bounds__(256) void export_kv_kernel(const uint16_t* __restrict__ k,
                                                         const uint16_t* __restrict__ vt,

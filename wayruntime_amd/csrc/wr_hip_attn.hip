@@ -699,6 +699,37 @@ int wr_hip_attn_append_dev(wr_hip_kv* kv, uint32_t layer, uint32_t pos, uint32_t
     return append_rows_locked<float>(kv, layer, pos, n_rows, k_f32_dev, v_f32_dev);
 }
 
+int wr_hip_attn_append_batched_dev(uint32_t n, wr_hip_kv* const* kv, uint32_t layer,
+                                   const uint32_t* pos, const float* k_f32_dev,
+                                   const float* v_f32_dev)
+{
+    if (!g.inited) return WR_HIP_ERR_STATE;
+    if (!kv || !pos || !k_f32_dev || !v_f32_dev) return WR_HIP_ERR_INVAL;
+    if (n == 0 || n > WR_HIP_BATCH_MAX) return WR_HIP_ERR_LIMIT;
+    AppendBatchArgs a;
+    memset(&a, 0, sizeof a);
+    for (uint32_t i = 0; i < n; i++) {
+        int rc = check_layer(kv[i], layer);
+        if (rc) return rc;
+        if (kv[i]->nkv != kv[0]->nkv || kv[i]->hd[layer] != kv[0]->hd[layer]) return WR_HIP_ERR_INVAL;
+        for (uint32_t j = 0; j < i; j++)
+            if (kv[i] == kv[j]) return WR_HIP_ERR_INVAL;
+        if (pos[i] >= kv[i]->max_ctx) return WR_HIP_ERR_CTX_FULL;      // nothing is written
+        a.k[i] = reinterpret_cast<uint16_t*>(kv[i]->slab + kv[i]->k_off[layer]);
+        a.vt[i] = reinterpret_cast<uint16_t*>(kv[i]->slab + kv[i]->vt_off[layer]);
+        a.pos[i] = pos[i];
+        a.ctx_pad[i] = kv[i]->ctx_pad;
+    }
+    a.k_src = k_f32_dev;
+    a.v_src = v_f32_dev;
+    a.nkv = kv[0]->nkv;
+    a.hd = kv[0]->hd[layer];
+    Locked lk;
+    hipLaunchKernelGGL(append_batch_kernel, dim3(n), dim3(256), 0, g.stream, a);
+    HIP_TRY(hipGetLastError(), "batched append launch", layer);
+    return WR_HIP_OK;
+}
+
 int wr_hip_attn_rope_dev(void* x_dev, const void* cos_sin_dev, uint32_t rows, uint32_t heads,
                          uint32_t hd, uint32_t n_rot)
 {

@@ -59,6 +59,8 @@ def load() -> C.CDLL:
         "wr_hip_attn_sync": (C.c_int, []),
         "wr_hip_attn_stream": (_vp, []),
         "wr_hip_attn_append_dev": (C.c_int, [_vp, _u32, _u32, _u32, _vp, _vp]),
+        "wr_hip_attn_append_batched_dev": (C.c_int, [_u32, C.POINTER(_vp), _u32, C.POINTER(_u32),
+                                                     _vp, _vp]),
         "wr_hip_attn_append_rope": (C.c_int, [_vp, _u32, _u32, _u32, _vp, _vp, _vp, _u32]),
         "wr_hip_attn_rope_dev": (C.c_int, [_vp, _vp, _u32, _u32, _u32, _u32]),
         "wr_hip_attn_decode_batched_dev": (C.c_int, [_u32, C.POINTER(_vp), _u32, C.POINTER(_u32),

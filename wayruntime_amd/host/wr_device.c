@@ -222,13 +222,14 @@ wr_status wrh_forward_rows_device(wr_model *m, wrh_workspace *hs, wrh_devspace *
         if (batch) {
             wr_hip_kv *kvs[WR_BATCH_MAX];
             uint32_t seq_k[WR_BATCH_MAX];
+            uint32_t at[WR_BATCH_MAX];
             for (uint32_t r = 0; r < R; r++) {
-                TRY(wr_hip_attn_append_dev(ss[r]->kv, L, ss[r]->pos, 1, ds->k + (size_t)r * kd,
-                                           ds->v + (size_t)r * kd), "kv append");
-                ss[r]->kv_rows[L] = ss[r]->pos + 1;
                 kvs[r] = ss[r]->kv;
+                at[r] = ss[r]->pos;
                 seq_k[r] = ss[r]->pos + 1;
             }
+            TRY(wr_hip_attn_append_batched_dev(R, kvs, L, at, ds->k, ds->v), "kv append");
+            for (uint32_t r = 0; r < R; r++) ss[r]->kv_rows[L] = ss[r]->pos + 1;
             TRY(wr_hip_attn_decode_batched_dev(R, kvs, L, seq_k, ds->q, ds->attn, nq, 0.0f, 0), "gqa");
         } else {
             wr_session *s = ss[0];
