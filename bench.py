@@ -36,11 +36,11 @@ MFMA_F16_PEAK_TFLOPS = 2500.0   # MI355X dense f16
 # HBM bytes one launch of decode_mfma_kernel<128> moves on the default workload
 # (16 sessions x 4096 ctx): rocprofv3 FETCH_SIZE + WRITE_SIZE per dispatch, each
 # scaled by what the same counter reads for a plain 256 MiB copy kernel
-# (FETCH_SIZE x 1.9998 KiB, WRITE_SIZE x 1.0000 KiB).  Counters cannot be read
+# (FETCH_SIZE x 1.99985 KiB, WRITE_SIZE x 1.00000 KiB).  Counters cannot be read
 # from inside this process, so the figure is carried here from the committed
 # counter summary (profiles/decode_prefill_traffic_pmc.txt) and reported only
 # for the workload it was measured on.
-PMC_TRAFFIC_BYTES = {(16, 4096): 270288670 + 863119}
+PMC_TRAFFIC_BYTES = {(16, 4096): 269496033 + 864256}
 
 
 def pooled16(pool16: np.ndarray, salt: int, n: int) -> np.ndarray:
