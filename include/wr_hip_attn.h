@@ -233,6 +233,24 @@ int wr_hip_proj_rows_dev(const wr_hip_weight *w, uint32_t rows,
                          const float *x_dev, uint32_t ldx,
                          const float *add_dev, float *y_dev, uint32_t ldy);
 
+/* The same product fed by a row step that only exists to feed it, so the
+ * intermediate rows are never written:
+ *   _norm_dev:   y = rmsnorm(x; norm_w_dev [n_in], eps) . W^T (+ add)   (the
+ *                attention / FFN / final norms, session.c:443, 509, 538, each
+ *                followed by products only)
+ *   _swiglu_dev: y = (silu(g) * u) . W^T (+ add), rows of gate_up_dev holding
+ *                g = [0, n_in) and u = [n_in, 2 n_in), ld >= 2 n_in
+ *                (session.c:521-534).
+ * Values are those of wr_hip_rows_rmsnorm_dev / wr_hip_rows_swiglu_dev followed
+ * by wr_hip_proj_rows_dev, bit for bit. */
+int wr_hip_proj_rows_norm_dev(const wr_hip_weight *w, uint32_t rows,
+                              const float *x_dev, uint32_t ldx,
+                              const float *norm_w_dev, float eps,
+                              const float *add_dev, float *y_dev, uint32_t ldy);
+int wr_hip_proj_rows_swiglu_dev(const wr_hip_weight *w, uint32_t rows,
+                                const float *gate_up_dev, uint32_t ld,
+                                const float *add_dev, float *y_dev, uint32_t ldy);
+
 /* ---- row steps between the projections and the attention path --------------
  * For callers that keep a layer's activations on the device.  All arguments
  * are device pointers (wr_hip_attn_dev_alloc), all calls are asynchronous on

@@ -262,6 +262,18 @@ int wr_hip_proj_rows_dev(const wr_hip_weight *w, uint32_t rows, const float *x, 
     (void)w; (void)rows; (void)x; (void)ldx; (void)add; (void)y; (void)ldy;
     return WR_HIP_ERR_STATE;
 }
+int wr_hip_proj_rows_norm_dev(const wr_hip_weight *w, uint32_t rows, const float *x, uint32_t ldx,
+                              const float *nw, float eps, const float *add, float *y, uint32_t ldy)
+{
+    (void)w; (void)rows; (void)x; (void)ldx; (void)nw; (void)eps; (void)add; (void)y; (void)ldy;
+    return WR_HIP_ERR_STATE;
+}
+int wr_hip_proj_rows_swiglu_dev(const wr_hip_weight *w, uint32_t rows, const float *gu, uint32_t ld,
+                                const float *add, float *y, uint32_t ldy)
+{
+    (void)w; (void)rows; (void)gu; (void)ld; (void)add; (void)y; (void)ldy;
+    return WR_HIP_ERR_STATE;
+}
 int wr_hip_rows_rmsnorm_dev(const float *x, uint32_t ldx, const float *w, uint32_t wn, float *out,
                             uint32_t ldo, uint32_t rows, uint32_t dim, float eps)
 {

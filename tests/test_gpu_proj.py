@@ -156,3 +156,45 @@ def test_error_contract():
     assert lib.wr_hip_proj_rows(None, 1, x.ctypes.data, y.ctypes.data) == hipattn.ERR_INVAL
     assert lib.wr_hip_proj_rows(h, 0, x.ctypes.data, y.ctypes.data) == hipattn.OK     # nothing to do
     lib.wr_hip_proj_weight_destroy(h)
+
+
+def test_fused_sources_equal_the_separate_steps():
+    # rmsnorm -> projection and swiglu -> projection in one call each must give
+    # the bits of the separate row step followed by the plain projection
+    lib = hipattn.lib()
+    rows, n_in, n_out = 11, 256, 96
+    x = synth.normal(51, (rows, n_in), std=2.0)
+    nw = synth.normal(52, (n_in,)) * np.float32(0.2) + np.float32(1.0)
+    gu = synth.normal(53, (rows, 2 * n_in), std=2.0)
+    add = synth.normal(54, (rows, n_out))
+    w16 = _w16(55, n_out, n_in, 0.1)
+    w = hipattn.Weight([w16])
+    D = hipattn.DeviceBuffer
+    xd, nwd, gud, addd = D.from_host(x), D.from_host(nw), D.from_host(gu), D.from_host(add)
+    tmp, y1, y2 = D(rows * n_in * 4), D(rows * n_out * 4), D(rows * n_out * 4)
+    eps = 1e-6
+    # norm
+    assert lib.wr_hip_rows_rmsnorm_dev(xd.p, n_in, nwd.p, n_in, tmp.p, n_in, rows, n_in, eps) == hipattn.OK
+    w.rows_dev(rows, tmp, n_in, y1, n_out, add_dev=addd)
+    assert lib.wr_hip_proj_rows_norm_dev(w.h, rows, xd.p, n_in, nwd.p, eps, addd.p, y2.p, n_out) == hipattn.OK
+    hipattn.sync()
+    a, b = y1.to_host((rows, n_out)), y2.to_host((rows, n_out))
+    assert a.tobytes() == b.tobytes()
+    want = oracle.matmul_w16(oracle.rmsnorm(x, nw, eps), w16) + add
+    assert np.max(np.abs(b - want)) <= 1e-5 * np.max(np.abs(want))
+    # swiglu
+    assert lib.wr_hip_rows_swiglu_dev(gud.p, 2 * n_in, tmp.p, n_in, rows, n_in) == hipattn.OK
+    w.rows_dev(rows, tmp, n_in, y1, n_out)
+    assert lib.wr_hip_proj_rows_swiglu_dev(w.h, rows, gud.p, 2 * n_in, None, y2.p, n_out) == hipattn.OK
+    hipattn.sync()
+    a, b = y1.to_host((rows, n_out)), y2.to_host((rows, n_out))
+    assert a.tobytes() == b.tobytes()
+    want = oracle.matmul_w16(oracle.silu_mul(np.ascontiguousarray(gu[:, :n_in]),
+                                             np.ascontiguousarray(gu[:, n_in:])), w16)
+    assert np.max(np.abs(b - want)) <= 1e-5 * np.max(np.abs(want))
+    # contracts: missing norm vector, gate/up stride too small
+    assert lib.wr_hip_proj_rows_norm_dev(w.h, rows, xd.p, n_in, None, eps, None, y2.p, n_out) == hipattn.ERR_INVAL
+    assert lib.wr_hip_proj_rows_swiglu_dev(w.h, rows, gud.p, n_in, None, y2.p, n_out) == hipattn.ERR_INVAL
+    for d in (xd, nwd, gud, addd, tmp, y1, y2):
+        d.free()
+    w.close()

@@ -21,9 +21,8 @@
 //       16g + m holds W[16nt + m][32kt + 8g .. +8]), one contiguous KiB per
 //       operand load; a wave streams the K/32 consecutive KiBs of its outputs.
 //   X   fragments [ceil(R/8)][K/32][64][8] halves, the matching B operands
-//       (lane 16g + c: column c, inputs 32kt + 8g .. +8), written by
-//       proj_prep_kernel, read by every wave (L2 / L1 hits), plus one F32
-//       scale per row (proj_scale_kernel).
+//       (lane 16g + c: column c, inputs 32kt + 8g .. +8), and one F32 scale
+//       per row, written by proj_prep_kernel, read by every wave (L2 / L1 hits).
 //
 // One wave owns 16 outputs for all rows; a workgroup is four waves = 64
 // outputs.  N must be a multiple of 16 and K a multiple of 32.
@@ -54,65 +53,120 @@ __global__ __launch_bounds__(256) void proj_pack_weights_kernel(const uint16_t* 
     tiles[unit] = *src;
 }
 
-// Per-row scale: scales[row] = 2^e with 2^e <= max|x[row]| < 2^(e+1) (1 for a
-// row of zeros).  One wave per row.
-__global__ __launch_bounds__(256) void proj_scale_kernel(const float* __restrict__ x, uint32_t ldx,
-                                                         float* __restrict__ scales, uint32_t R,
-                                                         uint32_t K)
-{
-    const uint32_t lane = threadIdx.x & 63;
-    const uint32_t row = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (row >= R) return;
-    float mx = 0.f;
-    for (uint32_t k = lane; k < K; k += 64) mx = fmaxf(mx, fabsf(x[(size_t)row * ldx + k]));
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) mx = fmaxf(mx, wave_xor_f32(mx, off));
-    if (lane == 0) {
-        uint32_t ex = (__float_as_uint(mx) >> 23) & 0xFFu;
-        if (ex == 0 || ex == 0xFF) ex = 127;              // zeros, subnormals, inf / NaN rows: no scaling
-        if (ex > 253) ex = 253;                           // keeps the inverse 2^-e a normal number
-        scales[row] = __uint_as_float(ex << 23);
-    }
-}
-
-// X[R][K] F32 -> B-operand fragments.  Row r is divided by its scale (exact: a
-// power of two), so its largest magnitude lies in [1, 2), and split into
+// X rows -> B-operand fragments and per-row scales, one workgroup per row
+// (rows past R, which pad the last group of eight, get zero fragments).
+//
+// The row is first brought to its final F32 values v[k] by one of three
+// sources, so that a normalisation or activation that only feeds a projection
+// never has to be written out:
+//   kProjSrcPlain    v = x
+//   kProjSrcRmsNorm  v = x * (1 / sqrt(mean x^2 + eps)) * w     (RMSNorm,
+//                    src/core/kernels.c:1276-1316, same expressions and the
+//                    same reduction tree as rmsnorm_rows_kernel)
+//   kProjSrcSwiglu   v = silu(g) * u, g = x[k], u = x[K + k]   (kernels.c:963-967)
+// Then scales[row] = 2^e with 2^e <= max|v| < 2^(e+1) (1 for a row of zeros),
+// v is divided by it (exact), so its largest magnitude lies in [1, 2), and
+// split into
 //   hi = binary16(v), flushed to zero below the normal range, and
 //   lo = binary16((v - hi) * 2^11),
 // i.e. v = hi + lo * 2^-11 to about 2^-22 |v| (2^-25 of the row's largest value
 // for elements so small that hi is flushed).  Keeping lo scaled up keeps both
 // terms in the normal binary16 range, so the result does not depend on how the
-// matrix cores treat subnormal inputs.  grid = (ceil(K/128), row groups): each
-// wave writes one k tile of one row group.
+// matrix cores treat subnormal inputs.
 constexpr float kProjLoScale = 2048.0f;
+constexpr int kProjSrcPlain = 0, kProjSrcRmsNorm = 1, kProjSrcSwiglu = 2;
 
-__global__ __launch_bounds__(256) void proj_prep_kernel(const float* __restrict__ x, uint32_t ldx,
-                                                        half8* __restrict__ frag,
-                                                        const float* __restrict__ scales, uint32_t R,
-                                                        uint32_t K)
+struct ProjPrepArgs {
+    const float* x;          // [R][ldx]
+    const float* norm_w;     // kProjSrcRmsNorm: [K]
+    half8* frag;             // [groups][K/32][64]
+    float* scales;           // [R]
+    uint32_t ldx, R, K;
+    float eps;
+};
+
+__device__ __forceinline__ float block_sum_256(float v, float* s4)
 {
-    const uint32_t grp = blockIdx.y;
-    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const uint32_t kt = blockIdx.x * 4 + wave;
-    if (kt >= K / 32) return;
-    const uint32_t c = lane & 15, g = lane >> 4;
-    const uint32_t row = grp * 8 + (c & 7);
-    half8 out;
 #pragma unroll
-    for (int j = 0; j < 8; j++) out[j] = (_Float16)0.0f;
-    if (row < R) {
-        // 1 / 2^e: exponent field 254 - field(2^e)
-        const float inv = __uint_as_float((254u << 23) - __float_as_uint(scales[row]));
-        const float* src = x + (size_t)row * ldx + kt * 32 + g * 8;
+    for (int off = 32; off >= 1; off >>= 1) v += wave_xor_f32(v, off);
+    if ((threadIdx.x & 63) == 0) s4[threadIdx.x >> 6] = v;
+    __syncthreads();
+    const float t = (s4[0] + s4[1]) + (s4[2] + s4[3]);
+    __syncthreads();
+    return t;
+}
+
+template <int SRC>
+__device__ __forceinline__ float proj_src_value(const ProjPrepArgs& a, const float* xr, uint32_t k,
+                                                float inv_rms)
+{
+    if constexpr (SRC == kProjSrcRmsNorm) {
+        return xr[k] * inv_rms * a.norm_w[k];
+    } else if constexpr (SRC == kProjSrcSwiglu) {
+        const float g = xr[k], u = xr[a.K + k];
+        const float sig = 1.0f / (1.0f + expf(-g));
+        return (g * sig) * u;
+    } else {
+        return xr[k];
+    }
+}
+
+template <int SRC>
+__global__ __launch_bounds__(256) void proj_prep_kernel(const ProjPrepArgs a)
+{
+    __shared__ float s4[4];
+    const uint32_t row = blockIdx.x, t = threadIdx.x;
+    const uint32_t ktiles = a.K / 32;
+    const uint32_t grp = row / 8, c = row % 8;
+    half8* frow = a.frag + (size_t)grp * ktiles * 64;
+    if (row >= a.R) {                                     // padding row of the last group
+        half8 z;
+#pragma unroll
+        for (int j = 0; j < 8; j++) z[j] = (_Float16)0.0f;
+        for (uint32_t q = t; q < a.K / 8; q += 256) {
+            const uint32_t kt = q >> 2, g = q & 3;
+            frow[(size_t)kt * 64 + 16 * g + c] = z;
+            frow[(size_t)kt * 64 + 16 * g + c + 8] = z;
+        }
+        return;
+    }
+    const float* xr = a.x + (size_t)row * a.ldx;
+    float inv_rms = 1.0f;
+    if constexpr (SRC == kProjSrcRmsNorm) {
+        float ss = 0.f;
+        for (uint32_t k = t; k < a.K; k += 256) {
+            const float v = xr[k];
+            ss += v * v;
+        }
+        inv_rms = 1.0f / sqrtf(block_sum_256(ss, s4) / (float)a.K + a.eps);
+    }
+    float mx = 0.f;
+    for (uint32_t k = t; k < a.K; k += 256) mx = fmaxf(mx, fabsf(proj_src_value<SRC>(a, xr, k, inv_rms)));
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) mx = fmaxf(mx, wave_xor_f32(mx, off));
+    if ((t & 63) == 0) s4[t >> 6] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(s4[0], s4[1]), fmaxf(s4[2], s4[3]));
+    uint32_t ex = (__float_as_uint(mx) >> 23) & 0xFFu;
+    if (ex == 0 || ex == 0xFF) ex = 127;                  // zeros, subnormals, inf / NaN rows: no scaling
+    if (ex > 253) ex = 253;                               // keeps the inverse 2^-e a normal number
+    if (t == 0) a.scales[row] = __uint_as_float(ex << 23);
+    const float inv = __uint_as_float((254u - ex) << 23);
+
+    for (uint32_t q = t; q < a.K / 8; q += 256) {         // 8 consecutive inputs per thread
+        half8 hi, lo;
 #pragma unroll
         for (int j = 0; j < 8; j++) {
-            const float v = src[j] * inv;
-            _Float16 hi = (_Float16)v;
-            if (fabsf((float)hi) < 6.103515625e-05f) hi = (_Float16)0.0f;      // 2^-14
-            out[j] = (c < 8) ? hi : (_Float16)((v - (float)hi) * kProjLoScale);
+            const float v = proj_src_value<SRC>(a, xr, q * 8 + j, inv_rms) * inv;
+            _Float16 h = (_Float16)v;
+            if (fabsf((float)h) < 6.103515625e-05f) h = (_Float16)0.0f;      // 2^-14
+            hi[j] = h;
+            lo[j] = (_Float16)((v - (float)h) * kProjLoScale);
         }
+        const uint32_t kt = q >> 2, g = q & 3;
+        frow[(size_t)kt * 64 + 16 * g + c] = hi;
+        frow[(size_t)kt * 64 + 16 * g + c + 8] = lo;
     }
-    frag[((size_t)grp * (K / 32) + kt) * 64 + lane] = out;
 }
 
 struct ProjArgs {

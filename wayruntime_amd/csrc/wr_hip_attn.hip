@@ -444,10 +444,18 @@ void launch_proj(const ProjArgs& a)
                 dim3(kProjThreads), a);
 }
 
-// y_dev[rows][ldy] = x_dev[rows][ldx] . W^T (+ add_dev), rows <= kProjMaxRows.
+// What feeds a projection: the rows as they are, their RMS normalisation, or
+// the gated activation of rows that hold gate and up values side by side.
+struct ProjSource {
+    int kind = kProjSrcPlain;
+    const float* norm_w = nullptr;
+    float eps = 0.f;
+};
+
+// y_dev[rows][ldy] = source(x_dev)[rows][n_in] . W^T (+ add_dev), rows <= kProjMaxRows.
 // Caller holds g.mu.
 int proj_chunk_locked(const wr_hip_weight* w, uint32_t rows, const float* x_dev, uint32_t ldx,
-                      const float* add_dev, float* y_dev, uint32_t ldy)
+                      const ProjSource& src, const float* add_dev, float* y_dev, uint32_t ldy)
 {
     uint32_t groups = 1;
     while (groups * 8 < rows) groups *= 2;
@@ -457,10 +465,22 @@ int proj_chunk_locked(const wr_hip_weight* w, uint32_t rows, const float* x_dev,
     if (rc) return rc;
     half8* frag = reinterpret_cast<half8*>(g.d_proj.p);
     float* scales = reinterpret_cast<float*>((uint8_t*)g.d_proj.p + frag_bytes);
-    hipLaunchKernelGGL(proj_scale_kernel, dim3((rows + 3) / 4), dim3(256), 0, g.stream, x_dev, ldx,
-                       scales, rows, w->n_in);
-    hipLaunchKernelGGL(proj_prep_kernel, dim3((ktiles + 3) / 4, groups), dim3(256), 0, g.stream, x_dev,
-                       ldx, frag, scales, rows, w->n_in);
+    ProjPrepArgs pa;
+    pa.x = x_dev;
+    pa.norm_w = src.norm_w;
+    pa.frag = frag;
+    pa.scales = scales;
+    pa.ldx = ldx;
+    pa.R = rows;
+    pa.K = w->n_in;
+    pa.eps = src.eps;
+    const dim3 pgrid(groups * 8), pblock(256);
+    if (src.kind == kProjSrcRmsNorm)
+        hipLaunchKernelGGL(proj_prep_kernel<kProjSrcRmsNorm>, pgrid, pblock, 0, g.stream, pa);
+    else if (src.kind == kProjSrcSwiglu)
+        hipLaunchKernelGGL(proj_prep_kernel<kProjSrcSwiglu>, pgrid, pblock, 0, g.stream, pa);
+    else
+        hipLaunchKernelGGL(proj_prep_kernel<kProjSrcPlain>, pgrid, pblock, 0, g.stream, pa);
     ProjArgs a;
     a.w = reinterpret_cast<const half8*>(w->tiles);
     a.xfrag = frag;
@@ -499,11 +519,11 @@ int proj_chunk_locked(const wr_hip_weight* w, uint32_t rows, const float* x_dev,
 }
 
 int proj_locked(const wr_hip_weight* w, uint32_t rows, const float* x_dev, uint32_t ldx,
-                const float* add_dev, float* y_dev, uint32_t ldy)
+                const ProjSource& src, const float* add_dev, float* y_dev, uint32_t ldy)
 {
     for (uint32_t done = 0; done < rows; done += kProjMaxRows) {
         const uint32_t n = rows - done < (uint32_t)kProjMaxRows ? rows - done : (uint32_t)kProjMaxRows;
-        int rc = proj_chunk_locked(w, n, x_dev + (size_t)done * ldx, ldx,
+        int rc = proj_chunk_locked(w, n, x_dev + (size_t)done * ldx, ldx, src,
                                    add_dev ? add_dev + (size_t)done * ldy : nullptr,
                                    y_dev + (size_t)done * ldy, ldy);
         if (rc) return rc;
@@ -1044,29 +1064,56 @@ void wr_hip_proj_weight_destroy(wr_hip_weight* w)
 }
 
 static int check_proj(const wr_hip_weight* w, uint32_t rows, const void* x, uint32_t ldx,
-                      const void* y, uint32_t ldy)
+                      uint32_t min_ldx, const void* y, uint32_t ldy)
 {
     if (!g.inited) return WR_HIP_ERR_STATE;
     if (!w || !x || !y) return WR_HIP_ERR_INVAL;
     if (rows == 0) return WR_HIP_OK;
-    if (ldx < w->n_in || ldy < w->n_out || ldy % 4 != 0) return WR_HIP_ERR_INVAL;
+    if (ldx < min_ldx || ldy < w->n_out || ldy % 4 != 0) return WR_HIP_ERR_INVAL;
     return WR_HIP_OK;
+}
+
+static int proj_dev_common(const wr_hip_weight* w, uint32_t rows, const float* x_dev, uint32_t ldx,
+                           uint32_t min_ldx, const ProjSource& src, const float* add_dev,
+                           float* y_dev, uint32_t ldy)
+{
+    int rc = check_proj(w, rows, x_dev, ldx, min_ldx, y_dev, ldy);
+    if (rc || rows == 0) return rc;
+    if (((uintptr_t)y_dev & 15) || (add_dev && ((uintptr_t)add_dev & 15))) return WR_HIP_ERR_INVAL;
+    Locked lk;
+    return proj_locked(w, rows, x_dev, ldx, src, add_dev, y_dev, ldy);
 }
 
 int wr_hip_proj_rows_dev(const wr_hip_weight* w, uint32_t rows, const float* x_dev, uint32_t ldx,
                          const float* add_dev, float* y_dev, uint32_t ldy)
 {
-    int rc = check_proj(w, rows, x_dev, ldx, y_dev, ldy);
-    if (rc || rows == 0) return rc;
-    if (((uintptr_t)y_dev & 15) || (add_dev && ((uintptr_t)add_dev & 15))) return WR_HIP_ERR_INVAL;
-    Locked lk;
-    return proj_locked(w, rows, x_dev, ldx, add_dev, y_dev, ldy);
+    return proj_dev_common(w, rows, x_dev, ldx, w ? w->n_in : 0, ProjSource(), add_dev, y_dev, ldy);
+}
+
+int wr_hip_proj_rows_norm_dev(const wr_hip_weight* w, uint32_t rows, const float* x_dev,
+                              uint32_t ldx, const float* norm_w_dev, float eps,
+                              const float* add_dev, float* y_dev, uint32_t ldy)
+{
+    if (g.inited && !norm_w_dev) return WR_HIP_ERR_INVAL;
+    ProjSource src;
+    src.kind = kProjSrcRmsNorm;
+    src.norm_w = norm_w_dev;
+    src.eps = eps;
+    return proj_dev_common(w, rows, x_dev, ldx, w ? w->n_in : 0, src, add_dev, y_dev, ldy);
+}
+
+int wr_hip_proj_rows_swiglu_dev(const wr_hip_weight* w, uint32_t rows, const float* gate_up_dev,
+                                uint32_t ld, const float* add_dev, float* y_dev, uint32_t ldy)
+{
+    ProjSource src;
+    src.kind = kProjSrcSwiglu;
+    return proj_dev_common(w, rows, gate_up_dev, ld, w ? 2 * w->n_in : 0, src, add_dev, y_dev, ldy);
 }
 
 int wr_hip_proj_rows(const wr_hip_weight* w, uint32_t rows, const float* x, float* y)
 {
     if (w && (w->n_out % 4 != 0)) return WR_HIP_ERR_INVAL;
-    int rc = check_proj(w, rows, x, w ? w->n_in : 0, y, w ? w->n_out : 0);
+    int rc = check_proj(w, rows, x, w ? w->n_in : 0, w ? w->n_in : 0, y, w ? w->n_out : 0);
     if (rc || rows == 0) return rc;
     const size_t xb = ((size_t)rows * w->n_in * sizeof(float) + 255) & ~(size_t)255;
     const size_t yb = (size_t)rows * w->n_out * sizeof(float);
@@ -1076,7 +1123,7 @@ int wr_hip_proj_rows(const wr_hip_weight* w, uint32_t rows, const float* x, floa
     float* dx = reinterpret_cast<float*>(g.d_stage.p);
     float* dy = reinterpret_cast<float*>((uint8_t*)g.d_stage.p + xb);
     rc = copy_up(dx, x, (size_t)rows * w->n_in * sizeof(float), 0);
-    if (rc == WR_HIP_OK) rc = proj_locked(w, rows, dx, w->n_in, nullptr, dy, w->n_out);
+    if (rc == WR_HIP_OK) rc = proj_locked(w, rows, dx, w->n_in, ProjSource(), nullptr, dy, w->n_out);
     if (rc == WR_HIP_OK) rc = copy_down_sync(y, dy, yb);
     return rc;
 }

@@ -74,6 +74,8 @@ def load() -> C.CDLL:
         "wr_hip_proj_weight_cols": (_u32, [_vp]),
         "wr_hip_proj_rows": (C.c_int, [_vp, _u32, _vp, _vp]),
         "wr_hip_proj_rows_dev": (C.c_int, [_vp, _u32, _vp, _u32, _vp, _vp, _u32]),
+        "wr_hip_proj_rows_norm_dev": (C.c_int, [_vp, _u32, _vp, _u32, _vp, C.c_float, _vp, _vp, _u32]),
+        "wr_hip_proj_rows_swiglu_dev": (C.c_int, [_vp, _u32, _vp, _u32, _vp, _vp, _u32]),
         "wr_hip_rows_rmsnorm_dev": (C.c_int, [_vp, _u32, _vp, _u32, _vp, _u32, _u32, _u32, C.c_float]),
         "wr_hip_rows_qkv_prep_dev": (C.c_int, [_vp, _u32, _u32, _u32, _u32, _u32, _vp, _vp, C.c_float,
                                                _vp, _u32, _vp, _vp, _vp]),

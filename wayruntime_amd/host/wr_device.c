@@ -140,23 +140,20 @@ int wrh_devspace_init(wrh_devspace *ws, const wr_model *m, uint32_t rows, uint32
     memset(ws, 0, sizeof *ws);
     const size_t hidden = m->hidden, qd = (size_t)m->n_q * m->head_dim, kd = (size_t)m->n_kv * m->head_dim;
     const size_t ffn = m->ffn, R = rows;
-    const size_t total = 2 * r64(R * hidden) + r64(R * (qd + 2 * kd)) + 2 * r64(R * qd) + 2 * r64(R * kd) +
-                         r64(R * 2 * ffn) + r64(R * ffn) + r64(R * m->head_dim) +
-                         r64((size_t)logit_rows * m->vocab);
+    const size_t total = r64(R * hidden) + r64(R * (qd + 2 * kd)) + 2 * r64(R * qd) + 2 * r64(R * kd) +
+                         r64(R * 2 * ffn) + r64(R * m->head_dim) + r64((size_t)logit_rows * m->vocab);
     float *b = wr_hip_attn_dev_alloc(total * sizeof(float));
     if (!b) return WR_ERR_NOMEM;
     ws->block = b;
     ws->rows_cap = rows;
     ws->logit_rows = logit_rows;
     ws->resid = b;   b += r64(R * hidden);
-    ws->normed = b;  b += r64(R * hidden);
     ws->qkv = b;     b += r64(R * (qd + 2 * kd));
     ws->q = b;       b += r64(R * qd);
     ws->attn = b;    b += r64(R * qd);
     ws->k = b;       b += r64(R * kd);
     ws->v = b;       b += r64(R * kd);
     ws->gu = b;      b += r64(R * 2 * ffn);
-    ws->act = b;     b += r64(R * ffn);
     ws->rope = b;    b += r64(R * m->head_dim);
     ws->logits = b;
     return WR_OK;
@@ -211,10 +208,8 @@ wr_status wrh_forward_rows_device(wr_model *m, wrh_workspace *hs, wrh_devspace *
 
     for (L = 0; L < m->n_layers; L++) {
         const dev_layer *dl = &d->L[L];
-        TRY(wr_hip_rows_rmsnorm_dev(ds->resid, hidden, dl->attn_norm, hidden, ds->normed, hidden, R,
-                                    hidden, m->rms_eps), "attn norm");
-        TRY(wr_hip_proj_rows_dev(dl->wqkv, R, ds->normed, hidden, NULL, ds->qkv, qd + 2 * kd),
-            "qkv projection");
+        TRY(wr_hip_proj_rows_norm_dev(dl->wqkv, R, ds->resid, hidden, dl->attn_norm, m->rms_eps, NULL,
+                                      ds->qkv, qd + 2 * kd), "attn norm + qkv projection");
         TRY(wr_hip_rows_qkv_prep_dev(ds->qkv, qd + 2 * kd, R, nq, nkv, hd, dl->q_norm, dl->k_norm,
                                      m->rms_eps, ds->rope, n_rot, ds->q, ds->k, ds->v), "qkv prep");
 
@@ -233,7 +228,12 @@ wr_status wrh_forward_rows_device(wr_model *m, wrh_workspace *hs, wrh_devspace *
             TRY(wr_hip_attn_decode_batched_dev(R, kvs, L, seq_k, ds->q, ds->attn, nq, 0.0f, 0), "gqa");
         } else {
             wr_session *s = ss[0];
-            TRY(wr_hip_attn_append_dev(s->kv, L, pos0, R, ds->k, ds->v), "kv append");
+            if (R == 1) {                          /* one launch instead of a K and a V kernel */
+                wr_hip_kv *one[1] = {s->kv};
+                TRY(wr_hip_attn_append_batched_dev(1, one, L, &pos0, ds->k, ds->v), "kv append");
+            } else {
+                TRY(wr_hip_attn_append_dev(s->kv, L, pos0, R, ds->k, ds->v), "kv append");
+            }
             s->kv_rows[L] = pos0 + R;
             if (prefill) {
                 TRY(wr_hip_attn_prefill_dev(s->kv, L, pos0, R, ds->q, ds->attn, nq, 0.0f, 0), "gqa");
@@ -245,20 +245,15 @@ wr_status wrh_forward_rows_device(wr_model *m, wrh_workspace *hs, wrh_devspace *
         }
         TRY(wr_hip_proj_rows_dev(dl->wo, R, ds->attn, qd, ds->resid, ds->resid, hidden),
             "output projection");
-        TRY(wr_hip_rows_rmsnorm_dev(ds->resid, hidden, dl->ffn_norm, hidden, ds->normed, hidden, R,
-                                    hidden, m->rms_eps), "ffn norm");
-        TRY(wr_hip_proj_rows_dev(dl->wgu, R, ds->normed, hidden, NULL, ds->gu, 2 * ffn),
-            "gate/up projection");
-        TRY(wr_hip_rows_swiglu_dev(ds->gu, 2 * ffn, ds->act, ffn, R, ffn), "swiglu");
-        TRY(wr_hip_proj_rows_dev(dl->wdown, R, ds->act, ffn, ds->resid, ds->resid, hidden),
-            "down projection");
+        TRY(wr_hip_proj_rows_norm_dev(dl->wgu, R, ds->resid, hidden, dl->ffn_norm, m->rms_eps, NULL,
+                                      ds->gu, 2 * ffn), "ffn norm + gate/up projection");
+        TRY(wr_hip_proj_rows_swiglu_dev(dl->wdown, R, ds->gu, 2 * ffn, ds->resid, ds->resid, hidden),
+            "swiglu + down projection");
     }
     L = m->n_layers;
-    TRY(wr_hip_rows_rmsnorm_dev(ds->resid, hidden, d->final_norm, hidden, ds->normed, hidden, R,
-                                hidden, m->rms_eps), "final norm");
     if (logits_host && logit_rows) {
-        TRY(wr_hip_proj_rows_dev(d->lm_head, logit_rows, ds->normed, hidden, NULL, ds->logits,
-                                 m->vocab), "lm head");
+        TRY(wr_hip_proj_rows_norm_dev(d->lm_head, logit_rows, ds->resid, hidden, d->final_norm,
+                                      m->rms_eps, NULL, ds->logits, m->vocab), "final norm + lm head");
         TRY(wr_hip_attn_d2h(logits_host, ds->logits, (size_t)logit_rows * m->vocab * sizeof(float)),
             "logits down");
     } else {

@@ -88,11 +88,11 @@ typedef struct wrh_workspace {
 /* Device scratch for R rows of the device walk (wr_device.c). */
 typedef struct wrh_devspace {
     uint32_t rows_cap, logit_rows;
-    float *resid, *normed;               /* [R][hidden] */
+    float *resid;                        /* [R][hidden] */
     float *qkv;                          /* [R][(n_q + 2 n_kv) * hd] */
     float *q, *attn;                     /* [R][n_q*hd] */
     float *k, *v;                        /* [R][n_kv*hd] */
-    float *gu, *act;                     /* [R][2 ffn], [R][ffn] */
+    float *gu;                           /* [R][2 ffn]: gate | up */
     float *rope;                         /* [R][hd/2][2] */
     float *logits;                       /* [logit_rows][vocab] */
     float *block;
