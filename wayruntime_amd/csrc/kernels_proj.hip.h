@@ -193,8 +193,9 @@ __device__ __forceinline__ void proj_step(f32x4 (&acc)[NT][GROUPS], const half8 
     }
 }
 
-// GROUPS = row groups of eight handled per launch, NT = 16-output tiles per
-// wave (templates, so the accumulators stay in registers).  A workgroup is four
+// GROUPS = row groups of eight per wave, NT = 16-output tiles per wave
+// (templates, so the accumulators stay in registers); grid.y walks further
+// runs of GROUPS row groups when a launch carries more rows than that.  A workgroup is four
 // waves.  With ksplit = 1 they own four consecutive runs of 16*NT outputs; with
 // ksplit = 2 or 4 that many waves share a run and take contiguous parts of the
 // input range (a narrow weight then still puts a thousand waves on the chip),
@@ -205,7 +206,7 @@ __device__ __forceinline__ void proj_step(f32x4 (&acc)[NT][GROUPS], const half8 
 template <int GROUPS, int NT>
 __global__ __launch_bounds__(kProjThreads) void proj_rows_kernel(const ProjArgs a)
 {
-    constexpr int KB = (NT == 1) ? kProjKBatch : kProjKBatch / 2;      // k-steps per register batch
+    constexpr int KB = kProjKBatch / NT;                               // k-steps per register batch
     // partial sums of the waves with part > 0: (4 / S) runs x (S - 1) parts <= 3 entries
     __shared__ f32x4 s_part[(GROUPS <= 2) ? 3 * NT * GROUPS * 64 : 1];
 
@@ -219,7 +220,9 @@ __global__ __launch_bounds__(kProjThreads) void proj_rows_kernel(const ProjArgs 
     const uint32_t ktiles = a.K / 32;
     const uint32_t kper = ktiles / S;                            // host guarantees divisibility
     const uint32_t k_begin = part * kper, k_end = k_begin + kper;
-    const half8* xp = a.xfrag + lane;
+    // blockIdx.y: which run of GROUPS row groups (prefill-sized row counts only)
+    const uint32_t group0 = blockIdx.y * GROUPS;
+    const half8* xp = a.xfrag + (size_t)group0 * ktiles * 64 + lane;
 
     f32x4 acc[NT][GROUPS];
 #pragma unroll
@@ -315,7 +318,7 @@ __global__ __launch_bounds__(kProjThreads) void proj_rows_kernel(const ProjArgs 
                     __int_as_float(__builtin_amdgcn_ds_bpermute(partner_addr, __float_as_int(v[i])));
                 v[i] += other * (1.0f / kProjLoScale);      // meaningful in the hi columns only
             }
-            const uint32_t row = gi * 8 + (c & 7);
+            const uint32_t row = (group0 + gi) * 8 + (c & 7);
             if (c < 8 && row < a.R && nt < ntiles) {
                 const float sc = a.scales[row];
                 const size_t o = (size_t)row * a.ldy + nt * 16 + g * 4;

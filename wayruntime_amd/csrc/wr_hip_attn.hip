@@ -436,11 +436,12 @@ struct Locked {
 namespace {
 
 template <int GROUPS, int NT>
-void launch_proj(const ProjArgs& a)
+void launch_proj(const ProjArgs& a, uint32_t groups)
 {
     const uint32_t runs = (a.N / 16 + NT - 1) / NT;              // runs of 16*NT outputs
     const uint32_t per_block = 4 / a.ksplit;
-    launch_main(proj_rows_kernel<GROUPS, NT>, dim3((runs + per_block - 1) / per_block),
+    launch_main(proj_rows_kernel<GROUPS, NT>,
+                dim3((runs + per_block - 1) / per_block, (groups + GROUPS - 1) / GROUPS),
                 dim3(kProjThreads), a);
 }
 
@@ -457,8 +458,9 @@ struct ProjSource {
 int proj_chunk_locked(const wr_hip_weight* w, uint32_t rows, const float* x_dev, uint32_t ldx,
                       const ProjSource& src, const float* add_dev, float* y_dev, uint32_t ldy)
 {
-    uint32_t groups = 1;
-    while (groups * 8 < rows) groups *= 2;
+    // row groups of eight, padded to what one wave takes (1, 2, or runs of 4)
+    uint32_t groups = (rows + 7) / 8;
+    if (groups > 2) groups = (groups + 3) / 4 * 4;
     const uint32_t ktiles = w->n_in / 32;
     const size_t frag_bytes = (size_t)groups * ktiles * 1024;
     int rc = ensure_device(g.d_proj, frag_bytes + kProjMaxRows * sizeof(float));
@@ -506,14 +508,12 @@ int proj_chunk_locked(const wr_hip_weight* w, uint32_t rows, const float* x_dev,
             ksplit *= 2;
     }
     a.ksplit = ksplit;
-    switch (groups) {
-    case 1: launch_proj<1, 1>(a); break;
-    case 2: launch_proj<2, 2>(a); break;
-    case 4: launch_proj<4, 1>(a); break;
-    case 8: launch_proj<8, 1>(a); break;
-    case 16: launch_proj<16, 1>(a); break;
-    default: launch_proj<32, 1>(a); break;
-    }
+    if (groups == 1)
+        launch_proj<1, 1>(a, groups);
+    else if (groups == 2)
+        launch_proj<2, 2>(a, groups);
+    else
+        launch_proj<4, 4>(a, groups);       // grid.y = groups / 4
     HIP_TRY(hipGetLastError(), "projection launch", 0);
     return WR_HIP_OK;
 }
