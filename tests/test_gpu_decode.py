@@ -358,3 +358,27 @@ def test_batched_append_writes_the_same_bits_as_single_appends():
         c.close()
     kd.free()
     vd.free()
+
+
+def test_work_list_at_its_largest():
+    # 16 sessions, each cut into the maximum of 64 key splits: 1024 work-list
+    # entries (the list's capacity), merged in-kernel; the longest-first order
+    # and the per-session results must be unaffected by the other sessions
+    nq, nkv, hd, S = 8, 2, 64, 16
+    ctxs = [2048 - 31 * i for i in range(S)]
+    caches, qs, wants = [], [], []
+    for i, ctx in enumerate(ctxs):
+        q = synth.normal(600 + i, (nq, hd))
+        _a, _b, k16, v16 = util.make_kv(700 + 2 * i, ctx, nkv, hd)
+        kv = hipattn.KVCache(1, hd, nkv, ctx)
+        kv.write_f16(0, 0, k16, v16)
+        caches.append(kv); qs.append(q)
+        wants.append(util.oracle_decode(q, k16, v16, ctx))
+    hipattn.set_tuning(32, False)                 # one 32-key tile per workgroup -> 64 splits each
+    outs = hipattn.decode_batched(caches, 0, ctxs, qs)
+    for i in range(S):
+        util.assert_close(outs[i], wants[i], f"session {i}")
+        assert np.array_equal(caches[i].decode(0, ctxs[i], qs[i]), outs[i]), f"session {i}"
+    hipattn.set_tuning(0, False)
+    for kv in caches:
+        kv.close()
