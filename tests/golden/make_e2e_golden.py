@@ -4,7 +4,7 @@
 Qwen3-0.6B-architecture model (28 layers, hidden 1024, 16/8 heads, head_dim 128,
 F16 weights N(0, 0.02) from seed 0x5EED0100).
 
-    python tests/golden/make_e2e_golden.py [--small | --small16]
+    python tests/golden/make_e2e_golden.py [--small | --small16 | --gemma]
 
 Workload: 128 prompt token ids uniform in [0, vocab) from splitmix64, prefill of
 the first 127, then 129 greedy steps (the last prompt token plus 128 generated
@@ -14,7 +14,10 @@ from "results differ".  --small writes the same for a 2-layer toy model
 (e2e_tiny_golden.npz) that the CPU-only tests can run in a second; --small16
 for a 3-layer toy model whose every dimension is a multiple of 32 (vocab 320),
 the smallest shape that can run with its weights on the device
-(e2e_small16_golden.npz).
+(e2e_small16_golden.npz); --gemma for a 6-layer toy model of the reference's
+Gemma family (local layers with a 16-key window and head_dim 32, global layers
+with head_dim 64 and partial rotary, the last two layers reading earlier
+layers' caches, logit soft cap): e2e_gemma_golden.npz.
 """
 from __future__ import annotations
 
@@ -38,6 +41,11 @@ TINY = gw.ModelShape(n_layers=2, hidden=64, ffn=128, n_q=4, n_kv=2, head_dim=32,
                      context=512)
 SMALL16 = gw.ModelShape(n_layers=3, hidden=128, ffn=256, n_q=4, n_kv=2, head_dim=64, vocab=320,
                         context=512)
+GEMMA_TOY = gw.ModelShape(arch="gemma4", n_layers=6, hidden=96, ffn=160, n_q=4, n_kv=2, head_dim=64,
+                          vocab=288, context=512, rope_base=1e6, head_dim_swa=32, sliding_window=16,
+                          shared_kv_layers=2, swa_pattern=(True, True, False, True, True, False),
+                          softcap=30.0, rope_base_swa=1e4)
+GEMMA_SEED, GEMMA_STD = 0x5EED0102, 0.08     # a seed whose greedy stream has top-2 gaps >= 0.02
 PROBES = 8
 
 
@@ -104,14 +112,19 @@ def run_reference(path: str, prompt: np.ndarray, n_steps: int, max_ctx: int):
 def main() -> None:
     small = "--small" in sys.argv
     small16 = "--small16" in sys.argv
+    gemma = "--gemma" in sys.argv
     oracle.build(ref=True)
-    shape = TINY if small else (SMALL16 if small16 else gw.QWEN3_0_6B)
-    n_prompt, n_steps = (12, 20) if small else ((40, 40) if small16 else (128, 129))
+    shape = TINY if small else (SMALL16 if small16 else (GEMMA_TOY if gemma else gw.QWEN3_0_6B))
+    n_prompt, n_steps = (12, 20) if small else ((40, 40) if (small16 or gemma) else (128, 129))
     out = os.path.join(HERE, "e2e_tiny_golden.npz" if small else
-                       ("e2e_small16_golden.npz" if small16 else "e2e_qwen3_golden.npz"))
+                       ("e2e_small16_golden.npz" if small16 else
+                        ("e2e_gemma_golden.npz" if gemma else "e2e_qwen3_golden.npz")))
     with tempfile.TemporaryDirectory(dir="/tmp") as d:
         path = os.path.join(d, "model.gguf")
-        gw.write_model(path, shape)
+        if gemma:
+            gw.write_model(path, shape, seed=GEMMA_SEED, std=GEMMA_STD)
+        else:
+            gw.write_model(path, shape)
         crc = file_crc(path)
         prompt = workload(shape, n_prompt)
         run_reference.vocab = shape.vocab

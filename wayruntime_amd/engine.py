@@ -21,6 +21,7 @@ WR_OK, WR_ERR_IO, WR_ERR_FORMAT, WR_ERR_UNSUPPORTED, WR_ERR_INVAL = 0, -1, -2, -
 WR_ERR_NOMEM, WR_ERR_CTX_FULL, WR_ERR_STATE, WR_ERR_LIMIT = -5, -6, -7, -8
 WR_ERR_BUSY, WR_ERR_INTERNAL = -9, -10
 WR_BATCH_MAX = 16
+WR_SWA_ENABLED, WR_SWA_DISABLED = 0, 1
 WR_CTR_ATTENTION_CALLS = 3
 
 
@@ -102,15 +103,15 @@ class Engine:
         assert self.lib.wr_engine_counters(self.h, out) == WR_OK
         return list(out)
 
-    def load(self, path: str, max_context: int = 0) -> "Model":
-        return Model(self, path, max_context)
+    def load(self, path: str, max_context: int = 0, swa_mode: int = WR_SWA_ENABLED) -> "Model":
+        return Model(self, path, max_context, swa_mode)
 
 
 class Model:
-    def __init__(self, eng: Engine, path: str, max_context: int = 0):
+    def __init__(self, eng: Engine, path: str, max_context: int = 0, swa_mode: int = WR_SWA_ENABLED):
         self.eng, self.lib = eng, eng.lib
         self.h = C.c_void_p()
-        p = ModelParams(max_context, 0, 0, 0)
+        p = ModelParams(max_context, 0, swa_mode, 0)
         rc = self.lib.wr_model_load(eng.h, path.encode(), C.byref(p), C.byref(self.h))
         if rc != WR_OK:
             raise EngineError(rc, "wr_model_load")

@@ -68,6 +68,7 @@ wr_status wrh_device_model_init(wr_model *m)
     const char *env = getenv("WAYRT_HOST_LAYERS");
     if (env && env[0] == '1') return WR_OK;
     if (!(wr_hip_attn_caps() & WR_HIP_CAP_PROJ)) return WR_OK;
+    if (m->is_gemma) return WR_OK;               /* the Gemma block runs on the host walk */
     const uint32_t qd = m->n_q * m->head_dim, kd = m->n_kv * m->head_dim;
     int ok = proj_dims_ok(&m->lm_head) && m->vocab % 16 == 0 && (qd + 2 * kd) % 16 == 0 &&
              m->hidden % 16 == 0 && (2 * m->ffn) % 16 == 0;

@@ -58,6 +58,17 @@ struct wr_model {
     float      rms_eps, rope_base;
     uint8_t    has_qk_norm, tied_head, all_f16;
 
+    /* Gemma family (reference: src/core/loader.c:576-628): sandwich norms,
+     * GeGLU, embedding scale, attention scale 1.0, per-layer head_dim and
+     * sliding window, KV-shared trailing layers, final-logit soft cap. */
+    uint8_t    is_gemma, has_swa, swa_mode;
+    uint8_t    swa[WRH_MAX_LAYERS];          /* 1 = sliding-window (local) layer */
+    uint32_t   head_dim_swa, sliding_window, kv_shared_layers;
+    uint32_t   hd_layer[WRH_MAX_LAYERS];     /* head_dim of each layer */
+    uint32_t   kv_src[WRH_MAX_LAYERS];       /* layer whose cache layer L reads (L itself if it owns one) */
+    float      rope_base_swa, embed_scale, attn_scale, logit_softcap;
+    wrh_vec    post_attn_norm[WRH_MAX_LAYERS], post_ffw_norm[WRH_MAX_LAYERS];
+
     wrh_weight embed, lm_head;
     wrh_vec    final_norm;
     wrh_vec    attn_norm[WRH_MAX_LAYERS], ffn_norm[WRH_MAX_LAYERS];
@@ -82,6 +93,7 @@ typedef struct wrh_workspace {
     float *gate, *up;                    /* [R][ffn]     */
     float *proj;                         /* [R][hidden]  */
     float *rope;                         /* [R][hd/2][2] (cos, sin) of the rows' angles */
+    float *rope_swa;                     /* the same for Gemma's sliding-window layers */
     void  *block;
 } wrh_workspace;
 
@@ -126,6 +138,10 @@ uint32_t wrh_rope_table(float *cos_sin, uint32_t hd, uint32_t pos, float theta,
                         uint32_t n_rot_pairs);
 void wrh_rope_apply(float *x, uint32_t heads, uint32_t hd, const float *cos_sin, uint32_t n_rot);
 void wrh_swiglu(wr_engine *e, float *gate, const float *up, uint64_t n);
+void wrh_geglu(wr_engine *e, float *gate, const float *up, uint64_t n);
+void wrh_softcap(float *x, uint64_t n, float cap);
+void wrh_scale(float *x, uint64_t n, float s);
+float wrh_tanh(float x);
 void wrh_add(float *acc, const float *x, uint64_t n);
 
 /* ---- model / gguf (wr_model.c) -------------------------------------------- */

@@ -89,3 +89,9 @@ float wrh_cos(float x)
     const float x2 = x * x, x4 = x2 * x2, x6 = x4 * x2;
     return 1.0f - x2 * 0.5f + x4 * (1.0f / 24.0f) - x6 * (1.0f / 720.0f);
 }
+
+/* reference: src/core/mathx.c:158-161 (2/(1+e^-2x) rounds once) */
+float wrh_tanh(float x)
+{
+    return 2.0f / (1.0f + wrh_exp(-2.0f * x)) - 1.0f;
+}

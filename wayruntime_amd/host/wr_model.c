@@ -267,11 +267,44 @@ typedef struct gguf_file {
     uint32_t head_count, head_count_kv, key_length, rope_dim_count, vocab_from_tokens;
     float    rms_eps, rope_base;
     uint32_t alignment;
+    /* Gemma family keys (reference: src/core/gguf.c:920-938) */
+    uint32_t key_length_swa, sliding_window, shared_kv_layers, has_swa_pattern, pl_emb_dim;
+    float    rope_base_swa, softcap;
+    uint8_t  swa_pattern[WRH_MAX_LAYERS];
 } gguf_file;
 
 static int key_is(const char *k, uint64_t klen, const char *lit)
 {
     return klen == strlen(lit) && memcmp(k, lit, klen) == 0;
+}
+
+/* Per-layer sliding-window flags: an array of any scalar type, non-zero = local
+ * layer (reference: src/core/gguf.c:850-881). */
+static void rd_swa_pattern(rd *r, gguf_file *g)
+{
+    const uint32_t et = (uint32_t)rd_int(r, 4);
+    const uint64_t n = rd_int(r, 8);
+    const int sb = scalar_bytes(et);
+    if (!sb) {
+        for (uint64_t i = 0; i < n && !r->bad; i++) rd_skip(r, et, 1);
+        return;
+    }
+    if (n > (uint64_t)(r->end - r->p) / (uint64_t)sb) {
+        r->bad = 1;
+        return;
+    }
+    for (uint64_t k = 0; k < n; k++) {
+        uint32_t u = 0;
+        float f = 0.0f;
+        if (et == GT_BOOL) {
+            u = (uint32_t)rd_int(r, 1);
+        } else {
+            rd_num(r, et, &u, &f);
+            if (f != 0.0f) u = 1;
+        }
+        if (k < WRH_MAX_LAYERS) g->swa_pattern[k] = (uint8_t)(u != 0);
+    }
+    g->has_swa_pattern = 1;
 }
 
 static int parse_gguf(wr_engine *e, gguf_file *g)
@@ -341,6 +374,13 @@ static int parse_gguf(wr_engine *e, gguf_file *g)
                 else if (key_is(sfx, sl, "attention.layer_norm_rms_epsilon")) rd_num(&r, t, NULL, &g->rms_eps);
                 else if (key_is(sfx, sl, "rope.freq_base")) rd_num(&r, t, NULL, &g->rope_base);
                 else if (key_is(sfx, sl, "rope.dimension_count")) rd_num(&r, t, &g->rope_dim_count, NULL);
+                else if (key_is(sfx, sl, "rope.freq_base_swa")) rd_num(&r, t, NULL, &g->rope_base_swa);
+                else if (key_is(sfx, sl, "attention.key_length_swa")) rd_num(&r, t, &g->key_length_swa, NULL);
+                else if (key_is(sfx, sl, "attention.sliding_window")) rd_num(&r, t, &g->sliding_window, NULL);
+                else if (key_is(sfx, sl, "attention.shared_kv_layers")) rd_num(&r, t, &g->shared_kv_layers, NULL);
+                else if (key_is(sfx, sl, "final_logit_softcapping")) rd_num(&r, t, NULL, &g->softcap);
+                else if (key_is(sfx, sl, "embedding_length_per_layer_input")) rd_num(&r, t, &g->pl_emb_dim, NULL);
+                else if (key_is(sfx, sl, "attention.sliding_window_pattern") && t == GT_ARR) rd_swa_pattern(&r, g);
                 else rd_skip(&r, t, 0);
             } else {
                 rd_skip(&r, t, 0);
@@ -487,9 +527,10 @@ wr_status wr_model_load(wr_engine *e, const char *path, const wr_model_params *p
     if (rc != WR_OK) goto fail;
 
     int is_qwen3 = strcmp(g.arch, "qwen3") == 0;
-    if (!is_qwen3 && strcmp(g.arch, "llama") != 0) {
+    const int is_gemma = strcmp(g.arch, "gemma4") == 0;
+    if (!is_qwen3 && !is_gemma && strcmp(g.arch, "llama") != 0) {
         wrh_logf(e, 0, "loader: architecture '%s' is not served by this engine "
-                      "(llama and qwen3 are)", g.arch);
+                      "(llama, qwen3 and gemma4 are)", g.arch);
         rc = WR_ERR_UNSUPPORTED;
         goto fail;
     }
@@ -533,15 +574,75 @@ wr_status wr_model_load(wr_engine *e, const char *path, const wr_model_params *p
     m->train_context = g.context_length;
     m->ffn = g.feed_forward_length;
     m->rope_base = (g.rope_base > 0.0f) ? g.rope_base : 10000.0f;
-    m->has_qk_norm = (uint8_t)is_qwen3;
-    m->rms_eps = (g.rms_eps > 0.0f) ? g.rms_eps : 1e-5f;
-    m->head_dim = g.key_length ? g.key_length : m->hidden / m->n_q;
+    m->has_qk_norm = (uint8_t)(is_qwen3 || is_gemma);
+    m->rms_eps = (g.rms_eps > 0.0f) ? g.rms_eps : (is_gemma ? 1e-6f : 1e-5f);
+    m->head_dim = g.key_length ? g.key_length : (is_gemma ? 0 : m->hidden / m->n_q);
+    if (is_gemma && m->head_dim == 0) {
+        wrh_logf(e, 0, "loader: gemma4 requires %s.attention.key_length", g.arch);
+        rc = WR_ERR_FORMAT;
+        goto fail;
+    }
     if (m->head_dim == 0) m->head_dim = 64;
+    m->attn_scale = 0.0f;                       /* 0 = 1/sqrt(head_dim) */
+    for (uint32_t l = 0; l < m->n_layers; l++) {
+        m->hd_layer[l] = m->head_dim;
+        m->kv_src[l] = l;
+    }
+    if (is_gemma) {
+        /* reference: src/core/loader.c:576-628 */
+        if (g.pl_emb_dim) {
+            wrh_logf(e, 0, "loader: per-layer input tables (embedding_length_per_layer_input=%u) are "
+                          "not served by this engine (WR_ERR_UNSUPPORTED)", g.pl_emb_dim);
+            rc = WR_ERR_UNSUPPORTED;
+            goto fail;
+        }
+        m->is_gemma = 1;
+        m->swa_mode = (uint8_t)p.swa_mode;
+        m->head_dim_swa = g.key_length_swa;
+        m->rope_base_swa = (g.rope_base_swa >= 1.0f) ? g.rope_base_swa : 10000.0f;
+        m->sliding_window = g.sliding_window;
+        m->kv_shared_layers = g.shared_kv_layers;
+        if (m->kv_shared_layers >= m->n_layers) {
+            wrh_logf(e, 0, "loader: shared_kv_layers %u >= block_count %u", m->kv_shared_layers,
+                    m->n_layers);
+            rc = WR_ERR_FORMAT;
+            goto fail;
+        }
+        m->has_swa = (uint8_t)(g.has_swa_pattern ? 1 : 0);
+        for (uint32_t l = 0; l < m->n_layers; l++) {
+            m->swa[l] = (uint8_t)(m->has_swa && g.swa_pattern[l]);
+            if (m->swa[l] && m->head_dim_swa) m->hd_layer[l] = m->head_dim_swa;
+        }
+        /* a shared layer reads the last earlier layer of its own kind that owns a
+         * cache (reference: src/core/session.c:115-134) */
+        if (m->kv_shared_layers) {
+            const uint32_t first_shared = m->n_layers - m->kv_shared_layers;
+            for (uint32_t l = first_shared; l < m->n_layers; l++)
+                for (int c = (int)first_shared - 1; c >= 0; c--)
+                    if (m->swa[c] == m->swa[l]) {
+                        m->kv_src[l] = (uint32_t)c;
+                        break;
+                    }
+        }
+        /* sqrt(hidden) by 24 Newton steps from the value itself, as the reference
+         * computes it (loader.c:46-54) */
+        float gs = (float)m->hidden;
+        for (int i = 0; i < 24; i++) gs = 0.5f * (gs + (float)m->hidden / gs);
+        m->embed_scale = gs;
+        m->attn_scale = 1.0f;                    /* the Q/K norms set the magnitude */
+        m->logit_softcap = g.softcap;
+        m->n_rot_pairs = m->head_dim / 8;        /* partial rotary on global layers */
+        if (m->head_dim_swa & 1) {
+            rc = WR_ERR_FORMAT;
+            goto fail;
+        }
+    }
     if (m->head_dim & 1) {
         rc = WR_ERR_FORMAT;
         goto fail;
     }
-    if (g.rope_dim_count && g.rope_dim_count < m->head_dim) m->n_rot_pairs = g.rope_dim_count / 2;
+    if (!is_gemma && g.rope_dim_count && g.rope_dim_count < m->head_dim)
+        m->n_rot_pairs = g.rope_dim_count / 2;
     if (p.max_context) {
         m->max_context = p.max_context;
     } else {
@@ -551,7 +652,6 @@ wr_status wr_model_load(wr_engine *e, const char *path, const wr_model_params *p
     }
 
     char nb[96];
-    const uint32_t qd = m->n_q * m->head_dim, kd = m->n_kv * m->head_dim;
     if ((rc = bind_matrix(e, &g, "token_embd.weight", m->vocab, m->hidden, 1, &m->embed)) < 0) goto fail;
     if ((rc = bind_vector(e, &g, "output_norm.weight", m->hidden, &m->final_norm)) < 0) goto fail;
     rc = bind_matrix(e, &g, "output.weight", m->vocab, m->hidden, 0, &m->lm_head);
@@ -577,15 +677,21 @@ wr_status wr_model_load(wr_engine *e, const char *path, const wr_model_params *p
             rc = WR_ERR_UNSUPPORTED;
             goto fail;
         }
+        const uint32_t hd_l = m->hd_layer[l];
+        const uint32_t qd = m->n_q * hd_l, kd = m->n_kv * hd_l;
         if ((rc = bind_vector(e, &g, NAME("attn_norm.weight"), m->hidden, &m->attn_norm[l])) < 0) goto fail;
         if ((rc = bind_matrix(e, &g, NAME("attn_q.weight"), qd, m->hidden, 1, &m->wq[l])) < 0) goto fail;
         if ((rc = bind_matrix(e, &g, NAME("attn_k.weight"), kd, m->hidden, 1, &m->wk[l])) < 0) goto fail;
         if ((rc = bind_matrix(e, &g, NAME("attn_v.weight"), kd, m->hidden, 1, &m->wv[l])) < 0) goto fail;
         if (m->has_qk_norm) {
-            if ((rc = bind_vector(e, &g, NAME("attn_q_norm.weight"), m->head_dim, &m->q_norm[l])) < 0) goto fail;
-            if ((rc = bind_vector(e, &g, NAME("attn_k_norm.weight"), m->head_dim, &m->k_norm[l])) < 0) goto fail;
+            if ((rc = bind_vector(e, &g, NAME("attn_q_norm.weight"), hd_l, &m->q_norm[l])) < 0) goto fail;
+            if ((rc = bind_vector(e, &g, NAME("attn_k_norm.weight"), hd_l, &m->k_norm[l])) < 0) goto fail;
         }
         if ((rc = bind_matrix(e, &g, NAME("attn_output.weight"), m->hidden, qd, 1, &m->wo[l])) < 0) goto fail;
+        if (m->is_gemma) {
+            if ((rc = bind_vector(e, &g, NAME("post_attention_norm.weight"), m->hidden, &m->post_attn_norm[l])) < 0) goto fail;
+            if ((rc = bind_vector(e, &g, NAME("post_ffw_norm.weight"), m->hidden, &m->post_ffw_norm[l])) < 0) goto fail;
+        }
         if ((rc = bind_vector(e, &g, NAME("ffn_norm.weight"), m->hidden, &m->ffn_norm[l])) < 0) goto fail;
         if ((rc = bind_matrix(e, &g, NAME("ffn_gate.weight"), m->ffn, m->hidden, 1, &m->w_gate[l])) < 0) goto fail;
         if ((rc = bind_matrix(e, &g, NAME("ffn_up.weight"), m->ffn, m->hidden, 1, &m->w_up[l])) < 0) goto fail;
@@ -653,6 +759,11 @@ wr_status wr_model_get_info(const wr_model *m, wr_model_info *out)
     out->rope_freq_base = m->rope_base;
     out->rms_eps = m->rms_eps;
     out->has_qk_norm = m->has_qk_norm;
+    out->is_gemma = m->is_gemma;
+    out->has_swa = m->has_swa;
+    out->head_dim_swa = m->head_dim_swa;
+    out->sliding_window = m->sliding_window;
+    out->logit_softcap = m->logit_softcap;
     out->tied_lm_head = m->tied_head;
     return WR_OK;
 }

@@ -224,6 +224,31 @@ void wrh_swiglu(wr_engine *e, float *gate, const float *up, uint64_t n)
     }
 }
 
+/* GeGLU, gelu_pytorch_tanh(gate) * up (reference: src/core/kernels.c:969-976 and
+ * wri_op_fused_gelu_mul). */
+void wrh_geglu(wr_engine *e, float *gate, const float *up, uint64_t n)
+{
+    if (e) __atomic_fetch_add(&e->ctr[WR_CTR_FUSED_CALLS], 1, __ATOMIC_RELAXED);
+    for (uint64_t i = 0; i < n; i++) {
+        const float x = gate[i];
+        const float x3 = x * x * x;
+        const float z = 0.7978845608f * (x + 0.044715f * x3);
+        gate[i] = 0.5f * x * (1.0f + wrh_tanh(z)) * up[i];
+    }
+}
+
+/* x = cap * tanh(x / cap): divides, as the reference does (src/core/kernels.c:1576-1584) */
+void wrh_softcap(float *x, uint64_t n, float cap)
+{
+    if (!x || cap <= 0.0f) return;
+    for (uint64_t i = 0; i < n; i++) x[i] = cap * wrh_tanh(x[i] / cap);
+}
+
+void wrh_scale(float *x, uint64_t n, float s)
+{
+    for (uint64_t i = 0; i < n; i++) x[i] *= s;
+}
+
 void wrh_add(float *acc, const float *x, uint64_t n)
 {
     for (uint64_t i = 0; i < n; i++) acc[i] = acc[i] + x[i];

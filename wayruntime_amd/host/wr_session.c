@@ -43,12 +43,15 @@ static size_t round64(size_t n) { return (n + 15) & ~(size_t)15; }   /* floats *
 int wrh_workspace_init(wrh_workspace *ws, const wr_model *m, uint32_t rows)
 {
     memset(ws, 0, sizeof *ws);
+    uint32_t hd_max = m->head_dim;
+    for (uint32_t l = 0; l < m->n_layers; l++)
+        if (m->hd_layer[l] > hd_max) hd_max = m->hd_layer[l];
     const size_t h = round64((size_t)rows * m->hidden);
-    const size_t qd = round64((size_t)rows * m->n_q * m->head_dim);
-    const size_t kd = round64((size_t)rows * m->n_kv * m->head_dim);
+    const size_t qd = round64((size_t)rows * m->n_q * hd_max);
+    const size_t kd = round64((size_t)rows * m->n_kv * hd_max);
     const size_t fd = round64((size_t)rows * m->ffn);
-    const size_t rd = round64((size_t)rows * m->head_dim);
-    const size_t total = 3 * h + 2 * qd + 2 * kd + 2 * fd + rd;
+    const size_t rd = round64((size_t)rows * hd_max);
+    const size_t total = 3 * h + 2 * qd + 2 * kd + 2 * fd + 2 * rd;
     float *b = NULL;
     if (posix_memalign((void **)&b, 64, total * sizeof(float)) != 0 || !b) return WR_ERR_NOMEM;
     ws->block = b;
@@ -62,7 +65,8 @@ int wrh_workspace_init(wrh_workspace *ws, const wr_model *m, uint32_t rows)
     ws->v = b;         b += kd;
     ws->gate = b;      b += fd;
     ws->up = b;        b += fd;
-    ws->rope = b;
+    ws->rope = b;      b += rd;
+    ws->rope_swa = b;
     return WR_OK;
 }
 
@@ -80,6 +84,118 @@ static wr_status op_fail(wr_engine *e, const char *what, uint32_t layer, int rc)
 {
     wrh_logf(e, 0, "session: %s failed at layer %u (rc=%d)", what, layer, rc);
     return (rc < 0) ? (wr_status)rc : WR_ERR_INTERNAL;
+}
+
+/* The Gemma-family block over R already embedded rows (reference:
+ * src/core/session.c:251-437 without the per-layer-input fold): sandwich norms
+ * (the sublayer outputs are normalised before they join the residual), Q/K
+ * RMSNorm per head, rotary embedding with the layer's own base (partial on
+ * global layers, full on sliding-window layers), a weightless RMSNorm of V
+ * before the append, attention with scale 1.0 and the layer's window over the
+ * layer's own cache or, for a KV-shared layer, over its source layer's
+ * (whose rows for these positions are already in place: sources precede
+ * their readers), GeGLU. */
+static wr_status forward_rows_gemma(wr_model *m, wrh_workspace *ws, uint32_t R,
+                                    wr_session *const *ss, uint32_t pos0, fwd_mode mode)
+{
+    wr_engine *e = m->engine;
+    const uint32_t hidden = m->hidden, nq = m->n_q, nkv = m->n_kv, ffn = m->ffn;
+    int rc;
+
+    if (m->embed_scale != 0.0f) wrh_scale(ws->residual, (uint64_t)R * hidden, m->embed_scale);
+
+    /* the rows' angles, once per kind of layer: global (partial rotary, the
+     * model's base) and sliding-window (full rotary, its own base and head_dim) */
+    const uint32_t hd_g = m->head_dim, hd_s = m->head_dim_swa ? m->head_dim_swa : m->head_dim;
+    const uint32_t nrot_g = (m->n_rot_pairs >= 1 && m->n_rot_pairs < hd_g / 2) ? m->n_rot_pairs : hd_g / 2;
+    const uint32_t nrot_s = hd_s / 2;
+    for (uint32_t r = 0; r < R; r++) {
+        const uint32_t p = (mode == FWD_BATCH) ? ss[r]->pos : pos0 + r;
+        (void)wrh_rope_table(ws->rope + (size_t)r * 2 * nrot_g, hd_g, p, m->rope_base, m->n_rot_pairs);
+        if (m->has_swa)
+            (void)wrh_rope_table(ws->rope_swa + (size_t)r * 2 * nrot_s, hd_s, p, m->rope_base_swa, 0);
+    }
+
+    for (uint32_t L = 0; L < m->n_layers; L++) {
+        const int local = m->swa[L];
+        const uint32_t hd = m->hd_layer[L], qd = nq * hd, kd = nkv * hd;
+        const uint32_t ksrc = m->kv_src[L];
+        const int shared = (ksrc != L);
+        const uint32_t window = (local && m->swa_mode != WR_SWA_DISABLED) ? m->sliding_window : 0u;
+        const float *tab = local ? ws->rope_swa : ws->rope;
+        const uint32_t n_rot = local ? nrot_s : nrot_g;
+        const size_t ts = (size_t)2 * n_rot;
+
+        wrh_rmsnorm(ws->residual, m->attn_norm[L].data, m->attn_norm[L].n, ws->normed, R, hidden,
+                    m->rms_eps);
+        wrh_matmul(e, ws->normed, R, hidden, &m->wq[L], ws->q, qd);
+        wrh_rmsnorm(ws->q, m->q_norm[L].data, m->q_norm[L].n, ws->q, R * nq, hd, m->rms_eps);
+        for (uint32_t r = 0; r < R; r++)
+            wrh_rope_apply(ws->q + (size_t)r * qd, nq, hd, tab + r * ts, n_rot);
+        if (!shared) {
+            wrh_matmul(e, ws->normed, R, hidden, &m->wk[L], ws->k, kd);
+            wrh_matmul(e, ws->normed, R, hidden, &m->wv[L], ws->v, kd);
+            wrh_rmsnorm(ws->k, m->k_norm[L].data, m->k_norm[L].n, ws->k, R * nkv, hd, m->rms_eps);
+            wrh_rmsnorm(ws->v, NULL, 0, ws->v, R * nkv, hd, m->rms_eps);
+        }
+
+        if (g_fail_attention_layer == (int)L) {
+            g_fail_attention_layer = -1;
+            return op_fail(e, "gqa (injected)", L, WR_ERR_INTERNAL);
+        }
+        if (mode == FWD_BATCH) {
+            wr_hip_kv *kvs[WR_BATCH_MAX];
+            uint32_t seq_k[WR_BATCH_MAX];
+            const float *qp[WR_BATCH_MAX];
+            float *op[WR_BATCH_MAX];
+            for (uint32_t r = 0; r < R; r++) {
+                if (!shared) {
+                    rc = wr_hip_attn_append_rope(ss[r]->kv, L, ss[r]->pos, 1, ws->k + (size_t)r * kd,
+                                                 ws->v + (size_t)r * kd, tab + r * ts, n_rot);
+                    if (rc != WR_HIP_OK) return (rc == WR_HIP_ERR_CTX_FULL) ? WR_ERR_CTX_FULL
+                                                                             : op_fail(e, "kv append", L, rc);
+                    ss[r]->kv_rows[L] = ss[r]->pos + 1;
+                }
+                kvs[r] = ss[r]->kv;
+                seq_k[r] = ss[r]->pos + 1;
+                qp[r] = ws->q + (size_t)r * qd;
+                op[r] = ws->attn + (size_t)r * qd;
+            }
+            rc = wr_hip_attn_decode_batched(R, kvs, ksrc, seq_k, qp, op, nq, m->attn_scale, window);
+        } else {
+            wr_session *s = ss[0];
+            if (!shared) {
+                rc = wr_hip_attn_append_rope(s->kv, L, pos0, R, ws->k, ws->v, tab, n_rot);
+                if (rc != WR_HIP_OK) return (rc == WR_HIP_ERR_CTX_FULL) ? WR_ERR_CTX_FULL
+                                                                         : op_fail(e, "kv append", L, rc);
+                s->kv_rows[L] = pos0 + R;
+            }
+            if (mode == FWD_STEP)
+                rc = wr_hip_attn_decode(s->kv, ksrc, pos0 + 1, ws->q, ws->attn, nq, m->attn_scale, window);
+            else
+                rc = wr_hip_attn_prefill(s->kv, ksrc, pos0, R, ws->q, ws->attn, nq, m->attn_scale,
+                                         window);
+        }
+        if (rc != WR_HIP_OK) return op_fail(e, "gqa", L, rc);
+
+        wrh_matmul(e, ws->attn, R, qd, &m->wo[L], ws->proj, hidden);
+        wrh_rmsnorm(ws->proj, m->post_attn_norm[L].data, m->post_attn_norm[L].n, ws->proj, R, hidden,
+                    m->rms_eps);
+        wrh_add(ws->residual, ws->proj, (uint64_t)R * hidden);
+
+        wrh_rmsnorm(ws->residual, m->ffn_norm[L].data, m->ffn_norm[L].n, ws->normed, R, hidden,
+                    m->rms_eps);
+        wrh_matmul(e, ws->normed, R, hidden, &m->w_gate[L], ws->gate, ffn);
+        wrh_matmul(e, ws->normed, R, hidden, &m->w_up[L], ws->up, ffn);
+        wrh_geglu(e, ws->gate, ws->up, (uint64_t)R * ffn);
+        wrh_matmul(e, ws->gate, R, ffn, &m->w_down[L], ws->proj, hidden);
+        wrh_rmsnorm(ws->proj, m->post_ffw_norm[L].data, m->post_ffw_norm[L].n, ws->proj, R, hidden,
+                    m->rms_eps);
+        wrh_add(ws->residual, ws->proj, (uint64_t)R * hidden);
+    }
+    wrh_rmsnorm(ws->residual, m->final_norm.data, m->final_norm.n, ws->normed, R, hidden,
+                m->rms_eps);
+    return WR_OK;
 }
 
 /* Forward pass minus the LM head over R rows.
@@ -100,6 +216,8 @@ static wr_status forward_rows(wr_model *m, wrh_workspace *ws, uint32_t R, wr_ses
         rc = wrh_embed(&m->embed, tokens[r], ws->residual + (size_t)r * hidden);
         if (rc != WR_OK) return op_fail(e, "embed", 0, rc);
     }
+
+    if (m->is_gemma) return forward_rows_gemma(m, ws, R, ss, pos0, mode);
 
     for (uint32_t L = 0; L < m->n_layers; L++) {
         wrh_rmsnorm(ws->residual, m->attn_norm[L].data, m->attn_norm[L].n, ws->normed, R, hidden,
@@ -212,8 +330,8 @@ wr_status wr_session_create(wr_model *m, const wr_session_params *params, wr_ses
     s->model = m;
     s->max_context = max_ctx;
     s->last_status = WR_OK;
-    uint32_t hds[WRH_MAX_LAYERS];
-    for (uint32_t L = 0; L < m->n_layers; L++) hds[L] = m->head_dim;
+    uint32_t hds[WRH_MAX_LAYERS];          /* 0 = no cache of its own (KV-shared layer) */
+    for (uint32_t L = 0; L < m->n_layers; L++) hds[L] = (m->kv_src[L] == L) ? m->hd_layer[L] : 0;
     int rc = wr_hip_attn_kv_create(m->n_layers, hds, m->n_kv, max_ctx, &s->kv);
     if (rc != WR_HIP_OK) {
         wrh_logf(m->engine, 0, "session: device cache allocation failed (rc=%d)", rc);
@@ -281,8 +399,10 @@ const float *wr_step(wr_session *s, uint32_t token)
                                          take_fail_layer(m), s->logits, 1);
         } else {
             st = forward_rows(m, &s->ws1, 1, one, &token, s->pos, FWD_STEP);
-            if (st == WR_OK)
+            if (st == WR_OK) {
                 wrh_matmul(m->engine, s->ws1.normed, 1, m->hidden, &m->lm_head, s->logits, m->vocab);
+                if (m->is_gemma) wrh_softcap(s->logits, m->vocab, m->logit_softcap);
+            }
         }
         if (st == WR_OK)
             __atomic_store_n(&s->pos, s->pos + 1, __ATOMIC_RELEASE);
@@ -401,6 +521,7 @@ int wr_batch_step(wr_session *const *sessions, const uint32_t *tokens, uint32_t 
     if (st == WR_OK) {
         /* one LM-head product for all n rows (reference: batch.c:45-104), then demux */
         if (!m->dev) wrh_matmul(m->engine, ws.normed, n, m->hidden, &m->lm_head, big, m->vocab);
+        if (m->is_gemma) wrh_softcap(big, (uint64_t)n * m->vocab, m->logit_softcap);
         for (uint32_t i = 0; i < n; i++)
             memcpy(sessions[i]->logits, big + (size_t)i * m->vocab, (size_t)m->vocab * sizeof(float));
         for (uint32_t i = 0; i < n; i++)
