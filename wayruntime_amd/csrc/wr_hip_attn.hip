@@ -495,7 +495,7 @@ int proj_chunk_locked(const wr_hip_weight* w, uint32_t rows, const float* x_dev,
     a.ldy = ldy;
     // Waves that share a run of outputs (contiguous parts of the inputs, summed
     // through LDS in a fixed order): enough that a narrow weight still gives
-    // about a thousand waves.  A function of the weight's shape only: a row's
+    // one to two thousand waves.  A function of the weight's shape only: a row's
     // sums are then split the same way whether it travels alone or with up to
     // fifteen others, so a batched step's rows equal the serial steps' bit
     // for bit (reference contract: src/core/batch.c:15-19).  Larger row counts
@@ -503,15 +503,17 @@ int proj_chunk_locked(const wr_hip_weight* w, uint32_t rows, const float* x_dev,
     const uint32_t tiles = w->n_out / 16;
     uint32_t ksplit = 1;
     if (groups <= 2) {
-        while (ksplit < 4 && tiles * ksplit < 1024 && ktiles % (ksplit * 2) == 0 &&
+        while (ksplit < 4 && tiles * ksplit < 2048 && ktiles % (ksplit * 2) == 0 &&
                ktiles / (ksplit * 2) >= 4)
             ksplit *= 2;
     }
     a.ksplit = ksplit;
     if (groups == 1)
         launch_proj<1, 1>(a, groups);
+    else if (groups == 2 && tiles * ksplit >= 2048)
+        launch_proj<2, 2>(a, groups);       // wide weight: two output tiles per operand load
     else if (groups == 2)
-        launch_proj<2, 2>(a, groups);
+        launch_proj<2, 1>(a, groups);       // narrow weight: every wave counts
     else
         launch_proj<4, 4>(a, groups);       // grid.y = groups / 4
     HIP_TRY(hipGetLastError(), "projection launch", 0);
