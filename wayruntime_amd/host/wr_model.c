@@ -103,6 +103,16 @@ wr_status wr_engine_create(const wr_engine_config *cfg, wr_engine **out)
         free(e);
         return (wr_status)rc;
     }
+    /* Keys per decode workgroup (0 / unset = the library's batch-oriented
+     * rule).  A deployment that serves one session at a time wants smaller
+     * splits: 256-512 keys halve the attention latency of a single long
+     * session.  The rule stays a function of the session alone either way, so
+     * batched steps still equal serial ones bit for bit. */
+    const char *kpw = getenv("WAYRT_DECODE_KEYS_PER_WG");
+    if (kpw && *kpw && atoi(kpw) > 0) {
+        wr_hip_attn_set_tuning((uint32_t)atoi(kpw), 0);
+        wrh_logf(e, 2, "engine: %d keys per decode workgroup (WAYRT_DECODE_KEYS_PER_WG)", atoi(kpw));
+    }
     wrh_logf(e, 2, "engine ready: version %s, %d host thread(s), device %s", wr_version(),
             e->n_threads, wr_hip_attn_device_name());
     *out = e;
