@@ -47,8 +47,11 @@ def pooled16(pool16: np.ndarray, salt: int, n: int) -> np.ndarray:
     """n F16 bit patterns drawn from a pool of truncated N(0,1) samples at a
     salted offset, sign-flipped for odd salts: distinct per (session, layer),
     still N(0,1), and cheap to make."""
-    off = (salt * 2654435761) % (pool16.size - n)
-    x = pool16[off:off + n].copy()
+    if n > pool16.size // 2:                      # long contexts: the pool repeated, rotated by the salt
+        x = np.resize(np.roll(pool16, -((salt * 40503) % pool16.size)), n)
+    else:
+        off = (salt * 2654435761) % (pool16.size - n)
+        x = pool16[off:off + n].copy()
     if salt & 1:
         x ^= np.uint16(0x8000)
     return x
@@ -68,6 +71,13 @@ def main() -> None:
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-proj", action="store_true")
     ap.add_argument("--keys-per-wg", type=int, default=0)
+    ap.add_argument("--workload", default="headline",
+                    choices=["headline", "ragged16", "long16", "long16-hd256", "batch1"],
+                    help="headline: 16 sessions x --ctx, 32/8/128 (the metric's configuration); "
+                         "ragged16: 16 sessions with contexts drawn from [256, 4096]; "
+                         "long16 / long16-hd256: 16 sessions x 32768 at 32/8/128 / 8/4/256; "
+                         "batch1: one session, 16/8/128, --ctx keys.  Other than headline they "
+                         "report the decode figures only")
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -80,6 +90,22 @@ def main() -> None:
     hipattn.init(0)
     nq, nkv, hd = 32, 8, 128
     S, ctx, L = args.sessions, args.ctx, args.layers
+    ctxs = None
+    if args.workload == "ragged16":
+        S = 16
+        ctxs = [int(c) for c in synth.ragged_contexts(synth.config_seed(3, 0), S, 256, 4096)]
+    elif args.workload in ("long16", "long16-hd256"):
+        S, ctx, L = 16, 32768, 2
+        if args.workload == "long16-hd256":
+            nq, nkv, hd = 8, 4, 256
+    elif args.workload == "batch1":
+        nq, S, L = 16, 1, max(L, 16)
+    if ctxs is None:
+        ctxs = [ctx] * S
+    secondary = args.workload != "headline"
+    if secondary:
+        args.no_prefill = args.no_proj = True
+        args.cpu_seconds = 0.0
     row = nkv * hd
 
     t0 = time.time()
@@ -87,20 +113,23 @@ def main() -> None:
     caches = []
     host_kv = {}                                    # (session) -> (k16, v16) of layer 0, for checks
     for s in range(S):
-        kv = hipattn.KVCache(L, hd, nkv, ctx)
+        c = ctxs[s]
+        kv = hipattn.KVCache(L, hd, nkv, c)
         for layer in range(L):
-            k16 = pooled16(pool16, 1 + 2 * (s * L + layer), ctx * row)
-            v16 = pooled16(pool16, 2 + 2 * (s * L + layer), ctx * row)
-            k16 = k16.reshape(ctx, nkv, hd)
-            v16 = v16.reshape(ctx, nkv, hd)
+            k16 = pooled16(pool16, 1 + 2 * (s * L + layer), c * row)
+            v16 = pooled16(pool16, 2 + 2 * (s * L + layer), c * row)
+            k16 = k16.reshape(c, nkv, hd)
+            v16 = v16.reshape(c, nkv, hd)
             kv.write_f16(layer, 0, k16, v16)
-            if layer == 0:
+            if layer == 0 and s == 0:
+                host_kv[s] = (k16, v16)
+            elif layer == 0 and not secondary:
                 host_kv[s] = (k16, v16)
         caches.append(kv)
     q_host = synth.normal(synth.config_seed(3, 1), (L, S, nq, hd))
     q_dev = hipattn.DeviceBuffer.from_host(q_host)
     out_dev = hipattn.DeviceBuffer(S * nq * hd * 4)
-    seq_k = [ctx] * S
+    seq_k = list(ctxs)
     step_q_bytes = S * nq * hd * 4
     setup_s = time.time() - t0
 
@@ -140,7 +169,7 @@ def main() -> None:
     hipattn.sync()
     wall = time.perf_counter() - t
     ms_per_step = wall * 1e3 / args.steps
-    bytes_per_step = 2 * 2 * nkv * hd * ctx * S              # K and V, two bytes each
+    bytes_per_step = 2 * 2 * nkv * hd * sum(ctxs)            # K and V, two bytes each
     value = bytes_per_step / (ms_per_step * 1e-3) / 1e9
 
     # ---- dominant kernel alone, per-launch events
@@ -151,9 +180,10 @@ def main() -> None:
     kern_ms, n_timed = hipattn.profile_end()
     kern_avg_ms = kern_ms / max(n_timed, 1)
     achieved = bytes_per_step / (kern_avg_ms * 1e-3) / 1e9
-    roofline = {"bound": "hbm", "kernel": "decode_mfma_kernel<128>", "achieved": round(achieved, 1),
+    roofline = {"bound": "hbm", "kernel": "decode_mfma_kernel<%d>" % hd, "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                "traffic": PMC_TRAFFIC_BYTES.get((S, ctx)), "kernel_avg_us": round(kern_avg_ms * 1e3, 2),
+                "traffic": PMC_TRAFFIC_BYTES.get((S, ctx)) if not secondary else None,
+                "kernel_avg_us": round(kern_avg_ms * 1e3, 2),
                 "bytes_per_launch": bytes_per_step}
 
     # ---- causal prefill (secondary figure of the metric)
@@ -267,9 +297,13 @@ def main() -> None:
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f16 cache, f32 accumulate",
         "data": "synthetic",
-        "config": {"workload": "batched decode attention, Llama-3-8B head shape 32/8/128, "
-                               "%d sessions x %d ctx, %d cache layers walked" % (S, ctx, L),
-                   "sessions": S, "ctx": ctx, "layers": L},
+        "config": {"workload": ("batched decode attention, Llama-3-8B head shape 32/8/128, "
+                                "%d sessions x %d ctx, %d cache layers walked" % (S, ctx, L))
+                   if not secondary else
+                   ("decode attention, head shape %d/%d/%d, %d session(s), contexts %d..%d "
+                    "(%s), %d cache layers walked" % (nq, nkv, hd, S, min(ctxs), max(ctxs),
+                                                      args.workload, L)),
+                   "sessions": S, "ctx": ctx if len(set(ctxs)) == 1 else ctxs, "layers": L},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
         "roofline": roofline, "cpu_baseline": cpu, "prefill": prefill, "projection": proj,
         "check": {"max_abs": max_abs, "rel_l2": rel_l2},
