@@ -24,8 +24,9 @@
 //       (lane 16g + c: column c, inputs 32kt + 8g .. +8), and one F32 scale
 //       per row, written by proj_prep_kernel, read by every wave (L2 / L1 hits).
 //
-// One wave owns 16 outputs for all rows; a workgroup is four waves = 64
-// outputs.  N must be a multiple of 16 and K a multiple of 32.
+// A wave owns one to four 16-output tiles for one to four row groups of eight;
+// a workgroup is four waves (see proj_rows_kernel).  N must be a multiple of
+// 16 and K a multiple of 32.
 #pragma once
 
 #include "common.hip.h"
