@@ -97,6 +97,35 @@ __device__ __forceinline__ float block_sum_256(float v, float* s4)
     return t;
 }
 
+__device__ __forceinline__ float block_max_256(float v, float* s4)
+{
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, wave_xor_f32(v, off));
+    if ((threadIdx.x & 63) == 0) s4[threadIdx.x >> 6] = v;
+    __syncthreads();
+    const float t = fmaxf(fmaxf(s4[0], s4[1]), fmaxf(s4[2], s4[3]));
+    __syncthreads();
+    return t;
+}
+
+// Sum of squares of a row by a 256-thread workgroup.  Thread t takes the
+// chunks of eight values t, t + 256, ... in order; the partial sums go through
+// a wave tree and the four waves are added pairwise.  Every kernel that
+// normalises a row uses this order, so a norm computed inside the fragment
+// kernel has the bits of rmsnorm_rows_kernel.
+__device__ __forceinline__ float row_sumsq_256(const float* __restrict__ xr, uint32_t K, float* s4)
+{
+    float ss = 0.f;
+    for (uint32_t k0 = threadIdx.x * 8; k0 < K; k0 += 2048) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const float v = (k0 + j < K) ? xr[k0 + j] : 0.f;
+            ss = fmaf(v, v, ss);          // explicit, so every copy of this sum rounds alike
+        }
+    }
+    return block_sum_256(ss, s4);
+}
+
 template <int SRC>
 __device__ __forceinline__ float proj_src_value(const ProjPrepArgs& a, const float* xr, uint32_t k,
                                                 float inv_rms)
@@ -112,19 +141,40 @@ __device__ __forceinline__ float proj_src_value(const ProjPrepArgs& a, const flo
     }
 }
 
-template <int SRC>
+__device__ __forceinline__ void proj_write_chunk(half8* frow, uint32_t q, uint32_t c,
+                                                 const float (&v)[8], float inv)
+{
+    half8 hi, lo;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const float s = v[j] * inv;
+        _Float16 h = (_Float16)s;
+        if (fabsf((float)h) < 6.103515625e-05f) h = (_Float16)0.0f;      // 2^-14
+        hi[j] = h;
+        lo[j] = (_Float16)((s - (float)h) * kProjLoScale);
+    }
+    const uint32_t kt = q >> 2, g = q & 3;
+    frow[(size_t)kt * 64 + 16 * g + c] = hi;
+    frow[(size_t)kt * 64 + 16 * g + c + 8] = lo;
+}
+
+// CH > 0: K <= 2048 * CH and the row's values are held in registers between
+// the passes (one read of the row: a single-row call is pure latency, and each
+// pass over global memory is a round trip).  CH = 0: any K, the passes re-read
+// (and re-compute) the row.
+template <int SRC, int CH>
 __global__ __launch_bounds__(256) void proj_prep_kernel(const ProjPrepArgs a)
 {
     __shared__ float s4[4];
     const uint32_t row = blockIdx.x, t = threadIdx.x;
-    const uint32_t ktiles = a.K / 32;
+    const uint32_t ktiles = a.K / 32, nchunks = a.K / 8;
     const uint32_t grp = row / 8, c = row % 8;
     half8* frow = a.frag + (size_t)grp * ktiles * 64;
     if (row >= a.R) {                                     // padding row of the last group
         half8 z;
 #pragma unroll
         for (int j = 0; j < 8; j++) z[j] = (_Float16)0.0f;
-        for (uint32_t q = t; q < a.K / 8; q += 256) {
+        for (uint32_t q = t; q < nchunks; q += 256) {
             const uint32_t kt = q >> 2, g = q & 3;
             frow[(size_t)kt * 64 + 16 * g + c] = z;
             frow[(size_t)kt * 64 + 16 * g + c + 8] = z;
@@ -132,41 +182,76 @@ __global__ __launch_bounds__(256) void proj_prep_kernel(const ProjPrepArgs a)
         return;
     }
     const float* xr = a.x + (size_t)row * a.ldx;
-    float inv_rms = 1.0f;
-    if constexpr (SRC == kProjSrcRmsNorm) {
-        float ss = 0.f;
-        for (uint32_t k = t; k < a.K; k += 256) {
-            const float v = xr[k];
-            ss += v * v;
-        }
-        inv_rms = 1.0f / sqrtf(block_sum_256(ss, s4) / (float)a.K + a.eps);
-    }
-    float mx = 0.f;
-    for (uint32_t k = t; k < a.K; k += 256) mx = fmaxf(mx, fabsf(proj_src_value<SRC>(a, xr, k, inv_rms)));
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) mx = fmaxf(mx, wave_xor_f32(mx, off));
-    if ((t & 63) == 0) s4[t >> 6] = mx;
-    __syncthreads();
-    mx = fmaxf(fmaxf(s4[0], s4[1]), fmaxf(s4[2], s4[3]));
-    uint32_t ex = (__float_as_uint(mx) >> 23) & 0xFFu;
-    if (ex == 0 || ex == 0xFF) ex = 127;                  // zeros, subnormals, inf / NaN rows: no scaling
-    if (ex > 253) ex = 253;                               // keeps the inverse 2^-e a normal number
-    if (t == 0) a.scales[row] = __uint_as_float(ex << 23);
-    const float inv = __uint_as_float((254u - ex) << 23);
 
-    for (uint32_t q = t; q < a.K / 8; q += 256) {         // 8 consecutive inputs per thread
-        half8 hi, lo;
+    if constexpr (CH > 0) {
+        float v[CH][8];
+        float ss = 0.f;
 #pragma unroll
-        for (int j = 0; j < 8; j++) {
-            const float v = proj_src_value<SRC>(a, xr, q * 8 + j, inv_rms) * inv;
-            _Float16 h = (_Float16)v;
-            if (fabsf((float)h) < 6.103515625e-05f) h = (_Float16)0.0f;      // 2^-14
-            hi[j] = h;
-            lo[j] = (_Float16)((v - (float)h) * kProjLoScale);
+        for (int i = 0; i < CH; i++) {
+            const uint32_t q = t + 256 * i;
+#pragma unroll
+            for (int j = 0; j < 8; j++) v[i][j] = (q < nchunks) ? xr[q * 8 + j] : 0.f;
+            if constexpr (SRC == kProjSrcRmsNorm) {
+#pragma unroll
+                for (int j = 0; j < 8; j++) ss = fmaf(v[i][j], v[i][j], ss);
+            }
         }
-        const uint32_t kt = q >> 2, g = q & 3;
-        frow[(size_t)kt * 64 + 16 * g + c] = hi;
-        frow[(size_t)kt * 64 + 16 * g + c + 8] = lo;
+        float mx = 0.f;
+        if constexpr (SRC == kProjSrcRmsNorm) {
+            const float inv_rms = 1.0f / sqrtf(block_sum_256(ss, s4) / (float)a.K + a.eps);
+#pragma unroll
+            for (int i = 0; i < CH; i++) {
+                const uint32_t q = t + 256 * i;
+#pragma unroll
+                for (int j = 0; j < 8; j++)
+                    v[i][j] = (q < nchunks) ? v[i][j] * inv_rms * a.norm_w[q * 8 + j] : 0.f;
+            }
+        } else if constexpr (SRC == kProjSrcSwiglu) {
+#pragma unroll
+            for (int i = 0; i < CH; i++) {
+                const uint32_t q = t + 256 * i;
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    const float g = v[i][j];
+                    const float u = (q < nchunks) ? xr[a.K + q * 8 + j] : 0.f;
+                    const float sig = 1.0f / (1.0f + expf(-g));
+                    v[i][j] = (g * sig) * u;
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < CH; i++)
+#pragma unroll
+            for (int j = 0; j < 8; j++) mx = fmaxf(mx, fabsf(v[i][j]));
+        mx = block_max_256(mx, s4);
+        uint32_t ex = (__float_as_uint(mx) >> 23) & 0xFFu;
+        if (ex == 0 || ex == 0xFF) ex = 127;              // zeros, subnormals, inf / NaN rows: no scaling
+        if (ex > 253) ex = 253;                           // keeps the inverse 2^-e a normal number
+        if (t == 0) a.scales[row] = __uint_as_float(ex << 23);
+        const float inv = __uint_as_float((254u - ex) << 23);
+#pragma unroll
+        for (int i = 0; i < CH; i++) {
+            const uint32_t q = t + 256 * i;
+            if (q < nchunks) proj_write_chunk(frow, q, c, v[i], inv);
+        }
+    } else {
+        float inv_rms = 1.0f;
+        if constexpr (SRC == kProjSrcRmsNorm)
+            inv_rms = 1.0f / sqrtf(row_sumsq_256(xr, a.K, s4) / (float)a.K + a.eps);
+        float mx = 0.f;
+        for (uint32_t k = t; k < a.K; k += 256) mx = fmaxf(mx, fabsf(proj_src_value<SRC>(a, xr, k, inv_rms)));
+        mx = block_max_256(mx, s4);
+        uint32_t ex = (__float_as_uint(mx) >> 23) & 0xFFu;
+        if (ex == 0 || ex == 0xFF) ex = 127;
+        if (ex > 253) ex = 253;
+        if (t == 0) a.scales[row] = __uint_as_float(ex << 23);
+        const float inv = __uint_as_float((254u - ex) << 23);
+        for (uint32_t q = t; q < nchunks; q += 256) {     // 8 consecutive inputs per thread
+            float v[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) v[j] = proj_src_value<SRC>(a, xr, q * 8 + j, inv_rms);
+            proj_write_chunk(frow, q, c, v, inv);
+        }
     }
 }
 

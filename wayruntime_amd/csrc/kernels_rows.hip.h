@@ -11,6 +11,7 @@
 #pragma once
 
 #include "common.hip.h"
+#include "kernels_proj.hip.h"      // row_sumsq_256: the one summation order of every row norm
 
 namespace wr {
 
@@ -33,15 +34,7 @@ __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const float* __restri
     __shared__ float s_sum[4];
     const uint32_t r = blockIdx.x;
     const float* xr = x + (size_t)r * ldx;
-    float ss = 0.f;
-    for (uint32_t j = threadIdx.x; j < dim; j += 256) {
-        const float v = xr[j];
-        ss += v * v;
-    }
-    ss = wave_sum_f32(ss);
-    if ((threadIdx.x & 63) == 0) s_sum[threadIdx.x >> 6] = ss;
-    __syncthreads();
-    const float total = (s_sum[0] + s_sum[1]) + (s_sum[2] + s_sum[3]);
+    const float total = row_sumsq_256(xr, dim, s_sum);
     const float inv_rms = 1.0f / sqrtf(total / (float)dim + eps);
     float* orow = out + (size_t)r * ldo;
     for (uint32_t j = threadIdx.x; j < dim; j += 256) {

@@ -477,12 +477,21 @@ int proj_chunk_locked(const wr_hip_weight* w, uint32_t rows, const float* x_dev,
     pa.K = w->n_in;
     pa.eps = src.eps;
     const dim3 pgrid(groups * 8), pblock(256);
+    const bool in_regs = w->n_in <= 4096;           // two chunks of eight values per thread
+#define WR_LAUNCH_PREP(SRC)                                                                          \
+    do {                                                                                             \
+        if (in_regs)                                                                                 \
+            hipLaunchKernelGGL(HIP_KERNEL_NAME(proj_prep_kernel<SRC, 2>), pgrid, pblock, 0, g.stream, pa); \
+        else                                                                                         \
+            hipLaunchKernelGGL(HIP_KERNEL_NAME(proj_prep_kernel<SRC, 0>), pgrid, pblock, 0, g.stream, pa); \
+    } while (0)
     if (src.kind == kProjSrcRmsNorm)
-        hipLaunchKernelGGL(proj_prep_kernel<kProjSrcRmsNorm>, pgrid, pblock, 0, g.stream, pa);
+        WR_LAUNCH_PREP(kProjSrcRmsNorm);
     else if (src.kind == kProjSrcSwiglu)
-        hipLaunchKernelGGL(proj_prep_kernel<kProjSrcSwiglu>, pgrid, pblock, 0, g.stream, pa);
+        WR_LAUNCH_PREP(kProjSrcSwiglu);
     else
-        hipLaunchKernelGGL(proj_prep_kernel<kProjSrcPlain>, pgrid, pblock, 0, g.stream, pa);
+        WR_LAUNCH_PREP(kProjSrcPlain);
+#undef WR_LAUNCH_PREP
     ProjArgs a;
     a.w = reinterpret_cast<const half8*>(w->tiles);
     a.xfrag = frag;
