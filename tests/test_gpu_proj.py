@@ -50,7 +50,11 @@ def _check(got, x, w16, what):
     (3, 320, 16, 1.0),            # ten input tiles: one batch and a tail; a single output tile
     (8, 32, 64, 1.0),             # one input tile
     (17, 512, 80, 0.1),           # rows pad to four groups of eight; outputs not a multiple of 64
-    (300, 256, 128, 0.1),         # more rows than one launch takes
+    (300, 256, 128, 0.1),         # prefill-sized: the register-tiled kernel, small tile
+    (64, 96, 48, 0.5),            # ... its smallest row count; three input tiles (odd), three output tiles
+    (100, 160, 80, 0.3),          # ... a last row group of four rows, five input tiles
+    (1030, 64, 32, 1.0),          # more rows than one launch takes: 1024 + a six-row launch
+    (1000, 1056, 4112, 0.02),     # the large tile, with a partial output panel, row panel and odd input tiles
 ])
 def test_projection_shapes_vs_oracle(rows, n_in, n_out, std):
     print("proj", rows, n_in, n_out, flush=True)
@@ -114,8 +118,9 @@ def test_row_magnitudes_do_not_matter():
     w.close()
 
 
-def test_device_form_with_strides_and_residual_add():
-    rows, n_in, n_out = 6, 128, 64
+@pytest.mark.parametrize("rows", [6, 70])           # the row kernel and the register-tiled one
+def test_device_form_with_strides_and_residual_add(rows):
+    n_in, n_out = 128, 64
     ldx, ldy = n_in + 32, n_out + 8
     x = synth.normal(31, (rows, ldx))
     add = synth.normal(32, (rows, ldy))

@@ -34,7 +34,7 @@
 namespace wr {
 
 constexpr int kProjThreads = 256;
-constexpr int kProjMaxRows = 256;                 // rows per launch (32 row groups)
+constexpr int kProjMaxRows = 1024;                // rows per launch (128 row groups)
 constexpr int kProjKBatch = 8;                    // k-steps (KiBs of W) a wave keeps in flight per buffer
 
 // Row-major F16 W[N][K] -> tile order.  One thread per 16-byte unit.
@@ -265,6 +265,36 @@ struct ProjArgs {
     uint32_t ksplit;         // waves of a workgroup that share one run of outputs: 1, 2 or 4
 };
 
+// Writes one accumulator tile.  Layout: lane 16g + c holds outputs 16nt + 4g .. +3
+// of column c; column c (< 8) is the hi term of row c of the group, column c + 8
+// its lo term.  The two are combined, the row's scale undone, the optional
+// residual added.  Tiles past N and rows past R are dropped.
+__device__ __forceinline__ void proj_store_tile(const ProjArgs& a, f32x4 v, uint32_t nt, uint32_t group,
+                                                int lane)
+{
+    const int c = lane & 15, g = lane >> 4;
+    const int partner_addr = (lane ^ 8) * 4;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const float other = __int_as_float(__builtin_amdgcn_ds_bpermute(partner_addr, __float_as_int(v[i])));
+        v[i] += other * (1.0f / kProjLoScale);      // meaningful in the hi columns only
+    }
+    const uint32_t row = group * 8 + (c & 7);
+    if (c < 8 && row < a.R && nt < a.N / 16) {
+        const float sc = a.scales[row];
+        const size_t o = (size_t)row * a.ldy + nt * 16 + g * 4;
+        f32x4 r;
+#pragma unroll
+        for (int i = 0; i < 4; i++) r[i] = v[i] * sc;
+        if (a.bias_rows) {
+            const f32x4 b = *reinterpret_cast<const f32x4*>(a.bias_rows + o);
+#pragma unroll
+            for (int i = 0; i < 4; i++) r[i] += b[i];
+        }
+        *reinterpret_cast<f32x4*>(a.y + o) = r;
+    }
+}
+
 // One wave-step: NT weight tiles against GROUPS operand fragments.
 template <int GROUPS, int NT>
 __device__ __forceinline__ void proj_step(f32x4 (&acc)[NT][GROUPS], const half8 (&wv)[NT],
@@ -388,38 +418,124 @@ __global__ __launch_bounds__(kProjThreads) void proj_rows_kernel(const ProjArgs 
     }
     if (!live) return;
 
-    // Accumulator layout: lane 16g + c holds outputs 16nt + 4g .. +3 of column c.
-    // Column c (< 8) is the hi term of row c, column c + 8 its lo term.
-    const int c = lane & 15, g = lane >> 4;
-    const int partner_addr = (lane ^ 8) * 4;
 #pragma unroll
-    for (int t = 0; t < NT; t++) {
-        const uint32_t nt = nt0 + t;
+    for (int t = 0; t < NT; t++)
 #pragma unroll
-        for (int gi = 0; gi < GROUPS; gi++) {
-            f32x4 v = acc[t][gi];
+        for (int gi = 0; gi < GROUPS; gi++) proj_store_tile(a, acc[t][gi], nt0 + t, group0 + gi, lane);
+}
+
+// Many rows (prefill chunks): a register-tiled GEMM on the same two layouts.
+// A wave owns NT x GROUPS accumulator tiles (16 NT outputs x 8 GROUPS rows):
+// every k-step loads NT weight tiles and GROUPS operand fragments, one KiB each
+// and both already in operand order, and feeds NT x GROUPS MFMAs, so a loaded
+// byte serves GROUPS (weights) or NT (rows) MFMAs instead of the four of
+// proj_rows_kernel.  The next k-step's operands are requested while this one's
+// MFMAs run (two register sets, the loop unrolled by two so no set is copied).
+//
+// KS = 1: a workgroup is 2 x 2 waves, each with its own tile and the whole input
+// range; the two waves of a row pair share weight tiles, the two of a column
+// pair share fragments (vector-cache hits).  For products large enough to give
+// every CU such a workgroup.
+// KS = 4: the four waves share one tile and take a quarter of the input range
+// each; their sums are added through LDS in wave order.  Four times the waves
+// and a quarter of the dependent k-steps: for products that would otherwise
+// leave a CU with one wave per SIMD waiting on its own loads.
+//
+// grid.x walks the output panels, so the workgroups the dispatcher deals
+// round-robin to the eight XCDs differ in output panel: one XCD's L2 holds an
+// eighth of the weight and all of the fragments.  Two workgroups per CU at
+// least (<= 256 registers), which also keeps the accumulators in ordinary
+// vector registers.
+template <int GROUPS, int NT, int KS>
+__global__ __launch_bounds__(kProjThreads, KS == 1 ? 2 : 3) void proj_gemm_kernel(const ProjArgs a)
+{
+    static_assert(KS == 1 || KS == 4, "whole range per wave, or four waves per tile");
+    __shared__ f32x4 s_red[KS == 4 ? 3 * NT * GROUPS * 64 : 1];
+    const int lane = threadIdx.x & 63;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t ktiles = a.K / 32, ntiles = a.N / 16, ngroups = (a.R + 7) / 8;
+    const uint32_t nt0 = (KS == 1 ? blockIdx.x * 2 + (wave & 1) : blockIdx.x) * NT;
+    const uint32_t group0 = (KS == 1 ? blockIdx.y * 2 + (wave >> 1) : blockIdx.y) * GROUPS;
+    if (nt0 >= ntiles || group0 >= ngroups) return;       // KS = 4: the same for all four waves
+    const uint32_t k_begin = KS == 1 ? 0 : ktiles * wave / 4;
+    const uint32_t k_end = KS == 1 ? ktiles : ktiles * (wave + 1) / 4;
+
+    // a tile or group past the end re-reads the last one; its result is dropped
+    const half8* wp[NT];
+    const half8* xp[GROUPS];
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const float other =
-                    __int_as_float(__builtin_amdgcn_ds_bpermute(partner_addr, __float_as_int(v[i])));
-                v[i] += other * (1.0f / kProjLoScale);      // meaningful in the hi columns only
-            }
-            const uint32_t row = (group0 + gi) * 8 + (c & 7);
-            if (c < 8 && row < a.R && nt < ntiles) {
-                const float sc = a.scales[row];
-                const size_t o = (size_t)row * a.ldy + nt * 16 + g * 4;
-                f32x4 r;
+    for (int t = 0; t < NT; t++)
+        wp[t] = a.w + (size_t)min(nt0 + t, ntiles - 1) * ktiles * 64;
 #pragma unroll
-                for (int i = 0; i < 4; i++) r[i] = v[i] * sc;
-                if (a.bias_rows) {
-                    const f32x4 b = *reinterpret_cast<const f32x4*>(a.bias_rows + o);
+    for (int gi = 0; gi < GROUPS; gi++)
+        xp[gi] = a.xfrag + (size_t)min(group0 + gi, ngroups - 1) * ktiles * 64;
+
+    f32x4 acc[NT][GROUPS];
 #pragma unroll
-                    for (int i = 0; i < 4; i++) r[i] += b[i];
+    for (int t = 0; t < NT; t++)
+#pragma unroll
+        for (int gi = 0; gi < GROUPS; gi++) acc[t][gi] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    half8 w0[NT], x0[GROUPS], w1[NT], x1[GROUPS];
+    auto load_set = [&](half8 (&wv)[NT], half8 (&xv)[GROUPS], uint32_t kt) {
+        const size_t o = (size_t)kt * 64 + lane;
+#pragma unroll
+        for (int t = 0; t < NT; t++) wv[t] = wp[t][o];
+#pragma unroll
+        for (int gi = 0; gi < GROUPS; gi++) xv[gi] = xp[gi][o];
+    };
+    auto mfma_set = [&](const half8 (&wv)[NT], const half8 (&xv)[GROUPS]) {
+#pragma unroll
+        for (int gi = 0; gi < GROUPS; gi++)
+#pragma unroll
+            for (int t = 0; t < NT; t++)
+                acc[t][gi] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wv[t], xv[gi], acc[t][gi], 0, 0, 0);
+    };
+
+    // loads inside the loop are unconditional (a k-step past the end re-reads the
+    // last one, unused), so the load counter the compiler waits on stays exact;
+    // a wave whose part of the range is empty (fewer than four k-steps) adds zeros
+    const uint32_t klast = ktiles - 1;
+    load_set(w0, x0, min(k_begin, klast));
+    uint32_t kt = k_begin;
+    for (; kt + 2 <= k_end; kt += 2) {
+        load_set(w1, x1, kt + 1);
+        mfma_set(w0, x0);
+        load_set(w0, x0, min(kt + 2, klast));
+        mfma_set(w1, x1);
+    }
+    if (kt < k_end) mfma_set(w0, x0);                     // odd number of k-steps
+
+    if constexpr (KS == 4) {
+        if (wave > 0) {
+#pragma unroll
+            for (int t = 0; t < NT; t++)
+#pragma unroll
+                for (int gi = 0; gi < GROUPS; gi++)
+                    s_red[(((wave - 1) * NT + t) * GROUPS + gi) * 64 + lane] = acc[t][gi];
+        }
+        __syncthreads();
+        if (wave > 0) return;
+        // wave order: 0 + 1 + 2 + 3; a real loop over the waves, so that at most
+        // one wave's partial tiles are in registers beside the accumulators
+#pragma unroll 1
+        for (int p = 0; p < 3; p++) {
+            const f32x4* from = s_red + (size_t)p * NT * GROUPS * 64 + lane;
+#pragma unroll
+            for (int t = 0; t < NT; t++)
+#pragma unroll
+                for (int gi = 0; gi < GROUPS; gi++) {
+                    const f32x4 o = from[(t * GROUPS + gi) * 64];
+#pragma unroll
+                    for (int i = 0; i < 4; i++) acc[t][gi][i] += o[i];
                 }
-                *reinterpret_cast<f32x4*>(a.y + o) = r;
-            }
         }
     }
+
+#pragma unroll
+    for (int t = 0; t < NT; t++)
+#pragma unroll
+        for (int gi = 0; gi < GROUPS; gi++) proj_store_tile(a, acc[t][gi], nt0 + t, group0 + gi, lane);
 }
 
 }  // namespace wr

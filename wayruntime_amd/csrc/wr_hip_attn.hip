@@ -445,6 +445,31 @@ void launch_proj(const ProjArgs& a, uint32_t groups)
                 dim3(kProjThreads), a);
 }
 
+// Prefill-sized row counts: the largest tile that still fills the chip.
+//   <8, 4, 1>  a workgroup covers 128 outputs x 128 rows (four wave tiles);
+//   <4, 4, 4>  64 outputs x 32 rows, its four waves split the input range;
+//   <4, 2, 4>  32 outputs x 32 rows, likewise.
+constexpr int kProjGemmMinRows = 64;
+
+template <int GROUPS, int NT, int KS>
+void launch_proj_gemm_tile(const ProjArgs& a, uint32_t groups)
+{
+    constexpr uint32_t wn = KS == 1 ? 2 * NT : NT, wg = KS == 1 ? 2 * GROUPS : GROUPS;
+    launch_main(proj_gemm_kernel<GROUPS, NT, KS>,
+                dim3((a.N / 16 + wn - 1) / wn, (groups + wg - 1) / wg), dim3(kProjThreads), a);
+}
+
+void launch_proj_gemm(const ProjArgs& a, uint32_t groups)
+{
+    const uint32_t nt = a.N / 16;
+    if (((nt + 7) / 8) * ((groups + 15) / 16) >= 256)
+        launch_proj_gemm_tile<8, 4, 1>(a, groups);
+    else if (((nt + 3) / 4) * ((groups + 3) / 4) >= 384)
+        launch_proj_gemm_tile<4, 4, 4>(a, groups);
+    else
+        launch_proj_gemm_tile<4, 2, 4>(a, groups);
+}
+
 // What feeds a projection: the rows as they are, their RMS normalisation, or
 // the gated activation of rows that hold gate and up values side by side.
 struct ProjSource {
@@ -460,7 +485,8 @@ int proj_chunk_locked(const wr_hip_weight* w, uint32_t rows, const float* x_dev,
 {
     // row groups of eight, padded to what one wave takes (1, 2, or runs of 4)
     uint32_t groups = (rows + 7) / 8;
-    if (groups > 2) groups = (groups + 3) / 4 * 4;
+    const bool gemm = rows >= (uint32_t)kProjGemmMinRows;  // the GEMM kernel clamps instead of padding
+    if (groups > 2 && !gemm) groups = (groups + 3) / 4 * 4;
     const uint32_t ktiles = w->n_in / 32;
     const size_t frag_bytes = (size_t)groups * ktiles * 1024;
     int rc = ensure_device(g.d_proj, frag_bytes + kProjMaxRows * sizeof(float));
@@ -517,7 +543,9 @@ int proj_chunk_locked(const wr_hip_weight* w, uint32_t rows, const float* x_dev,
             ksplit *= 2;
     }
     a.ksplit = ksplit;
-    if (groups == 1)
+    if (gemm)
+        launch_proj_gemm(a, groups);
+    else if (groups == 1)
         launch_proj<1, 1>(a, groups);
     else if (groups == 2 && tiles * ksplit >= 2048)
         launch_proj<2, 2>(a, groups);       // wide weight: two output tiles per operand load

@@ -436,7 +436,8 @@ int wr_prefill(wr_session *s, const uint32_t *ids, uint32_t n)
         wrh_workspace ws;
         wrh_devspace ds;
         memset(&ds, 0, sizeof ds);
-        const uint32_t chunk = n < WRH_PREFILL_CHUNK ? n : WRH_PREFILL_CHUNK;
+        const uint32_t cap = m->dev ? WRH_DEVICE_PREFILL_CHUNK : WRH_PREFILL_CHUNK;
+        const uint32_t chunk = n < cap ? n : cap;
         if (st == WR_OK && wrh_workspace_init(&ws, m, chunk) != WR_OK) st = WR_ERR_NOMEM;
         if (st == WR_OK) {
             if (m->dev && wrh_devspace_init(&ds, m, chunk, 0) != WR_OK) st = WR_ERR_NOMEM;
