@@ -50,11 +50,13 @@ def _check(got, x, w16, what):
     (3, 320, 16, 1.0),            # ten input tiles: one batch and a tail; a single output tile
     (8, 32, 64, 1.0),             # one input tile
     (17, 512, 80, 0.1),           # rows pad to four groups of eight; outputs not a multiple of 64
-    (300, 256, 128, 0.1),         # prefill-sized: the register-tiled kernel, small tile
-    (64, 96, 48, 0.5),            # ... its smallest row count; three input tiles (odd), three output tiles
+    (300, 256, 128, 0.1),         # prefill-sized rows: the register GEMM, 32 x 32 tiles, inputs split over four waves
+    (64, 96, 48, 0.5),            # ... its smallest row count; three input tiles (a wave with none), three output tiles
     (100, 160, 80, 0.3),          # ... a last row group of four rows, five input tiles
+    (300, 160, 2512, 0.2),        # ... 64 x 32 tiles, a partial last tile both ways
     (1030, 64, 32, 1.0),          # more rows than one launch takes: 1024 + a six-row launch
-    (1000, 1056, 4112, 0.02),     # the large tile, with a partial output panel, row panel and odd input tiles
+    (500, 96, 4112, 0.3),         # LDS-staged GEMM, 128 x 64 tiles: partial output and row panels, odd input tiles
+    (1000, 1056, 4112, 0.02),     # LDS-staged GEMM, 128 x 128 tiles, likewise
 ])
 def test_projection_shapes_vs_oracle(rows, n_in, n_out, std):
     print("proj", rows, n_in, n_out, flush=True)

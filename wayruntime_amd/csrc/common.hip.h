@@ -124,4 +124,35 @@ __device__ __forceinline__ float wave_pair32_sum(float v)
     return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
+// Tells the compiler that a pointer is the same in every lane (keeps the
+// arithmetic on it in scalar registers).
+__device__ __forceinline__ const unsigned char* uniform_ptr(const unsigned char* p)
+{
+    const uint64_t b = reinterpret_cast<uint64_t>(p);
+    // the builtin returns a signed int: widen through uint32_t, or a low half
+    // with its top bit set would smear ones over the high half
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)b);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(b >> 32));
+    return reinterpret_cast<const unsigned char*>((uint64_t)lo | ((uint64_t)hi << 32));
+}
+
+// One 64 x 16-byte load from global memory straight into LDS.  The LDS address
+// (wave-uniform, in M0) receives lane 0's 16 bytes, lane i's go 16*i further.
+__device__ __forceinline__ void lds_direct_load(uint32_t lds_addr, const unsigned char* base,
+                                                uint32_t lane_off)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(lds_addr), "v"(lane_off), "s"(base)
+                 : "memory");
+}
+
+// Workgroup barrier that waits for this wave's LDS traffic only.  __syncthreads()
+// also drains outstanding global loads, which would pull the tiles being
+// prefetched for later iterations back onto the critical path.
+__device__ __forceinline__ void lds_barrier()
+{
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 }  // namespace wr

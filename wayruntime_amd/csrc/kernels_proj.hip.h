@@ -424,41 +424,29 @@ __global__ __launch_bounds__(kProjThreads) void proj_rows_kernel(const ProjArgs 
         for (int gi = 0; gi < GROUPS; gi++) proj_store_tile(a, acc[t][gi], nt0 + t, group0 + gi, lane);
 }
 
-// Many rows (prefill chunks): a register-tiled GEMM on the same two layouts.
-// A wave owns NT x GROUPS accumulator tiles (16 NT outputs x 8 GROUPS rows):
-// every k-step loads NT weight tiles and GROUPS operand fragments, one KiB each
-// and both already in operand order, and feeds NT x GROUPS MFMAs, so a loaded
-// byte serves GROUPS (weights) or NT (rows) MFMAs instead of the four of
-// proj_rows_kernel.  The next k-step's operands are requested while this one's
-// MFMAs run (two register sets, the loop unrolled by two so no set is copied).
-//
-// KS = 1: a workgroup is 2 x 2 waves, each with its own tile and the whole input
-// range; the two waves of a row pair share weight tiles, the two of a column
-// pair share fragments (vector-cache hits).  For products large enough to give
-// every CU such a workgroup.
-// KS = 4: the four waves share one tile and take a quarter of the input range
-// each; their sums are added through LDS in wave order.  Four times the waves
-// and a quarter of the dependent k-steps: for products that would otherwise
-// leave a CU with one wave per SIMD waiting on its own loads.
-//
-// grid.x walks the output panels, so the workgroups the dispatcher deals
-// round-robin to the eight XCDs differ in output panel: one XCD's L2 holds an
-// eighth of the weight and all of the fragments.  Two workgroups per CU at
-// least (<= 256 registers), which also keeps the accumulators in ordinary
-// vector registers.
-template <int GROUPS, int NT, int KS>
-__global__ __launch_bounds__(kProjThreads, KS == 1 ? 2 : 3) void proj_gemm_kernel(const ProjArgs a)
+// Many rows (prefill chunks), products too small to fill the chip with the
+// LDS-staged tiles below: a register-tiled GEMM on the same two layouts.  The
+// four waves of a workgroup share one tile of NT x GROUPS accumulator tiles
+// (16 NT outputs x 8 GROUPS rows) and take a quarter of the input range each;
+// their sums are added through LDS in wave order.  Every k-step loads NT weight
+// tiles and GROUPS operand fragments, one KiB each and both already in operand
+// order, and feeds NT x GROUPS MFMAs; the next k-step's operands are requested
+// while this one's MFMAs run (two register sets, the loop unrolled by two so no
+// set is copied).  Small tiles and the split range put several waves on every
+// SIMD and keep the chains of dependent k-steps short: these products are
+// bound by load latency, not by bytes.  grid.x walks the outputs, so the
+// workgroups the dispatcher deals round-robin to the eight XCDs differ in
+// output tile.  At least three workgroups per CU (<= 168 registers), which
+// also keeps the accumulators in ordinary vector registers.
+template <int GROUPS, int NT>
+__global__ __launch_bounds__(kProjThreads, 3) void proj_gemm_split_kernel(const ProjArgs a)
 {
-    static_assert(KS == 1 || KS == 4, "whole range per wave, or four waves per tile");
-    __shared__ f32x4 s_red[KS == 4 ? 3 * NT * GROUPS * 64 : 1];
+    __shared__ f32x4 s_red[3 * NT * GROUPS * 64];
     const int lane = threadIdx.x & 63;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t ktiles = a.K / 32, ntiles = a.N / 16, ngroups = (a.R + 7) / 8;
-    const uint32_t nt0 = (KS == 1 ? blockIdx.x * 2 + (wave & 1) : blockIdx.x) * NT;
-    const uint32_t group0 = (KS == 1 ? blockIdx.y * 2 + (wave >> 1) : blockIdx.y) * GROUPS;
-    if (nt0 >= ntiles || group0 >= ngroups) return;       // KS = 4: the same for all four waves
-    const uint32_t k_begin = KS == 1 ? 0 : ktiles * wave / 4;
-    const uint32_t k_end = KS == 1 ? ktiles : ktiles * (wave + 1) / 4;
+    const uint32_t nt0 = blockIdx.x * NT, group0 = blockIdx.y * GROUPS;
+    const uint32_t k_begin = ktiles * wave / 4, k_end = ktiles * (wave + 1) / 4;
 
     // a tile or group past the end re-reads the last one; its result is dropped
     const half8* wp[NT];
@@ -506,32 +494,130 @@ __global__ __launch_bounds__(kProjThreads, KS == 1 ? 2 : 3) void proj_gemm_kerne
     }
     if (kt < k_end) mfma_set(w0, x0);                     // odd number of k-steps
 
-    if constexpr (KS == 4) {
-        if (wave > 0) {
+    if (wave > 0) {
 #pragma unroll
-            for (int t = 0; t < NT; t++)
+        for (int t = 0; t < NT; t++)
 #pragma unroll
-                for (int gi = 0; gi < GROUPS; gi++)
-                    s_red[(((wave - 1) * NT + t) * GROUPS + gi) * 64 + lane] = acc[t][gi];
-        }
-        __syncthreads();
-        if (wave > 0) return;
-        // wave order: 0 + 1 + 2 + 3; a real loop over the waves, so that at most
-        // one wave's partial tiles are in registers beside the accumulators
-#pragma unroll 1
-        for (int p = 0; p < 3; p++) {
-            const f32x4* from = s_red + (size_t)p * NT * GROUPS * 64 + lane;
-#pragma unroll
-            for (int t = 0; t < NT; t++)
-#pragma unroll
-                for (int gi = 0; gi < GROUPS; gi++) {
-                    const f32x4 o = from[(t * GROUPS + gi) * 64];
-#pragma unroll
-                    for (int i = 0; i < 4; i++) acc[t][gi][i] += o[i];
-                }
-        }
+            for (int gi = 0; gi < GROUPS; gi++)
+                s_red[(((wave - 1) * NT + t) * GROUPS + gi) * 64 + lane] = acc[t][gi];
     }
+    __syncthreads();
+    if (wave > 0) return;
+    // wave order: 0 + 1 + 2 + 3; a real loop over the waves, so that at most
+    // one wave's partial tiles are in registers beside the accumulators
+#pragma unroll 1
+    for (int p = 0; p < 3; p++) {
+        const f32x4* from = s_red + (size_t)p * NT * GROUPS * 64 + lane;
+#pragma unroll
+        for (int t = 0; t < NT; t++)
+#pragma unroll
+            for (int gi = 0; gi < GROUPS; gi++) {
+                const f32x4 o = from[(t * GROUPS + gi) * 64];
+#pragma unroll
+                for (int i = 0; i < 4; i++) acc[t][gi][i] += o[i];
+            }
+    }
+#pragma unroll
+    for (int t = 0; t < NT; t++)
+#pragma unroll
+        for (int gi = 0; gi < GROUPS; gi++) proj_store_tile(a, acc[t][gi], nt0 + t, group0 + gi, lane);
+}
 
+// Many rows, products that fill the chip with 128-output x 128-row workgroup
+// tiles (2 x 2 waves of 64 x 64): operands staged through LDS.  Per k-step the
+// workgroup needs 8 weight tiles and 16 operand fragments, 24 KiB that are
+// already in operand order: every wave copies six of them with direct-to-LDS
+// loads (no registers, so the copies run two k-steps ahead of the MFMAs in a
+// ring of three stages), and reads the 4 + 8 KiB of its own wave tile back with
+// 128-bit LDS reads, lane i at 16 i: conflict free.  Against loading the wave
+// tile's operands into registers directly the vector cache moves half the
+// bytes per MFMA and the prefetch depth costs no registers.  grid.x walks the
+// output panels, so one XCD's L2 holds an eighth of the weight and all of the
+// fragments.
+//
+// Step kt: wait for this wave's copies of stage kt (the six of stage kt + 1 may
+// still be in flight), workgroup barrier (everybody's copies of stage kt have
+// landed, and everybody has finished reading stage kt - 1), start the copies
+// of stage kt + 2 into the slot of stage kt - 1, then read and multiply.
+//
+// GROUPS = 8 is the tile described above; GROUPS = 4 halves the rows (128
+// outputs x 64 rows, 16 KiB per stage) for products with too few rows to fill
+// the chip with the large one.
+constexpr int kGemmRing = 3;
+template <int GROUPS>
+constexpr size_t gemm_lds_bytes()
+{
+    return (size_t)kGemmRing * (8 + 2 * GROUPS) * 1024;   // KiB per stage: 8 weight tiles, 2 GROUPS fragments
+}
+
+template <int GROUPS>
+__global__ __launch_bounds__(kProjThreads, 2) void proj_gemm_lds_kernel(const ProjArgs a)
+{
+    extern __shared__ __attribute__((aligned(16))) unsigned char gemm_smem[];
+    constexpr int NT = 4, CHUNKS = 2 * NT + 2 * GROUPS, CPW = CHUNKS / 4;   // chunks a wave copies per stage
+    constexpr uint32_t STAGE = CHUNKS * 1024;
+    const int lane = threadIdx.x & 63;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t ktiles = a.K / 32, ntiles = a.N / 16, ngroups = (a.R + 7) / 8;
+    const uint32_t klast = ktiles - 1;
+    const uint32_t nt_wg = blockIdx.x * 2 * NT, g_wg = blockIdx.y * 2 * GROUPS;
+    const uint32_t lds0 = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)gemm_smem);
+
+    // chunk c of a stage: weight tile nt_wg + c (c < 8) or fragment group g_wg + c - 8;
+    // one past the end re-reads the last one, and its results are dropped
+    const unsigned char* src[CPW];
+#pragma unroll
+    for (int i = 0; i < CPW; i++) {
+        const uint32_t c = wave * CPW + i;
+        const unsigned char* p =
+            c < 2 * NT ? reinterpret_cast<const unsigned char*>(a.w) + (size_t)min(nt_wg + c, ntiles - 1) * ktiles * 1024
+                       : reinterpret_cast<const unsigned char*>(a.xfrag) +
+                             (size_t)min(g_wg + c - 2 * NT, ngroups - 1) * ktiles * 1024;
+        src[i] = uniform_ptr(p);
+    }
+    const uint32_t lane_off = lane * 16;
+    auto issue = [&](uint32_t kt) {                        // a k-step past the end copies the last one again
+        const size_t k = (size_t)min(kt, klast) * 1024;
+        const uint32_t to = lds0 + (kt % kGemmRing) * STAGE + wave * CPW * 1024;
+#pragma unroll
+        for (int i = 0; i < CPW; i++) lds_direct_load(to + i * 1024, src[i] + k, lane_off);
+    };
+
+    f32x4 acc[NT][GROUPS];
+#pragma unroll
+    for (int t = 0; t < NT; t++)
+#pragma unroll
+        for (int gi = 0; gi < GROUPS; gi++) acc[t][gi] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    issue(0);
+    issue(1);
+    const uint32_t w_off = (wave & 1) * NT * 1024 + lane * 16;
+    const uint32_t x_off = (2 * NT + (wave >> 1) * GROUPS) * 1024 + lane * 16;
+    for (uint32_t kt = 0; kt < ktiles; kt++) {
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(CPW) : "memory");
+        issue(kt + 2);
+        const unsigned char* st = gemm_smem + (kt % kGemmRing) * STAGE;
+        half8 wv[NT], xv[GROUPS];
+#pragma unroll
+        for (int t = 0; t < NT; t++) wv[t] = *reinterpret_cast<const half8*>(st + w_off + t * 1024);
+#pragma unroll
+        for (int gi = 0; gi < GROUPS; gi++) xv[gi] = *reinterpret_cast<const half8*>(st + x_off + gi * 1024);
+#pragma unroll
+        for (int gi = 0; gi < GROUPS; gi++)
+#pragma unroll
+            for (int t = 0; t < NT; t++)
+                acc[t][gi] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wv[t], xv[gi], acc[t][gi], 0, 0, 0);
+        // all twelve operand reads first (their latency overlaps, and the first
+        // MFMAs hide the rest), then the MFMAs: left alone the scheduler reads
+        // two fragments at a time and waits for each pair
+        __builtin_amdgcn_sched_group_barrier(0x100, NT + GROUPS, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, NT * GROUPS, 0);
+    }
+    // the last two steps' copies still target the ring
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+    const uint32_t nt0 = nt_wg + (wave & 1) * NT, group0 = g_wg + (wave >> 1) * GROUPS;
+    if (nt0 >= ntiles || group0 >= ngroups) return;
 #pragma unroll
     for (int t = 0; t < NT; t++)
 #pragma unroll

@@ -445,29 +445,33 @@ void launch_proj(const ProjArgs& a, uint32_t groups)
                 dim3(kProjThreads), a);
 }
 
-// Prefill-sized row counts: the largest tile that still fills the chip.
-//   <8, 4, 1>  a workgroup covers 128 outputs x 128 rows (four wave tiles);
-//   <4, 4, 4>  64 outputs x 32 rows, its four waves split the input range;
-//   <4, 2, 4>  32 outputs x 32 rows, likewise.
+// Prefill-sized row counts: the largest tile that still gives every CU a workgroup.
+//   LDS-staged, 128 outputs x 128 rows per workgroup;
+//   LDS-staged, 128 x 64;
+//   registers, 64 x 32, the four waves split the input range;
+//   registers, 32 x 32, likewise.
 constexpr int kProjGemmMinRows = 64;
 
-template <int GROUPS, int NT, int KS>
-void launch_proj_gemm_tile(const ProjArgs& a, uint32_t groups)
+template <int GROUPS, int NT>
+void launch_proj_gemm_split(const ProjArgs& a, uint32_t groups)
 {
-    constexpr uint32_t wn = KS == 1 ? 2 * NT : NT, wg = KS == 1 ? 2 * GROUPS : GROUPS;
-    launch_main(proj_gemm_kernel<GROUPS, NT, KS>,
-                dim3((a.N / 16 + wn - 1) / wn, (groups + wg - 1) / wg), dim3(kProjThreads), a);
+    launch_main(proj_gemm_split_kernel<GROUPS, NT>,
+                dim3((a.N / 16 + NT - 1) / NT, (groups + GROUPS - 1) / GROUPS), dim3(kProjThreads), a);
 }
 
 void launch_proj_gemm(const ProjArgs& a, uint32_t groups)
 {
-    const uint32_t nt = a.N / 16;
-    if (((nt + 7) / 8) * ((groups + 15) / 16) >= 256)
-        launch_proj_gemm_tile<8, 4, 1>(a, groups);
+    const uint32_t nt = a.N / 16, panels = (nt + 7) / 8;
+    if (panels * ((groups + 15) / 16) >= 256)
+        launch_main(proj_gemm_lds_kernel<8>, dim3(panels, (groups + 15) / 16), dim3(kProjThreads), a,
+                    gemm_lds_bytes<8>());
+    else if (panels * ((groups + 7) / 8) >= 256)
+        launch_main(proj_gemm_lds_kernel<4>, dim3(panels, (groups + 7) / 8), dim3(kProjThreads), a,
+                    gemm_lds_bytes<4>());
     else if (((nt + 3) / 4) * ((groups + 3) / 4) >= 384)
-        launch_proj_gemm_tile<4, 4, 4>(a, groups);
+        launch_proj_gemm_split<4, 4>(a, groups);
     else
-        launch_proj_gemm_tile<4, 2, 4>(a, groups);
+        launch_proj_gemm_split<4, 2>(a, groups);
 }
 
 // What feeds a projection: the rows as they are, their RMS normalisation, or
@@ -619,7 +623,10 @@ int wr_hip_attn_init(int device)
             e = hipFuncSetAttribute(reinterpret_cast<const void*>(prefill_split_kernel<128>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize,
                                     (int)split_smem_bytes<128>());
-        if (e != hipSuccess) rc = hip_fail(e, "prefill LDS size", 0);
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute(reinterpret_cast<const void*>(proj_gemm_lds_kernel<8>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)gemm_lds_bytes<8>());
+        if (e != hipSuccess) rc = hip_fail(e, "kernel LDS size", 0);
     }
     if (rc != WR_HIP_OK) {
         g.inited = false;
