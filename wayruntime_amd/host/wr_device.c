@@ -181,13 +181,50 @@ static wr_status dev_fail(wr_engine *e, const char *what, uint32_t layer, int rc
         if (rc != WR_HIP_OK) return dev_fail(e, what, L, rc);  \
     } while (0)
 
+/* Host part of a pass: embedding rows and rotary angles of R tokens into the
+ * host workspace, rows in parallel (the angles go through the reference's
+ * scalar polynomials: four microseconds a position on one core). */
+static wr_status stage_rows(wr_model *m, wrh_workspace *hs, uint32_t R, wr_session *const *ss,
+                            const uint32_t *tokens, uint32_t pos0, int batch)
+{
+    const uint32_t hidden = m->hidden, hd = m->head_dim;
+    const uint32_t n_rot = (m->n_rot_pairs >= 1 && m->n_rot_pairs < hd / 2) ? m->n_rot_pairs : hd / 2;
+    const size_t ts = (size_t)2 * n_rot;
+    const wr_engine *e = m->engine;
+    const int threads = (e && e->n_threads > 0) ? e->n_threads : 1;
+    int bad = WR_OK;
+#pragma omp parallel for num_threads(threads) schedule(static) if (R >= 32)
+    for (uint32_t r = 0; r < R; r++) {
+        const int rc = wrh_embed(&m->embed, tokens[r], hs->residual + (size_t)r * hidden);
+        if (rc != WR_OK) __atomic_store_n(&bad, rc, __ATOMIC_RELAXED);
+        const uint32_t p = batch ? ss[r]->pos : pos0 + r;
+        (void)wrh_rope_table(hs->rope + r * ts, hd, p, m->rope_base, m->n_rot_pairs);
+    }
+    return (wr_status)bad;
+}
+
+/* Stages the rows of the NEXT pass of a prefill; called between a pass's last
+ * launch and its wait for the device, so the host's share of a pass costs no
+ * wall time from the second pass on. */
+void wrh_stage_next_rows(wr_model *m, wrh_workspace *hs, uint32_t R, const uint32_t *tokens,
+                         uint32_t pos0)
+{
+    hs->staged_rows = 0;
+    if (stage_rows(m, hs, R, NULL, tokens, pos0, 0) != WR_OK) return;   /* the pass itself reports it */
+    hs->staged_tokens = tokens;
+    hs->staged_rows = R;
+    hs->staged_pos0 = pos0;
+}
+
 /* Same contract as the host walk's forward_rows (wr_session.c), plus: when
  * logits_host is not NULL, the LM head runs for the first `logit_rows` rows
- * and their logits [logit_rows][vocab] are brought down. */
+ * and their logits [logit_rows][vocab] are brought down; when next_rows is not
+ * zero (prefill), the host stages that many further tokens (tokens + R, at
+ * pos0 + R) while the device works. */
 wr_status wrh_forward_rows_device(wr_model *m, wrh_workspace *hs, wrh_devspace *ds, uint32_t R,
                                   wr_session *const *ss, const uint32_t *tokens, uint32_t pos0,
                                   int batch, int prefill, int fail_layer, float *logits_host,
-                                  uint32_t logit_rows)
+                                  uint32_t logit_rows, uint32_t next_rows)
 {
     wr_engine *e = m->engine;
     const struct wrh_dev_model *d = m->dev;
@@ -198,11 +235,11 @@ wr_status wrh_forward_rows_device(wr_model *m, wrh_workspace *hs, wrh_devspace *
     uint32_t L = 0;
     int rc;
 
-    for (uint32_t r = 0; r < R; r++) {
-        rc = wrh_embed(&m->embed, tokens[r], hs->residual + (size_t)r * hidden);
+    const int staged = !batch && hs->staged_rows == R && hs->staged_tokens == tokens && hs->staged_pos0 == pos0;
+    hs->staged_rows = 0;
+    if (!staged) {
+        rc = stage_rows(m, hs, R, ss, tokens, pos0, batch);
         if (rc != WR_OK) return dev_fail(e, "embed", 0, rc);
-        const uint32_t p = batch ? ss[r]->pos : pos0 + r;
-        (void)wrh_rope_table(hs->rope + r * ts, hd, p, m->rope_base, m->n_rot_pairs);
     }
     TRY(wr_hip_attn_h2d(ds->resid, hs->residual, (size_t)R * hidden * sizeof(float)), "rows up");
     TRY(wr_hip_attn_h2d(ds->rope, hs->rope, (size_t)R * ts * sizeof(float)), "angles up");
@@ -258,6 +295,8 @@ wr_status wrh_forward_rows_device(wr_model *m, wrh_workspace *hs, wrh_devspace *
         TRY(wr_hip_attn_d2h(logits_host, ds->logits, (size_t)logit_rows * m->vocab * sizeof(float)),
             "logits down");
     } else {
+        /* both uploads above were synchronous: the host buffers are free again */
+        if (next_rows) wrh_stage_next_rows(m, hs, next_rows, tokens + R, pos0 + R);
         TRY(wr_hip_attn_sync(), "sync");
     }
     return WR_OK;

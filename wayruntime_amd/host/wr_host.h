@@ -96,6 +96,10 @@ typedef struct wrh_workspace {
     float *rope;                         /* [R][hd/2][2] (cos, sin) of the rows' angles */
     float *rope_swa;                     /* the same for Gemma's sliding-window layers */
     void  *block;
+    /* device walk: `residual` and `rope` already hold the embedded rows and
+     * angles of these tokens (staged while the device worked on the rows before) */
+    const uint32_t *staged_tokens;
+    uint32_t staged_rows, staged_pos0;
 } wrh_workspace;
 
 /* Device scratch for R rows of the device walk (wr_device.c). */
@@ -161,7 +165,7 @@ void      wrh_devspace_free(wrh_devspace *ws);
 wr_status wrh_forward_rows_device(wr_model *m, wrh_workspace *hs, wrh_devspace *ds, uint32_t R,
                                   wr_session *const *ss, const uint32_t *tokens, uint32_t pos0,
                                   int batch, int prefill, int fail_layer, float *logits_host,
-                                  uint32_t logit_rows);
+                                  uint32_t logit_rows, uint32_t next_rows);
 
 /* Test hook: make the attention call of `layer` fail with WR_ERR_INTERNAL once
  * (layer < 0 disarms).  The device is not involved: the failure is raised on

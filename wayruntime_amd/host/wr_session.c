@@ -396,7 +396,7 @@ const float *wr_step(wr_session *s, uint32_t token)
         wr_session *one[1] = {s};
         if (m->dev) {
             st = wrh_forward_rows_device(m, &s->ws1, &s->ds1, 1, one, &token, s->pos, 0, 0,
-                                         take_fail_layer(m), s->logits, 1);
+                                         take_fail_layer(m), s->logits, 1, 0);
         } else {
             st = forward_rows(m, &s->ws1, 1, one, &token, s->pos, FWD_STEP);
             if (st == WR_OK) {
@@ -444,10 +444,11 @@ int wr_prefill(wr_session *s, const uint32_t *ids, uint32_t n)
             wr_session *one[1] = {s};
             for (uint32_t done = 0; done < n && st == WR_OK; done += chunk) {
                 const uint32_t rows = (n - done < chunk) ? n - done : chunk;
-                if (m->dev)
+                if (m->dev) {
+                    const uint32_t left = n - done - rows;             /* staged while the device works */
                     st = wrh_forward_rows_device(m, &ws, &ds, rows, one, ids + done, s->pos, 0, 1,
-                                                 take_fail_layer(m), NULL, 0);
-                else
+                                                 take_fail_layer(m), NULL, 0, left < chunk ? left : chunk);
+                } else
                     st = forward_rows(m, &ws, rows, one, ids + done, s->pos, FWD_PREFILL);
                 if (st == WR_OK) __atomic_store_n(&s->pos, s->pos + rows, __ATOMIC_RELEASE);
             }
@@ -514,7 +515,7 @@ int wr_batch_step(wr_session *const *sessions, const uint32_t *tokens, uint32_t 
     if (st == WR_OK) {
         if (m->dev)
             st = wrh_forward_rows_device(m, &ws, &ds, n, sessions, tokens, 0, 1, 0,
-                                         take_fail_layer(m), big, n);
+                                         take_fail_layer(m), big, n, 0);
         else
             st = forward_rows(m, &ws, n, sessions, tokens, 0, FWD_BATCH);
     }
