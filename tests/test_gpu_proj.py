@@ -205,3 +205,42 @@ def test_fused_sources_equal_the_separate_steps():
     for d in (xd, nwd, gud, addd, tmp, y1, y2):
         d.free()
     w.close()
+
+
+@pytest.mark.parametrize("n_in", [256, 1056, 2080, 4128])
+def test_fused_sources_with_many_rows(n_in):
+    # 64 rows and more: the fragment kernel that takes a row group per workgroup
+    # (values held in registers up to 4096 inputs, re-read beyond) and the GEMM
+    # kernels.  The row sums of the norm are formed in another order than in the
+    # separate row step, so the comparison is with the oracle, to rounding; the
+    # gated activation has no sum and stays bit-identical to the separate steps.
+    lib = hipattn.lib()
+    rows, n_out = 77, 48
+    x = synth.normal(61 + n_in, (rows, n_in), std=2.0)
+    nw = synth.normal(62, (n_in,)) * np.float32(0.2) + np.float32(1.0)
+    gu = synth.normal(63 + n_in, (rows, 2 * n_in), std=2.0)
+    add = synth.normal(64, (rows, n_out))
+    w16 = _w16(65, n_out, n_in, 0.1)
+    w = hipattn.Weight([w16])
+    D = hipattn.DeviceBuffer
+    xd, nwd, gud, addd = D.from_host(x), D.from_host(nw), D.from_host(gu), D.from_host(add)
+    tmp, y1, y2 = D(rows * n_in * 4), D(rows * n_out * 4), D(rows * n_out * 4)
+    eps = 1e-6
+    assert lib.wr_hip_proj_rows_norm_dev(w.h, rows, xd.p, n_in, nwd.p, eps, addd.p, y2.p, n_out) == hipattn.OK
+    hipattn.sync()
+    got = y2.to_host((rows, n_out))
+    normed = oracle.rmsnorm(x, nw, eps)
+    want = oracle.matmul_w16(normed, w16) + add
+    mag = np.abs(normed.astype(np.float64)) @ np.abs(_widen(w16)).T + np.abs(add)
+    assert np.all(np.abs(got - want) <= 1e-6 * np.sqrt(n_in) * mag)
+    assert lib.wr_hip_rows_swiglu_dev(gud.p, 2 * n_in, tmp.p, n_in, rows, n_in) == hipattn.OK
+    w.rows_dev(rows, tmp, n_in, y1, n_out)
+    assert lib.wr_hip_proj_rows_swiglu_dev(w.h, rows, gud.p, 2 * n_in, None, y2.p, n_out) == hipattn.OK
+    hipattn.sync()
+    a, b = y1.to_host((rows, n_out)), y2.to_host((rows, n_out))
+    assert a.tobytes() == b.tobytes()
+    act = oracle.silu_mul(np.ascontiguousarray(gu[:, :n_in]), np.ascontiguousarray(gu[:, n_in:]))
+    _check(b, act, w16, f"swiglu {n_in}")
+    for d in (xd, nwd, gud, addd, tmp, y1, y2):
+        d.free()
+    w.close()

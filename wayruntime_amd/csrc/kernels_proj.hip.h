@@ -255,6 +255,154 @@ __global__ __launch_bounds__(256) void proj_prep_kernel(const ProjPrepArgs a)
     }
 }
 
+// The fragment kernel for many rows: one workgroup per row GROUP of eight.
+// Thread t serves row t % 8 of the group and the chunks of eight inputs t / 8,
+// t / 8 + 32, ...: a wave reads 256 contiguous bytes of each of its eight rows
+// per step and writes the hi and lo terms of eight chunks as whole 128-byte
+// lines (the eight rows' 16-byte units of one chunk are neighbours in the
+// fragment), where the one-row kernel's writes touch 16 bytes of a line each.
+// Same sources, expressions and scaling as proj_prep_kernel; the row sums are
+// formed in a different order (each thread over its own chunks, then the 32
+// threads of the row), so a normalised row agrees with the one-row kernel's to
+// rounding, not bit for bit: only launches of 64 rows and more come here.
+//
+// CH > 0: K <= 256 * CH and the row group's values stay in registers between
+// the passes; CH = 0: any K, the passes re-read and re-compute.
+__device__ __forceinline__ float group_rows_sum(float v, float (*s)[8], int lane, int wave, int c)
+{
+    v += wave_xor_f32(v, 8);
+    v += wave_xor_f32(v, 16);
+    v += wave_xor_f32(v, 32);
+    if (lane < 8) s[wave][lane] = v;
+    __syncthreads();
+    const float t = (s[0][c] + s[1][c]) + (s[2][c] + s[3][c]);
+    __syncthreads();
+    return t;
+}
+
+__device__ __forceinline__ float group_rows_max(float v, float (*s)[8], int lane, int wave, int c)
+{
+    v = fmaxf(v, wave_xor_f32(v, 8));
+    v = fmaxf(v, wave_xor_f32(v, 16));
+    v = fmaxf(v, wave_xor_f32(v, 32));
+    if (lane < 8) s[wave][lane] = v;
+    __syncthreads();
+    const float t = fmaxf(fmaxf(s[0][c], s[1][c]), fmaxf(s[2][c], s[3][c]));
+    __syncthreads();
+    return t;
+}
+
+// the eight values of chunk q of a row, from the row's source
+template <int SRC>
+__device__ __forceinline__ void proj_src_chunk(const ProjPrepArgs& a, const float* xr, uint32_t q,
+                                               float inv_rms, float (&v)[8])
+{
+    const f32x4 lo = *reinterpret_cast<const f32x4*>(xr + q * 8), hi = *reinterpret_cast<const f32x4*>(xr + q * 8 + 4);
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        v[j] = lo[j];
+        v[4 + j] = hi[j];
+    }
+    if constexpr (SRC == kProjSrcRmsNorm) {
+        const f32x4 wl = *reinterpret_cast<const f32x4*>(a.norm_w + q * 8),
+                    wh = *reinterpret_cast<const f32x4*>(a.norm_w + q * 8 + 4);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            v[j] = v[j] * inv_rms * wl[j];
+            v[4 + j] = v[4 + j] * inv_rms * wh[j];
+        }
+    } else if constexpr (SRC == kProjSrcSwiglu) {
+        const f32x4 ul = *reinterpret_cast<const f32x4*>(xr + a.K + q * 8),
+                    uh = *reinterpret_cast<const f32x4*>(xr + a.K + q * 8 + 4);
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const float g = v[j], u = j < 4 ? ul[j] : uh[j - 4];
+            const float sig = 1.0f / (1.0f + expf(-g));
+            v[j] = (g * sig) * u;
+        }
+    }
+}
+
+template <int SRC, int CH>
+__global__ __launch_bounds__(256) void proj_prep_group_kernel(const ProjPrepArgs a)
+{
+    __shared__ float s48[4][8];
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int c = t & 7;
+    const uint32_t col = t >> 3;                                  // 0..31
+    const uint32_t grp = blockIdx.x, row = grp * 8 + c;
+    const uint32_t ktiles = a.K / 32, nchunks = a.K / 8;
+    half8* frow = a.frag + (size_t)grp * ktiles * 64;
+    const bool live = row < a.R;                                  // rows past R pad the last group with zeros
+    const float* xr = a.x + (size_t)(live ? row : a.R - 1) * a.ldx;
+
+    // rows need 16-byte alignment for the vector loads: ldx and K are multiples
+    // of four floats (the host checks), the base comes from the allocator
+    float inv_rms = 1.0f;
+    if constexpr (SRC == kProjSrcRmsNorm) {
+        float ss = 0.f;
+        for (uint32_t q = col; q < nchunks; q += 32) {
+            const f32x4 lo = *reinterpret_cast<const f32x4*>(xr + q * 8), hi = *reinterpret_cast<const f32x4*>(xr + q * 8 + 4);
+#pragma unroll
+            for (int j = 0; j < 4; j++) ss = fmaf(lo[j], lo[j], ss);
+#pragma unroll
+            for (int j = 0; j < 4; j++) ss = fmaf(hi[j], hi[j], ss);
+        }
+        inv_rms = 1.0f / sqrtf(group_rows_sum(ss, s48, lane, wave, c) / (float)a.K + a.eps);
+    }
+
+    float held[CH > 0 ? CH : 1][8];
+    float mx = 0.f;
+    if constexpr (CH > 0) {
+#pragma unroll
+        for (int i = 0; i < CH; i++) {
+            const uint32_t q = col + 32 * i;
+            if (q < nchunks) {
+                proj_src_chunk<SRC>(a, xr, q, inv_rms, held[i]);
+#pragma unroll
+                for (int j = 0; j < 8; j++) mx = fmaxf(mx, fabsf(held[i][j]));
+            }
+        }
+    } else {
+        for (uint32_t q = col; q < nchunks; q += 32) {
+            float v[8];
+            proj_src_chunk<SRC>(a, xr, q, inv_rms, v);
+#pragma unroll
+            for (int j = 0; j < 8; j++) mx = fmaxf(mx, fabsf(v[j]));
+        }
+    }
+    mx = group_rows_max(mx, s48, lane, wave, c);
+    uint32_t ex = (__float_as_uint(mx) >> 23) & 0xFFu;
+    if (ex == 0 || ex == 0xFF) ex = 127;              // zeros, subnormals, inf / NaN rows: no scaling
+    if (ex > 253) ex = 253;                           // keeps the inverse 2^-e a normal number
+    if (col == 0 && live) a.scales[row] = __uint_as_float(ex << 23);
+    const float inv = __uint_as_float((254u - ex) << 23);
+
+    if constexpr (CH > 0) {
+#pragma unroll
+        for (int i = 0; i < CH; i++) {
+            const uint32_t q = col + 32 * i;
+            if (q < nchunks) {
+                if (!live) {
+#pragma unroll
+                    for (int j = 0; j < 8; j++) held[i][j] = 0.f;
+                }
+                proj_write_chunk(frow, q, c, held[i], inv);
+            }
+        }
+    } else {
+        for (uint32_t q = col; q < nchunks; q += 32) {
+            float v[8];
+            proj_src_chunk<SRC>(a, xr, q, inv_rms, v);
+            if (!live) {
+#pragma unroll
+                for (int j = 0; j < 8; j++) v[j] = 0.f;
+            }
+            proj_write_chunk(frow, q, c, v, inv);
+        }
+    }
+}
+
 struct ProjArgs {
     const half8* w;          // tile order
     const half8* xfrag;      // [groups][K/32][64]

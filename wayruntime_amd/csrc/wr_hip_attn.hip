@@ -508,9 +508,24 @@ int proj_chunk_locked(const wr_hip_weight* w, uint32_t rows, const float* x_dev,
     pa.eps = src.eps;
     const dim3 pgrid(groups * 8), pblock(256);
     const bool in_regs = w->n_in <= 4096;           // two chunks of eight values per thread
+    // many rows: a workgroup per row group (whole-line writes); it reads rows
+    // with 16-byte loads
+    const bool by_group = gemm && ldx % 4 == 0 && ((uintptr_t)x_dev & 15) == 0 &&
+                          ((uintptr_t)src.norm_w & 15) == 0;
+    const uint32_t kin = w->n_in;
+#define WR_LAUNCH_PREP_GROUP(SRC, CH) \
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(proj_prep_group_kernel<SRC, CH>), dim3(groups), pblock, 0, g.stream, pa)
 #define WR_LAUNCH_PREP(SRC)                                                                          \
     do {                                                                                             \
-        if (in_regs)                                                                                 \
+        if (by_group && kin <= 1024)                                                                 \
+            WR_LAUNCH_PREP_GROUP(SRC, 4);                                                            \
+        else if (by_group && kin <= 2048)                                                            \
+            WR_LAUNCH_PREP_GROUP(SRC, 8);                                                            \
+        else if (by_group && kin <= 4096)                                                            \
+            WR_LAUNCH_PREP_GROUP(SRC, 16);                                                           \
+        else if (by_group)                                                                           \
+            WR_LAUNCH_PREP_GROUP(SRC, 0);                                                            \
+        else if (in_regs)                                                                            \
             hipLaunchKernelGGL(HIP_KERNEL_NAME(proj_prep_kernel<SRC, 2>), pgrid, pblock, 0, g.stream, pa); \
         else                                                                                         \
             hipLaunchKernelGGL(HIP_KERNEL_NAME(proj_prep_kernel<SRC, 0>), pgrid, pblock, 0, g.stream, pa); \
@@ -522,6 +537,7 @@ int proj_chunk_locked(const wr_hip_weight* w, uint32_t rows, const float* x_dev,
     else
         WR_LAUNCH_PREP(kProjSrcPlain);
 #undef WR_LAUNCH_PREP
+#undef WR_LAUNCH_PREP_GROUP
     ProjArgs a;
     a.w = reinterpret_cast<const half8*>(w->tiles);
     a.xfrag = frag;

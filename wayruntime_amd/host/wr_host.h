@@ -23,7 +23,7 @@
 #define WRH_MAX_LAYERS   64          /* reference: WR_MAX_LAYERS, src/core/internal.h:184 */
 #define WRH_DEFAULT_CTX  4096        /* reference: WR_DEFAULT_MAX_CONTEXT, internal.h:194 */
 #define WRH_PREFILL_CHUNK 256        /* rows per layer-major prefill pass, host walk */
-#define WRH_DEVICE_PREFILL_CHUNK 1024 /* ... device walk: one projection launch takes this many rows */
+#define WRH_DEVICE_PREFILL_CHUNK 4096 /* ... device walk: long passes give the attention kernel enough position blocks to fill the chip */
 
 /* ---- scalar math with the reference's polynomials (wr_math.c) ------------- */
 float wrh_exp(float x);
