@@ -14,8 +14,9 @@ wall time per step (whole step: split-K kernel + combine).  `roofline` is for
 the split-K kernel alone, timed with per-launch events.  `cpu_baseline` is the
 CPU oracle (a bit-exact restatement of the reference op) on the same data, one
 core, on a bounded sample.  `prefill` reports causal prefill attention,
-`projection` the row projections either side of the path (proj_rows_kernel,
-HBM-bound on the F16 weight bytes).
+`projection` the row projections either side of the path: 16 rows
+(proj_rows_kernel, HBM-bound on the F16 weight bytes) and a 1024-row prefill
+pass (proj_gemm_lds_kernel, MFMA-bound).
 """
 from __future__ import annotations
 
@@ -240,6 +241,30 @@ def main() -> None:
                           "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)}
             for w in ws:
                 w.close()
+            xd.free()
+            yd.free()
+        # the same weights against a prefill pass of 1024 rows: MFMA-bound.  The
+        # activations travel as two half-precision terms, so the matrix cores do
+        # twice the useful multiply-adds; both rates are given.
+        rows = 1024
+        for name, n_out, n_in in (("qkv 6144x4096", 6144, 4096), ("gate_up 28672x4096", 28672, 4096),
+                                  ("down 4096x14336", 4096, 14336)):
+            w = hipattn.Weight([rng.integers(0, 0x3C00, size=(n_out, n_in), dtype=np.uint16)])
+            xd = hipattn.DeviceBuffer.from_host(synth.normal(10, (rows, n_in)))
+            yd = hipattn.DeviceBuffer(rows * n_out * 4)
+            reps = 10
+            for _ in range(2):
+                w.rows_dev(rows, xd, n_in, yd, n_out)
+            hipattn.profile_begin(reps)
+            for _ in range(reps):
+                w.rows_dev(rows, xd, n_in, yd, n_out)
+            pms, pn = hipattn.profile_end()
+            us = pms / max(pn, 1) * 1e3
+            tf = 2.0 * rows * n_out * n_in / (us * 1e-6) / 1e12
+            proj[name + " x 1024 rows"] = {"rows": rows, "kernel_us": round(us, 2), "TFLOP/s": round(tf, 1),
+                                           "mfma_TFLOP/s": round(2 * tf, 1),
+                                           "frac_of_f16_peak": round(2 * tf / MFMA_F16_PEAK_TFLOPS, 4)}
+            w.close()
             xd.free()
             yd.free()
 

@@ -708,7 +708,16 @@ __global__ __launch_bounds__(kProjThreads, 2) void proj_gemm_lds_kernel(const Pr
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t ktiles = a.K / 32, ntiles = a.N / 16, ngroups = (a.R + 7) / 8;
     const uint32_t klast = ktiles - 1;
-    const uint32_t nt_wg = blockIdx.x * 2 * NT, g_wg = blockIdx.y * 2 * GROUPS;
+    // Workgroup -> tile.  The dispatcher deals consecutive workgroups round-robin
+    // to the eight XCDs; XCD x takes the output panels x, x + 8, ..., and runs
+    // through all row panels of one before the next, so the workgroups resident
+    // on an XCD at one time share a few weight panels (fetched once into its L2)
+    // and the fragments of all rows.
+    const uint32_t nx = (ntiles + 2 * NT - 1) / (2 * NT), ny = (ngroups + 2 * GROUPS - 1) / (2 * GROUPS);
+    const uint32_t xcd = blockIdx.x % 8, slot = blockIdx.x / 8;
+    const uint32_t px = (slot / ny) * 8 + xcd, py = slot % ny;
+    if (px >= nx) return;                                 // the grid is padded to eight equal shares
+    const uint32_t nt_wg = px * 2 * NT, g_wg = py * 2 * GROUPS;
     const uint32_t lds0 = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)gemm_smem);
 
     // chunk c of a stage: weight tile nt_wg + c (c < 8) or fragment group g_wg + c - 8;

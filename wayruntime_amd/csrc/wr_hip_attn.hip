@@ -445,9 +445,9 @@ void launch_proj(const ProjArgs& a, uint32_t groups)
                 dim3(kProjThreads), a);
 }
 
-// Prefill-sized row counts: the largest tile that still gives every CU a workgroup.
-//   LDS-staged, 128 outputs x 128 rows per workgroup;
-//   LDS-staged, 128 x 64;
+// Prefill-sized row counts: the largest tile that still fills the chip.
+//   LDS-staged, 128 outputs x 128 rows per workgroup, from two workgroups per CU;
+//   LDS-staged, 128 x 64, from one per CU;
 //   registers, 64 x 32, the four waves split the input range;
 //   registers, 32 x 32, likewise.
 constexpr int kProjGemmMinRows = 64;
@@ -462,11 +462,13 @@ void launch_proj_gemm_split(const ProjArgs& a, uint32_t groups)
 void launch_proj_gemm(const ProjArgs& a, uint32_t groups)
 {
     const uint32_t nt = a.N / 16, panels = (nt + 7) / 8;
-    if (panels * ((groups + 15) / 16) >= 256)
-        launch_main(proj_gemm_lds_kernel<8>, dim3(panels, (groups + 15) / 16), dim3(kProjThreads), a,
+    // one-dimensional grids: eight equal shares of output panels, times the row panels
+    const uint32_t share = (panels + 7) / 8 * 8;
+    if (panels * ((groups + 15) / 16) >= 512)
+        launch_main(proj_gemm_lds_kernel<8>, dim3(share * ((groups + 15) / 16)), dim3(kProjThreads), a,
                     gemm_lds_bytes<8>());
     else if (panels * ((groups + 7) / 8) >= 256)
-        launch_main(proj_gemm_lds_kernel<4>, dim3(panels, (groups + 7) / 8), dim3(kProjThreads), a,
+        launch_main(proj_gemm_lds_kernel<4>, dim3(share * ((groups + 7) / 8)), dim3(kProjThreads), a,
                     gemm_lds_bytes<4>());
     else if (((nt + 3) / 4) * ((groups + 3) / 4) >= 384)
         launch_proj_gemm_split<4, 4>(a, groups);
