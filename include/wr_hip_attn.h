@@ -277,6 +277,25 @@ int wr_hip_rows_qkv_prep_dev(const float *qkv_dev, uint32_t ld, uint32_t rows,
                              float eps, const float *cos_sin_dev, uint32_t n_rot,
                              float *q_out_dev, float *k_out_dev, float *v_out_dev);
 
+/* qkv_append: qkv_prep and the cache append in one launch, for callers whose
+ * K and V rows exist only to be appended (src/core/session.c:459-486: the norm,
+ * the rotation, then wri_kv_append for K and V).  Q leaves as in qkv_prep; the
+ * rotated K heads and the V heads are truncated to binary16 as in
+ * wr_hip_attn_append and written into the cache(s) directly.  Head counts and
+ * head_dim of K and V are the cache's (layer `layer`).
+ *   n_kv == 1: the rows are positions pos[0], pos[0]+1, ... of kv[0];
+ *   n_kv == rows (<= WR_HIP_BATCH_MAX, distinct caches of one geometry): row i
+ *   is position pos[i] of kv[i] (the batched step).
+ * All or nothing: a position past a cache's max_ctx returns
+ * WR_HIP_ERR_CTX_FULL before anything is written.  head_dim <= 512
+ * (WR_HIP_ERR_LIMIT beyond; use qkv_prep + append).  Q and the cache bits
+ * equal those of qkv_prep followed by the append, bit for bit. */
+int wr_hip_rows_qkv_append_dev(const float *qkv_dev, uint32_t ld, uint32_t rows, uint32_t nq,
+                               const float *q_norm_dev, const float *k_norm_dev, float eps,
+                               const float *cos_sin_dev, uint32_t n_rot, uint32_t n_kv,
+                               wr_hip_kv *const *kv, uint32_t layer, const uint32_t *pos,
+                               float *q_out_dev);
+
 /* swiglu: act[r][j] = silu(gu[r][j]) * gu[r][ffn + j] for rows of a stacked
  * gate/up projection (wri_op_fused_silu_mul, src/core/kernels.c:1243-1258 with
  * silu at :963-967; called at session.c:523-526). */

@@ -289,6 +289,15 @@ int wr_hip_rows_qkv_prep_dev(const float *qkv, uint32_t ld, uint32_t rows, uint3
     (void)cs; (void)n_rot; (void)q; (void)k; (void)v;
     return WR_HIP_ERR_STATE;
 }
+int wr_hip_rows_qkv_append_dev(const float *qkv, uint32_t ld, uint32_t rows, uint32_t nq,
+                               const float *qn, const float *kn, float eps, const float *cs,
+                               uint32_t n_rot, uint32_t n_kv, wr_hip_kv *const *kv, uint32_t layer,
+                               const uint32_t *pos, float *q)
+{
+    (void)qkv; (void)ld; (void)rows; (void)nq; (void)qn; (void)kn; (void)eps; (void)cs; (void)n_rot;
+    (void)n_kv; (void)kv; (void)layer; (void)pos; (void)q;
+    return WR_HIP_ERR_STATE;
+}
 int wr_hip_rows_swiglu_dev(const float *gu, uint32_t ld, float *act, uint32_t ldo, uint32_t rows,
                            uint32_t ffn)
 {

@@ -125,3 +125,72 @@ def test_error_contract():
     assert lib.wr_hip_rows_qkv_prep_dev(d.p, 24, 1, 1, 1, 8, None, None, 1e-6, None, 4, d.p, d.p, d.p) == hipattn.ERR_INVAL
     assert lib.wr_hip_rows_swiglu_dev(d.p, 8, d.p, 8, 1, 8) == hipattn.ERR_INVAL                    # stride < 2 ffn
     d.free()
+
+
+import ctypes as C
+
+
+@pytest.mark.parametrize("rows,nq,nkv,hd,norm,pos,batch", [
+    (70, 16, 8, 128, True, 13, False),      # three cache blocks, both ends partial
+    (1, 16, 8, 128, True, 77, False),       # one decode row
+    (33, 4, 2, 64, False, 0, False),        # no norm; head_dim 64 (the pair sits in two lanes)
+    (5, 8, 4, 256, True, 31, False),        # crosses a block boundary after one row
+    (5, 16, 8, 128, True, 0, True),         # batched step: row i to session i at its own position
+    (16, 32, 8, 128, False, 0, True),
+])
+def test_qkv_append_equals_prep_then_append(rows, nq, nkv, hd, norm, pos, batch):
+    # the fused launch against the two-step path: Q rows and the cache contents, bit for bit
+    print("qkv_append", rows, nq, nkv, hd, norm, pos, batch, flush=True)
+    lib = hipattn.lib()
+    width = (nq + 2 * nkv) * hd
+    ld = width + 16
+    qkv = synth.normal(7 * hd + rows, (rows, ld), std=1.5)
+    qn = synth.normal(1, (hd,)) * np.float32(0.1) + np.float32(1.0)
+    kn = synth.normal(2, (hd,)) * np.float32(0.1) + np.float32(1.0)
+    qd, kd = nq * hd, nkv * hd
+    eps = 1e-6
+    n_kv = rows if batch else 1
+    positions = [3 + 37 * i for i in range(rows)] if batch else [pos]
+    if batch:
+        tab = np.concatenate([oracle.rope_table(1, hd, p, 1e6, 0) for p in positions])
+    else:
+        tab = oracle.rope_table(rows, hd, pos, 1e6, 0)
+    n_rot = tab.shape[1]
+    ctx = 1024
+    two_step = [hipattn.KVCache(1, hd, nkv, ctx) for _ in range(n_kv)]
+    fused = [hipattn.KVCache(1, hd, nkv, ctx) for _ in range(n_kv)]
+    bufs = [_dev(qkv), _dev(qn), _dev(kn), _dev(tab), _dev(np.zeros((rows, qd))), _dev(np.zeros((rows, kd))),
+            _dev(np.zeros((rows, kd))), _dev(np.full((rows, qd), 5.0))]
+    xd, qnd, knd, td, qo, ko, vo, qo2 = bufs
+    qnp, knp = (qnd.p, knd.p) if norm else (None, None)
+    assert lib.wr_hip_rows_qkv_prep_dev(xd.p, ld, rows, nq, nkv, hd, qnp, knp, eps, td.p, n_rot,
+                                        qo.p, ko.p, vo.p) == hipattn.OK
+    if batch:
+        kvp = (C.c_void_p * n_kv)(*[c.h for c in two_step])
+        pp = (C.c_uint32 * n_kv)(*positions)
+        assert lib.wr_hip_attn_append_batched_dev(n_kv, kvp, 0, pp, ko.p, vo.p) == hipattn.OK
+    else:
+        hipattn.append_dev(two_step[0], 0, pos, rows, ko, vo)
+    kvp = (C.c_void_p * n_kv)(*[c.h for c in fused])
+    pp = (C.c_uint32 * n_kv)(*positions)
+    assert lib.wr_hip_rows_qkv_append_dev(xd.p, ld, rows, nq, qnp, knp, eps, td.p, n_rot, n_kv, kvp, 0, pp,
+                                          qo2.p) == hipattn.OK
+    hipattn.sync()
+    assert qo.to_host((rows, qd)).tobytes() == qo2.to_host((rows, qd)).tobytes()
+    for a, b, p in zip(two_step, fused, positions if batch else [pos]):
+        n = 1 if batch else rows
+        lo = max(0, p - 40)
+        ka, va = a.read_f16(0, lo, p + n - lo + 40)      # neighbours too: nothing else may be written
+        kb, vb = b.read_f16(0, lo, p + n - lo + 40)
+        assert ka.tobytes() == kb.tobytes() and va.tobytes() == vb.tobytes()
+    # contracts: all or nothing past the end of a cache; one cache or one per row; distinct caches
+    pp_bad = (C.c_uint32 * n_kv)(*([ctx - (0 if batch else rows - 1)] * n_kv))
+    assert lib.wr_hip_rows_qkv_append_dev(xd.p, ld, rows, nq, qnp, knp, eps, td.p, n_rot, n_kv, kvp, 0, pp_bad,
+                                          qo2.p) == hipattn.ERR_CTX_FULL
+    if rows > 2:
+        assert lib.wr_hip_rows_qkv_append_dev(xd.p, ld, rows, nq, qnp, knp, eps, td.p, n_rot, 2, kvp, 0, pp,
+                                              qo2.p) == hipattn.ERR_INVAL
+    for c in two_step + fused:
+        c.close()
+    for b in bufs:
+        b.free()

@@ -102,6 +102,122 @@ __global__ __launch_bounds__(64) void qkv_prep_kernel(const QkvPrepArgs a)
     }
 }
 
+// qkv_prep and the cache append in one launch: Q heads leave as rotated F32
+// rows, K heads go through the same norm and rotation and are truncated to F16
+// straight into the cache's K tiles, V heads are truncated and turned into the
+// block-transposed Vt.  The arithmetic is qkv_prep_kernel's (one wave per row
+// and head, the same wave sum) and the conversion is the append kernels', so Q
+// and the cache bits equal the two-step path's bit for bit.
+//
+// Two shapes of call:
+//   rows of ONE session at consecutive positions pos[0] ... (prefill, a step):
+//     grid.x walks the cache's 32-position blocks the rows touch;
+//   ONE row for each of n sessions (batched step): grid.x = session.
+// grid.y = head (nq + 2 nkv), 256 threads: wave w takes the block's positions
+// w, w + 4, ...  A V workgroup gathers its block in LDS and writes each
+// dimension's positions as one run, like append_v_kernel.
+struct QkvAppendArgs {
+    const float* qkv;        // [rows][ld]
+    const float* q_norm;
+    const float* k_norm;
+    const float* cos_sin;    // [rows][n_rot][2]
+    float* q_out;            // [rows][nq][hd]
+    uint16_t* k[16];
+    uint16_t* vt[16];
+    uint32_t pos[16];
+    uint32_t ctx_pad[16];
+    uint32_t ld, nq, nkv, hd, n_rot, rows;
+    uint32_t per_session;    // 1: row i belongs to session i; 0: all rows to session 0 from pos[0]
+    float eps;
+};
+
+__global__ __launch_bounds__(256) void qkv_append_kernel(const QkvAppendArgs a)
+{
+#pragma clang fp contract(off)
+    extern __shared__ __attribute__((aligned(16))) unsigned char qkv_smem[];
+    const uint32_t h = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t hd = a.hd, half = hd / 2;
+    const uint32_t sess = a.per_session ? blockIdx.x : 0;
+    const uint32_t pos0 = a.pos[sess], ctx_pad = a.ctx_pad[sess];
+    // positions of this workgroup: [p_begin, p_end), rows row0 ...
+    uint32_t p_begin, p_end, row0;
+    if (a.per_session) {
+        p_begin = pos0;
+        p_end = pos0 + 1;
+        row0 = blockIdx.x;
+    } else {
+        const uint32_t blk = pos0 / kVBlock + blockIdx.x;
+        p_begin = max(blk * kVBlock, pos0);
+        p_end = min((blk + 1) * kVBlock, pos0 + a.rows);
+        row0 = p_begin - pos0;
+    }
+    const uint32_t np = p_end - p_begin;                  // 1 .. 32
+
+    if (h >= a.nq + a.nkv) {
+        // V head: rows -> F16 -> tile[d][position in block] -> runs along positions
+        const uint32_t kvh = h - a.nq - a.nkv;
+        uint16_t (*tile)[kVBlock + 2] = reinterpret_cast<uint16_t (*)[kVBlock + 2]>(qkv_smem);
+        for (uint32_t i = wave; i < np; i += 4) {
+            const float* src = a.qkv + (size_t)(row0 + i) * a.ld + (size_t)h * hd;
+            for (uint32_t j = lane; j < hd; j += 64) tile[j][i] = f32_to_f16_trunc(src[j]);
+        }
+        __syncthreads();
+        uint16_t* vt = a.vt[sess];
+        for (uint32_t idx = threadIdx.x; idx < hd * np; idx += 256) {
+            const uint32_t d = idx / np, i = idx % np;
+            vt[vt_offset(kvh, ctx_pad, p_begin + i, d, hd)] = tile[d][i];
+        }
+        return;
+    }
+
+    const bool is_q = h < a.nq;
+    const float* nw = is_q ? a.q_norm : a.k_norm;
+    float* s = reinterpret_cast<float*>(qkv_smem) + (size_t)wave * hd;   // this wave's row
+    // the same trip count in every wave (the barrier needs it); a wave past its
+    // positions repeats the block's last one and stores nothing
+    for (uint32_t i0 = 0; i0 < np; i0 += 4) {
+        const bool mine = i0 + wave < np;
+        const uint32_t i = mine ? i0 + wave : np - 1;
+        const uint32_t r = row0 + i;
+        const float* src = a.qkv + (size_t)r * a.ld + (size_t)h * hd;
+        float ss = 0.f;
+        for (uint32_t j = lane; j < hd; j += 64) {
+            const float v = src[j];
+            s[j] = v;
+            ss += v * v;
+        }
+        if (nw) {
+            ss = wave_sum_f32(ss);
+            const float inv_rms = 1.0f / sqrtf(ss / (float)hd + a.eps);
+            for (uint32_t j = lane; j < hd; j += 64) s[j] = s[j] * inv_rms * nw[j];
+        }
+        __syncthreads();
+        const float* cs = a.cos_sin + (size_t)r * a.n_rot * 2;
+        for (uint32_t j = lane; j < half; j += 64) {
+            const float x0 = s[j], x1 = s[j + half];
+            float y0 = x0, y1 = x1;
+            if (j < a.n_rot) {
+                const float c = cs[2 * j], sn = cs[2 * j + 1];
+                const float a0 = x0 * c, b0 = x1 * sn, a1 = x0 * sn, b1 = x1 * c;
+                y0 = a0 - b0;
+                y1 = a1 + b1;
+            }
+            if (!mine) continue;
+            if (is_q) {
+                float* dst = a.q_out + ((size_t)r * a.nq + h) * hd;
+                dst[j] = y0;
+                dst[j + half] = y1;
+            } else {
+                uint16_t* k = a.k[sess];
+                const uint32_t kvh = h - a.nq, p = p_begin + i;
+                k[k_offset(kvh, ctx_pad, p, j, hd)] = f32_to_f16_trunc(y0);
+                k[k_offset(kvh, ctx_pad, p, j + half, hd)] = f32_to_f16_trunc(y1);
+            }
+        }
+        __syncthreads();                                  // s is rewritten by the next position
+    }
+}
+
 // act[r][j] = silu(gu[r][j]) * gu[r][ffn + j],  silu(x) = x / (1 + exp(-x))
 __global__ __launch_bounds__(256) void swiglu_rows_kernel(const float* __restrict__ gu, uint32_t ld,
                                                           float* __restrict__ act, uint32_t ldo,

@@ -8,6 +8,7 @@
 #include <hip/hip_runtime.h>
 #include <hip/hip_ext.h>
 
+#include <algorithm>
 #include <atomic>
 #include <cmath>
 #include <cstdarg>
@@ -1237,6 +1238,59 @@ int wr_hip_rows_qkv_prep_dev(const float* qkv_dev, uint32_t ld, uint32_t rows, u
     Locked lk;
     hipLaunchKernelGGL(qkv_prep_kernel, dim3(rows, nq + 2 * nkv), dim3(64), 0, g.stream, a);
     HIP_TRY(hipGetLastError(), "qkv prep launch", 0);
+    return WR_HIP_OK;
+}
+
+int wr_hip_rows_qkv_append_dev(const float* qkv_dev, uint32_t ld, uint32_t rows, uint32_t nq,
+                               const float* q_norm_dev, const float* k_norm_dev, float eps,
+                               const float* cos_sin_dev, uint32_t n_rot, uint32_t n_kv,
+                               wr_hip_kv* const* kv, uint32_t layer, const uint32_t* pos,
+                               float* q_out_dev)
+{
+    if (!g.inited) return WR_HIP_ERR_STATE;
+    if (!qkv_dev || !q_out_dev || !kv || !pos || nq == 0) return WR_HIP_ERR_INVAL;
+    if (n_kv == 0 || (n_kv != 1 && n_kv != rows)) return WR_HIP_ERR_INVAL;
+    if (n_kv > WR_HIP_BATCH_MAX) return WR_HIP_ERR_LIMIT;
+    QkvAppendArgs a;
+    memset(&a, 0, sizeof a);
+    for (uint32_t i = 0; i < n_kv; i++) {
+        int rc = check_layer(kv[i], layer);
+        if (rc) return rc;
+        if (kv[i]->nkv != kv[0]->nkv || kv[i]->hd[layer] != kv[0]->hd[layer]) return WR_HIP_ERR_INVAL;
+        for (uint32_t j = 0; j < i; j++)
+            if (kv[i] == kv[j]) return WR_HIP_ERR_INVAL;
+        const uint64_t end = (uint64_t)pos[i] + (n_kv == 1 ? rows : 1);
+        if (end > kv[i]->max_ctx) return WR_HIP_ERR_CTX_FULL;         // nothing is written
+        a.k[i] = reinterpret_cast<uint16_t*>(kv[i]->slab + kv[i]->k_off[layer]);
+        a.vt[i] = reinterpret_cast<uint16_t*>(kv[i]->slab + kv[i]->vt_off[layer]);
+        a.pos[i] = pos[i];
+        a.ctx_pad[i] = kv[i]->ctx_pad;
+    }
+    const uint32_t nkv = kv[0]->nkv, hd = kv[0]->hd[layer];
+    if (hd < 2 || (hd & 1)) return WR_HIP_ERR_INVAL;
+    if (hd > 512) return WR_HIP_ERR_LIMIT;                // the V block gathered in LDS: hd * 68 bytes
+    if ((uint64_t)ld < (uint64_t)(nq + 2 * nkv) * hd) return WR_HIP_ERR_INVAL;
+    if (n_rot > hd / 2 || (n_rot > 0 && !cos_sin_dev)) return WR_HIP_ERR_INVAL;
+    if ((q_norm_dev == nullptr) != (k_norm_dev == nullptr)) return WR_HIP_ERR_INVAL;
+    if (rows == 0) return WR_HIP_OK;
+    a.qkv = qkv_dev;
+    a.q_norm = q_norm_dev;
+    a.k_norm = k_norm_dev;
+    a.cos_sin = cos_sin_dev;
+    a.q_out = q_out_dev;
+    a.ld = ld;
+    a.nq = nq;
+    a.nkv = nkv;
+    a.hd = hd;
+    a.n_rot = n_rot;
+    a.rows = rows;
+    a.per_session = (n_kv > 1 || rows == 1) ? 1 : 0;
+    a.eps = eps;
+    const uint32_t gx = a.per_session ? rows : (pos[0] + rows - 1) / kVBlock - pos[0] / kVBlock + 1;
+    const size_t lds = std::max((size_t)4 * hd * sizeof(float), (size_t)hd * (kVBlock + 2) * sizeof(uint16_t));
+    Locked lk;
+    hipLaunchKernelGGL(qkv_append_kernel, dim3(gx, nq + 2 * nkv), dim3(256), lds, g.stream, a);
+    HIP_TRY(hipGetLastError(), "qkv append launch", layer);
     return WR_HIP_OK;
 }
 

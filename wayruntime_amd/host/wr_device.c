@@ -71,7 +71,8 @@ wr_status wrh_device_model_init(wr_model *m)
     if (m->is_gemma) return WR_OK;               /* the Gemma block runs on the host walk */
     const uint32_t qd = m->n_q * m->head_dim, kd = m->n_kv * m->head_dim;
     int ok = proj_dims_ok(&m->lm_head) && m->vocab % 16 == 0 && (qd + 2 * kd) % 16 == 0 &&
-             m->hidden % 16 == 0 && (2 * m->ffn) % 16 == 0;
+             m->hidden % 16 == 0 && (2 * m->ffn) % 16 == 0 &&
+             m->head_dim <= 512;                  /* the fused Q/K/V split + append */
     for (uint32_t l = 0; l < m->n_layers && ok; l++)
         ok = proj_dims_ok(&m->wq[l]) && proj_dims_ok(&m->wk[l]) && proj_dims_ok(&m->wv[l]) &&
              proj_dims_ok(&m->wo[l]) && proj_dims_ok(&m->w_gate[l]) && proj_dims_ok(&m->w_up[l]) &&
@@ -248,9 +249,7 @@ wr_status wrh_forward_rows_device(wr_model *m, wrh_workspace *hs, wrh_devspace *
         const dev_layer *dl = &d->L[L];
         TRY(wr_hip_proj_rows_norm_dev(dl->wqkv, R, ds->resid, hidden, dl->attn_norm, m->rms_eps, NULL,
                                       ds->qkv, qd + 2 * kd), "attn norm + qkv projection");
-        TRY(wr_hip_rows_qkv_prep_dev(ds->qkv, qd + 2 * kd, R, nq, nkv, hd, dl->q_norm, dl->k_norm,
-                                     m->rms_eps, ds->rope, n_rot, ds->q, ds->k, ds->v), "qkv prep");
-
+        /* Q/K/V split, per-head norms, rotation and the cache append in one launch */
         if (fail_layer == (int)L) return dev_fail(e, "gqa (injected)", L, WR_ERR_INTERNAL);
         if (batch) {
             wr_hip_kv *kvs[WR_BATCH_MAX];
@@ -261,22 +260,19 @@ wr_status wrh_forward_rows_device(wr_model *m, wrh_workspace *hs, wrh_devspace *
                 at[r] = ss[r]->pos;
                 seq_k[r] = ss[r]->pos + 1;
             }
-            TRY(wr_hip_attn_append_batched_dev(R, kvs, L, at, ds->k, ds->v), "kv append");
+            TRY(wr_hip_rows_qkv_append_dev(ds->qkv, qd + 2 * kd, R, nq, dl->q_norm, dl->k_norm, m->rms_eps,
+                                           ds->rope, n_rot, R, kvs, L, at, ds->q), "qkv split + kv append");
             for (uint32_t r = 0; r < R; r++) ss[r]->kv_rows[L] = ss[r]->pos + 1;
             TRY(wr_hip_attn_decode_batched_dev(R, kvs, L, seq_k, ds->q, ds->attn, nq, 0.0f, 0), "gqa");
         } else {
             wr_session *s = ss[0];
-            if (R == 1) {                          /* one launch instead of a K and a V kernel */
-                wr_hip_kv *one[1] = {s->kv};
-                TRY(wr_hip_attn_append_batched_dev(1, one, L, &pos0, ds->k, ds->v), "kv append");
-            } else {
-                TRY(wr_hip_attn_append_dev(s->kv, L, pos0, R, ds->k, ds->v), "kv append");
-            }
+            wr_hip_kv *one[1] = {s->kv};
+            TRY(wr_hip_rows_qkv_append_dev(ds->qkv, qd + 2 * kd, R, nq, dl->q_norm, dl->k_norm, m->rms_eps,
+                                           ds->rope, n_rot, 1, one, L, &pos0, ds->q), "qkv split + kv append");
             s->kv_rows[L] = pos0 + R;
             if (prefill) {
                 TRY(wr_hip_attn_prefill_dev(s->kv, L, pos0, R, ds->q, ds->attn, nq, 0.0f, 0), "gqa");
             } else {
-                wr_hip_kv *one[1] = {s->kv};
                 const uint32_t sk = pos0 + 1;
                 TRY(wr_hip_attn_decode_batched_dev(1, one, L, &sk, ds->q, ds->attn, nq, 0.0f, 0), "gqa");
             }
