@@ -507,6 +507,23 @@ __global__ __launch_bounds__(kProjThreads) void proj_rows_kernel(const ProjArgs 
         // loop are unconditional and the last batch is peeled, so the
         // compiler's load counting keeps the prefetched batch in flight.
         half8 wa[KB][NT], wb[KB][NT];
+        // The operand fragments travel a batch ahead with the weights: read when
+        // needed they are cache hits, but a round trip to L2 per batch on a
+        // chain of four to thirty batches that is the launch's critical path.
+        half8 xa[KB][GROUPS], xb[KB][GROUPS];
+        auto load_x = [&](half8 (&xv)[KB][GROUPS], uint32_t k0) {
+#pragma unroll
+            for (int u = 0; u < KB; u++)
+#pragma unroll
+                for (int gi = 0; gi < GROUPS; gi++) xv[u][gi] = xp[((size_t)gi * ktiles + k0 + u) * 64];
+        };
+        auto step = [&](const half8 (&wv)[NT], const half8 (&xv)[GROUPS]) {
+#pragma unroll
+            for (int gi = 0; gi < GROUPS; gi++)
+#pragma unroll
+                for (int t = 0; t < NT; t++)
+                    acc[t][gi] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wv[t], xv[gi], acc[t][gi], 0, 0, 0);
+        };
         uint32_t kt = k_begin;
         const uint32_t full_end = k_begin + kper / KB * KB;
         if (kt < full_end) {
@@ -515,22 +532,27 @@ __global__ __launch_bounds__(kProjThreads) void proj_rows_kernel(const ProjArgs 
 #pragma unroll
                 for (int t = 0; t < NT; t++)
                     wa[u][t] = __builtin_nontemporal_load(&wp[t][(size_t)(kt + u) * 64]);
+            load_x(xa, kt);
             while (kt + 2 * KB <= full_end) {
 #pragma unroll
                 for (int u = 0; u < KB; u++)
 #pragma unroll
                     for (int t = 0; t < NT; t++)
                         wb[u][t] = __builtin_nontemporal_load(&wp[t][(size_t)(kt + KB + u) * 64]);
+                load_x(xb, kt + KB);
 #pragma unroll
-                for (int u = 0; u < KB; u++) proj_step<GROUPS, NT>(acc, wa[u], xp, ktiles, kt + u);
+                for (int u = 0; u < KB; u++) step(wa[u], xa[u]);
 #pragma unroll
-                for (int u = 0; u < KB; u++)
+                for (int u = 0; u < KB; u++) {
 #pragma unroll
                     for (int t = 0; t < NT; t++) wa[u][t] = wb[u][t];
+#pragma unroll
+                    for (int gi = 0; gi < GROUPS; gi++) xa[u][gi] = xb[u][gi];
+                }
                 kt += KB;
             }
 #pragma unroll
-            for (int u = 0; u < KB; u++) proj_step<GROUPS, NT>(acc, wa[u], xp, ktiles, kt + u);
+            for (int u = 0; u < KB; u++) step(wa[u], xa[u]);
             kt += KB;
         }
         for (; kt < k_end; kt++) {                               // part not a multiple of the batch
