@@ -246,3 +246,38 @@ def test_fused_sources_with_many_rows(n_in):
     for d in (xd, nwd, gud, addd, tmp, y1, y2):
         d.free()
     w.close()
+
+
+@pytest.mark.parametrize("n_in,n_out", [(1024, 4096), (3072, 1024), (2048, 48), (14336, 64), (96, 16)])
+def test_one_row_equals_its_row_of_two(n_in, n_out):
+    # A single row takes the kernel that builds its operand terms in LDS; two rows
+    # take the fragment launch and then the product.  Same values, same order of
+    # every sum: the row's bits must not depend on the company it keeps (the
+    # reference's batch contract, src/core/batch.c:15-19).  All three sources.
+    lib = hipattn.lib()
+    x = synth.normal(71 + n_in, (2, n_in), std=2.0)
+    nw = synth.normal(72, (n_in,)) * np.float32(0.2) + np.float32(1.0)
+    gu = synth.normal(73 + n_in, (2, 2 * n_in), std=2.0)
+    add = synth.normal(74, (2, n_out))
+    w16 = _w16(75, n_out, n_in, 0.1)
+    w = hipattn.Weight([w16])
+    D = hipattn.DeviceBuffer
+    xd, nwd, gud, addd = D.from_host(x), D.from_host(nw), D.from_host(gu), D.from_host(add)
+    y1, y2 = D(n_out * 4), D(2 * n_out * 4)
+    eps = 1e-6
+    for what, one, two in (
+        ("plain", lambda: w.rows_dev(1, xd, n_in, y1, n_out, add_dev=addd),
+         lambda: w.rows_dev(2, xd, n_in, y2, n_out, add_dev=addd)),
+        ("norm", lambda: lib.wr_hip_proj_rows_norm_dev(w.h, 1, xd.p, n_in, nwd.p, eps, None, y1.p, n_out),
+         lambda: lib.wr_hip_proj_rows_norm_dev(w.h, 2, xd.p, n_in, nwd.p, eps, None, y2.p, n_out)),
+        ("swiglu", lambda: lib.wr_hip_proj_rows_swiglu_dev(w.h, 1, gud.p, 2 * n_in, None, y1.p, n_out),
+         lambda: lib.wr_hip_proj_rows_swiglu_dev(w.h, 2, gud.p, 2 * n_in, None, y2.p, n_out)),
+    ):
+        assert one() in (None, hipattn.OK) and two() in (None, hipattn.OK)
+        hipattn.sync()
+        a, b = y1.to_host((1, n_out)), y2.to_host((2, n_out))
+        assert a[0].tobytes() == b[0].tobytes(), what
+    _check(w.rows(x[:1]), x[:1], w16, "one row")
+    for d in (xd, nwd, gud, addd, y1, y2):
+        d.free()
+    w.close()

@@ -418,8 +418,9 @@ struct ProjArgs {
 // its lo term.  The two are combined, the row's scale undone, the optional
 // residual added.  Tiles past N and rows past R are dropped.
 __device__ __forceinline__ void proj_store_tile(const ProjArgs& a, f32x4 v, uint32_t nt, uint32_t group,
-                                                int lane)
+                                                int lane, const float* scales = nullptr)
 {
+    if (!scales) scales = a.scales;
     const int c = lane & 15, g = lane >> 4;
     const int partner_addr = (lane ^ 8) * 4;
 #pragma unroll
@@ -429,7 +430,7 @@ __device__ __forceinline__ void proj_store_tile(const ProjArgs& a, f32x4 v, uint
     }
     const uint32_t row = group * 8 + (c & 7);
     if (c < 8 && row < a.R && nt < a.N / 16) {
-        const float sc = a.scales[row];
+        const float sc = scales[row];
         const size_t o = (size_t)row * a.ldy + nt * 16 + g * 4;
         f32x4 r;
 #pragma unroll
@@ -592,6 +593,116 @@ __global__ __launch_bounds__(kProjThreads) void proj_rows_kernel(const ProjArgs 
     for (int t = 0; t < NT; t++)
 #pragma unroll
         for (int gi = 0; gi < GROUPS; gi++) proj_store_tile(a, acc[t][gi], nt0 + t, group0 + gi, lane);
+}
+
+// One row (a decode step): proj_rows_kernel<1, 1> with the fragment kernel
+// folded in.  Every workgroup builds the row's operand terms in its own LDS
+// (4 bytes per input: hi and lo of the one live column pair) while its first
+// batch of weights is on the way, instead of reading fragments a launch before
+// it wrote: a decode step is a chain of dependent launches of a few
+// microseconds each, and this removes four of ten per layer.  The row's values,
+// the scale and the order of every sum are those of proj_prep_kernel followed
+// by proj_rows_kernel<1, 1> (same helpers, same loops), so the result has the
+// same bits: a serial step still equals its row of a batched step.
+template <int SRC>
+__global__ __launch_bounds__(kProjThreads) void proj_row1_kernel(const ProjArgs a, const ProjPrepArgs p)
+{
+    constexpr int KB = kProjKBatch;
+    extern __shared__ __attribute__((aligned(16))) unsigned char row1_smem[];
+    half8* sfrag = reinterpret_cast<half8*>(row1_smem);           // [K/8][2]: hi, lo of chunk q
+    __shared__ f32x4 s_part[3 * 64];
+    __shared__ float s4[4];
+    __shared__ float s_scale;
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t t = threadIdx.x;
+    const uint32_t S = a.ksplit;
+    const uint32_t slot = wave / S, part = wave % S;
+    const uint32_t nt0 = blockIdx.x * (4 / S) + slot;
+    const uint32_t ntiles = a.N / 16;
+    const bool live = nt0 < ntiles;
+    const uint32_t ktiles = a.K / 32, nchunks = a.K / 8;
+    const uint32_t kper = ktiles / S;
+    const uint32_t k_begin = part * kper, k_end = k_begin + kper;
+    const half8* wp = a.w + (size_t)(live ? nt0 : ntiles - 1) * ktiles * 64 + lane;
+
+    // the first batch of weights leaves before the row is touched
+    half8 wa[KB], wb[KB];
+    uint32_t kt = k_begin;
+    const uint32_t full_end = k_begin + kper / KB * KB;
+    if (kt < full_end) {
+#pragma unroll
+        for (int u = 0; u < KB; u++) wa[u] = __builtin_nontemporal_load(&wp[(size_t)(kt + u) * 64]);
+    }
+
+    // the row's terms, as proj_prep_kernel forms them
+    const float* xr = p.x;
+    float inv_rms = 1.0f;
+    if constexpr (SRC == kProjSrcRmsNorm)
+        inv_rms = 1.0f / sqrtf(row_sumsq_256(xr, a.K, s4) / (float)a.K + p.eps);
+    float mx = 0.f;
+    for (uint32_t k = t; k < a.K; k += 256) mx = fmaxf(mx, fabsf(proj_src_value<SRC>(p, xr, k, inv_rms)));
+    mx = block_max_256(mx, s4);
+    uint32_t ex = (__float_as_uint(mx) >> 23) & 0xFFu;
+    if (ex == 0 || ex == 0xFF) ex = 127;
+    if (ex > 253) ex = 253;
+    if (t == 0) s_scale = __uint_as_float(ex << 23);
+    const float inv = __uint_as_float((254u - ex) << 23);
+    for (uint32_t q = t; q < nchunks; q += 256) {
+        half8 hi, lo;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const float sv = proj_src_value<SRC>(p, xr, q * 8 + j, inv_rms) * inv;
+            _Float16 h = (_Float16)sv;
+            if (fabsf((float)h) < 6.103515625e-05f) h = (_Float16)0.0f;      // 2^-14
+            hi[j] = h;
+            lo[j] = (_Float16)((sv - (float)h) * kProjLoScale);
+        }
+        sfrag[q * 2] = hi;
+        sfrag[q * 2 + 1] = lo;
+    }
+    __syncthreads();
+
+    // B operand of k-step kt: column 0 = hi, column 8 = lo of row 0, the rest zero
+    const int c = lane & 15, g = lane >> 4;
+    const bool has = (c & 7) == 0;
+    const half8* my = sfrag + g * 2 + (c >> 3);
+    half8 zero;
+#pragma unroll
+    for (int j = 0; j < 8; j++) zero[j] = (_Float16)0.0f;
+    f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+    auto step = [&](const half8& wv, uint32_t k) {
+        const half8 xb = has ? my[(size_t)k * 8] : zero;
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(wv, xb, acc, 0, 0, 0);
+    };
+    if (kt < full_end) {
+        while (kt + 2 * KB <= full_end) {
+#pragma unroll
+            for (int u = 0; u < KB; u++) wb[u] = __builtin_nontemporal_load(&wp[(size_t)(kt + KB + u) * 64]);
+#pragma unroll
+            for (int u = 0; u < KB; u++) step(wa[u], kt + u);
+#pragma unroll
+            for (int u = 0; u < KB; u++) wa[u] = wb[u];
+            kt += KB;
+        }
+#pragma unroll
+        for (int u = 0; u < KB; u++) step(wa[u], kt + u);
+        kt += KB;
+    }
+    for (; kt < k_end; kt++) step(__builtin_nontemporal_load(&wp[(size_t)kt * 64]), kt);
+
+    if (S > 1) {                                                 // uniform over the workgroup
+        if (part > 0) s_part[(slot * (S - 1) + (part - 1)) * 64 + lane] = acc;
+        __syncthreads();
+        if (part > 0) return;
+        for (uint32_t pp = 1; pp < S; pp++) {
+            const f32x4 o = s_part[(slot * (S - 1) + (pp - 1)) * 64 + lane];
+#pragma unroll
+            for (int i = 0; i < 4; i++) acc[i] += o[i];
+        }
+    }
+    if (!live) return;
+    proj_store_tile(a, acc, nt0, 0, lane, &s_scale);
 }
 
 // Many rows (prefill chunks), products too small to fill the chip with the

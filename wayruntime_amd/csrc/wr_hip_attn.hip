@@ -162,6 +162,18 @@ int copy_down_sync(void* dst_host, const void* src_dev, size_t bytes)
     return WR_HIP_OK;
 }
 
+template <typename Kern, typename A0, typename A1>
+void launch_main(Kern kernel, dim3 grid, dim3 block, const A0& a0, const A1& a1, size_t lds_bytes)
+{
+    if (g.profiling && g.ev_used + 2 <= g.ev.size()) {
+        hipExtLaunchKernelGGL(kernel, grid, block, lds_bytes, g.stream, g.ev[g.ev_used],
+                              g.ev[g.ev_used + 1], 0, a0, a1);
+        g.ev_used += 2;
+    } else {
+        hipLaunchKernelGGL(kernel, grid, block, lds_bytes, g.stream, a0, a1);
+    }
+}
+
 template <typename Kern, typename Args>
 void launch_main(Kern kernel, dim3 grid, dim3 block, const Args& args, size_t lds_bytes = 0)
 {
@@ -452,6 +464,7 @@ void launch_proj(const ProjArgs& a, uint32_t groups)
 //   registers, 64 x 32, the four waves split the input range;
 //   registers, 32 x 32, likewise.
 constexpr int kProjGemmMinRows = 64;
+constexpr size_t kProjRow1MaxLds = 60 * 1024;      // inputs up to 15 360 take the one-row kernel
 
 template <int GROUPS, int NT>
 void launch_proj_gemm_split(const ProjArgs& a, uint32_t groups)
@@ -495,6 +508,8 @@ int proj_chunk_locked(const wr_hip_weight* w, uint32_t rows, const float* x_dev,
     const bool gemm = rows >= (uint32_t)kProjGemmMinRows;  // the GEMM kernel clamps instead of padding
     if (groups > 2 && !gemm) groups = (groups + 3) / 4 * 4;
     const uint32_t ktiles = w->n_in / 32;
+    // one row: the fragment step runs inside the product's kernel (4 bytes of LDS per input)
+    const bool row1 = rows == 1 && (size_t)w->n_in * 4 <= kProjRow1MaxLds;
     const size_t frag_bytes = (size_t)groups * ktiles * 1024;
     int rc = ensure_device(g.d_proj, frag_bytes + kProjMaxRows * sizeof(float));
     if (rc) return rc;
@@ -533,7 +548,9 @@ int proj_chunk_locked(const wr_hip_weight* w, uint32_t rows, const float* x_dev,
         else                                                                                         \
             hipLaunchKernelGGL(HIP_KERNEL_NAME(proj_prep_kernel<SRC, 0>), pgrid, pblock, 0, g.stream, pa); \
     } while (0)
-    if (src.kind == kProjSrcRmsNorm)
+    if (row1)
+        ;                                           // no fragment launch
+    else if (src.kind == kProjSrcRmsNorm)
         WR_LAUNCH_PREP(kProjSrcRmsNorm);
     else if (src.kind == kProjSrcSwiglu)
         WR_LAUNCH_PREP(kProjSrcSwiglu);
@@ -566,7 +583,16 @@ int proj_chunk_locked(const wr_hip_weight* w, uint32_t rows, const float* x_dev,
             ksplit *= 2;
     }
     a.ksplit = ksplit;
-    if (gemm)
+    if (row1) {
+        const dim3 grid((tiles + 4 / ksplit - 1) / (4 / ksplit)), block(kProjThreads);
+        const size_t lds = (size_t)w->n_in * 4;
+        if (src.kind == kProjSrcRmsNorm)
+            launch_main(proj_row1_kernel<kProjSrcRmsNorm>, grid, block, a, pa, lds);
+        else if (src.kind == kProjSrcSwiglu)
+            launch_main(proj_row1_kernel<kProjSrcSwiglu>, grid, block, a, pa, lds);
+        else
+            launch_main(proj_row1_kernel<kProjSrcPlain>, grid, block, a, pa, lds);
+    } else if (gemm)
         launch_proj_gemm(a, groups);
     else if (groups == 1)
         launch_proj<1, 1>(a, groups);
