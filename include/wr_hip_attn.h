@@ -159,6 +159,11 @@ int wr_hip_attn_prefill(wr_hip_kv *kv, uint32_t layer, uint32_t p0,
  * form q_dev and out_dev are [n, nq, hd] contiguous. */
 void *wr_hip_attn_dev_alloc(size_t bytes);
 void  wr_hip_attn_dev_free(void *p);
+/* Page-locked host memory: copies to and from it run at the link's rate and
+ * need no staging (a 10 MB block of logits comes down five times faster than
+ * into pageable memory).  Freed with wr_hip_attn_host_free before shutdown. */
+void *wr_hip_attn_host_alloc(size_t bytes);
+void  wr_hip_attn_host_free(void *p);
 int   wr_hip_attn_h2d(void *dst_dev, const void *src_host, size_t bytes);
 int   wr_hip_attn_d2h(void *dst_host, const void *src_dev, size_t bytes);
 int   wr_hip_attn_sync(void);

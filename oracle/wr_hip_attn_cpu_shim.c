@@ -289,6 +289,8 @@ int wr_hip_rows_qkv_prep_dev(const float *qkv, uint32_t ld, uint32_t rows, uint3
     (void)cs; (void)n_rot; (void)q; (void)k; (void)v;
     return WR_HIP_ERR_STATE;
 }
+void *wr_hip_attn_host_alloc(size_t bytes) { return malloc(bytes); }
+void wr_hip_attn_host_free(void *p) { free(p); }
 int wr_hip_rows_qkv_append_dev(const float *qkv, uint32_t ld, uint32_t rows, uint32_t nq,
                                const float *qn, const float *kn, float eps, const float *cs,
                                uint32_t n_rot, uint32_t n_kv, wr_hip_kv *const *kv, uint32_t layer,

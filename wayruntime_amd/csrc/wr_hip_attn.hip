@@ -1054,6 +1054,23 @@ void wr_hip_attn_dev_free(void* p)
     (void)hipFree(p);
 }
 
+void* wr_hip_attn_host_alloc(size_t bytes)
+{
+    if (!g.inited || bytes == 0) return nullptr;
+    Locked lk;
+    void* p = nullptr;
+    if (hipHostMalloc(&p, bytes, hipHostMallocDefault) != hipSuccess) return nullptr;
+    return p;
+}
+
+void wr_hip_attn_host_free(void* p)
+{
+    if (!g.inited || !p) return;
+    Locked lk;
+    (void)hipStreamSynchronize(g.stream);
+    (void)hipHostFree(p);
+}
+
 int wr_hip_attn_h2d(void* dst_dev, const void* src_host, size_t bytes)
 {
     if (!g.inited) return WR_HIP_ERR_STATE;

@@ -82,6 +82,8 @@ def load() -> C.CDLL:
         "wr_hip_rows_qkv_append_dev": (C.c_int, [_vp, _u32, _u32, _u32, _vp, _vp, C.c_float, _vp, _u32, _u32,
                                                  C.POINTER(_vp), _u32, C.POINTER(_u32), _vp]),
         "wr_hip_rows_swiglu_dev": (C.c_int, [_vp, _u32, _vp, _u32, _u32, _u32]),
+        "wr_hip_attn_host_alloc": (_vp, [C.c_size_t]),
+        "wr_hip_attn_host_free": (None, [_vp]),
         "wr_hip_attn_set_tuning": (None, [_u32, C.c_int]),
         "wr_hip_attn_profile_begin": (C.c_int, [_u32]),
         "wr_hip_attn_profile_end": (C.c_int, [C.POINTER(C.c_double), C.POINTER(_u32)]),

@@ -167,6 +167,84 @@ void wrh_devspace_free(wrh_devspace *ws)
     memset(ws, 0, sizeof *ws);
 }
 
+/* ---------------------------------------------------------- kept scratch -- */
+
+static void scratch_destroy(struct wrh_scratch *sc)
+{
+    if (!sc) return;
+    wrh_devspace_free(&sc->ds);
+    wrh_workspace_free(&sc->ws);
+    if (sc->logits_host) wr_hip_attn_host_free(sc->logits_host);
+    free(sc);
+}
+
+static struct wrh_scratch *scratch_create(const wr_model *m, uint32_t rows, uint32_t logit_rows)
+{
+    struct wrh_scratch *sc = calloc(1, sizeof *sc);
+    if (!sc) return NULL;
+    sc->rows = rows;
+    sc->logit_rows = logit_rows;
+    int ok = wrh_workspace_init(&sc->ws, m, rows) == WR_OK;
+    ok = ok && wrh_devspace_init(&sc->ds, m, rows, logit_rows) == WR_OK;
+    if (ok && logit_rows) {
+        sc->logits_host = wr_hip_attn_host_alloc((size_t)logit_rows * m->vocab * sizeof(float));
+        ok = sc->logits_host != NULL;
+    }
+    if (!ok) {
+        scratch_destroy(sc);
+        return NULL;
+    }
+    return sc;
+}
+
+struct wrh_scratch *wrh_scratch_acquire(wr_model *m, int kind, uint32_t rows, uint32_t logit_rows)
+{
+    struct wrh_scratch **slot = kind ? &m->prefill_scratch : &m->batch_scratch;
+    pthread_mutex_lock(&m->lock);
+    struct wrh_scratch *sc = *slot;
+    if (sc && sc->busy) {                              /* a concurrent call has it */
+        pthread_mutex_unlock(&m->lock);
+        return scratch_create(m, rows, logit_rows);
+    }
+    if (sc && (sc->rows < rows || sc->logit_rows < logit_rows)) {
+        *slot = NULL;                                  /* too small: replace */
+        scratch_destroy(sc);
+        sc = NULL;
+    }
+    if (!sc) {
+        /* a batch set is sized for the largest batch once; a prefill set for this call */
+        const uint32_t r = kind ? rows : WR_BATCH_MAX;
+        sc = scratch_create(m, r > rows ? r : rows, kind ? logit_rows : WR_BATCH_MAX);
+        if (sc) {
+            sc->cached = 1;
+            *slot = sc;
+        }
+    }
+    if (sc) sc->busy = 1;
+    pthread_mutex_unlock(&m->lock);
+    return sc;
+}
+
+void wrh_scratch_release(wr_model *m, struct wrh_scratch *sc)
+{
+    if (!sc) return;
+    if (!sc->cached) {
+        scratch_destroy(sc);
+        return;
+    }
+    pthread_mutex_lock(&m->lock);
+    sc->busy = 0;
+    sc->ws.staged_rows = 0;
+    pthread_mutex_unlock(&m->lock);
+}
+
+void wrh_scratch_free_all(wr_model *m)
+{
+    scratch_destroy(m->batch_scratch);
+    scratch_destroy(m->prefill_scratch);
+    m->batch_scratch = m->prefill_scratch = NULL;
+}
+
 /* --------------------------------------------------------------- forward -- */
 
 static wr_status dev_fail(wr_engine *e, const char *what, uint32_t layer, int rc)

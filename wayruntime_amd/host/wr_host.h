@@ -78,6 +78,12 @@ struct wr_model {
     wrh_weight w_gate[WRH_MAX_LAYERS], w_up[WRH_MAX_LAYERS], w_down[WRH_MAX_LAYERS];
 
     struct wrh_dev_model *dev;   /* device copies of the weights, NULL on the host walk */
+    /* Scratch of the device walk's multi-row calls, kept between calls (a
+     * 16-session step otherwise spends a third of its time allocating device
+     * memory and faulting in ten megabytes of logits): one set for
+     * wr_batch_step, one for wr_prefill.  A call that finds its set taken by a
+     * concurrent call allocates its own as before. */
+    struct wrh_scratch *batch_scratch, *prefill_scratch;
 
     void           *map;         /* mmap of the GGUF file */
     size_t          map_bytes;
@@ -102,6 +108,14 @@ typedef struct wrh_workspace {
     uint32_t staged_rows, staged_pos0;
 } wrh_workspace;
 
+struct wrh_scratch;
+/* Takes the model's cached set (kind 0 = batch, 1 = prefill) when it is free,
+ * growing it to rows / logit_rows; otherwise returns a fresh one.  NULL when
+ * memory runs out.  Release returns it (a fresh one is freed). */
+struct wrh_scratch *wrh_scratch_acquire(wr_model *m, int kind, uint32_t rows, uint32_t logit_rows);
+void wrh_scratch_release(wr_model *m, struct wrh_scratch *sc);
+void wrh_scratch_free_all(wr_model *m);
+
 /* Device scratch for R rows of the device walk (wr_device.c). */
 typedef struct wrh_devspace {
     uint32_t rows_cap, logit_rows;
@@ -114,6 +128,16 @@ typedef struct wrh_devspace {
     float *logits;                       /* [logit_rows][vocab] */
     float *block;
 } wrh_devspace;
+
+/* Everything a multi-row call of the device walk needs besides the model. */
+struct wrh_scratch {
+    wrh_workspace ws;                    /* host rows (embedding, angles) */
+    wrh_devspace  ds;
+    float        *logits_host;           /* page-locked, [logit_rows][vocab]; NULL when logit_rows == 0 */
+    uint32_t      rows, logit_rows;
+    int           cached;                /* belongs to the model (else freed on release) */
+    int           busy;
+};
 
 struct wr_session {
     wr_model       *model;

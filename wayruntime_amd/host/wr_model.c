@@ -745,6 +745,7 @@ void wr_model_free(wr_model *m)
         return;
     }
     if (m->engine && m->engine->models_live) m->engine->models_live--;
+    wrh_scratch_free_all(m);
     wrh_device_model_free(m);
     munmap(m->map, m->map_bytes);
     pthread_mutex_destroy(&m->lock);

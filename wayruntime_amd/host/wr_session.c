@@ -433,27 +433,32 @@ int wr_prefill(wr_session *s, const uint32_t *ids, uint32_t n)
          * whole call before anything is written */
         for (uint32_t i = 0; i < n && st == WR_OK; i++)
             if (ids[i] >= m->vocab) st = WR_ERR_INVAL;
-        wrh_workspace ws;
-        wrh_devspace ds;
-        memset(&ds, 0, sizeof ds);
         const uint32_t cap = m->dev ? WRH_DEVICE_PREFILL_CHUNK : WRH_PREFILL_CHUNK;
         const uint32_t chunk = n < cap ? n : cap;
-        if (st == WR_OK && wrh_workspace_init(&ws, m, chunk) != WR_OK) st = WR_ERR_NOMEM;
-        if (st == WR_OK) {
-            if (m->dev && wrh_devspace_init(&ds, m, chunk, 0) != WR_OK) st = WR_ERR_NOMEM;
-            wr_session *one[1] = {s};
+        wr_session *one[1] = {s};
+        if (st == WR_OK && m->dev) {
+            /* device walk: scratch kept by the model between calls */
+            struct wrh_scratch *sc = wrh_scratch_acquire(m, 1, chunk, 0);
+            if (!sc) st = WR_ERR_NOMEM;
             for (uint32_t done = 0; done < n && st == WR_OK; done += chunk) {
                 const uint32_t rows = (n - done < chunk) ? n - done : chunk;
-                if (m->dev) {
-                    const uint32_t left = n - done - rows;             /* staged while the device works */
-                    st = wrh_forward_rows_device(m, &ws, &ds, rows, one, ids + done, s->pos, 0, 1,
-                                                 take_fail_layer(m), NULL, 0, left < chunk ? left : chunk);
-                } else
-                    st = forward_rows(m, &ws, rows, one, ids + done, s->pos, FWD_PREFILL);
+                const uint32_t left = n - done - rows;                 /* staged while the device works */
+                st = wrh_forward_rows_device(m, &sc->ws, &sc->ds, rows, one, ids + done, s->pos, 0, 1,
+                                             take_fail_layer(m), NULL, 0, left < chunk ? left : chunk);
                 if (st == WR_OK) __atomic_store_n(&s->pos, s->pos + rows, __ATOMIC_RELEASE);
             }
-            wrh_devspace_free(&ds);
-            wrh_workspace_free(&ws);
+            wrh_scratch_release(m, sc);
+        } else if (st == WR_OK) {
+            wrh_workspace ws;
+            if (wrh_workspace_init(&ws, m, chunk) != WR_OK) st = WR_ERR_NOMEM;
+            if (st == WR_OK) {
+                for (uint32_t done = 0; done < n && st == WR_OK; done += chunk) {
+                    const uint32_t rows = (n - done < chunk) ? n - done : chunk;
+                    st = forward_rows(m, &ws, rows, one, ids + done, s->pos, FWD_PREFILL);
+                    if (st == WR_OK) __atomic_store_n(&s->pos, s->pos + rows, __ATOMIC_RELEASE);
+                }
+                wrh_workspace_free(&ws);
+            }
         }
         if (st != WR_OK) {
             __atomic_store_n(&s->pos, pos_entry, __ATOMIC_RELEASE);
@@ -501,25 +506,24 @@ int wr_batch_step(wr_session *const *sessions, const uint32_t *tokens, uint32_t 
     wrh_workspace ws;
     float *big = NULL;
     int have_ws = 0;
-    if (st == WR_OK) {
+    struct wrh_scratch *sc = NULL;
+    if (st == WR_OK && m->dev) {
+        /* device walk: rows, device scratch and page-locked logits kept by the model */
+        sc = wrh_scratch_acquire(m, 0, n, n);
+        if (!sc) st = WR_ERR_NOMEM;
+        if (st == WR_OK)
+            st = wrh_forward_rows_device(m, &sc->ws, &sc->ds, n, sessions, tokens, 0, 1, 0,
+                                         take_fail_layer(m), sc->logits_host, n, 0);
+        big = sc ? sc->logits_host : NULL;
+    } else if (st == WR_OK) {
         if (wrh_workspace_init(&ws, m, n) == WR_OK) have_ws = 1;
         else st = WR_ERR_NOMEM;
+        if (st == WR_OK) {
+            big = malloc((size_t)n * m->vocab * sizeof(float));
+            if (!big) st = WR_ERR_NOMEM;
+        }
+        if (st == WR_OK) st = forward_rows(m, &ws, n, sessions, tokens, 0, FWD_BATCH);
     }
-    if (st == WR_OK) {
-        big = malloc((size_t)n * m->vocab * sizeof(float));
-        if (!big) st = WR_ERR_NOMEM;
-    }
-    wrh_devspace ds;
-    memset(&ds, 0, sizeof ds);
-    if (st == WR_OK && m->dev && wrh_devspace_init(&ds, m, n, n) != WR_OK) st = WR_ERR_NOMEM;
-    if (st == WR_OK) {
-        if (m->dev)
-            st = wrh_forward_rows_device(m, &ws, &ds, n, sessions, tokens, 0, 1, 0,
-                                         take_fail_layer(m), big, n, 0);
-        else
-            st = forward_rows(m, &ws, n, sessions, tokens, 0, FWD_BATCH);
-    }
-    wrh_devspace_free(&ds);
     if (st == WR_OK) {
         /* one LM-head product for all n rows (reference: batch.c:45-104), then demux */
         if (!m->dev) wrh_matmul(m->engine, ws.normed, n, m->hidden, &m->lm_head, big, m->vocab);
@@ -531,7 +535,8 @@ int wr_batch_step(wr_session *const *sessions, const uint32_t *tokens, uint32_t 
     } else {
         for (uint32_t i = 0; i < n; i++) kv_rollback(sessions[i]);      /* nobody advanced */
     }
-    free(big);
+    if (sc) wrh_scratch_release(m, sc);
+    else free(big);
     if (have_ws) wrh_workspace_free(&ws);
 
     for (uint32_t i = 0; i < n; i++)
