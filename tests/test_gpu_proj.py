@@ -54,11 +54,13 @@ def _check(got, x, w16, what):
     (64, 96, 48, 0.5),            # ... its smallest row count; three input tiles (a wave with none), three output tiles
     (100, 160, 80, 0.3),          # ... a last row group of four rows, five input tiles
     (300, 160, 2512, 0.2),        # ... 64 x 32 tiles, a partial last tile both ways
-    (1030, 64, 32, 1.0),          # more rows than one launch takes: 1024 + a six-row launch
+    (4102, 64, 32, 1.0),          # more rows than one launch takes: 4096 + a six-row launch
     (500, 96, 4112, 0.3),         # LDS-staged GEMM, 128 x 64 tiles: partial output and row panels, odd input tiles
     (1000, 1056, 4112, 0.02),     # ... 33 input tiles
     (1000, 96, 8208, 0.3),        # LDS-staged GEMM, 128 x 128 tiles: partial output and row panels, three input tiles
     (1000, 32, 8208, 0.5),        # ... a single input tile (the ring's prologue covers the whole product)
+    (2040, 96, 4112, 0.3),        # LDS-staged GEMM, eight waves, 256 x 128 tiles: partial panels, three input tiles
+    (2040, 32, 4112, 0.5),        # ... a single input tile
 ])
 def test_projection_shapes_vs_oracle(rows, n_in, n_out, std):
     print("proj", rows, n_in, n_out, flush=True)

@@ -34,7 +34,7 @@
 namespace wr {
 
 constexpr int kProjThreads = 256;
-constexpr int kProjMaxRows = 1024;                // rows per launch (128 row groups)
+constexpr int kProjMaxRows = 4096;                // rows per launch (512 row groups)
 constexpr int kProjKBatch = 8;                    // k-steps (KiBs of W) a wave keeps in flight per buffer
 
 // Row-major F16 W[N][K] -> tile order.  One thread per 16-byte unit.
@@ -824,21 +824,27 @@ __global__ __launch_bounds__(kProjThreads, 3) void proj_gemm_split_kernel(const 
 // GROUPS = 8 is the tile described above; GROUPS = 4 halves the rows (128
 // outputs x 64 rows, 16 KiB per stage) for products with too few rows to fill
 // the chip with the large one.
-constexpr int kGemmRing = 3;
-template <int GROUPS>
+// WN = waves side by side along the outputs (2 or 4; two wave rows always),
+// RING = stages.  <8, 2, 3>: the tile above.  <4, 2, 3>: 128 x 64 for products
+// with too few rows to fill the chip with the large one.  <8, 4, 4>: eight
+// waves, 256 outputs x 128 rows, 32 KiB per stage copied three k-steps ahead,
+// one workgroup per CU: a third fewer bytes per MFMA than the four-wave tile.
+template <int GROUPS, int WN, int RING>
 constexpr size_t gemm_lds_bytes()
 {
-    return (size_t)kGemmRing * (8 + 2 * GROUPS) * 1024;   // KiB per stage: 8 weight tiles, 2 GROUPS fragments
+    return (size_t)RING * (WN * 4 + 2 * GROUPS) * 1024;   // KiB per stage: 4 WN weight tiles, 2 GROUPS fragments
 }
 
-template <int GROUPS>
-__global__ __launch_bounds__(kProjThreads, 2) void proj_gemm_lds_kernel(const ProjArgs a)
+template <int GROUPS, int WN, int RING>
+__global__ __launch_bounds__(128 * WN, WN == 2 ? 2 : 1) void proj_gemm_lds_kernel(const ProjArgs a)
 {
     extern __shared__ __attribute__((aligned(16))) unsigned char gemm_smem[];
-    constexpr int NT = 4, CHUNKS = 2 * NT + 2 * GROUPS, CPW = CHUNKS / 4;   // chunks a wave copies per stage
+    constexpr int NT = 4, WAVES = 2 * WN, CHUNKS = WN * NT + 2 * GROUPS, CPW = CHUNKS / WAVES;
+    static_assert(CHUNKS % WAVES == 0, "every wave copies the same number of chunks");
     constexpr uint32_t STAGE = CHUNKS * 1024;
     const int lane = threadIdx.x & 63;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t wn = wave % WN, wr = wave / WN;
     const uint32_t ktiles = a.K / 32, ntiles = a.N / 16, ngroups = (a.R + 7) / 8;
     const uint32_t klast = ktiles - 1;
     // Workgroup -> tile.  The dispatcher deals consecutive workgroups round-robin
@@ -846,29 +852,29 @@ __global__ __launch_bounds__(kProjThreads, 2) void proj_gemm_lds_kernel(const Pr
     // through all row panels of one before the next, so the workgroups resident
     // on an XCD at one time share a few weight panels (fetched once into its L2)
     // and the fragments of all rows.
-    const uint32_t nx = (ntiles + 2 * NT - 1) / (2 * NT), ny = (ngroups + 2 * GROUPS - 1) / (2 * GROUPS);
+    const uint32_t nx = (ntiles + WN * NT - 1) / (WN * NT), ny = (ngroups + 2 * GROUPS - 1) / (2 * GROUPS);
     const uint32_t xcd = blockIdx.x % 8, slot = blockIdx.x / 8;
     const uint32_t px = (slot / ny) * 8 + xcd, py = slot % ny;
     if (px >= nx) return;                                 // the grid is padded to eight equal shares
-    const uint32_t nt_wg = px * 2 * NT, g_wg = py * 2 * GROUPS;
+    const uint32_t nt_wg = px * WN * NT, g_wg = py * 2 * GROUPS;
     const uint32_t lds0 = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)gemm_smem);
 
-    // chunk c of a stage: weight tile nt_wg + c (c < 8) or fragment group g_wg + c - 8;
-    // one past the end re-reads the last one, and its results are dropped
+    // chunk c of a stage: weight tile nt_wg + c (c < WN * NT) or fragment group
+    // g_wg + c - WN * NT; one past the end re-reads the last one, and its results are dropped
     const unsigned char* src[CPW];
 #pragma unroll
     for (int i = 0; i < CPW; i++) {
         const uint32_t c = wave * CPW + i;
         const unsigned char* p =
-            c < 2 * NT ? reinterpret_cast<const unsigned char*>(a.w) + (size_t)min(nt_wg + c, ntiles - 1) * ktiles * 1024
-                       : reinterpret_cast<const unsigned char*>(a.xfrag) +
-                             (size_t)min(g_wg + c - 2 * NT, ngroups - 1) * ktiles * 1024;
+            c < WN * NT ? reinterpret_cast<const unsigned char*>(a.w) + (size_t)min(nt_wg + c, ntiles - 1) * ktiles * 1024
+                        : reinterpret_cast<const unsigned char*>(a.xfrag) +
+                              (size_t)min(g_wg + c - WN * NT, ngroups - 1) * ktiles * 1024;
         src[i] = uniform_ptr(p);
     }
     const uint32_t lane_off = lane * 16;
     auto issue = [&](uint32_t kt) {                        // a k-step past the end copies the last one again
         const size_t k = (size_t)min(kt, klast) * 1024;
-        const uint32_t to = lds0 + (kt % kGemmRing) * STAGE + wave * CPW * 1024;
+        const uint32_t to = lds0 + (kt % RING) * STAGE + wave * CPW * 1024;
 #pragma unroll
         for (int i = 0; i < CPW; i++) lds_direct_load(to + i * 1024, src[i] + k, lane_off);
     };
@@ -879,14 +885,15 @@ __global__ __launch_bounds__(kProjThreads, 2) void proj_gemm_lds_kernel(const Pr
 #pragma unroll
         for (int gi = 0; gi < GROUPS; gi++) acc[t][gi] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    issue(0);
-    issue(1);
-    const uint32_t w_off = (wave & 1) * NT * 1024 + lane * 16;
-    const uint32_t x_off = (2 * NT + (wave >> 1) * GROUPS) * 1024 + lane * 16;
+#pragma unroll
+    for (int st0 = 0; st0 < RING - 1; st0++) issue(st0);
+    const uint32_t w_off = wn * NT * 1024 + lane * 16;
+    const uint32_t x_off = (WN * NT + wr * GROUPS) * 1024 + lane * 16;
     for (uint32_t kt = 0; kt < ktiles; kt++) {
-        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(CPW) : "memory");
-        issue(kt + 2);
-        const unsigned char* st = gemm_smem + (kt % kGemmRing) * STAGE;
+        // this wave's copies of stage kt have landed; those of the RING - 2 stages after it may be in flight
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(CPW * (RING - 2)) : "memory");
+        issue(kt + RING - 1);
+        const unsigned char* st = gemm_smem + (kt % RING) * STAGE;
         half8 wv[NT], xv[GROUPS];
 #pragma unroll
         for (int t = 0; t < NT; t++) wv[t] = *reinterpret_cast<const half8*>(st + w_off + t * 1024);
@@ -897,16 +904,16 @@ __global__ __launch_bounds__(kProjThreads, 2) void proj_gemm_lds_kernel(const Pr
 #pragma unroll
             for (int t = 0; t < NT; t++)
                 acc[t][gi] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wv[t], xv[gi], acc[t][gi], 0, 0, 0);
-        // all twelve operand reads first (their latency overlaps, and the first
-        // MFMAs hide the rest), then the MFMAs: left alone the scheduler reads
-        // two fragments at a time and waits for each pair
+        // all operand reads first (their latency overlaps, and the first MFMAs
+        // hide the rest), then the MFMAs: left alone the scheduler reads two
+        // fragments at a time and waits for each pair
         __builtin_amdgcn_sched_group_barrier(0x100, NT + GROUPS, 0);
         __builtin_amdgcn_sched_group_barrier(0x008, NT * GROUPS, 0);
     }
-    // the last two steps' copies still target the ring
+    // the last steps' copies still target the ring
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
-    const uint32_t nt0 = nt_wg + (wave & 1) * NT, group0 = g_wg + (wave >> 1) * GROUPS;
+    const uint32_t nt0 = nt_wg + wn * NT, group0 = g_wg + wr * GROUPS;
     if (nt0 >= ntiles || group0 >= ngroups) return;
 #pragma unroll
     for (int t = 0; t < NT; t++)

@@ -459,7 +459,8 @@ void launch_proj(const ProjArgs& a, uint32_t groups)
 }
 
 // Prefill-sized row counts: the largest tile that still fills the chip.
-//   LDS-staged, 128 outputs x 128 rows per workgroup, from two workgroups per CU;
+//   LDS-staged, eight waves, 256 outputs x 128 rows per workgroup, from one workgroup per CU;
+//   LDS-staged, 128 x 128, from two workgroups per CU;
 //   LDS-staged, 128 x 64, from one per CU;
 //   registers, 64 x 32, the four waves split the input range;
 //   registers, 32 x 32, likewise.
@@ -478,12 +479,16 @@ void launch_proj_gemm(const ProjArgs& a, uint32_t groups)
     const uint32_t nt = a.N / 16, panels = (nt + 7) / 8;
     // one-dimensional grids: eight equal shares of output panels, times the row panels
     const uint32_t share = (panels + 7) / 8 * 8;
-    if (panels * ((groups + 15) / 16) >= 512)
-        launch_main(proj_gemm_lds_kernel<8>, dim3(share * ((groups + 15) / 16)), dim3(kProjThreads), a,
-                    gemm_lds_bytes<8>());
+    const uint32_t wide = (nt + 15) / 16, wshare = (wide + 7) / 8 * 8;
+    if (wide * ((groups + 15) / 16) >= 256)
+        launch_main(proj_gemm_lds_kernel<8, 4, 4>, dim3(wshare * ((groups + 15) / 16)), dim3(512), a,
+                    gemm_lds_bytes<8, 4, 4>());
+    else if (panels * ((groups + 15) / 16) >= 512)
+        launch_main(proj_gemm_lds_kernel<8, 2, 3>, dim3(share * ((groups + 15) / 16)), dim3(kProjThreads), a,
+                    gemm_lds_bytes<8, 2, 3>());
     else if (panels * ((groups + 7) / 8) >= 256)
-        launch_main(proj_gemm_lds_kernel<4>, dim3(share * ((groups + 7) / 8)), dim3(kProjThreads), a,
-                    gemm_lds_bytes<4>());
+        launch_main(proj_gemm_lds_kernel<4, 2, 3>, dim3(share * ((groups + 7) / 8)), dim3(kProjThreads), a,
+                    gemm_lds_bytes<4, 2, 3>());
     else if (((nt + 3) / 4) * ((groups + 3) / 4) >= 384)
         launch_proj_gemm_split<4, 4>(a, groups);
     else
@@ -669,8 +674,11 @@ int wr_hip_attn_init(int device)
                                     hipFuncAttributeMaxDynamicSharedMemorySize,
                                     (int)split_smem_bytes<128>());
         if (e == hipSuccess)
-            e = hipFuncSetAttribute(reinterpret_cast<const void*>(proj_gemm_lds_kernel<8>),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)gemm_lds_bytes<8>());
+            e = hipFuncSetAttribute(reinterpret_cast<const void*>(proj_gemm_lds_kernel<8, 2, 3>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)gemm_lds_bytes<8, 2, 3>());
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute(reinterpret_cast<const void*>(proj_gemm_lds_kernel<8, 4, 4>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)gemm_lds_bytes<8, 4, 4>());
         if (e != hipSuccess) rc = hip_fail(e, "kernel LDS size", 0);
     }
     if (rc != WR_HIP_OK) {
