@@ -255,6 +255,11 @@ int wr_hip_proj_rows_norm_dev(const wr_hip_weight *w, uint32_t rows,
 int wr_hip_proj_rows_swiglu_dev(const wr_hip_weight *w, uint32_t rows,
                                 const float *gate_up_dev, uint32_t ld,
                                 const float *add_dev, float *y_dev, uint32_t ldy);
+/* the same with the tanh form of GELU in place of SiLU (wri_op_fused_gelu_mul,
+ * src/core/kernels.c:969-976; Gemma's FFN, session.c:376-381) */
+int wr_hip_proj_rows_geglu_dev(const wr_hip_weight *w, uint32_t rows,
+                               const float *gate_up_dev, uint32_t ld,
+                               const float *add_dev, float *y_dev, uint32_t ldy);
 
 /* ---- row steps between the projections and the attention path --------------
  * For callers that keep a layer's activations on the device.  All arguments
@@ -268,6 +273,13 @@ int wr_hip_proj_rows_swiglu_dev(const wr_hip_weight *w, uint32_t rows,
 int wr_hip_rows_rmsnorm_dev(const float *x_dev, uint32_t ldx, const float *w_dev,
                             uint32_t wn, float *out_dev, uint32_t ldo,
                             uint32_t rows, uint32_t dim, float eps);
+
+/* rmsnorm_add: acc[r][j] += the same normalised value (Gemma's sandwich norms:
+ * a sublayer's output is normalised before it joins the residual,
+ * src/core/session.c:355-359, 391-395). */
+int wr_hip_rows_rmsnorm_add_dev(const float *x_dev, uint32_t ldx, const float *w_dev,
+                                uint32_t wn, float *acc_dev, uint32_t lda,
+                                uint32_t rows, uint32_t dim, float eps);
 
 /* qkv_prep: rows of a stacked projection [nq heads | nkv K heads | nkv V heads]
  * (row stride ld) are split into Q [rows, nq, hd], K and V [rows, nkv, hd].
@@ -295,11 +307,16 @@ int wr_hip_rows_qkv_prep_dev(const float *qkv_dev, uint32_t ld, uint32_t rows,
  * WR_HIP_ERR_CTX_FULL before anything is written.  head_dim <= 512
  * (WR_HIP_ERR_LIMIT beyond; use qkv_prep + append).  Q and the cache bits
  * equal those of qkv_prep followed by the append, bit for bit. */
+#define WR_HIP_QKV_V_NORM 1u   /* V heads get a weightless RMSNorm before they are stored (Gemma,
+                                  src/core/session.c:318-323) */
+#define WR_HIP_QKV_Q_ONLY 2u   /* the rows hold Q heads only and nothing is appended: a layer that
+                                  reads another layer's cache (session.c:108-134); `layer` names
+                                  the cache layer whose head_dim the Q heads have */
 int wr_hip_rows_qkv_append_dev(const float *qkv_dev, uint32_t ld, uint32_t rows, uint32_t nq,
                                const float *q_norm_dev, const float *k_norm_dev, float eps,
                                const float *cos_sin_dev, uint32_t n_rot, uint32_t n_kv,
                                wr_hip_kv *const *kv, uint32_t layer, const uint32_t *pos,
-                               float *q_out_dev);
+                               float *q_out_dev, uint32_t flags);
 
 /* swiglu: act[r][j] = silu(gu[r][j]) * gu[r][ffn + j] for rows of a stacked
  * gate/up projection (wri_op_fused_silu_mul, src/core/kernels.c:1243-1258 with

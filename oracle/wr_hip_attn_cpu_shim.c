@@ -294,10 +294,22 @@ void wr_hip_attn_host_free(void *p) { free(p); }
 int wr_hip_rows_qkv_append_dev(const float *qkv, uint32_t ld, uint32_t rows, uint32_t nq,
                                const float *qn, const float *kn, float eps, const float *cs,
                                uint32_t n_rot, uint32_t n_kv, wr_hip_kv *const *kv, uint32_t layer,
-                               const uint32_t *pos, float *q)
+                               const uint32_t *pos, float *q, uint32_t flags)
 {
     (void)qkv; (void)ld; (void)rows; (void)nq; (void)qn; (void)kn; (void)eps; (void)cs; (void)n_rot;
-    (void)n_kv; (void)kv; (void)layer; (void)pos; (void)q;
+    (void)n_kv; (void)kv; (void)layer; (void)pos; (void)q; (void)flags;
+    return WR_HIP_ERR_STATE;
+}
+int wr_hip_rows_rmsnorm_add_dev(const float *x, uint32_t ldx, const float *w, uint32_t wn, float *acc,
+                                uint32_t lda, uint32_t rows, uint32_t dim, float eps)
+{
+    (void)x; (void)ldx; (void)w; (void)wn; (void)acc; (void)lda; (void)rows; (void)dim; (void)eps;
+    return WR_HIP_ERR_STATE;
+}
+int wr_hip_proj_rows_geglu_dev(const wr_hip_weight *w, uint32_t rows, const float *gu, uint32_t ld,
+                               const float *add, float *y, uint32_t ldy)
+{
+    (void)w; (void)rows; (void)gu; (void)ld; (void)add; (void)y; (void)ldy;
     return WR_HIP_ERR_STATE;
 }
 int wr_hip_rows_swiglu_dev(const float *gu, uint32_t ld, float *act, uint32_t ldo, uint32_t rows,

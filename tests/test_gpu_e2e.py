@@ -88,8 +88,8 @@ def test_small16_model_stream_on_device(eng, tmp_path, walk):
     m.close()
 
 
-def test_gemma_family_stream_on_device(eng, tmp_path):
-    # The reference's Gemma block on the host walk with the device's attention:
+def test_gemma_family_stream_on_device(eng, tmp_path, walk):
+    # The reference's Gemma block, on the device walk and on the host walk with the device's attention:
     # head_dim 64 on global layers and 32 on sliding-window layers (16-key
     # window, skipped tiles), scale_override 1.0, two layers that read an earlier
     # layer's cache, partial rotary, logit soft cap.  Probe tolerance: scale-1.0
@@ -104,7 +104,7 @@ def test_gemma_family_stream_on_device(eng, tmp_path):
         pytest.skip("random-init model file differs from the one the golden stream was made with")
     m = eng.load(p)
     got, forced, probe = _run_stream(m, g, len(g["prompt"]))
-    print("gemma: forced", forced, "probe err", probe, flush=True)
+    print("gemma", walk, ": forced", forced, "probe err", probe, flush=True)
     assert forced == len(g["tokens"]) and np.array_equal(got, g["tokens"]) and probe < 5e-3
     m.close()
 
@@ -134,12 +134,16 @@ def test_qwen3_0_6b_greedy_stream_matches_reference(eng, tmp_path, walk):
     os.remove(p)
 
 
-def test_batched_step_equals_serial_on_device(eng, tmp_path, walk):
-    p = str(tmp_path / "small16.gguf")
-    gw.write_model(p, SMALL16)
+@pytest.mark.parametrize("family", ["qwen3", "gemma"])
+def test_batched_step_equals_serial_on_device(eng, tmp_path, walk, family):
+    p = str(tmp_path / "model.gguf")
+    if family == "gemma":       # sliding-window layers, shared caches, per-layer head_dim in the batched walk
+        gw.write_model(p, GEMMA_TOY, seed=GEMMA_SEED, std=GEMMA_STD)
+    else:
+        gw.write_model(p, SMALL16)
     m = eng.load(p)
     n = 12                                  # more than eight rows: two row groups in the projections
-    prompts = [workload(SMALL16, 4 + 7 * i) for i in range(n)]
+    prompts = [workload(gw.ModelShape(vocab=m.vocab), 4 + 7 * i) for i in range(n)]
     batch = [m.session(128) for _ in range(n)]
     serial = [m.session(128) for _ in range(n)]
     for i in range(n):

@@ -283,3 +283,28 @@ def test_one_row_equals_its_row_of_two(n_in, n_out):
     for d in (xd, nwd, gud, addd, y1, y2):
         d.free()
     w.close()
+
+
+@pytest.mark.parametrize("rows", [1, 11, 70])
+def test_geglu_source(rows):
+    # gelu_tanh(gate) * up feeding a projection (Gemma's FFN), against the closed
+    # form in float64; one row, a few rows and a prefill-sized count take three
+    # different fragment paths
+    lib = hipattn.lib()
+    n_in, n_out = 256, 48
+    gu = synth.normal(95 + rows, (rows, 2 * n_in), std=2.0)
+    w16 = _w16(96, n_out, n_in, 0.1)
+    w = hipattn.Weight([w16])
+    D = hipattn.DeviceBuffer
+    gud, y = D.from_host(gu), D(rows * n_out * 4)
+    assert lib.wr_hip_proj_rows_geglu_dev(w.h, rows, gud.p, 2 * n_in, None, y.p, n_out) == hipattn.OK
+    hipattn.sync()
+    g, u = gu[:, :n_in].astype(np.float64), gu[:, n_in:].astype(np.float64)
+    act = 0.5 * g * (1.0 + np.tanh(0.7978845608 * (g + 0.044715 * g ** 3))) * u
+    want = act @ _widen(w16).T
+    got = y.to_host((rows, n_out)).astype(np.float64)
+    mag = np.abs(act) @ np.abs(_widen(w16)).T
+    assert np.all(np.abs(got - want) <= 2e-6 * np.sqrt(n_in) * mag + 1e-30)
+    gud.free()
+    y.free()
+    w.close()

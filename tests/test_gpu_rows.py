@@ -174,7 +174,7 @@ def test_qkv_append_equals_prep_then_append(rows, nq, nkv, hd, norm, pos, batch)
     kvp = (C.c_void_p * n_kv)(*[c.h for c in fused])
     pp = (C.c_uint32 * n_kv)(*positions)
     assert lib.wr_hip_rows_qkv_append_dev(xd.p, ld, rows, nq, qnp, knp, eps, td.p, n_rot, n_kv, kvp, 0, pp,
-                                          qo2.p) == hipattn.OK
+                                          qo2.p, 0) == hipattn.OK
     hipattn.sync()
     assert qo.to_host((rows, qd)).tobytes() == qo2.to_host((rows, qd)).tobytes()
     for a, b, p in zip(two_step, fused, positions if batch else [pos]):
@@ -186,11 +186,87 @@ def test_qkv_append_equals_prep_then_append(rows, nq, nkv, hd, norm, pos, batch)
     # contracts: all or nothing past the end of a cache; one cache or one per row; distinct caches
     pp_bad = (C.c_uint32 * n_kv)(*([ctx - (0 if batch else rows - 1)] * n_kv))
     assert lib.wr_hip_rows_qkv_append_dev(xd.p, ld, rows, nq, qnp, knp, eps, td.p, n_rot, n_kv, kvp, 0, pp_bad,
-                                          qo2.p) == hipattn.ERR_CTX_FULL
+                                          qo2.p, 0) == hipattn.ERR_CTX_FULL
     if rows > 2:
         assert lib.wr_hip_rows_qkv_append_dev(xd.p, ld, rows, nq, qnp, knp, eps, td.p, n_rot, 2, kvp, 0, pp,
-                                              qo2.p) == hipattn.ERR_INVAL
+                                              qo2.p, 0) == hipattn.ERR_INVAL
     for c in two_step + fused:
         c.close()
     for b in bufs:
+        b.free()
+
+
+def test_rmsnorm_add_accumulates_into_the_residual():
+    rows, dim = 5, 1024
+    x = synth.normal(81, (rows, dim), std=3.0)
+    w = synth.normal(82, (dim,)) * np.float32(0.1) + np.float32(1.0)
+    acc = synth.normal(83, (rows, dim + 8))
+    xd, wd, ad = _dev(x), _dev(w), _dev(acc)
+    assert hipattn.lib().wr_hip_rows_rmsnorm_add_dev(xd.p, dim, wd.p, dim, ad.p, dim + 8, rows, dim, 1e-6) == hipattn.OK
+    hipattn.sync()
+    got = ad.to_host((rows, dim + 8))
+    want = acc[:, :dim].astype(np.float64) + oracle.rmsnorm(x, w, 1e-6).astype(np.float64)
+    _close(got[:, :dim], want)
+    assert np.array_equal(got[:, dim:], acc[:, dim:])     # padding columns untouched
+    for b in (xd, wd, ad):
+        b.free()
+
+
+def _f16_ulps(a16, b16):
+    # distance in binary16 steps between two arrays of bit patterns of the same sign
+    return np.abs(a16.astype(np.int32) - b16.astype(np.int32))
+
+
+def test_qkv_append_gemma_flags():
+    # V_NORM: the V heads get a weightless RMSNorm before they are truncated into
+    # the cache; Q_ONLY: rows of Q heads only, nothing is appended (a layer that
+    # reads another layer's cache)
+    lib = hipattn.lib()
+    rows, nq, nkv, hd, pos = 9, 4, 2, 64, 30
+    width = (nq + 2 * nkv) * hd
+    qkv = synth.normal(91, (rows, width), std=1.5)
+    qn = synth.normal(1, (hd,)) * np.float32(0.1) + np.float32(1.0)
+    kn = synth.normal(2, (hd,)) * np.float32(0.1) + np.float32(1.0)
+    tab = oracle.rope_table(rows, hd, pos, 1e6, 0)
+    n_rot = tab.shape[1]
+    qd, kd = nq * hd, nkv * hd
+    eps = 1e-6
+    kv = hipattn.KVCache(1, hd, nkv, 256)
+    bufs = [_dev(qkv), _dev(qn), _dev(kn), _dev(tab), _dev(np.zeros((rows, qd))), _dev(np.zeros((rows, qd))),
+            _dev(np.zeros((rows, kd))), _dev(np.zeros((rows, kd)))]
+    xd, qnd, knd, td, q1, q2, ko, vo = bufs
+    kvp = (C.c_void_p * 1)(kv.h)
+    pp = (C.c_uint32 * 1)(pos)
+    assert lib.wr_hip_rows_qkv_append_dev(xd.p, width, rows, nq, qnd.p, knd.p, eps, td.p, n_rot, 1, kvp, 0, pp,
+                                          q1.p, hipattn.QKV_V_NORM) == hipattn.OK
+    hipattn.sync()
+    k16, v16 = kv.read_f16(0, pos, rows)
+    v_in = np.ascontiguousarray(qkv[:, qd + kd:]).reshape(rows, nkv, hd)
+    want_v = synth.f32_to_f16_trunc(oracle.rmsnorm(v_in, None, eps))
+    assert _f16_ulps(v16, want_v).max() <= 1              # a last-bit difference in F32 can move the truncation
+    assert (_f16_ulps(v16, want_v) > 0).mean() < 0.01
+    # K is what the unflagged call stores
+    kv2 = hipattn.KVCache(1, hd, nkv, 256)
+    kvp2 = (C.c_void_p * 1)(kv2.h)
+    assert lib.wr_hip_rows_qkv_append_dev(xd.p, width, rows, nq, qnd.p, knd.p, eps, td.p, n_rot, 1, kvp2, 0, pp,
+                                          q2.p, 0) == hipattn.OK
+    hipattn.sync()
+    k16b, _ = kv2.read_f16(0, pos, rows)
+    assert k16.tobytes() == k16b.tobytes()
+    assert q1.to_host((rows, qd)).tobytes() == q2.to_host((rows, qd)).tobytes()
+    # Q_ONLY on rows that hold the Q heads alone: the same Q, and the cache stays as it is
+    q_rows = np.ascontiguousarray(qkv[:, :qd])
+    qx = _dev(q_rows)
+    before = kv2.read_f16(0, 0, 256)
+    assert lib.wr_hip_rows_qkv_append_dev(qx.p, qd, rows, nq, qnd.p, None, eps, td.p, n_rot, 1, kvp2, 0, pp,
+                                          q1.p, hipattn.QKV_Q_ONLY) == hipattn.OK
+    hipattn.sync()
+    assert q1.to_host((rows, qd)).tobytes() == q2.to_host((rows, qd)).tobytes()
+    after = kv2.read_f16(0, 0, 256)
+    assert before[0].tobytes() == after[0].tobytes() and before[1].tobytes() == after[1].tobytes()
+    assert lib.wr_hip_rows_qkv_append_dev(qx.p, qd, rows, nq, qnd.p, None, eps, td.p, n_rot, 1, kvp2, 0, pp,
+                                          q1.p, 8) == hipattn.ERR_INVAL
+    for c in (kv, kv2):
+        c.close()
+    for b in bufs + [qx]:
         b.free()

@@ -65,6 +65,7 @@ __global__ __launch_bounds__(256) void proj_pack_weights_kernel(const uint16_t* 
 //                    src/core/kernels.c:1276-1316, same expressions and the
 //                    same reduction tree as rmsnorm_rows_kernel)
 //   kProjSrcSwiglu   v = silu(g) * u, g = x[k], u = x[K + k]   (kernels.c:963-967)
+//   kProjSrcGeglu    v = gelu_tanh(g) * u, same operands      (kernels.c:969-976)
 // Then scales[row] = 2^e with 2^e <= max|v| < 2^(e+1) (1 for a row of zeros),
 // v is divided by it (exact), so its largest magnitude lies in [1, 2), and
 // split into
@@ -75,7 +76,7 @@ __global__ __launch_bounds__(256) void proj_pack_weights_kernel(const uint16_t* 
 // terms in the normal binary16 range, so the result does not depend on how the
 // matrix cores treat subnormal inputs.
 constexpr float kProjLoScale = 2048.0f;
-constexpr int kProjSrcPlain = 0, kProjSrcRmsNorm = 1, kProjSrcSwiglu = 2;
+constexpr int kProjSrcPlain = 0, kProjSrcRmsNorm = 1, kProjSrcSwiglu = 2, kProjSrcGeglu = 3;
 
 struct ProjPrepArgs {
     const float* x;          // [R][ldx]
@@ -126,16 +127,29 @@ __device__ __forceinline__ float row_sumsq_256(const float* __restrict__ xr, uin
     return block_sum_256(ss, s4);
 }
 
+// the two gated activations: SiLU(g) * u and the tanh form of GELU(g) * u
+template <int SRC>
+__device__ __forceinline__ float proj_gated(float g, float u)
+{
+    if constexpr (SRC == kProjSrcGeglu) {
+        const float x3 = g * g * g;
+        const float z = 0.7978845608f * (g + 0.044715f * x3);
+        const float th = 2.0f / (1.0f + expf(-2.0f * z)) - 1.0f;
+        return 0.5f * g * (1.0f + th) * u;
+    } else {
+        const float sig = 1.0f / (1.0f + expf(-g));
+        return (g * sig) * u;
+    }
+}
+
 template <int SRC>
 __device__ __forceinline__ float proj_src_value(const ProjPrepArgs& a, const float* xr, uint32_t k,
                                                 float inv_rms)
 {
     if constexpr (SRC == kProjSrcRmsNorm) {
         return xr[k] * inv_rms * a.norm_w[k];
-    } else if constexpr (SRC == kProjSrcSwiglu) {
-        const float g = xr[k], u = xr[a.K + k];
-        const float sig = 1.0f / (1.0f + expf(-g));
-        return (g * sig) * u;
+    } else if constexpr (SRC == kProjSrcSwiglu || SRC == kProjSrcGeglu) {
+        return proj_gated<SRC>(xr[k], xr[a.K + k]);
     } else {
         return xr[k];
     }
@@ -206,16 +220,14 @@ __global__ __launch_bounds__(256) void proj_prep_kernel(const ProjPrepArgs a)
                 for (int j = 0; j < 8; j++)
                     v[i][j] = (q < nchunks) ? v[i][j] * inv_rms * a.norm_w[q * 8 + j] : 0.f;
             }
-        } else if constexpr (SRC == kProjSrcSwiglu) {
+        } else if constexpr (SRC == kProjSrcSwiglu || SRC == kProjSrcGeglu) {
 #pragma unroll
             for (int i = 0; i < CH; i++) {
                 const uint32_t q = t + 256 * i;
 #pragma unroll
                 for (int j = 0; j < 8; j++) {
-                    const float g = v[i][j];
                     const float u = (q < nchunks) ? xr[a.K + q * 8 + j] : 0.f;
-                    const float sig = 1.0f / (1.0f + expf(-g));
-                    v[i][j] = (g * sig) * u;
+                    v[i][j] = proj_gated<SRC>(v[i][j], u);
                 }
             }
         }
@@ -311,15 +323,11 @@ __device__ __forceinline__ void proj_src_chunk(const ProjPrepArgs& a, const floa
             v[j] = v[j] * inv_rms * wl[j];
             v[4 + j] = v[4 + j] * inv_rms * wh[j];
         }
-    } else if constexpr (SRC == kProjSrcSwiglu) {
+    } else if constexpr (SRC == kProjSrcSwiglu || SRC == kProjSrcGeglu) {
         const f32x4 ul = *reinterpret_cast<const f32x4*>(xr + a.K + q * 8),
                     uh = *reinterpret_cast<const f32x4*>(xr + a.K + q * 8 + 4);
 #pragma unroll
-        for (int j = 0; j < 8; j++) {
-            const float g = v[j], u = j < 4 ? ul[j] : uh[j - 4];
-            const float sig = 1.0f / (1.0f + expf(-g));
-            v[j] = (g * sig) * u;
-        }
+        for (int j = 0; j < 8; j++) v[j] = proj_gated<SRC>(v[j], j < 4 ? ul[j] : uh[j - 4]);
     }
 }
 

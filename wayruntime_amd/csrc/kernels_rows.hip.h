@@ -24,12 +24,13 @@ __device__ __forceinline__ float wave_sum_f32(float v)
     return v;
 }
 
-// out[r][j] = x[r][j] * (1 / sqrt(mean_j x^2 + eps)) * w[j % wn]   (wn == 0: no weight)
+// out[r][j] = x[r][j] * (1 / sqrt(mean_j x^2 + eps)) * w[j % wn]   (wn == 0: no weight),
+// or out[r][j] += that when `accumulate` (a normalised sublayer output joining the residual)
 // One workgroup of 256 threads per row.
 __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const float* __restrict__ x, uint32_t ldx,
                                                            const float* __restrict__ w, uint32_t wn,
                                                            float* __restrict__ out, uint32_t ldo,
-                                                           uint32_t dim, float eps)
+                                                           uint32_t dim, float eps, int accumulate)
 {
     __shared__ float s_sum[4];
     const uint32_t r = blockIdx.x;
@@ -39,7 +40,8 @@ __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const float* __restri
     float* orow = out + (size_t)r * ldo;
     for (uint32_t j = threadIdx.x; j < dim; j += 256) {
         const float ww = wn ? w[j % wn] : 1.0f;
-        orow[j] = xr[j] * inv_rms * ww;
+        const float v = xr[j] * inv_rms * ww;
+        orow[j] = accumulate ? orow[j] + v : v;
     }
 }
 
@@ -128,6 +130,7 @@ struct QkvAppendArgs {
     uint32_t ctx_pad[16];
     uint32_t ld, nq, nkv, hd, n_rot, rows;
     uint32_t per_session;    // 1: row i belongs to session i; 0: all rows to session 0 from pos[0]
+    uint32_t v_norm;         // 1: V heads get a weightless RMSNorm before they are stored
     float eps;
 };
 
@@ -159,7 +162,18 @@ __global__ __launch_bounds__(256) void qkv_append_kernel(const QkvAppendArgs a)
         uint16_t (*tile)[kVBlock + 2] = reinterpret_cast<uint16_t (*)[kVBlock + 2]>(qkv_smem);
         for (uint32_t i = wave; i < np; i += 4) {
             const float* src = a.qkv + (size_t)(row0 + i) * a.ld + (size_t)h * hd;
-            for (uint32_t j = lane; j < hd; j += 64) tile[j][i] = f32_to_f16_trunc(src[j]);
+            float inv_rms = 1.0f;
+            if (a.v_norm) {                               // wave-uniform
+                float ss = 0.f;
+                for (uint32_t j = lane; j < hd; j += 64) {
+                    const float v = src[j];
+                    ss += v * v;
+                }
+                ss = wave_sum_f32(ss);
+                inv_rms = 1.0f / sqrtf(ss / (float)hd + a.eps);
+            }
+            for (uint32_t j = lane; j < hd; j += 64)
+                tile[j][i] = f32_to_f16_trunc(a.v_norm ? src[j] * inv_rms : src[j]);
         }
         __syncthreads();
         uint16_t* vt = a.vt[sess];

@@ -559,6 +559,8 @@ int proj_chunk_locked(const wr_hip_weight* w, uint32_t rows, const float* x_dev,
         WR_LAUNCH_PREP(kProjSrcRmsNorm);
     else if (src.kind == kProjSrcSwiglu)
         WR_LAUNCH_PREP(kProjSrcSwiglu);
+    else if (src.kind == kProjSrcGeglu)
+        WR_LAUNCH_PREP(kProjSrcGeglu);
     else
         WR_LAUNCH_PREP(kProjSrcPlain);
 #undef WR_LAUNCH_PREP
@@ -595,6 +597,8 @@ int proj_chunk_locked(const wr_hip_weight* w, uint32_t rows, const float* x_dev,
             launch_main(proj_row1_kernel<kProjSrcRmsNorm>, grid, block, a, pa, lds);
         else if (src.kind == kProjSrcSwiglu)
             launch_main(proj_row1_kernel<kProjSrcSwiglu>, grid, block, a, pa, lds);
+        else if (src.kind == kProjSrcGeglu)
+            launch_main(proj_row1_kernel<kProjSrcGeglu>, grid, block, a, pa, lds);
         else
             launch_main(proj_row1_kernel<kProjSrcPlain>, grid, block, a, pa, lds);
     } else if (gemm)
@@ -1226,6 +1230,14 @@ int wr_hip_proj_rows_swiglu_dev(const wr_hip_weight* w, uint32_t rows, const flo
     return proj_dev_common(w, rows, gate_up_dev, ld, w ? 2 * w->n_in : 0, src, add_dev, y_dev, ldy);
 }
 
+int wr_hip_proj_rows_geglu_dev(const wr_hip_weight* w, uint32_t rows, const float* gate_up_dev,
+                               uint32_t ld, const float* add_dev, float* y_dev, uint32_t ldy)
+{
+    ProjSource src;
+    src.kind = kProjSrcGeglu;
+    return proj_dev_common(w, rows, gate_up_dev, ld, w ? 2 * w->n_in : 0, src, add_dev, y_dev, ldy);
+}
+
 int wr_hip_proj_rows(const wr_hip_weight* w, uint32_t rows, const float* x, float* y)
 {
     if (w && (w->n_out % 4 != 0)) return WR_HIP_ERR_INVAL;
@@ -1255,8 +1267,22 @@ int wr_hip_rows_rmsnorm_dev(const float* x_dev, uint32_t ldx, const float* w_dev
     if (rows == 0) return WR_HIP_OK;
     Locked lk;
     hipLaunchKernelGGL(rmsnorm_rows_kernel, dim3(rows), dim3(256), 0, g.stream, x_dev, ldx, w_dev, wn,
-                       out_dev, ldo, dim, eps);
+                       out_dev, ldo, dim, eps, 0);
     HIP_TRY(hipGetLastError(), "rmsnorm launch", 0);
+    return WR_HIP_OK;
+}
+
+int wr_hip_rows_rmsnorm_add_dev(const float* x_dev, uint32_t ldx, const float* w_dev, uint32_t wn,
+                                float* acc_dev, uint32_t lda, uint32_t rows, uint32_t dim, float eps)
+{
+    if (!g.inited) return WR_HIP_ERR_STATE;
+    if (!x_dev || !acc_dev || dim == 0 || ldx < dim || lda < dim) return WR_HIP_ERR_INVAL;
+    if (wn > 0 && !w_dev) return WR_HIP_ERR_INVAL;
+    if (rows == 0) return WR_HIP_OK;
+    Locked lk;
+    hipLaunchKernelGGL(rmsnorm_rows_kernel, dim3(rows), dim3(256), 0, g.stream, x_dev, ldx, w_dev, wn,
+                       acc_dev, lda, dim, eps, 1);
+    HIP_TRY(hipGetLastError(), "rmsnorm + add launch", 0);
     return WR_HIP_OK;
 }
 
@@ -1296,10 +1322,12 @@ int wr_hip_rows_qkv_append_dev(const float* qkv_dev, uint32_t ld, uint32_t rows,
                                const float* q_norm_dev, const float* k_norm_dev, float eps,
                                const float* cos_sin_dev, uint32_t n_rot, uint32_t n_kv,
                                wr_hip_kv* const* kv, uint32_t layer, const uint32_t* pos,
-                               float* q_out_dev)
+                               float* q_out_dev, uint32_t flags)
 {
     if (!g.inited) return WR_HIP_ERR_STATE;
     if (!qkv_dev || !q_out_dev || !kv || !pos || nq == 0) return WR_HIP_ERR_INVAL;
+    if (flags & ~(uint32_t)(WR_HIP_QKV_V_NORM | WR_HIP_QKV_Q_ONLY)) return WR_HIP_ERR_INVAL;
+    const bool q_only = (flags & WR_HIP_QKV_Q_ONLY) != 0;
     if (n_kv == 0 || (n_kv != 1 && n_kv != rows)) return WR_HIP_ERR_INVAL;
     if (n_kv > WR_HIP_BATCH_MAX) return WR_HIP_ERR_LIMIT;
     QkvAppendArgs a;
@@ -1311,7 +1339,7 @@ int wr_hip_rows_qkv_append_dev(const float* qkv_dev, uint32_t ld, uint32_t rows,
         for (uint32_t j = 0; j < i; j++)
             if (kv[i] == kv[j]) return WR_HIP_ERR_INVAL;
         const uint64_t end = (uint64_t)pos[i] + (n_kv == 1 ? rows : 1);
-        if (end > kv[i]->max_ctx) return WR_HIP_ERR_CTX_FULL;         // nothing is written
+        if (!q_only && end > kv[i]->max_ctx) return WR_HIP_ERR_CTX_FULL;   // nothing is written
         a.k[i] = reinterpret_cast<uint16_t*>(kv[i]->slab + kv[i]->k_off[layer]);
         a.vt[i] = reinterpret_cast<uint16_t*>(kv[i]->slab + kv[i]->vt_off[layer]);
         a.pos[i] = pos[i];
@@ -1320,10 +1348,11 @@ int wr_hip_rows_qkv_append_dev(const float* qkv_dev, uint32_t ld, uint32_t rows,
     const uint32_t nkv = kv[0]->nkv, hd = kv[0]->hd[layer];
     if (hd < 2 || (hd & 1)) return WR_HIP_ERR_INVAL;
     if (hd > 512) return WR_HIP_ERR_LIMIT;                // the V block gathered in LDS: hd * 68 bytes
-    if ((uint64_t)ld < (uint64_t)(nq + 2 * nkv) * hd) return WR_HIP_ERR_INVAL;
+    if ((uint64_t)ld < (uint64_t)(nq + (q_only ? 0 : 2 * nkv)) * hd) return WR_HIP_ERR_INVAL;
     if (n_rot > hd / 2 || (n_rot > 0 && !cos_sin_dev)) return WR_HIP_ERR_INVAL;
-    if ((q_norm_dev == nullptr) != (k_norm_dev == nullptr)) return WR_HIP_ERR_INVAL;
+    if (!q_only && (q_norm_dev == nullptr) != (k_norm_dev == nullptr)) return WR_HIP_ERR_INVAL;
     if (rows == 0) return WR_HIP_OK;
+    a.v_norm = (flags & WR_HIP_QKV_V_NORM) ? 1 : 0;
     a.qkv = qkv_dev;
     a.q_norm = q_norm_dev;
     a.k_norm = k_norm_dev;
@@ -1340,7 +1369,7 @@ int wr_hip_rows_qkv_append_dev(const float* qkv_dev, uint32_t ld, uint32_t rows,
     const uint32_t gx = a.per_session ? rows : (pos[0] + rows - 1) / kVBlock - pos[0] / kVBlock + 1;
     const size_t lds = std::max((size_t)4 * hd * sizeof(float), (size_t)hd * (kVBlock + 2) * sizeof(uint16_t));
     Locked lk;
-    hipLaunchKernelGGL(qkv_append_kernel, dim3(gx, nq + 2 * nkv), dim3(256), lds, g.stream, a);
+    hipLaunchKernelGGL(qkv_append_kernel, dim3(gx, nq + (q_only ? 0 : 2 * nkv)), dim3(256), lds, g.stream, a);
     HIP_TRY(hipGetLastError(), "qkv append launch", layer);
     return WR_HIP_OK;
 }

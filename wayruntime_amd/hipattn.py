@@ -16,6 +16,7 @@ HIP_SO = os.environ.get("WR_HIP_ATTN_LIB") or os.path.join(PKG, "libwr_hip_attn.
 OK = 0
 ERR_UNSUPPORTED, ERR_INVAL, ERR_NOMEM, ERR_CTX_FULL = -3, -4, -5, -6
 ERR_STATE, ERR_LIMIT, ERR_INTERNAL = -7, -8, -10
+QKV_V_NORM, QKV_Q_ONLY = 1, 2          # flags of wr_hip_rows_qkv_append_dev
 ATTN_MAX_SEQ = 131072
 BATCH_MAX = 16
 
@@ -80,7 +81,9 @@ def load() -> C.CDLL:
         "wr_hip_rows_qkv_prep_dev": (C.c_int, [_vp, _u32, _u32, _u32, _u32, _u32, _vp, _vp, C.c_float,
                                                _vp, _u32, _vp, _vp, _vp]),
         "wr_hip_rows_qkv_append_dev": (C.c_int, [_vp, _u32, _u32, _u32, _vp, _vp, C.c_float, _vp, _u32, _u32,
-                                                 C.POINTER(_vp), _u32, C.POINTER(_u32), _vp]),
+                                                 C.POINTER(_vp), _u32, C.POINTER(_u32), _vp, _u32]),
+        "wr_hip_rows_rmsnorm_add_dev": (C.c_int, [_vp, _u32, _vp, _u32, _vp, _u32, _u32, _u32, C.c_float]),
+        "wr_hip_proj_rows_geglu_dev": (C.c_int, [_vp, _u32, _vp, _u32, _vp, _vp, _u32]),
         "wr_hip_rows_swiglu_dev": (C.c_int, [_vp, _u32, _vp, _u32, _u32, _u32]),
         "wr_hip_attn_host_alloc": (_vp, [C.c_size_t]),
         "wr_hip_attn_host_free": (None, [_vp]),

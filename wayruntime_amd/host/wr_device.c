@@ -7,7 +7,10 @@
  * host walk.  Per call the host embeds the rows and works out the rotary
  * angles (the reference's polynomial sin / cos and range reduction stay on the
  * host), sends both up once, runs the layers without coming back, and brings
- * down the logits (wr_step, wr_batch_step) or nothing (wr_prefill).
+ * down the logits (wr_step, wr_batch_step) or nothing (wr_prefill).  The Gemma
+ * family's block (session.c:251-437) takes the same walk with its own steps:
+ * per-layer head_dim, two rotary tables, layers that read another layer's
+ * cache, the weightless V norm, sandwich norms, GeGLU, attention scale 1.
  *
  * Sums run in a different order than on the host (matrix-core tiles, tree
  * reductions), so activations agree with the host walk to F32 rounding, not
@@ -21,8 +24,9 @@
 #include <string.h>
 
 typedef struct dev_layer {
-    wr_hip_weight *wqkv, *wo, *wgu, *wdown;
+    wr_hip_weight *wqkv, *wo, *wgu, *wdown;                   /* wqkv holds Q only on a layer without its own cache */
     const float *attn_norm, *ffn_norm, *q_norm, *k_norm;      /* device */
+    const float *post_attn_norm, *post_ffw_norm;              /* Gemma */
 } dev_layer;
 
 struct wrh_dev_model {
@@ -68,15 +72,17 @@ wr_status wrh_device_model_init(wr_model *m)
     const char *env = getenv("WAYRT_HOST_LAYERS");
     if (env && env[0] == '1') return WR_OK;
     if (!(wr_hip_attn_caps() & WR_HIP_CAP_PROJ)) return WR_OK;
-    if (m->is_gemma) return WR_OK;               /* the Gemma block runs on the host walk */
-    const uint32_t qd = m->n_q * m->head_dim, kd = m->n_kv * m->head_dim;
-    int ok = proj_dims_ok(&m->lm_head) && m->vocab % 16 == 0 && (qd + 2 * kd) % 16 == 0 &&
-             m->hidden % 16 == 0 && (2 * m->ffn) % 16 == 0 &&
-             m->head_dim <= 512;                  /* the fused Q/K/V split + append */
-    for (uint32_t l = 0; l < m->n_layers && ok; l++)
-        ok = proj_dims_ok(&m->wq[l]) && proj_dims_ok(&m->wk[l]) && proj_dims_ok(&m->wv[l]) &&
+    int ok = proj_dims_ok(&m->lm_head) && m->vocab % 16 == 0 && m->hidden % 16 == 0 &&
+             (2 * m->ffn) % 16 == 0;
+    for (uint32_t l = 0; l < m->n_layers && ok; l++) {
+        const uint32_t hd = m->hd_layer[l], qd = m->n_q * hd, kd = m->n_kv * hd;
+        const int shared = m->kv_src[l] != l;
+        ok = hd <= 512 &&                          /* the fused Q/K/V split + append */
+             (qd + (shared ? 0 : 2 * kd)) % 16 == 0 && proj_dims_ok(&m->wq[l]) &&
+             (shared || (proj_dims_ok(&m->wk[l]) && proj_dims_ok(&m->wv[l]))) &&
              proj_dims_ok(&m->wo[l]) && proj_dims_ok(&m->w_gate[l]) && proj_dims_ok(&m->w_up[l]) &&
              proj_dims_ok(&m->w_down[l]);
+    }
     if (!ok) {
         wrh_logf(m->engine, 2, "device layers: model keeps the host walk (needs F16 matrices, "
                               "inputs a multiple of 32, outputs of 16)");
@@ -87,38 +93,42 @@ wr_status wrh_device_model_init(wr_model *m)
     if (!d) return WR_ERR_NOMEM;
     m->dev = d;
     int rc = WR_HIP_OK;
-    /* norm vectors: [final | per layer: attn, ffn, (q, k)] */
-    const size_t per_layer = 2 * (size_t)m->hidden + (m->has_qk_norm ? 2 * (size_t)m->head_dim : 0);
-    const size_t n_vec = m->hidden + per_layer * m->n_layers;
+    /* norm vectors: [final | per layer: attn, ffn, (q, k), (post-attn, post-ffn)] */
+    size_t n_vec = m->hidden;
+    for (uint32_t l = 0; l < m->n_layers; l++)
+        n_vec += m->attn_norm[l].n + m->ffn_norm[l].n + m->q_norm[l].n + m->k_norm[l].n +
+                 m->post_attn_norm[l].n + m->post_ffw_norm[l].n;
     float *host = malloc(n_vec * sizeof(float));
     d->vecs = wr_hip_attn_dev_alloc(n_vec * sizeof(float));
     if (!host || !d->vecs) rc = WR_HIP_ERR_NOMEM;
     if (rc == WR_HIP_OK) {
         size_t at = 0;
-        memcpy(host + at, m->final_norm.data, m->hidden * sizeof(float));
-        d->final_norm = d->vecs + at;
-        at += m->hidden;
+#define PUT(vec, dst)                                                   \
+        do {                                                            \
+            if ((vec).n) {                                              \
+                memcpy(host + at, (vec).data, (vec).n * sizeof(float)); \
+                (dst) = d->vecs + at;                                   \
+                at += (vec).n;                                          \
+            }                                                           \
+        } while (0)
+        PUT(m->final_norm, d->final_norm);
         for (uint32_t l = 0; l < m->n_layers; l++) {
-            memcpy(host + at, m->attn_norm[l].data, m->hidden * sizeof(float));
-            d->L[l].attn_norm = d->vecs + at;
-            at += m->hidden;
-            memcpy(host + at, m->ffn_norm[l].data, m->hidden * sizeof(float));
-            d->L[l].ffn_norm = d->vecs + at;
-            at += m->hidden;
-            if (m->has_qk_norm) {
-                memcpy(host + at, m->q_norm[l].data, m->head_dim * sizeof(float));
-                d->L[l].q_norm = d->vecs + at;
-                at += m->head_dim;
-                memcpy(host + at, m->k_norm[l].data, m->head_dim * sizeof(float));
-                d->L[l].k_norm = d->vecs + at;
-                at += m->head_dim;
-            }
+            PUT(m->attn_norm[l], d->L[l].attn_norm);
+            PUT(m->ffn_norm[l], d->L[l].ffn_norm);
+            PUT(m->q_norm[l], d->L[l].q_norm);
+            PUT(m->k_norm[l], d->L[l].k_norm);
+            PUT(m->post_attn_norm[l], d->L[l].post_attn_norm);
+            PUT(m->post_ffw_norm[l], d->L[l].post_ffw_norm);
         }
+#undef PUT
         rc = wr_hip_attn_h2d(d->vecs, host, n_vec * sizeof(float));
     }
     free(host);
     for (uint32_t l = 0; l < m->n_layers && rc == WR_HIP_OK; l++) {
-        rc = stack(&d->L[l].wqkv, &m->wq[l], &m->wk[l], &m->wv[l]);
+        if (m->kv_src[l] != l)
+            rc = stack(&d->L[l].wqkv, &m->wq[l], NULL, NULL);
+        else
+            rc = stack(&d->L[l].wqkv, &m->wq[l], &m->wk[l], &m->wv[l]);
         if (rc == WR_HIP_OK) rc = stack(&d->L[l].wo, &m->wo[l], NULL, NULL);
         if (rc == WR_HIP_OK) rc = stack(&d->L[l].wgu, &m->w_gate[l], &m->w_up[l], NULL);
         if (rc == WR_HIP_OK) rc = stack(&d->L[l].wdown, &m->w_down[l], NULL, NULL);
@@ -140,23 +150,28 @@ static size_t r64(size_t n) { return (n + 63) & ~(size_t)63; }       /* floats: 
 int wrh_devspace_init(wrh_devspace *ws, const wr_model *m, uint32_t rows, uint32_t logit_rows)
 {
     memset(ws, 0, sizeof *ws);
-    const size_t hidden = m->hidden, qd = (size_t)m->n_q * m->head_dim, kd = (size_t)m->n_kv * m->head_dim;
+    size_t hd = m->head_dim;
+    for (uint32_t l = 0; l < m->n_layers; l++)
+        if (m->hd_layer[l] > hd) hd = m->hd_layer[l];
+    const size_t hidden = m->hidden, qd = (size_t)m->n_q * hd, kd = (size_t)m->n_kv * hd;
     const size_t ffn = m->ffn, R = rows;
-    const size_t total = r64(R * hidden) + r64(R * (qd + 2 * kd)) + 2 * r64(R * qd) + 2 * r64(R * kd) +
-                         r64(R * 2 * ffn) + r64(R * m->head_dim) + r64((size_t)logit_rows * m->vocab);
+    const size_t total = 2 * r64(R * hidden) + r64(R * (qd + 2 * kd)) + 2 * r64(R * qd) + 2 * r64(R * kd) +
+                         r64(R * 2 * ffn) + 2 * r64(R * hd) + r64((size_t)logit_rows * m->vocab);
     float *b = wr_hip_attn_dev_alloc(total * sizeof(float));
     if (!b) return WR_ERR_NOMEM;
     ws->block = b;
     ws->rows_cap = rows;
     ws->logit_rows = logit_rows;
     ws->resid = b;   b += r64(R * hidden);
+    ws->proj = b;    b += r64(R * hidden);
     ws->qkv = b;     b += r64(R * (qd + 2 * kd));
     ws->q = b;       b += r64(R * qd);
     ws->attn = b;    b += r64(R * qd);
     ws->k = b;       b += r64(R * kd);
     ws->v = b;       b += r64(R * kd);
     ws->gu = b;      b += r64(R * 2 * ffn);
-    ws->rope = b;    b += r64(R * m->head_dim);
+    ws->rope = b;    b += r64(R * hd);
+    ws->rope_swa = b; b += r64(R * hd);
     ws->logits = b;
     return WR_OK;
 }
@@ -269,15 +284,23 @@ static wr_status stage_rows(wr_model *m, wrh_workspace *hs, uint32_t R, wr_sessi
     const uint32_t hidden = m->hidden, hd = m->head_dim;
     const uint32_t n_rot = (m->n_rot_pairs >= 1 && m->n_rot_pairs < hd / 2) ? m->n_rot_pairs : hd / 2;
     const size_t ts = (size_t)2 * n_rot;
+    /* Gemma: scaled embeddings, and a second table for the sliding-window
+     * layers (their own head_dim and base, full rotation; session.c:262-283) */
+    const uint32_t hd_s = m->head_dim_swa ? m->head_dim_swa : hd;
+    const size_t ts_s = hd_s;                             /* hd_s / 2 pairs of two */
+    const int swa = m->is_gemma && m->has_swa;
     const wr_engine *e = m->engine;
     const int threads = (e && e->n_threads > 0) ? e->n_threads : 1;
     int bad = WR_OK;
 #pragma omp parallel for num_threads(threads) schedule(static) if (R >= 32)
     for (uint32_t r = 0; r < R; r++) {
-        const int rc = wrh_embed(&m->embed, tokens[r], hs->residual + (size_t)r * hidden);
+        float *row = hs->residual + (size_t)r * hidden;
+        const int rc = wrh_embed(&m->embed, tokens[r], row);
         if (rc != WR_OK) __atomic_store_n(&bad, rc, __ATOMIC_RELAXED);
+        if (m->is_gemma && m->embed_scale != 0.0f) wrh_scale(row, hidden, m->embed_scale);
         const uint32_t p = batch ? ss[r]->pos : pos0 + r;
         (void)wrh_rope_table(hs->rope + r * ts, hd, p, m->rope_base, m->n_rot_pairs);
+        if (swa) (void)wrh_rope_table(hs->rope_swa + r * ts_s, hd_s, p, m->rope_base_swa, 0);
     }
     return (wr_status)bad;
 }
@@ -308,7 +331,7 @@ wr_status wrh_forward_rows_device(wr_model *m, wrh_workspace *hs, wrh_devspace *
     wr_engine *e = m->engine;
     const struct wrh_dev_model *d = m->dev;
     const uint32_t hidden = m->hidden, hd = m->head_dim, nq = m->n_q, nkv = m->n_kv;
-    const uint32_t qd = nq * hd, kd = nkv * hd, ffn = m->ffn;
+    const uint32_t ffn = m->ffn;
     const uint32_t n_rot = (m->n_rot_pairs >= 1 && m->n_rot_pairs < hd / 2) ? m->n_rot_pairs : hd / 2;
     const size_t ts = (size_t)2 * n_rot;
     uint32_t L = 0;
@@ -322,11 +345,27 @@ wr_status wrh_forward_rows_device(wr_model *m, wrh_workspace *hs, wrh_devspace *
     }
     TRY(wr_hip_attn_h2d(ds->resid, hs->residual, (size_t)R * hidden * sizeof(float)), "rows up");
     TRY(wr_hip_attn_h2d(ds->rope, hs->rope, (size_t)R * ts * sizeof(float)), "angles up");
+    const int gemma = m->is_gemma;
+    const uint32_t hd_s = m->head_dim_swa ? m->head_dim_swa : hd;
+    if (gemma && m->has_swa)
+        TRY(wr_hip_attn_h2d(ds->rope_swa, hs->rope_swa, (size_t)R * hd_s * sizeof(float)), "angles up");
+    const float scale = gemma ? m->attn_scale : 0.0f;
 
     for (L = 0; L < m->n_layers; L++) {
         const dev_layer *dl = &d->L[L];
+        /* per layer (Gemma; constant elsewhere): head_dim, rotary table, window, whose cache */
+        const uint32_t hdl = m->hd_layer[L], qd = nq * hdl, kd = nkv * hdl;
+        const uint32_t ksrc = m->kv_src[L];
+        const int shared = ksrc != L;
+        const int local = gemma && m->swa[L];
+        const uint32_t window = (local && m->swa_mode != WR_SWA_DISABLED) ? m->sliding_window : 0u;
+        const float *tab = local ? ds->rope_swa : ds->rope;
+        const uint32_t nr = local ? hd_s / 2 : n_rot;
+        const uint32_t width = qd + (shared ? 0 : 2 * kd);
+        const uint32_t flags = shared ? WR_HIP_QKV_Q_ONLY : (gemma ? WR_HIP_QKV_V_NORM : 0u);
+
         TRY(wr_hip_proj_rows_norm_dev(dl->wqkv, R, ds->resid, hidden, dl->attn_norm, m->rms_eps, NULL,
-                                      ds->qkv, qd + 2 * kd), "attn norm + qkv projection");
+                                      ds->qkv, width), "attn norm + qkv projection");
         /* Q/K/V split, per-head norms, rotation and the cache append in one launch */
         if (fail_layer == (int)L) return dev_fail(e, "gqa (injected)", L, WR_ERR_INTERNAL);
         if (batch) {
@@ -338,29 +377,45 @@ wr_status wrh_forward_rows_device(wr_model *m, wrh_workspace *hs, wrh_devspace *
                 at[r] = ss[r]->pos;
                 seq_k[r] = ss[r]->pos + 1;
             }
-            TRY(wr_hip_rows_qkv_append_dev(ds->qkv, qd + 2 * kd, R, nq, dl->q_norm, dl->k_norm, m->rms_eps,
-                                           ds->rope, n_rot, R, kvs, L, at, ds->q), "qkv split + kv append");
-            for (uint32_t r = 0; r < R; r++) ss[r]->kv_rows[L] = ss[r]->pos + 1;
-            TRY(wr_hip_attn_decode_batched_dev(R, kvs, L, seq_k, ds->q, ds->attn, nq, 0.0f, 0), "gqa");
+            TRY(wr_hip_rows_qkv_append_dev(ds->qkv, width, R, nq, dl->q_norm, shared ? NULL : dl->k_norm,
+                                           m->rms_eps, tab, nr, R, kvs, ksrc, at, ds->q, flags),
+                "qkv split + kv append");
+            if (!shared)
+                for (uint32_t r = 0; r < R; r++) ss[r]->kv_rows[L] = ss[r]->pos + 1;
+            TRY(wr_hip_attn_decode_batched_dev(R, kvs, ksrc, seq_k, ds->q, ds->attn, nq, scale, window), "gqa");
         } else {
             wr_session *s = ss[0];
             wr_hip_kv *one[1] = {s->kv};
-            TRY(wr_hip_rows_qkv_append_dev(ds->qkv, qd + 2 * kd, R, nq, dl->q_norm, dl->k_norm, m->rms_eps,
-                                           ds->rope, n_rot, 1, one, L, &pos0, ds->q), "qkv split + kv append");
-            s->kv_rows[L] = pos0 + R;
+            TRY(wr_hip_rows_qkv_append_dev(ds->qkv, width, R, nq, dl->q_norm, shared ? NULL : dl->k_norm,
+                                           m->rms_eps, tab, nr, 1, one, ksrc, &pos0, ds->q, flags),
+                "qkv split + kv append");
+            if (!shared) s->kv_rows[L] = pos0 + R;
             if (prefill) {
-                TRY(wr_hip_attn_prefill_dev(s->kv, L, pos0, R, ds->q, ds->attn, nq, 0.0f, 0), "gqa");
+                TRY(wr_hip_attn_prefill_dev(s->kv, ksrc, pos0, R, ds->q, ds->attn, nq, scale, window), "gqa");
             } else {
                 const uint32_t sk = pos0 + 1;
-                TRY(wr_hip_attn_decode_batched_dev(1, one, L, &sk, ds->q, ds->attn, nq, 0.0f, 0), "gqa");
+                TRY(wr_hip_attn_decode_batched_dev(1, one, ksrc, &sk, ds->q, ds->attn, nq, scale, window), "gqa");
             }
         }
-        TRY(wr_hip_proj_rows_dev(dl->wo, R, ds->attn, qd, ds->resid, ds->resid, hidden),
-            "output projection");
-        TRY(wr_hip_proj_rows_norm_dev(dl->wgu, R, ds->resid, hidden, dl->ffn_norm, m->rms_eps, NULL,
-                                      ds->gu, 2 * ffn), "ffn norm + gate/up projection");
-        TRY(wr_hip_proj_rows_swiglu_dev(dl->wdown, R, ds->gu, 2 * ffn, ds->resid, ds->resid, hidden),
-            "swiglu + down projection");
+        if (gemma) {
+            /* sandwich norms: the sublayer output is normalised, then joins the residual */
+            TRY(wr_hip_proj_rows_dev(dl->wo, R, ds->attn, qd, NULL, ds->proj, hidden), "output projection");
+            TRY(wr_hip_rows_rmsnorm_add_dev(ds->proj, hidden, dl->post_attn_norm, hidden, ds->resid, hidden, R,
+                                            hidden, m->rms_eps), "post-attention norm + residual");
+            TRY(wr_hip_proj_rows_norm_dev(dl->wgu, R, ds->resid, hidden, dl->ffn_norm, m->rms_eps, NULL,
+                                          ds->gu, 2 * ffn), "ffn norm + gate/up projection");
+            TRY(wr_hip_proj_rows_geglu_dev(dl->wdown, R, ds->gu, 2 * ffn, NULL, ds->proj, hidden),
+                "geglu + down projection");
+            TRY(wr_hip_rows_rmsnorm_add_dev(ds->proj, hidden, dl->post_ffw_norm, hidden, ds->resid, hidden, R,
+                                            hidden, m->rms_eps), "post-ffn norm + residual");
+        } else {
+            TRY(wr_hip_proj_rows_dev(dl->wo, R, ds->attn, qd, ds->resid, ds->resid, hidden),
+                "output projection");
+            TRY(wr_hip_proj_rows_norm_dev(dl->wgu, R, ds->resid, hidden, dl->ffn_norm, m->rms_eps, NULL,
+                                          ds->gu, 2 * ffn), "ffn norm + gate/up projection");
+            TRY(wr_hip_proj_rows_swiglu_dev(dl->wdown, R, ds->gu, 2 * ffn, ds->resid, ds->resid, hidden),
+                "swiglu + down projection");
+        }
     }
     L = m->n_layers;
     if (logits_host && logit_rows) {

@@ -125,6 +125,8 @@ typedef struct wrh_devspace {
     float *k, *v;                        /* [R][n_kv*hd] */
     float *gu;                           /* [R][2 ffn]: gate | up */
     float *rope;                         /* [R][hd/2][2] */
+    float *rope_swa;                     /* the same for Gemma's sliding-window layers */
+    float *proj;                         /* [R][hidden]: a sublayer output on its way through a post-norm */
     float *logits;                       /* [logit_rows][vocab] */
     float *block;
 } wrh_devspace;

@@ -397,6 +397,7 @@ const float *wr_step(wr_session *s, uint32_t token)
         if (m->dev) {
             st = wrh_forward_rows_device(m, &s->ws1, &s->ds1, 1, one, &token, s->pos, 0, 0,
                                          take_fail_layer(m), s->logits, 1, 0);
+            if (st == WR_OK && m->is_gemma) wrh_softcap(s->logits, m->vocab, m->logit_softcap);
         } else {
             st = forward_rows(m, &s->ws1, 1, one, &token, s->pos, FWD_STEP);
             if (st == WR_OK) {
