@@ -16,7 +16,9 @@ CPU oracle (a bit-exact restatement of the reference op) on the same data, one
 core, on a bounded sample.  `prefill` reports causal prefill attention,
 `projection` the row projections either side of the path: 16 rows
 (proj_rows_kernel, HBM-bound on the F16 weight bytes) and a 1024-row prefill
-pass (proj_gemm_lds_kernel, MFMA-bound).
+pass (proj_gemm_lds_kernel, MFMA-bound); `end_to_end` the host engine on a
+random-init Qwen3-0.6B-shaped model (python -m wayruntime_amd.e2e_timing in a
+child process).
 """
 from __future__ import annotations
 
@@ -71,6 +73,7 @@ def main() -> None:
                     help="budget for the CPU baseline sample (0 disables it)")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-proj", action="store_true")
+    ap.add_argument("--no-e2e", action="store_true")
     ap.add_argument("--keys-per-wg", type=int, default=0)
     ap.add_argument("--workload", default="headline",
                     choices=["headline", "ragged16", "long16", "long16-hd256", "batch1"],
@@ -105,7 +108,7 @@ def main() -> None:
         ctxs = [ctx] * S
     secondary = args.workload != "headline"
     if secondary:
-        args.no_prefill = args.no_proj = True
+        args.no_prefill = args.no_proj = args.no_e2e = True
         args.cpu_seconds = 0.0
     row = nkv * hd
 
@@ -334,6 +337,21 @@ def main() -> None:
                                     "sample": "%d threads x %d calls, %.1f s" % (n_thr, rounds, t_par)},
                "host": "%s, %d cpus visible" % (cpu_model, os.cpu_count() or 0)}
 
+    # ---- the host engine end to end on a random-init Qwen3-0.6B-shaped model
+    # (secondary figures): a child process, so this process's device state and
+    # the engine's do not meet.  A failure is reported, not fatal.
+    e2e = None
+    if not args.no_e2e:
+        import subprocess
+        try:
+            res = subprocess.run([sys.executable, "-m", "wayruntime_amd.e2e_timing", "--json", "--reps", "2"],
+                                 cwd=ROOT, capture_output=True, text=True, timeout=240)
+            last = [ln for ln in res.stdout.splitlines() if ln.startswith("{")]
+            e2e = json.loads(last[-1]) if res.returncode == 0 and last else {
+                "error": "exit %d: %s" % (res.returncode, (res.stderr or res.stdout)[-200:])}
+        except Exception as exc:                      # timeout, missing model space, ...
+            e2e = {"error": repr(exc)[:200]}
+
     line = {
         "metric": "decode-attn HBM GB/s (% peak) at 16 sess x 4K ctx; prefill attn TFLOP/s",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
@@ -349,6 +367,7 @@ def main() -> None:
                    "sessions": S, "ctx": ctx if len(set(ctxs)) == 1 else ctxs, "layers": L},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
         "roofline": roofline, "cpu_baseline": cpu, "prefill": prefill, "projection": proj,
+        "end_to_end": e2e,
         "check": {"max_abs": max_abs, "rel_l2": rel_l2},
         "device": hipattn.device_name(), "setup_s": round(setup_s, 1),
     }

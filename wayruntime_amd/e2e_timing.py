@@ -30,6 +30,7 @@ def main() -> int:
     ap.add_argument("--prompt", type=int, nargs="*", default=[511, 2047, 4095])
     ap.add_argument("--reps", type=int, default=3)
     ap.add_argument("--skip-decode", action="store_true")
+    ap.add_argument("--json", action="store_true", help="one JSON line with the figures at the end")
     ap.add_argument("--model", default=os.path.join(tempfile.gettempdir(), "wayruntime_amd_qwen3_0_6b.gguf"))
     args = ap.parse_args()
     if args.host:
@@ -42,6 +43,7 @@ def main() -> int:
     m = eng.load(args.model, max_context=ctx)
     walk = "host walk" if args.host else "device walk"
     print(f"{walk}: load {time.perf_counter() - t:.2f} s", flush=True)
+    figures = {"model": "Qwen3-0.6B shape, random init, F16", "walk": walk}
     for n in args.prompt:
         toks = prompt_tokens(m.vocab, n)
         best = None
@@ -53,6 +55,8 @@ def main() -> int:
             best = dt if best is None else min(best, dt)
             s.close()
         print(f"{walk}: prefill {n} tokens: {best * 1e3:.1f} ms ({n / best:.0f} tok/s)", flush=True)
+        figures[f"prefill_{n}_ms"] = round(best * 1e3, 2)
+        figures[f"prefill_{n}_tok_s"] = round(n / best)
     if not args.skip_decode:
         toks = prompt_tokens(m.vocab, 512)
         s = m.session(ctx)
@@ -65,6 +69,7 @@ def main() -> int:
             tok = int(np.argmax(s.step(tok)))
         dt = (time.perf_counter() - t) / steps
         print(f"{walk}: decode step at context ~520: {dt * 1e3:.2f} ms/token ({1 / dt:.0f} tok/s)", flush=True)
+        figures["decode_ms_per_token"] = round(dt * 1e3, 3)
         ss = [m.session(1024) for _ in range(16)]
         for i, x in enumerate(ss):
             assert x.prefill(toks[:100 + i]) == 100 + i
@@ -80,10 +85,15 @@ def main() -> int:
         dt = (time.perf_counter() - t) / steps
         print(f"{walk}: batched step, 16 sessions: {dt * 1e3:.2f} ms/step ({16 / dt:.0f} tok/s aggregate)",
               flush=True)
+        figures["batch16_ms_per_step"] = round(dt * 1e3, 3)
+        figures["batch16_tok_s"] = round(16 / dt)
         for x in ss + [s]:
             x.close()
     m.close()
     eng.close()
+    if args.json:
+        import json
+        print(json.dumps(figures), flush=True)
     return 0
 
 
