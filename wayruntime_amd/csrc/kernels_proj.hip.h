@@ -430,10 +430,12 @@ __device__ __forceinline__ void proj_store_tile(const ProjArgs& a, f32x4 v, uint
 {
     if (!scales) scales = a.scales;
     const int c = lane & 15, g = lane >> 4;
-    const int partner_addr = (lane ^ 8) * 4;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        const float other = __int_as_float(__builtin_amdgcn_ds_bpermute(partner_addr, __float_as_int(v[i])));
+        // the lo column of row c is eight lanes on in the same row of sixteen: a
+        // rotation by eight inside the row (DPP row_ror:8), no trip through LDS
+        const float other = __int_as_float(
+            __builtin_amdgcn_update_dpp(0, __float_as_int(v[i]), 0x128, 0xF, 0xF, false));
         v[i] += other * (1.0f / kProjLoScale);      // meaningful in the hi columns only
     }
     const uint32_t row = group * 8 + (c & 7);
