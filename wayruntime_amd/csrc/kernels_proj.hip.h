@@ -24,9 +24,14 @@
 //       (lane 16g + c: column c, inputs 32kt + 8g .. +8), and one F32 scale
 //       per row, written by proj_prep_kernel, read by every wave (L2 / L1 hits).
 //
-// A wave owns one to four 16-output tiles for one to four row groups of eight;
-// a workgroup is four waves (see proj_rows_kernel).  N must be a multiple of
-// 16 and K a multiple of 32.
+// Kernels, by row count of a launch:
+//   1 row        proj_row1_kernel: the fragment step inside the product;
+//   2 .. 63      proj_prep_kernel, then proj_rows_kernel (a wave owns one to four
+//                16-output tiles for one to four row groups; HBM-bound);
+//   64 .. 4096   proj_prep_group_kernel, then an MFMA-bound GEMM:
+//                proj_gemm_lds_kernel (operands staged through LDS) where its
+//                tiles fill the chip, proj_gemm_split_kernel below that.
+// N must be a multiple of 16 and K a multiple of 32.
 #pragma once
 
 #include "common.hip.h"
