@@ -173,3 +173,48 @@ def test_batched_step_equals_serial_on_device(eng, tmp_path, walk, family):
     for s in batch + serial + [small]:
         s.close()
     m.close()
+
+
+def test_concurrent_calls_on_one_model(eng, tmp_path, walk):
+    # Two threads drive disjoint groups of sessions of one model at the same time
+    # (batched steps, a prefill, single steps).  The model keeps one scratch set
+    # per kind of call; the call that finds it taken allocates its own.  Results
+    # must equal the same calls made one after another.
+    import threading
+    p = str(tmp_path / "small16.gguf")
+    gw.write_model(p, SMALL16)
+    m = eng.load(p)
+    shape = gw.ModelShape(vocab=m.vocab)
+
+    def run(group_seed, out):
+        ss = [m.session(256) for _ in range(5)]
+        for i, s in enumerate(ss):
+            assert s.prefill(workload(shape, 9 + 5 * i + group_seed)) == 9 + 5 * i + group_seed
+        toks = [3 + group_seed + i for i in range(5)]
+        trace = []
+        for step in range(8):
+            rc, lb = E.batch_step(ss, toks)
+            assert rc == 5
+            toks = [int(np.argmax(x)) for x in lb]
+            trace.append(list(toks))
+            if step == 3:                                   # a single step and a longer prefill in between
+                trace.append(int(np.argmax(ss[0].step(toks[0]))))
+                extra = m.session(256)
+                assert extra.prefill(workload(shape, 70 + group_seed)) == 70 + group_seed
+                trace.append(int(np.argmax(extra.step(1))))
+                extra.close()
+                toks[0] = trace[-2]
+        for s in ss:
+            s.close()
+        out.append(trace)
+
+    serial = []
+    for seed in (0, 1):
+        run(seed, serial)
+    for _ in range(3):                                      # a few rounds: the interleaving differs every time
+        a, b = [], []
+        ta = threading.Thread(target=run, args=(0, a))
+        tb = threading.Thread(target=run, args=(1, b))
+        ta.start(); tb.start(); ta.join(); tb.join()
+        assert a and b and a[0] == serial[0] and b[0] == serial[1]
+    m.close()
