@@ -308,3 +308,25 @@ def test_geglu_source(rows):
     gud.free()
     y.free()
     w.close()
+
+
+def test_projection_random_shapes():
+    # a seeded sweep over row counts, input and output widths that crosses every
+    # kernel-selection boundary (1 row, 2-63 rows, the four GEMM tilings, more
+    # rows than a launch takes), checked against the oracle like the fixed cases
+    rng = np.random.default_rng(20240607)
+    row_choices = [1, 2, 7, 8, 9, 16, 17, 40, 63, 64, 65, 127, 128, 129, 500, 1023, 1025, 2047, 4096, 4100]
+    done = 0
+    for case in range(28):
+        rows = int(rng.choice(row_choices))
+        n_in = 32 * int(rng.integers(1, 40))
+        budget = max(16, int(2.5e8 / (rows * n_in)) // 16 * 16)
+        n_out = 16 * int(rng.integers(1, min(520, budget // 16) + 1))
+        print("random proj", case, rows, n_in, n_out, flush=True)
+        x = synth.normal(1000 + case, (rows, n_in), std=float(rng.choice([0.01, 1.0, 30.0])))
+        w16 = _w16(2000 + case, n_out, n_in, 0.2)
+        w = hipattn.Weight([w16])
+        _check(w.rows(x), x, w16, f"case {case}: {rows}x{n_in}x{n_out}")
+        w.close()
+        done += 1
+    assert done == 28
