@@ -292,7 +292,7 @@ static wr_status stage_rows(wr_model *m, wrh_workspace *hs, uint32_t R, wr_sessi
     const wr_engine *e = m->engine;
     const int threads = (e && e->n_threads > 0) ? e->n_threads : 1;
     int bad = WR_OK;
-#pragma omp parallel for num_threads(threads) schedule(static) if (R >= 32)
+#pragma omp parallel for num_threads(threads) schedule(static) if (R >= 4)
     for (uint32_t r = 0; r < R; r++) {
         float *row = hs->residual + (size_t)r * hidden;
         const int rc = wrh_embed(&m->embed, tokens[r], row);
