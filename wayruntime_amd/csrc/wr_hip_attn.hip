@@ -72,7 +72,7 @@ struct Lib {
 } g;
 
 constexpr float kLog2e = 1.4426950408889634f;
-constexpr uint32_t kDefaultTilesPerWg = 64;  // split-K decode: 2048 keys per workgroup
+constexpr uint32_t kDefaultTilesPerWg = 32;  // split-K decode: 1024 keys per workgroup
 constexpr uint32_t kMaxHeads = 4096;        // query heads per session the ticket array is sized for
 constexpr size_t kPinSmall = 1u << 20;      // host copies up to this size go through pinned staging
 
@@ -263,9 +263,11 @@ int decode_locked(uint32_t n, wr_hip_kv* const* kv, uint32_t layer, const uint32
     // key range), never at the rest of the batch: a session's arithmetic is then
     // the same whether it is stepped alone or with others, which is what makes
     // the batched step bit-identical to serial steps (reference contract:
-    // src/core/batch.c:15-19).  About 1 MiB of K+V per workgroup (2048 keys at
-    // head_dim 128, 1024 at 256) measured best for 16 sessions of 4096; from
-    // 16K keys up an eighth of the session per workgroup measured better
+    // src/core/batch.c:15-19).  Half a MiB of K+V per workgroup (1024 keys at
+    // head_dim 128, 512 at 256): 16 sessions of 4096 run as fast with it as
+    // with twice that, and a single session's chain of tiles is half as long
+    // (one session of 8192 keys: 27 -> 17 us); from
+    // 8K keys up an eighth of the session per workgroup measured better
     // (fewer partials and workgroup turnovers: 82 % -> 86 % of HBM peak at
     // 16 x 32768).  The session's tiles are spread evenly over the workgroups,
     // and the floor keeps the in-kernel merge within kMaxSplits partials.
