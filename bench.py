@@ -43,7 +43,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0   # MI355X dense f16
 # from inside this process, so the figure is carried here from the committed
 # counter summary (profiles/decode_prefill_traffic_pmc.txt) and reported only
 # for the workload it was measured on.
-PMC_TRAFFIC_BYTES = {(16, 4096): 269496033 + 864256}
+PMC_TRAFFIC_BYTES = {(16, 4096): 270032800 + 1462272}
 
 
 def pooled16(pool16: np.ndarray, salt: int, n: int) -> np.ndarray:
