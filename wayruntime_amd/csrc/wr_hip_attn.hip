@@ -482,10 +482,17 @@ void launch_proj_gemm(const ProjArgs& a, uint32_t groups)
     // one-dimensional grids: eight equal shares of output panels, times the row panels
     const uint32_t share = (panels + 7) / 8 * 8;
     const uint32_t wide = (nt + 15) / 16, wshare = (wide + 7) / 8 * 8;
-    if (wide * ((groups + 15) / 16) >= 256)
+    // The eight-wave tile runs one workgroup per CU, in rounds of 256: when its
+    // last round would leave more than 15 % of the CUs idle, the four-wave tile
+    // (two per CU, half the work each) loses less (2047 rows x 6144 outputs:
+    // 384 eight-wave tiles, 1.5 rounds, 83 us; 768 four-wave tiles 65 us).
+    const uint32_t n_wide = wide * ((groups + 15) / 16), n_big = panels * ((groups + 15) / 16);
+    const uint32_t rounds = (n_wide + 255) / 256;
+    const bool wide_fills = n_wide >= 256 && (n_wide * 100 >= rounds * 256 * 85 || n_big < 512);
+    if (wide_fills)
         launch_main(proj_gemm_lds_kernel<8, 4, 4>, dim3(wshare * ((groups + 15) / 16)), dim3(512), a,
                     gemm_lds_bytes<8, 4, 4>());
-    else if (panels * ((groups + 15) / 16) >= 512)
+    else if (n_big >= 512)
         launch_main(proj_gemm_lds_kernel<8, 2, 3>, dim3(share * ((groups + 15) / 16)), dim3(kProjThreads), a,
                     gemm_lds_bytes<8, 2, 3>());
     else if (panels * ((groups + 7) / 8) >= 256)
