@@ -850,7 +850,11 @@ constexpr size_t gemm_lds_bytes()
     return (size_t)RING * (WN * 4 + 2 * GROUPS) * 1024;   // KiB per stage: 4 WN weight tiles, 2 GROUPS fragments
 }
 
-template <int GROUPS, int WN, int RING>
+// PIPE: the operand reads of the next k-step are issued before this one's MFMAs
+// (two register sets), for launches that leave a SIMD with a single wave and
+// nobody else to cover its LDS latency; needs one more ring stage, because a
+// stage is now read one k-step before it is used.
+template <int GROUPS, int WN, int RING, bool PIPE = false>
 __global__ __launch_bounds__(128 * WN, WN == 2 ? 2 : 1) void proj_gemm_lds_kernel(const ProjArgs a)
 {
     extern __shared__ __attribute__((aligned(16))) unsigned char gemm_smem[];
@@ -904,6 +908,45 @@ __global__ __launch_bounds__(128 * WN, WN == 2 ? 2 : 1) void proj_gemm_lds_kerne
     for (int st0 = 0; st0 < RING - 1; st0++) issue(st0);
     const uint32_t w_off = wn * NT * 1024 + lane * 16;
     const uint32_t x_off = (WN * NT + wr * GROUPS) * 1024 + lane * 16;
+    if constexpr (PIPE) {
+        static_assert(RING >= 4, "a stage is read while the one before it is multiplied");
+        half8 w0[NT], x0[GROUPS], w1[NT], x1[GROUPS];
+        auto read_ops = [&](half8 (&wv)[NT], half8 (&xv)[GROUPS], uint32_t kt) {
+            const unsigned char* st = gemm_smem + (kt % RING) * STAGE;
+#pragma unroll
+            for (int t = 0; t < NT; t++) wv[t] = *reinterpret_cast<const half8*>(st + w_off + t * 1024);
+#pragma unroll
+            for (int gi = 0; gi < GROUPS; gi++) xv[gi] = *reinterpret_cast<const half8*>(st + x_off + gi * 1024);
+        };
+        auto mfmas = [&](const half8 (&wv)[NT], const half8 (&xv)[GROUPS]) {
+#pragma unroll
+            for (int gi = 0; gi < GROUPS; gi++)
+#pragma unroll
+                for (int t = 0; t < NT; t++)
+                    acc[t][gi] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wv[t], xv[gi], acc[t][gi], 0, 0, 0);
+        };
+        // stage 0 into the first register set
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(CPW * (RING - 2)) : "memory");
+        read_ops(w0, x0, 0);
+        // Step kt: everybody's copies of stage kt + 1 have landed (the barrier),
+        // the copies of stage kt + RING - 1 go to the slot of stage kt - 1, whose
+        // last reads were waited for before the MFMAs of step kt - 1 were issued;
+        // then the reads of stage kt + 1, then the MFMAs of stage kt.  Two steps
+        // per iteration so that no register set is copied; a step past the end
+        // reads a stage that holds a repeat of the last one and is not used.
+        uint32_t kt = 0;
+        for (; kt + 2 <= ktiles; kt += 2) {
+            asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(CPW * (RING - 3)) : "memory");
+            issue(kt + RING - 1);
+            read_ops(w1, x1, kt + 1);
+            mfmas(w0, x0);
+            asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(CPW * (RING - 3)) : "memory");
+            issue(kt + RING);
+            read_ops(w0, x0, kt + 2);
+            mfmas(w1, x1);
+        }
+        if (kt < ktiles) mfmas(w0, x0);                   // odd number of k-steps
+    } else
     for (uint32_t kt = 0; kt < ktiles; kt++) {
         // this wave's copies of stage kt have landed; those of the RING - 2 stages after it may be in flight
         asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(CPW * (RING - 2)) : "memory");

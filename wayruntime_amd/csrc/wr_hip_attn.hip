@@ -463,7 +463,7 @@ void launch_proj(const ProjArgs& a, uint32_t groups)
 // Prefill-sized row counts: the largest tile that still fills the chip.
 //   LDS-staged, eight waves, 256 outputs x 128 rows per workgroup, from one workgroup per CU;
 //   LDS-staged, 128 x 128, from two workgroups per CU;
-//   LDS-staged, 128 x 64, from one per CU;
+//   LDS-staged, 128 x 64, from one per CU (software-pipelined: a SIMD may hold a single wave);
 //   registers, 64 x 32, the four waves split the input range;
 //   registers, 32 x 32, likewise.
 constexpr int kProjGemmMinRows = 64;
@@ -496,8 +496,8 @@ void launch_proj_gemm(const ProjArgs& a, uint32_t groups)
         launch_main(proj_gemm_lds_kernel<8, 2, 3>, dim3(share * ((groups + 15) / 16)), dim3(kProjThreads), a,
                     gemm_lds_bytes<8, 2, 3>());
     else if (panels * ((groups + 7) / 8) >= 256)
-        launch_main(proj_gemm_lds_kernel<4, 2, 3>, dim3(share * ((groups + 7) / 8)), dim3(kProjThreads), a,
-                    gemm_lds_bytes<4, 2, 3>());
+        launch_main(proj_gemm_lds_kernel<4, 2, 4, true>, dim3(share * ((groups + 7) / 8)), dim3(kProjThreads), a,
+                    gemm_lds_bytes<4, 2, 4>());
     else if (((nt + 3) / 4) * ((groups + 3) / 4) >= 384)
         launch_proj_gemm_split<4, 4>(a, groups);
     else
@@ -689,6 +689,9 @@ int wr_hip_attn_init(int device)
         if (e == hipSuccess)
             e = hipFuncSetAttribute(reinterpret_cast<const void*>(proj_gemm_lds_kernel<8, 2, 3>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)gemm_lds_bytes<8, 2, 3>());
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute(reinterpret_cast<const void*>(proj_gemm_lds_kernel<4, 2, 4, true>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)gemm_lds_bytes<4, 2, 4>());
         if (e == hipSuccess)
             e = hipFuncSetAttribute(reinterpret_cast<const void*>(proj_gemm_lds_kernel<8, 4, 4>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)gemm_lds_bytes<8, 4, 4>());
