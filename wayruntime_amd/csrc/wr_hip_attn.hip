@@ -495,7 +495,10 @@ void launch_proj_gemm(const ProjArgs& a, uint32_t groups)
     else if (n_big >= 512)
         launch_main(proj_gemm_lds_kernel<8, 2, 3>, dim3(share * ((groups + 15) / 16)), dim3(kProjThreads), a,
                     gemm_lds_bytes<8, 2, 3>());
-    else if (panels * ((groups + 7) / 8) >= 256)
+    else if (panels * ((groups + 7) / 8) >= 512)          // two and more per CU cover each other's latency
+        launch_main(proj_gemm_lds_kernel<4, 2, 3>, dim3(share * ((groups + 7) / 8)), dim3(kProjThreads), a,
+                    gemm_lds_bytes<4, 2, 3>());
+    else if (panels * ((groups + 7) / 8) >= 256)          // one per CU, one wave per SIMD: pipelined reads
         launch_main(proj_gemm_lds_kernel<4, 2, 4, true>, dim3(share * ((groups + 7) / 8)), dim3(kProjThreads), a,
                     gemm_lds_bytes<4, 2, 4>());
     else if (((nt + 3) / 4) * ((groups + 3) / 4) >= 384)
