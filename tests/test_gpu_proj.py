@@ -55,8 +55,10 @@ def _check(got, x, w16, what):
     (100, 160, 80, 0.3),          # ... a last row group of four rows, five input tiles
     (300, 160, 2512, 0.2),        # ... 64 x 32 tiles, a partial last tile both ways
     (4102, 64, 32, 1.0),          # more rows than one launch takes: 4096 + a six-row launch
-    (500, 96, 4112, 0.3),         # LDS-staged GEMM, 128 x 64 tiles: partial output and row panels, odd input tiles
-    (1000, 1056, 4112, 0.02),     # ... 33 input tiles
+    (500, 96, 4112, 0.3),         # LDS-staged GEMM, 128 x 64 tiles, pipelined reads: partial panels, odd input tiles
+    (500, 32, 4112, 0.5),         # ... a single input tile
+    (500, 128, 4112, 0.3),        # ... an even number of them
+    (1000, 1056, 4112, 0.02),     # ... the plain 128 x 64 tile (two workgroups per CU), 33 input tiles
     (1000, 96, 8208, 0.3),        # LDS-staged GEMM, 128 x 128 tiles: partial output and row panels, three input tiles
     (1000, 32, 8208, 0.5),        # ... a single input tile (the ring's prologue covers the whole product)
     (2040, 96, 4112, 0.3),        # LDS-staged GEMM, eight waves, 256 x 128 tiles: partial panels, three input tiles
