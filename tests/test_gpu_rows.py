@@ -130,20 +130,28 @@ def test_error_contract():
 import ctypes as C
 
 
-@pytest.mark.parametrize("rows,nq,nkv,hd,norm,pos,batch", [
-    (70, 16, 8, 128, True, 13, False),      # three cache blocks, both ends partial
-    (1, 16, 8, 128, True, 77, False),       # one decode row
-    (33, 4, 2, 64, False, 0, False),        # no norm; head_dim 64 (the pair sits in two lanes)
-    (5, 8, 4, 256, True, 31, False),        # crosses a block boundary after one row
-    (5, 16, 8, 128, True, 0, True),         # batched step: row i to session i at its own position
-    (16, 32, 8, 128, False, 0, True),
+@pytest.mark.parametrize("rows,nq,nkv,hd,norm,pos,batch,rot_pairs,pad", [
+    (70, 16, 8, 128, True, 13, False, 0, 16),      # three cache blocks, both ends partial
+    (1, 16, 8, 128, True, 77, False, 0, 16),       # one decode row
+    (33, 4, 2, 64, False, 0, False, 0, 16),        # no norm; head_dim 64 (the pair sits in two lanes)
+    (5, 8, 4, 256, True, 31, False, 0, 16),        # crosses a block boundary after one row
+    (5, 16, 8, 128, True, 0, True, 0, 16),         # batched step: row i to session i at its own position
+    (16, 32, 8, 128, False, 0, True, 0, 16),
+    # head dims 128 and 256 take the eight-lanes-per-position path when rows,
+    # tables and vectors are 16-byte aligned and the rotated pairs come in
+    # eights; the cases below sit on both sides of each condition
+    (70, 8, 4, 128, True, 13, False, 24, 16),      # partial rotation, pairs in eights
+    (40, 8, 4, 128, True, 5, False, 20, 16),       # partial rotation, not in eights: one wave per position
+    (40, 8, 4, 128, True, 5, False, 0, 3),         # row stride not a multiple of four floats: likewise
+    (67, 4, 2, 256, False, 30, False, 40, 8),      # head_dim 256, no norm, partial rotation
+    (7, 4, 2, 256, True, 0, True, 0, 4),           # head_dim 256, batched step
 ])
-def test_qkv_append_equals_prep_then_append(rows, nq, nkv, hd, norm, pos, batch):
+def test_qkv_append_equals_prep_then_append(rows, nq, nkv, hd, norm, pos, batch, rot_pairs, pad):
     # the fused launch against the two-step path: Q rows and the cache contents, bit for bit
-    print("qkv_append", rows, nq, nkv, hd, norm, pos, batch, flush=True)
+    print("qkv_append", rows, nq, nkv, hd, norm, pos, batch, rot_pairs, pad, flush=True)
     lib = hipattn.lib()
     width = (nq + 2 * nkv) * hd
-    ld = width + 16
+    ld = width + pad
     qkv = synth.normal(7 * hd + rows, (rows, ld), std=1.5)
     qn = synth.normal(1, (hd,)) * np.float32(0.1) + np.float32(1.0)
     kn = synth.normal(2, (hd,)) * np.float32(0.1) + np.float32(1.0)
@@ -152,10 +160,11 @@ def test_qkv_append_equals_prep_then_append(rows, nq, nkv, hd, norm, pos, batch)
     n_kv = rows if batch else 1
     positions = [3 + 37 * i for i in range(rows)] if batch else [pos]
     if batch:
-        tab = np.concatenate([oracle.rope_table(1, hd, p, 1e6, 0) for p in positions])
+        tab = np.concatenate([oracle.rope_table(1, hd, p, 1e6, rot_pairs) for p in positions])
     else:
-        tab = oracle.rope_table(rows, hd, pos, 1e6, 0)
+        tab = oracle.rope_table(rows, hd, pos, 1e6, rot_pairs)
     n_rot = tab.shape[1]
+    assert n_rot == (rot_pairs or hd // 2)
     ctx = 1024
     two_step = [hipattn.KVCache(1, hd, nkv, ctx) for _ in range(n_kv)]
     fused = [hipattn.KVCache(1, hd, nkv, ctx) for _ in range(n_kv)]
@@ -217,12 +226,14 @@ def _f16_ulps(a16, b16):
     return np.abs(a16.astype(np.int32) - b16.astype(np.int32))
 
 
-def test_qkv_append_gemma_flags():
+@pytest.mark.parametrize("hd", [64, 128, 256])
+def test_qkv_append_gemma_flags(hd):
     # V_NORM: the V heads get a weightless RMSNorm before they are truncated into
     # the cache; Q_ONLY: rows of Q heads only, nothing is appended (a layer that
     # reads another layer's cache)
+    print("qkv_append flags", hd, flush=True)
     lib = hipattn.lib()
-    rows, nq, nkv, hd, pos = 9, 4, 2, 64, 30
+    rows, nq, nkv, pos = 9, 4, 2, 30
     width = (nq + 2 * nkv) * hd
     qkv = synth.normal(91, (rows, width), std=1.5)
     qn = synth.normal(1, (hd,)) * np.float32(0.1) + np.float32(1.0)

@@ -131,8 +131,148 @@ struct QkvAppendArgs {
     uint32_t ld, nq, nkv, hd, n_rot, rows;
     uint32_t per_session;    // 1: row i belongs to session i; 0: all rows to session 0 from pos[0]
     uint32_t v_norm;         // 1: V heads get a weightless RMSNorm before they are stored
+    uint32_t row8;           // hd / 64 (2 or 4) when qkv_append_row8 may serve the call, else 0
     float eps;
 };
+
+// wave_sum_f32 over a row whose 64 partial sums sit eight to a lane in eight
+// neighbouring lanes (lane `part` of the eight holds partial sums 8 part ..
+// 8 part + 7).  The wave sum pairs partial sums 32, 16, 8, 4, 2, 1 apart, in
+// that order: the first three are the lanes 4, 2, 1 away, the last three are
+// in the lane.  The same additions, hence the same bits.
+__device__ __forceinline__ float row8_sum_f32(float (&s)[8])
+{
+#pragma unroll
+    for (int m = 4; m >= 1; m >>= 1)
+#pragma unroll
+        for (int e = 0; e < 8; e++) s[e] += wave_xor_f32(s[e], m);
+    const float b0 = s[0] + s[4], b1 = s[1] + s[5], b2 = s[2] + s[6], b3 = s[3] + s[7];
+    const float c0 = b0 + b2, c1 = b1 + b3;
+    return c0 + c1;
+}
+
+// One workgroup's share of qkv_append_kernel for head dims of 128 and 256
+// (NJ = hd / 64) with everything 16-byte aligned: eight lanes per position, all
+// 32 positions of the block at once.  Lane `part` of a position holds the
+// elements 64 c + 8 part + e (c < NJ, e < 8), i.e. what the lanes 8 part .. + 7
+// of qkv_append_kernel's wave hold, so the sum of squares runs through the same
+// additions, a rotation pair (j, j + hd/2) is in one lane, and every load and
+// store is a run of 32 bytes (16 for a K chunk).  No loop over positions and no
+// barrier on the Q and K paths: one round trip to memory instead of eight.
+template <int NJ>
+__device__ __forceinline__ void qkv_append_row8(const QkvAppendArgs& a, unsigned char* smem, uint32_t h,
+                                                uint32_t sess, uint32_t ctx_pad, uint32_t p_begin,
+                                                uint32_t np, uint32_t row0)
+{
+#pragma clang fp contract(off)
+    constexpr uint32_t HD = 64 * NJ;
+    const uint32_t i = threadIdx.x >> 3, part = threadIdx.x & 7;
+    const bool live = i < np;
+    const uint32_t r = row0 + (live ? i : 0);
+    const float* src = a.qkv + (size_t)r * a.ld + (size_t)h * HD + part * 8;
+    float x[NJ][8];
+#pragma unroll
+    for (int c = 0; c < NJ; c++) {
+        f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = lo;
+        if (live) {
+            lo = *reinterpret_cast<const f32x4*>(src + c * 64);
+            hi = *reinterpret_cast<const f32x4*>(src + c * 64 + 4);
+        }
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            x[c][e] = lo[e];
+            x[c][4 + e] = hi[e];
+        }
+    }
+    const bool is_v = h >= a.nq + a.nkv, is_q = h < a.nq;
+    const float* nw = is_v ? nullptr : (is_q ? a.q_norm : a.k_norm);
+    if (is_v ? a.v_norm != 0 : nw != nullptr) {           // workgroup-uniform
+        float s[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            float ss = 0.f;
+#pragma unroll
+            for (int c = 0; c < NJ; c++) ss += x[c][e] * x[c][e];
+            s[e] = ss;
+        }
+        const float inv_rms = 1.0f / sqrtf(row8_sum_f32(s) / (float)HD + a.eps);
+#pragma unroll
+        for (int c = 0; c < NJ; c++) {
+            if (is_v) {
+#pragma unroll
+                for (int e = 0; e < 8; e++) x[c][e] = x[c][e] * inv_rms;
+            } else {
+                const f32x4 wl = *reinterpret_cast<const f32x4*>(nw + c * 64 + part * 8);
+                const f32x4 wh = *reinterpret_cast<const f32x4*>(nw + c * 64 + part * 8 + 4);
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    x[c][e] = x[c][e] * inv_rms * wl[e];
+                    x[c][4 + e] = x[c][4 + e] * inv_rms * wh[e];
+                }
+            }
+        }
+    }
+
+    if (is_v) {
+        const uint32_t kvh = h - a.nq - a.nkv;
+        uint16_t (*tile)[kVBlock + 2] = reinterpret_cast<uint16_t (*)[kVBlock + 2]>(smem);
+        if (live) {
+#pragma unroll
+            for (int c = 0; c < NJ; c++)
+#pragma unroll
+                for (int e = 0; e < 8; e++) tile[c * 64 + part * 8 + e][i] = f32_to_f16_trunc(x[c][e]);
+        }
+        __syncthreads();
+        uint16_t* vt = a.vt[sess];
+        for (uint32_t idx = threadIdx.x; idx < HD * np; idx += 256) {
+            const uint32_t d = idx / np, ii = idx % np;
+            vt[vt_offset(kvh, ctx_pad, p_begin + ii, d, HD)] = tile[d][ii];
+        }
+        return;
+    }
+
+    // rotation of the pairs (j, j + hd/2), j = 64 c + 8 part + e for c < NJ / 2
+    const float* cs = a.cos_sin + (size_t)r * a.n_rot * 2;
+#pragma unroll
+    for (int c = 0; c < NJ / 2; c++) {
+        const uint32_t j0 = c * 64 + part * 8;
+        if (live && j0 < a.n_rot) {                       // n_rot is a multiple of eight here
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const f32x4 t = *reinterpret_cast<const f32x4*>(cs + 2 * j0 + 4 * q);
+#pragma unroll
+                for (int u = 0; u < 2; u++) {
+                    const float co = t[2 * u], sn = t[2 * u + 1];
+                    const float x0 = x[c][2 * q + u], x1 = x[c + NJ / 2][2 * q + u];
+                    const float a0 = x0 * co, b0 = x1 * sn, a1 = x0 * sn, b1 = x1 * co;
+                    x[c][2 * q + u] = a0 - b0;
+                    x[c + NJ / 2][2 * q + u] = a1 + b1;
+                }
+            }
+        }
+    }
+    if (!live) return;
+    if (is_q) {
+        float* dst = a.q_out + ((size_t)r * a.nq + h) * HD + part * 8;
+#pragma unroll
+        for (int c = 0; c < NJ; c++) {
+            *reinterpret_cast<f32x4*>(dst + c * 64) = f32x4{x[c][0], x[c][1], x[c][2], x[c][3]};
+            *reinterpret_cast<f32x4*>(dst + c * 64 + 4) = f32x4{x[c][4], x[c][5], x[c][6], x[c][7]};
+        }
+    } else {
+        uint16_t* k = a.k[sess];
+        const uint32_t kvh = h - a.nq, p = p_begin + i;
+#pragma unroll
+        for (int c = 0; c < NJ; c++) {
+            uint32_t w[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                w[e] = (uint32_t)f32_to_f16_trunc(x[c][2 * e]) | ((uint32_t)f32_to_f16_trunc(x[c][2 * e + 1]) << 16);
+            *reinterpret_cast<u32x4*>(k + k_offset(kvh, ctx_pad, p, c * 64 + part * 8, HD)) =
+                u32x4{w[0], w[1], w[2], w[3]};
+        }
+    }
+}
 
 __global__ __launch_bounds__(256) void qkv_append_kernel(const QkvAppendArgs a)
 {
@@ -155,6 +295,9 @@ __global__ __launch_bounds__(256) void qkv_append_kernel(const QkvAppendArgs a)
         row0 = p_begin - pos0;
     }
     const uint32_t np = p_end - p_begin;                  // 1 .. 32
+
+    if (a.row8 == 2) return qkv_append_row8<2>(a, qkv_smem, h, sess, ctx_pad, p_begin, np, row0);
+    if (a.row8 == 4) return qkv_append_row8<4>(a, qkv_smem, h, sess, ctx_pad, p_begin, np, row0);
 
     if (h >= a.nq + a.nkv) {
         // V head: rows -> F16 -> tile[d][position in block] -> runs along positions

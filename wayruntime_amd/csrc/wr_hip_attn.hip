@@ -1381,6 +1381,13 @@ int wr_hip_rows_qkv_append_dev(const float* qkv_dev, uint32_t ld, uint32_t rows,
     a.rows = rows;
     a.per_session = (n_kv > 1 || rows == 1) ? 1 : 0;
     a.eps = eps;
+    {
+        // eight lanes per position with 16-byte accesses where the shapes and
+        // the addresses allow it (every model on the device walk does)
+        const uintptr_t addrs = (uintptr_t)qkv_dev | (uintptr_t)q_out_dev | (uintptr_t)cos_sin_dev |
+                                (uintptr_t)q_norm_dev | (uintptr_t)k_norm_dev;
+        if ((hd == 128 || hd == 256) && n_rot % 8 == 0 && ld % 4 == 0 && addrs % 16 == 0) a.row8 = hd / 64;
+    }
     const uint32_t gx = a.per_session ? rows : (pos[0] + rows - 1) / kVBlock - pos[0] / kVBlock + 1;
     const size_t lds = std::max((size_t)4 * hd * sizeof(float), (size_t)hd * (kVBlock + 2) * sizeof(uint16_t));
     Locked lk;
