@@ -342,35 +342,23 @@ __device__ __forceinline__ void prefill_block(const PrefillArgs& a, PrefillSmem<
     PrefillStage<HD> s0, s1;
     uint32_t tile = t_first;
     prefill_fetch<HD>(s0, kbase, vtbase, tile, tid);
-    if constexpr (HD < 256)
-        if (tile + 1 <= t_last) prefill_fetch<HD>(s1, kbase, vtbase, tile + 1, tid);
+    if (tile + 1 <= t_last) prefill_fetch<HD>(s1, kbase, vtbase, tile + 1, tid);
 
     PrefillRows<HD> R;
     prefill_rows_init<HD>(R, a, row0, head, n, g);
     const int krow = prefill_key_perm(n);                 // LDS row this lane feeds to MFMA row n
 
-    if constexpr (HD >= 256) {
-        // wide heads: one staging set (the second would not fit the register file)
-        for (int buf = 0;; buf ^= 1) {
-            prefill_stash<HD>(sm, buf, s0, tile, kv_valid, tid);
-            lds_barrier();
-            if (tile + 1 <= t_last) prefill_fetch<HD>(s0, kbase, vtbase, tile + 1, tid);
-            prefill_compute<HD, true>(R, sm.k[buf], sm.v[buf], tile, n, g, krow);
-            if (++tile > t_last) break;
-        }
-    } else {
-        for (;;) {
-            prefill_stash<HD>(sm, 0, s0, tile, kv_valid, tid);
-            lds_barrier();
-            if (tile + 2 <= t_last) prefill_fetch<HD>(s0, kbase, vtbase, tile + 2, tid);
-            prefill_compute<HD, true>(R, sm.k[0], sm.v[0], tile, n, g, krow);
-            if (++tile > t_last) break;
-            prefill_stash<HD>(sm, 1, s1, tile, kv_valid, tid);
-            lds_barrier();
-            if (tile + 2 <= t_last) prefill_fetch<HD>(s1, kbase, vtbase, tile + 2, tid);
-            prefill_compute<HD, true>(R, sm.k[1], sm.v[1], tile, n, g, krow);
-            if (++tile > t_last) break;
-        }
+    for (;;) {
+        prefill_stash<HD>(sm, 0, s0, tile, kv_valid, tid);
+        lds_barrier();
+        if (tile + 2 <= t_last) prefill_fetch<HD>(s0, kbase, vtbase, tile + 2, tid);
+        prefill_compute<HD, true>(R, sm.k[0], sm.v[0], tile, n, g, krow);
+        if (++tile > t_last) break;
+        prefill_stash<HD>(sm, 1, s1, tile, kv_valid, tid);
+        lds_barrier();
+        if (tile + 2 <= t_last) prefill_fetch<HD>(s1, kbase, vtbase, tile + 2, tid);
+        prefill_compute<HD, true>(R, sm.k[1], sm.v[1], tile, n, g, krow);
+        if (++tile > t_last) break;
     }
     prefill_rows_store<HD>(R, a, row0, head, n, g);
 }
@@ -379,7 +367,7 @@ __device__ __forceinline__ void prefill_block(const PrefillArgs& a, PrefillSmem<
 // block (blocks-1-x) and then block x: a long block and a short one, so every
 // workgroup streams the same number of tiles despite the causal triangle.
 template <int HD>
-__global__ __launch_bounds__(kPrefillThreads, 2) void prefill_mfma_kernel(const PrefillArgs a)
+__global__ __launch_bounds__(kPrefillThreads, 1) void prefill_mfma_kernel(const PrefillArgs a)
 {
     __shared__ __attribute__((aligned(16))) PrefillSmem<HD> sm;
     const uint32_t G = a.group;
