@@ -134,11 +134,14 @@ def test_qwen3_0_6b_greedy_stream_matches_reference(eng, tmp_path, walk):
     os.remove(p)
 
 
-@pytest.mark.parametrize("family", ["qwen3", "gemma"])
+@pytest.mark.parametrize("family", ["qwen3", "qwen3-hd128", "gemma"])
 def test_batched_step_equals_serial_on_device(eng, tmp_path, walk, family):
     p = str(tmp_path / "model.gguf")
     if family == "gemma":       # sliding-window layers, shared caches, per-layer head_dim in the batched walk
         gw.write_model(p, GEMMA_TOY, seed=GEMMA_SEED, std=GEMMA_STD)
+    elif family == "qwen3-hd128":   # the head_dim of the real models: the wide-access row kernels
+        gw.write_model(p, gw.ModelShape(n_layers=2, hidden=256, ffn=512, n_q=4, n_kv=2, head_dim=128,
+                                        vocab=320, context=512))
     else:
         gw.write_model(p, SMALL16)
     m = eng.load(p)
