@@ -63,6 +63,9 @@ def _check(got, x, w16, what):
     (1000, 32, 8208, 0.5),        # ... a single input tile (the ring's prologue covers the whole product)
     (2040, 96, 4112, 0.3),        # LDS-staged GEMM, eight waves, 256 x 128 tiles: partial panels, three input tiles
     (2040, 32, 4112, 0.5),        # ... a single input tile
+    (500, 1088, 4112, 0.02),      # ... 34 input tiles, partial panels
+    (2047, 2048, 1024, 0.02),     # the output projection of a 2047-token prompt (Qwen3-0.6B): one 128 x 64 tile per CU
+    (1000, 2048, 1040, 0.02),     # too few LDS tiles for the chip: the register GEMM with a long contraction
 ])
 def test_projection_shapes_vs_oracle(rows, n_in, n_out, std):
     print("proj", rows, n_in, n_out, flush=True)
@@ -70,6 +73,19 @@ def test_projection_shapes_vs_oracle(rows, n_in, n_out, std):
     w16 = _w16(n_out + 3, n_out, n_in, std)
     w = hipattn.Weight([w16])
     _check(w.rows(x), x, w16, f"{rows}x{n_in}x{n_out}")
+    w.close()
+
+
+@pytest.mark.parametrize("rows,n_in,n_out", [(2047, 2048, 1024), (1000, 2048, 1040)])
+def test_repeated_launches_give_the_same_bits(rows, n_in, n_out):
+    # no sum in these kernels depends on the order in which waves or workgroups finish
+    print("proj repeat", rows, n_in, n_out, flush=True)
+    x = synth.normal(5, (rows, n_in))
+    w16 = _w16(6, n_out, n_in, 0.02)
+    w = hipattn.Weight([w16])
+    first = w.rows(x)
+    for _ in range(4):
+        assert w.rows(x).tobytes() == first.tobytes()
     w.close()
 
 
@@ -126,9 +142,11 @@ def test_row_magnitudes_do_not_matter():
     w.close()
 
 
-@pytest.mark.parametrize("rows", [6, 70])           # the row kernel and the register-tiled one
-def test_device_form_with_strides_and_residual_add(rows):
-    n_in, n_out = 128, 64
+@pytest.mark.parametrize("rows,n_in,n_out", [
+    (6, 128, 64), (70, 128, 64),    # the row kernel and the register-tiled one
+    (1000, 2048, 1040),             # a GEMM-sized launch
+])
+def test_device_form_with_strides_and_residual_add(rows, n_in, n_out):
     ldx, ldy = n_in + 32, n_out + 8
     x = synth.normal(31, (rows, ldx))
     add = synth.normal(32, (rows, ldy))
@@ -143,6 +161,11 @@ def test_device_form_with_strides_and_residual_add(rows):
     plain = w.rows(np.ascontiguousarray(x[:, :n_in]))
     assert np.array_equal(y[:, :n_out], plain + add[:, :n_out])
     assert np.all(y[:, n_out:] == 7.0)              # padding columns are not touched
+    # in place: the residual is the output buffer (the device walk's h += W . x)
+    w.rows_dev(rows, xd, ldx, ad, ldy, add_dev=ad)
+    hipattn.sync()
+    y2 = ad.to_host((rows, ldy))
+    assert np.array_equal(y2[:, :n_out], y[:, :n_out]) and np.array_equal(y2[:, n_out:], add[:, n_out:])
     for b in (xd, ad, yd):
         b.free()
     w.close()
