@@ -47,6 +47,7 @@ def _setup(nq, nkv, hd, p0, T, seed, theta=None, extra_rows=0):
     (16, 8, 128, 0, 400, 64),       # sliding window
     (32, 8, 128, 50, 300, 33),
     (8, 4, 256, 0, 300, 100),
+    (16, 8, 256, 40, 700, 0),       # head_dim 256 behind a non-empty cache: blocks of 2 to 24 tiles, odd and even
 ])
 def test_prefill_matches_serial_stepping_oracle(nq, nkv, hd, p0, T, win):
     print("prefill", nq, nkv, hd, p0, T, win, flush=True)
