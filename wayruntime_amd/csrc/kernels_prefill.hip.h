@@ -18,6 +18,7 @@ struct PrefillArgs {
     float* out;              // [T][nq][hd]
     uint32_t p0, T, nq, nkv, group, hd, ctx_pad, window;
     float qscale;            // softmax scale * log2(e)
+    uint32_t single;         // MFMA kernels: one position block per workgroup (grid = blocks) instead of a pair
 };
 
 // Any head_dim / group: one workgroup per (row, head), vector ALU only.
@@ -366,6 +367,8 @@ __device__ __forceinline__ void prefill_block(const PrefillArgs& a, PrefillSmem<
 // grid = (ceil(blocks / 2), KV heads x head chunks).  Workgroup x takes position
 // block (blocks-1-x) and then block x: a long block and a short one, so every
 // workgroup streams the same number of tiles despite the causal triangle.
+// a.single: grid.x = blocks and workgroup x takes block (blocks-1-x) only (the
+// long blocks start first); for launches whose pairs would leave CUs idle.
 template <int HD>
 __global__ __launch_bounds__(kPrefillThreads, 1) void prefill_mfma_kernel(const PrefillArgs a)
 {
@@ -378,7 +381,7 @@ __global__ __launch_bounds__(kPrefillThreads, 1) void prefill_mfma_kernel(const 
     const uint32_t nblk = (a.T + BP - 1) / BP;
     const uint32_t lo = blockIdx.x, hi = nblk - 1 - blockIdx.x;
     prefill_block<HD>(a, sm, hi, kvh, hc);
-    if (hi != lo) {
+    if (!a.single && hi != lo) {
         __syncthreads();                                  // LDS buffers change hands
         prefill_block<HD>(a, sm, lo, kvh, hc);
     }
@@ -951,6 +954,7 @@ __device__ __forceinline__ void split_block(const PrefillArgs& a, unsigned char*
 // L2 keeps seeing the same few heads' K / Vt.  Workgroup y takes position block
 // (blocks-1-y) and then block y: a long block and a short one, so every
 // workgroup streams the same number of tiles despite the causal triangle.
+// a.single: grid.y = blocks, one block per workgroup, long blocks first.
 template <int HD>
 __global__ __launch_bounds__(kSplitThreads, 1) void prefill_split_kernel(const PrefillArgs a)
 {
@@ -962,8 +966,9 @@ __global__ __launch_bounds__(kSplitThreads, 1) void prefill_split_kernel(const P
     const uint32_t BP = 32 * (4 / Gw);
     const uint32_t nblk = (a.T + BP - 1) / BP;
     const uint32_t lo = blockIdx.y, hi = nblk - 1 - blockIdx.y;
+    const int passes = a.single ? 1 : 2;
 #pragma unroll 1
-    for (int pass = 0; pass < 2; pass++) {
+    for (int pass = 0; pass < passes; pass++) {
         if (pass) {
             if (hi == lo) break;
             __syncthreads();                              // LDS changes hands

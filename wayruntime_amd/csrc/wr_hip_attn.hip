@@ -406,15 +406,22 @@ int prefill_locked(wr_hip_kv* kv, uint32_t layer, uint32_t p0, uint32_t T, const
         const uint32_t Gw = G < 4 ? G : 4;
         const uint32_t BP = 32 * (4 / Gw);
         const uint32_t nblk = (T + BP - 1) / BP;
-        const uint32_t npairs = (nblk + 1) / 2, ny = kv->nkv * (G / Gw);
+        const uint32_t ny = kv->nkv * (G / Gw);
+        // A long and a short block per workgroup balance the causal triangle, but
+        // every block pays its own prologue and epilogue: when the pairs would
+        // not even give every CU a workgroup, one block per workgroup finishes
+        // with the longest block instead of with a pair's sum plus a second
+        // prologue and epilogue.
+        a.single = ((nblk + 1) / 2) * ny < 256 ? 1 : 0;
+        const uint32_t nwg = a.single ? nblk : (nblk + 1) / 2;
         if (hd == 64)
-            launch_main(prefill_split_kernel<64>, dim3(ny, npairs), dim3(kSplitThreads), a,
+            launch_main(prefill_split_kernel<64>, dim3(ny, nwg), dim3(kSplitThreads), a,
                         split_smem_bytes<64>());
         else if (hd == 128)
-            launch_main(prefill_split_kernel<128>, dim3(ny, npairs), dim3(kSplitThreads), a,
+            launch_main(prefill_split_kernel<128>, dim3(ny, nwg), dim3(kSplitThreads), a,
                         split_smem_bytes<128>());
         else   // 256: one wave per SIMD (the accumulators alone need 256 registers)
-            launch_main(prefill_mfma_kernel<256>, dim3(npairs, ny), dim3(kPrefillThreads), a);
+            launch_main(prefill_mfma_kernel<256>, dim3(nwg, ny), dim3(kPrefillThreads), a);
     } else {
         launch_main(prefill_generic_kernel, dim3(T, nq), dim3(kDecodeThreads), a);
     }
