@@ -107,13 +107,18 @@ def test_prefill_ignores_rows_that_were_never_appended():
     kv.close()
 
 
-@pytest.mark.parametrize("nq,nkv,theta,T", [(16, 8, 1e6, 2048), (32, 8, 5e5, 2048), (32, 8, 5e5, 4096)])
-def test_prefill_workload_sizes_after_rope_sampled_rows(nq, nkv, theta, T):
+@pytest.mark.parametrize("nq,nkv,theta,T,hd", [
+    (16, 8, 1e6, 2048, 128),        # Qwen3: one position block per workgroup (the pairs would not fill the chip)
+    (32, 8, 5e5, 2048, 128),        # Llama-3: a long and a short block per workgroup
+    (32, 8, 5e5, 4096, 128),
+    (32, 8, 5e5, 2048, 64),         # paired blocks at the other head dims
+    (32, 8, 5e5, 2048, 256),
+])
+def test_prefill_workload_sizes_after_rope_sampled_rows(nq, nkv, theta, T, hd):
     # the prefill workload: Q/K/V N(0,1), rotated (theta 1e6 Qwen3, 5e5 Llama-3),
     # appended to an empty cache; the CPU loop is quadratic, so the oracle checks a
     # spread of rows and properties cover the rest
-    hd = 128
-    print("prefill workload", nq, nkv, T, flush=True)
+    print("prefill workload", nq, nkv, T, hd, flush=True)
     kv, q, k16, v16 = _setup(nq, nkv, hd, 0, T, seed=synth.config_seed(4, nq + T % 97), theta=theta)
     got = kv.prefill(0, 0, q)
     assert not np.isnan(got).any()
