@@ -1,7 +1,7 @@
 """Builds the gfx950 shared library in-tree (``wayruntime_amd/libwr_hip_attn.so``).
 
     python -m wayruntime_amd.build            # compile
-    python -m wayruntime_amd.build --temps    # also keep ISA / resource usage under _work/temps
+    python -m wayruntime_amd.build --temps    # also keep ISA / resource usage under build/temps
 """
 from __future__ import annotations
 
@@ -25,7 +25,7 @@ HIPCC_FLAGS = [
 def build_hip(keep_temps: bool = False) -> str:
     cmd = ["hipcc"] + HIPCC_FLAGS
     if keep_temps:
-        tmp = os.path.join(ROOT, "_work", "temps")
+        tmp = os.path.join(ROOT, "build", "temps")
         os.makedirs(tmp, exist_ok=True)
         cmd += ["-save-temps=obj"]
     cmd += ["-o", HIP_SO, HIP_SRC]
@@ -39,7 +39,7 @@ def build_hip(keep_temps: bool = False) -> str:
     if keep_temps:
         for f in os.listdir(PKG):
             if f.startswith("wr_hip_attn-") or f.startswith("wr_hip_attn.hip-"):
-                os.replace(os.path.join(PKG, f), os.path.join(ROOT, "_work", "temps", f))
+                os.replace(os.path.join(PKG, f), os.path.join(ROOT, "build", "temps", f))
     return HIP_SO
 
 
