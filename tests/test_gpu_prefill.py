@@ -136,6 +136,25 @@ def test_prefill_workload_sizes_after_rope_sampled_rows(nq, nkv, theta, T, hd):
     kv.close()
 
 
+@pytest.mark.parametrize("nq,nkv,hd,p0,T,win", [
+    (32, 8, 128, 100, 2048, 500),   # a long and a short block per workgroup, behind a non-empty cache, windowed
+    (32, 8, 64, 37, 2048, 0),
+    (32, 8, 256, 64, 2048, 300),
+])
+def test_prefill_paired_blocks_with_offset_and_window_sampled_rows(nq, nkv, hd, p0, T, win):
+    # launches large enough for the paired form (256 workgroups and more), with
+    # the options the small cases above exercise on the one-block form
+    print("prefill paired", nq, nkv, hd, p0, T, win, flush=True)
+    kv, q, k16, v16 = _setup(nq, nkv, hd, p0, T, seed=4000 + hd + p0)
+    got = kv.prefill(0, p0, q, 0.0, win)
+    assert not np.isnan(got).any()
+    rows = sorted(set([0, 1, 30, 31, 32, 33, 63, 64, 65, 127, 128, 400, 500, 501, 1023, 1024, T // 2 + 17,
+                       T - 33, T - 32, T - 2, T - 1]))
+    want = oracle.causal_prefill(q, k16, v16, p0=p0, window=win, rows=rows, threads=8)
+    print("  errors", util.assert_close(got[rows], want[rows]), flush=True)
+    kv.close()
+
+
 def test_prefill_error_contract():
     lib = hipattn.lib()
     kv = hipattn.KVCache(1, 128, 8, 64)
