@@ -13,7 +13,9 @@ Prints ONE JSON line.  `value` is algorithmic K/V bytes per step divided by
 wall time per step (whole step: split-K kernel + combine).  `roofline` is for
 the split-K kernel alone, timed with per-launch events.  `cpu_baseline` is the
 CPU oracle (a bit-exact restatement of the reference op) on the same data, one
-core, on a bounded sample.  `prefill` reports causal prefill attention,
+core, on a bounded sample.  `prefill` reports causal prefill attention
+(the metric's T = 2048 launch checked against the oracle on sampled rows;
+`other_shapes`: the same launch timed at other head shapes and lengths),
 `projection` the row projections either side of the path: 16 rows
 (proj_rows_kernel, HBM-bound on the F16 weight bytes) and a 1024-row prefill
 pass (proj_gemm_lds_kernel, MFMA-bound); `end_to_end` the host engine on a
@@ -215,6 +217,31 @@ def main() -> None:
                    "max_abs_err_sampled_rows": perr}
         qp_dev.free()
         op_dev.free()
+        # the same launch at other head shapes and lengths (timing only: their
+        # parity is the GPU tests'), caches written directly as F16 bit patterns
+        others = []
+        for onq, onkv, ohd, oT in ((32, 8, 128, 4096), (16, 8, 128, 2048), (16, 8, 256, 2048), (32, 8, 128, 512)):
+            okv = hipattn.KVCache(1, ohd, onkv, oT)
+            rngp = np.random.default_rng(oT + ohd)
+            bits = rngp.integers(0x3000, 0x3C00, size=(2, oT, onkv, ohd), dtype=np.uint16)
+            bits |= (rngp.integers(0, 2, size=bits.shape, dtype=np.uint16) << 15)
+            okv.write_f16(0, 0, bits[0], bits[1])
+            oq = synth.normal(synth.config_seed(4, 2), (oT, onq, ohd))
+            oq_dev = hipattn.DeviceBuffer.from_host(oq)
+            oo_dev = hipattn.DeviceBuffer(oq.nbytes)
+            hipattn.prefill_dev(okv, 0, 0, oT, oq_dev, oo_dev, onq)
+            hipattn.profile_begin(reps)
+            for _ in range(reps):
+                hipattn.prefill_dev(okv, 0, 0, oT, oq_dev, oo_dev, onq)
+            oms, on = hipattn.profile_end()
+            o_avg = oms / max(on, 1)
+            otfl = 4.0 * onq * ohd * oT * (oT + 1) / 2.0 / (o_avg * 1e-3) / 1e12
+            others.append({"shape": f"{onq}/{onkv}/{ohd}", "T": oT, "ms": round(o_avg, 4), "tflops": round(otfl, 1),
+                           "frac_of_f16_mfma_peak": round(otfl / MFMA_F16_PEAK_TFLOPS, 4)})
+            oq_dev.free()
+            oo_dev.free()
+            okv.close()
+        prefill["other_shapes"] = others
 
     # ---- row projections either side of the attention path (secondary figure):
     # 16 rows through Llama-3-8B-sized F16 weights, HBM-bound on the weight
