@@ -199,6 +199,30 @@ int wr_hip_attn_prefill_dev(wr_hip_kv *kv, uint32_t layer, uint32_t p0,
                             uint32_t nq, float scale_override,
                             uint32_t window);
 
+/* wr_hip_attn_decode_batched_dev for callers that cannot allocate device
+ * memory (code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc).  It has no counterpart in the reference.  Same arguments,
+ * same kernels and the same results bit for bit; the difference is where the
+ * split-K tickets and partial rows live: in a fixed array of
+ * WR_HIP_NOALLOC_SCRATCH_BYTES that is part of the library's device image
+ * (every device the library runs on holds it until the process ends) instead
+ * of a buffer the library grows on demand.  The call makes no hipMalloc,
+ * hipFree or other allocating call.  Limits: nq <= WR_HIP_NOALLOC_MAX_HEADS,
+ * and n * nq * max_splits * (hd + 2) * 4 bytes of partials must fit the array
+ * behind its first 64 KiB (with the automatic split rule a session has at most
+ * 8 key splits: 16 sessions of 32 heads x 128 need 2.1 MB); beyond either,
+ * WR_HIP_ERR_LIMIT and nothing is launched.  All calls on one device share the
+ * array: the library's stream runs them one after the other, but a caller must
+ * not let two of them overlap on one device by other means (two processes'
+ * worth of streams replaying captured launches, say): they would race. */
+#define WR_HIP_NOALLOC_SCRATCH_BYTES (20u * 1024u * 1024u)
+#define WR_HIP_NOALLOC_MAX_HEADS     1024u
+int wr_hip_attn_decode_batched_dev_noalloc(uint32_t n, wr_hip_kv *const *kv,
+                                           uint32_t layer, const uint32_t *seq_k,
+                                           const float *q_dev, float *out_dev,
+                                           uint32_t nq, float scale_override,
+                                           uint32_t window);
+
 /* What this build of the library offers beyond the attention path proper
  * (bit mask).  A caller that wants the projections and row steps below on the
  * device checks WR_HIP_CAP_PROJ first and otherwise keeps them on the host. */

@@ -1,0 +1,137 @@
+"""The decode entry point that allocates nothing
+(wr_hip_attn_decode_batched_dev_noalloc) against the ordinary one
+(wr_hip_attn_decode_batched_dev), through the C ABI: same kernels, same key
+partition, so the outputs must be equal bit for bit; both are also checked
+against the CPU oracle (max-abs 2e-3, rel-L2 1e-3).  Two calls in a row share
+the fixed scratch array, the second with a smaller input."""
+import numpy as np
+import pytest
+
+from tests import util
+from wayruntime_amd import hipattn, synth
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _device():
+    hipattn.init()
+    yield
+    hipattn.set_tuning(0, False)
+
+
+def _sessions(seed, ctxs, nkv, hd):
+    caches, kvs = [], []
+    for i, ctx in enumerate(ctxs):
+        _a, _b, k16, v16 = util.make_kv(seed + 2 * i, int(ctx), nkv, hd)
+        kv = hipattn.KVCache(1, hd, nkv, int(ctx))
+        kv.write_f16(0, 0, k16, v16)
+        caches.append(kv)
+        kvs.append((k16, v16))
+    return caches, kvs
+
+
+def _both(caches, ctxs, q, nq, hd):
+    """Outputs of the ordinary and of the no-alloc entry point for one step."""
+    n = len(caches)
+    q_dev = hipattn.DeviceBuffer.from_host(q)
+    # the two outputs start from different garbage so that a launch that wrote
+    # nothing cannot pass
+    o_ref = hipattn.DeviceBuffer.from_host(np.full((n, nq, hd), 7.0, dtype=np.float32))
+    o_new = hipattn.DeviceBuffer.from_host(np.full((n, nq, hd), -9.0, dtype=np.float32))
+    hipattn.decode_batched_dev(caches, 0, ctxs, q_dev, o_ref, nq)
+    rc = hipattn.decode_batched_dev_noalloc(caches, 0, ctxs, q_dev, o_new, nq)
+    assert rc == hipattn.OK, rc
+    hipattn.sync()
+    ref = o_ref.to_host((n, nq, hd))
+    new = o_new.to_host((n, nq, hd))
+    for b in (q_dev, o_ref, o_new):
+        b.free()
+    return ref, new
+
+
+def test_no_alloc_decode_equals_the_ordinary_entry_point_twice_in_a_row():
+    nq, nkv, hd = 32, 8, 128
+    # first call: 16 ragged sessions, several key splits each (in-kernel merge
+    # through the scratch array); second call: fewer, shorter sessions, so the
+    # array still holds the first call's partials and tickets
+    ctx_a = [4096, 300, 2500, 1111, 4000, 257, 3333, 2048, 1025, 777, 3900, 1500, 2222, 640, 3071, 999]
+    ctx_b = [1000, 2000, 45]
+    caches, kvs = _sessions(7100, ctx_a, nkv, hd)
+    try:
+        for call, (idx, seed) in enumerate([(list(range(16)), 7200), ([3, 7, 5], 7300)]):
+            use = [caches[i] for i in idx]
+            ctxs = [ctx_a[i] for i in idx] if call == 0 else ctx_b
+            q = synth.normal(seed, (len(use), nq, hd))
+            print("no-alloc call", call, "ctx", ctxs, flush=True)
+            ref, new = _both(use, ctxs, q, nq, hd)
+            assert np.array_equal(ref, new), f"call {call}: outputs differ from the ordinary entry point"
+            for j, i in enumerate(idx):
+                want = util.oracle_decode(q[j], kvs[i][0], kvs[i][1], int(ctxs[j]))
+                util.assert_close(new[j], want, f"call {call} session {j}")
+    finally:
+        for kv in caches:
+            kv.close()
+
+
+def test_no_alloc_decode_with_the_finest_partition_and_a_window():
+    # 64 key splits per session (forced), head_dim 256, sliding window: the
+    # largest ticket / partial footprint per head, then a one-split call
+    nq, nkv, hd = 8, 4, 256
+    ctxs = [2048, 2048, 1999]
+    caches, kvs = _sessions(7400, ctxs, nkv, hd)
+    try:
+        hipattn.set_tuning(32, False)
+        q = synth.normal(7500, (3, nq, hd))
+        n = len(caches)
+        q_dev = hipattn.DeviceBuffer.from_host(q)
+        o_ref = hipattn.DeviceBuffer(q.nbytes)
+        o_new = hipattn.DeviceBuffer(q.nbytes)
+        hipattn.decode_batched_dev(caches, 0, ctxs, q_dev, o_ref, nq, 0.0, 1500)
+        assert hipattn.decode_batched_dev_noalloc(caches, 0, ctxs, q_dev, o_new, nq, 0.0, 1500) == hipattn.OK
+        hipattn.sync()
+        assert np.array_equal(o_ref.to_host((n, nq, hd)), o_new.to_host((n, nq, hd)))
+        hipattn.set_tuning(0, False)
+        small = [20, 31, 7]                     # one split each: no scratch use at all
+        hipattn.decode_batched_dev(caches, 0, small, q_dev, o_ref, nq)
+        assert hipattn.decode_batched_dev_noalloc(caches, 0, small, q_dev, o_new, nq) == hipattn.OK
+        hipattn.sync()
+        got = o_new.to_host((n, nq, hd))
+        assert np.array_equal(o_ref.to_host((n, nq, hd)), got)
+        for j in range(n):
+            util.assert_close(got[j], util.oracle_decode(q[j], kvs[j][0], kvs[j][1], small[j]),
+                              f"session {j}")
+        for b in (q_dev, o_ref, o_new):
+            b.free()
+    finally:
+        hipattn.set_tuning(0, False)
+        for kv in caches:
+            kv.close()
+
+
+def test_no_alloc_decode_refuses_what_does_not_fit():
+    # 16 sessions x 32 heads x 64 splits x (256 + 2) floats = 33.8 MB of partials:
+    # more than the fixed array; refused with WR_HIP_ERR_LIMIT, nothing launched,
+    # and the ordinary entry point still serves the same call
+    nq, nkv, hd, S = 32, 8, 256, 16
+    ctxs = [2048] * S
+    caches = [hipattn.KVCache(1, hd, nkv, 2048) for _ in range(S)]   # zero-filled caches
+    try:
+        hipattn.set_tuning(32, False)
+        q = synth.normal(7600, (S, nq, hd))
+        q_dev = hipattn.DeviceBuffer.from_host(q)
+        o_dev = hipattn.DeviceBuffer.from_host(np.full((S, nq, hd), 5.0, dtype=np.float32))
+        assert hipattn.decode_batched_dev_noalloc(caches, 0, ctxs, q_dev, o_dev, nq) == hipattn.ERR_LIMIT
+        hipattn.sync()
+        assert np.all(o_dev.to_host((S, nq, hd)) == 5.0)             # untouched
+        hipattn.decode_batched_dev(caches, 0, ctxs, q_dev, o_dev, nq)
+        hipattn.sync()
+        assert np.all(o_dev.to_host((S, nq, hd)) == 0.0)             # V is all zero
+        # more heads than the fixed ticket array holds
+        assert hipattn.decode_batched_dev_noalloc(caches[:1], 0, [8], q_dev, o_dev, 2048) == hipattn.ERR_LIMIT
+        q_dev.free()
+        o_dev.free()
+    finally:
+        hipattn.set_tuning(0, False)
+        for kv in caches:
+            kv.close()

@@ -28,6 +28,26 @@
 
 using namespace wr;
 
+// Scratch of wr_hip_attn_decode_batched_dev_noalloc, the one entry point that
+// allocates nothing: the split-K tickets (first kNoAllocTicketBytes) and the
+// partial rows (the rest).  Every device the library runs on holds its own copy
+// until the process ends.  In host code the array's name is only a stand-in: the
+// device address is asked for once per device at init (hipGetSymbolAddress) and
+// kept in Lib::noalloc_ws; host code uses that pointer, never the name.
+constexpr size_t kNoAllocTicketBytes = 64u * 1024u;            // 16 sessions x 1024 heads
+constexpr size_t kNoAllocScratchBytes = 20u * 1024u * 1024u;   // tickets + partials
+constexpr uint32_t kNoAllocMaxHeads = (uint32_t)(kNoAllocTicketBytes / sizeof(uint32_t) / WR_HIP_BATCH_MAX);
+constexpr int kMaxDevices = 16;
+static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
+
+// Clears n 32-bit words (tickets).  A kernel rather than a memset call so that a
+// caller may record the launch into a graph.
+__global__ void fill_u32_kernel(uint32_t* p, uint32_t n, uint32_t v)
+{
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = v;
+}
+
 struct wr_hip_weight {
     uint32_t n_out, n_in;
     void* tiles;                 // F16, tile order (kernels_proj.hip.h)
@@ -60,6 +80,7 @@ struct Lib {
     Buffer d_part;               // split-K partials
     Buffer d_proj;               // projection operand fragments and row scales
     uint32_t* d_counters = nullptr;   // split-K tickets, zero whenever no launch is in flight
+    unsigned char* noalloc_ws[kMaxDevices] = {};   // device address of `scratch`, per device
     Buffer h_pin;                // pinned host staging
     std::atomic<uint64_t> calls{0};
     wr_hip_log_fn log_fn = nullptr;
@@ -236,9 +257,17 @@ int check_append(const wr_hip_kv* kv, uint32_t layer, uint32_t pos, uint32_t n_r
     return WR_HIP_OK;
 }
 
+// Where a launch keeps its split-K tickets and partial rows: the library's own
+// growable buffers (ws == nullptr), or a fixed workspace that is never grown.
+struct DecodeWorkspace {
+    unsigned char* ws = nullptr;     // tickets at 0, partials from ticket_bytes on
+    size_t ticket_bytes = 0;
+    size_t bytes = 0;
+};
+
 int decode_locked(uint32_t n, wr_hip_kv* const* kv, uint32_t layer, const uint32_t* seq_k,
                   const float* q_dev, float* out_dev, uint32_t nq, float scale_override,
-                  uint32_t window)
+                  uint32_t window, const DecodeWorkspace& fixed = DecodeWorkspace())
 {
     const uint32_t hd = kv[0]->hd[layer], nkv = kv[0]->nkv;
     const uint32_t group = nq / nkv;
@@ -326,17 +355,36 @@ int decode_locked(uint32_t n, wr_hip_kv* const* kv, uint32_t layer, const uint32
     a.group = group;
     a.hd = hd;
     a.max_splits = max_splits;
-    a.counters = g.d_counters;
+    a.counters = fixed.ws ? reinterpret_cast<uint32_t*>(fixed.ws) : g.d_counters;
     const float scale = (scale_override > 0.0f) ? scale_override : 1.0f / sqrtf((float)hd);
     a.qscale = scale * kLog2e;
 
     if (max_splits > 1) {
         const size_t po = (size_t)n * nq * max_splits * hd * sizeof(float);
         const size_t pml = (size_t)n * nq * max_splits * 2 * sizeof(float);
-        int rc = ensure_device(g.d_part, po + pml);
-        if (rc) return rc;
-        a.part_o = reinterpret_cast<float*>(g.d_part.p);
-        a.part_ml = reinterpret_cast<float*>((uint8_t*)g.d_part.p + po);
+        uint8_t* base;
+        if (fixed.ws) {
+            if (fixed.ticket_bytes + po + pml > fixed.bytes) {
+                logmsg(0, "decode (no-alloc form): %zu bytes of split-K partials exceed the fixed "
+                          "workspace of %zu bytes (layer %u)", po + pml, fixed.bytes - fixed.ticket_bytes,
+                       layer);
+                return WR_HIP_ERR_LIMIT;
+            }
+            base = fixed.ws + fixed.ticket_bytes;
+        } else {
+            int rc = ensure_device(g.d_part, po + pml);
+            if (rc) return rc;
+            base = reinterpret_cast<uint8_t*>(g.d_part.p);
+        }
+        a.part_o = reinterpret_cast<float*>(base);
+        a.part_ml = reinterpret_cast<float*>(base + po);
+        if (fixed.ws) {
+            // the array keeps the last call's contents: the tickets this launch
+            // uses must start at zero
+            const uint32_t words = n * (use_mfma ? nkv : nq);
+            hipLaunchKernelGGL(fill_u32_kernel, dim3((words + 255) / 256), dim3(256), 0, g.stream,
+                               a.counters, words, 0u);
+        }
     }
 
     if (use_mfma) {
@@ -687,6 +735,20 @@ int wr_hip_attn_init(int device)
         if (e != hipSuccess) rc = hip_fail(e, "ticket array", 0);
     }
     if (rc == WR_HIP_OK) {
+        // device address of the no-alloc entry point's scratch array, once per
+        // device, with that device current
+        if (device >= kMaxDevices) {
+            rc = WR_HIP_ERR_LIMIT;
+        } else if (!g.noalloc_ws[device]) {
+            void* p = nullptr;
+            hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+            if (e != hipSuccess || !p)
+                rc = hip_fail(e, "address of the no-alloc scratch array", 0);
+            else
+                g.noalloc_ws[device] = reinterpret_cast<unsigned char*>(p);
+        }
+    }
+    if (rc == WR_HIP_OK) {
         // the two-waves-per-SIMD prefill kernels stage more than the 64 KiB a
         // kernel may use without asking
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(prefill_split_kernel<64>),
@@ -999,6 +1061,27 @@ int wr_hip_attn_decode_batched_dev(uint32_t n, wr_hip_kv* const* kv, uint32_t la
     if (rc) return rc;
     Locked lk;
     return decode_locked(n, kv, layer, seq_k, q_dev, out_dev, nq, scale_override, window);
+}
+
+int wr_hip_attn_decode_batched_dev_noalloc(uint32_t n, wr_hip_kv* const* kv, uint32_t layer,
+                                           const uint32_t* seq_k, const float* q_dev,
+                                           float* out_dev, uint32_t nq, float scale_override,
+                                           uint32_t window)
+{
+    int rc = check_decode(n, kv, layer, seq_k, q_dev, out_dev, nq);
+    if (rc) return rc;
+    if (nq > kNoAllocMaxHeads) {
+        logmsg(0, "decode (no-alloc form): %u query heads exceed the %u the fixed ticket array holds",
+               nq, kNoAllocMaxHeads);
+        return WR_HIP_ERR_LIMIT;
+    }
+    Locked lk;
+    DecodeWorkspace fixed;
+    fixed.ws = g.noalloc_ws[g.device];
+    fixed.ticket_bytes = kNoAllocTicketBytes;
+    fixed.bytes = kNoAllocScratchBytes;
+    if (!fixed.ws) return WR_HIP_ERR_STATE;
+    return decode_locked(n, kv, layer, seq_k, q_dev, out_dev, nq, scale_override, window, fixed);
 }
 
 int wr_hip_attn_decode_batched(uint32_t n, wr_hip_kv* const* kv, uint32_t layer,

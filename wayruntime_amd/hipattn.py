@@ -66,6 +66,9 @@ def load() -> C.CDLL:
         "wr_hip_attn_rope_dev": (C.c_int, [_vp, _vp, _u32, _u32, _u32, _u32]),
         "wr_hip_attn_decode_batched_dev": (C.c_int, [_u32, C.POINTER(_vp), _u32, C.POINTER(_u32),
                                                      _vp, _vp, _u32, C.c_float, _u32]),
+        "wr_hip_attn_decode_batched_dev_noalloc": (C.c_int, [_u32, C.POINTER(_vp), _u32,
+                                                             C.POINTER(_u32), _vp, _vp, _u32,
+                                                             C.c_float, _u32]),
         "wr_hip_attn_prefill_dev": (C.c_int, [_vp, _u32, _u32, _u32, _vp, _vp, _u32, C.c_float,
                                               _u32]),
         "wr_hip_proj_weight_create": (C.c_int, [_u32, C.POINTER(_vp), C.POINTER(_u32), _u32,
@@ -275,6 +278,17 @@ def decode_batched_dev(caches, layer: int, seq_k, q_dev: DeviceBuffer, out_dev: 
     sk = (_u32 * n)(*[int(s) for s in seq_k])
     _check(lib().wr_hip_attn_decode_batched_dev(n, kvp, layer, sk, q_dev.p, out_dev.p, nq,
                                                 scale_override, window), "decode_batched_dev")
+
+
+def decode_batched_dev_noalloc(caches, layer: int, seq_k, q_dev: DeviceBuffer,
+                               out_dev: DeviceBuffer, nq: int, scale_override: float = 0.0,
+                               window: int = 0) -> int:
+    """The form that allocates nothing; returns the wr_status."""
+    n = len(caches)
+    kvp = (_vp * n)(*[c.h for c in caches])
+    sk = (_u32 * n)(*[int(s) for s in seq_k])
+    return lib().wr_hip_attn_decode_batched_dev_noalloc(n, kvp, layer, sk, q_dev.p, out_dev.p, nq,
+                                                        scale_override, window)
 
 
 def prefill_dev(cache: KVCache, layer: int, p0: int, T: int, q_dev: DeviceBuffer,
