@@ -16,7 +16,10 @@ CPU oracle (a bit-exact restatement of the reference op) on the same data, one
 core, on a bounded sample.  `prefill` reports causal prefill attention
 (the metric's T = 2048 launch checked against the oracle on sampled rows;
 `other_shapes`: the same launch timed at other head shapes and lengths),
-`projection` the row projections either side of the path: 16 rows
+`decode_configs` the other decode workloads (16 ragged sessions, 16 x 32768 at
+both long-context head shapes, one session at 128 / 512 / 2048 / 8192 keys),
+each with its kernel time, rate, fraction of the HBM peak and an oracle check of
+one session; `projection` the row projections either side of the path: 16 rows
 (proj_rows_kernel, HBM-bound on the F16 weight bytes) and a 1024-row prefill
 pass (proj_gemm_lds_kernel, MFMA-bound); `end_to_end` the host engine on a
 random-init Qwen3-0.6B-shaped model (python -m wayruntime_amd.e2e_timing in a
@@ -38,14 +41,31 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0           # MI355X HBM3E
 MFMA_F16_PEAK_TFLOPS = 2500.0   # MI355X dense f16
 
-# HBM bytes one launch of decode_mfma_kernel<128> moves on the default workload
-# (16 sessions x 4096 ctx): rocprofv3 FETCH_SIZE + WRITE_SIZE per dispatch, each
-# scaled by what the same counter reads for a plain 256 MiB copy kernel
-# (FETCH_SIZE x 1.99985 KiB, WRITE_SIZE x 1.00000 KiB).  Counters cannot be read
-# from inside this process, so the figure is carried here from the committed
-# counter summary (profiles/decode_prefill_traffic_pmc.txt) and reported only
-# for the workload it was measured on.
-PMC_TRAFFIC_BYTES = {(16, 4096): 270032800 + 1462272}
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "decode_prefill_traffic_pmc.txt")
+DECODE_KERNEL_SRC = os.path.join(ROOT, "wayruntime_amd", "csrc", "kernels_decode.hip.h")
+
+
+def pmc_traffic_bytes(sessions: int, ctx: int):
+    """HBM bytes one launch of the decode kernel moves on the default workload:
+    rocprofv3 FETCH_SIZE + WRITE_SIZE per dispatch, each scaled by what the same
+    counter reads for a plain copy kernel of known size.  Counters cannot be read
+    from inside this process, so the figure is read from the committed counter
+    summary, which names the workload and the SHA-1 of the kernel source it was
+    measured on (line `bench.traffic decode SxCTX fetch_bytes=.. write_bytes=..
+    kernel_sha1=..`).  Another workload, or a kernel source that has changed
+    since, gives None rather than a stale number."""
+    import hashlib
+    try:
+        sha = hashlib.sha1(open(DECODE_KERNEL_SRC, "rb").read()).hexdigest()
+        for ln in open(TRAFFIC_PROFILE):
+            f = ln.split()
+            if len(f) >= 6 and f[0] == "bench.traffic" and f[1] == "decode" and f[2] == "%dx%d" % (sessions, ctx):
+                kv = dict(x.split("=", 1) for x in f[3:])
+                if kv.get("kernel_sha1") == sha:
+                    return int(kv["fetch_bytes"]) + int(kv["write_bytes"])
+    except (OSError, ValueError, KeyError):
+        pass
+    return None
 
 
 def pooled16(pool16: np.ndarray, salt: int, n: int) -> np.ndarray:
@@ -62,6 +82,113 @@ def pooled16(pool16: np.ndarray, salt: int, n: int) -> np.ndarray:
     return x
 
 
+def batch1_rotation(ctx: int):
+    """(layers, replicas) for a one-session workload of `ctx` keys (4096 bytes per
+    key): enough distinct copies that the working set passes 600 MB."""
+    layers = 64
+    per_cache = 4096 * ctx * layers
+    return layers, max(1, -(-600_000_000 // per_cache))
+
+
+class _Off:                                         # device pointer at an offset
+    def __init__(self, p):
+        self.p = p
+
+
+class DecodeWorkload:
+    """S sessions of one head shape with the given context lengths, resident in
+    HBM.  `replicas` independent copies of the session set with `layers` cache
+    layers each are walked by successive steps, so that the bytes a step reads
+    were last touched (replicas x layers) steps ago and cannot sit in the
+    last-level cache (256 MB)."""
+
+    def __init__(self, hipattn, synth, pool16, nq, nkv, hd, ctxs, layers, replicas=1, keep_host="first"):
+        self.h, self.nq, self.nkv, self.hd = hipattn, nq, nkv, hd
+        self.ctxs, self.L, self.R, self.S = list(ctxs), layers, replicas, len(ctxs)
+        row = nkv * hd
+        self.caches, self.host_kv = [], {}
+        for r in range(replicas):
+            group = []
+            for s_i, c in enumerate(self.ctxs):
+                kv = hipattn.KVCache(layers, hd, nkv, c)
+                for layer in range(layers):
+                    salt = 2 * ((r * self.S + s_i) * layers + layer)
+                    k16 = pooled16(pool16, 1 + salt, c * row).reshape(c, nkv, hd)
+                    v16 = pooled16(pool16, 2 + salt, c * row).reshape(c, nkv, hd)
+                    kv.write_f16(layer, 0, k16, v16)
+                    if r == 0 and layer == 0 and (s_i == 0 or keep_host == "all"):
+                        self.host_kv[s_i] = (k16, v16)
+                group.append(kv)
+            self.caches.append(group)
+        self.q_host = synth.normal(synth.config_seed(3, 1), (layers, self.S, nq, hd))
+        self.q_dev = hipattn.DeviceBuffer.from_host(self.q_host)
+        self.out_dev = hipattn.DeviceBuffer(self.S * nq * hd * 4)
+        self.step_q_bytes = self.S * nq * hd * 4
+        self.bytes_per_step = 2 * 2 * nkv * hd * sum(self.ctxs)      # K and V, two bytes each
+
+    def step(self, i: int) -> None:
+        group = self.caches[i % self.R]
+        layer = (i // self.R) % self.L
+        self.h.decode_batched_dev(group, layer, self.ctxs, _Off(self.q_dev.p + layer * self.step_q_bytes),
+                                  self.out_dev, self.nq)
+
+    def check(self, oracle):
+        """Session 0, layer 0 of replica 0 against the oracle: (max_abs, rel_l2)."""
+        self.step(0)
+        self.h.sync()
+        got = self.out_dev.to_host((self.S, self.nq, self.hd))
+        k16, v16 = self.host_kv[0]
+        want0 = oracle.attention(self.q_host[0, 0][None], k16, v16)[0]
+        return (float(np.max(np.abs(got[0] - want0))),
+                float(np.linalg.norm(got[0] - want0) / np.linalg.norm(want0)))
+
+    def time_steps(self, steps: int, warmup: int) -> float:
+        """ms per step, wall clock around `steps` launches (stream drained on both sides)."""
+        for i in range(warmup):
+            self.step(i)
+        self.h.sync()
+        t = time.perf_counter()
+        for i in range(steps):
+            self.step(i)
+        self.h.sync()
+        return (time.perf_counter() - t) * 1e3 / steps
+
+    def time_kernel(self, n: int) -> float:
+        """mean duration (ms) of the split-K kernel alone, per-launch events on the library stream"""
+        self.h.profile_begin(n)
+        for i in range(n):
+            self.step(i)
+        ms, timed = self.h.profile_end()
+        return ms / max(timed, 1)
+
+    def close(self):
+        for group in self.caches:
+            for kv in group:
+                kv.close()
+        self.q_dev.free()
+        self.out_dev.free()
+
+
+def decode_config(hipattn, synth, oracle, pool16, name, nq, nkv, hd, ctxs, layers, replicas, steps, warmup):
+    """One secondary decode workload: kernel time, rate, fraction of peak, oracle check."""
+    w = DecodeWorkload(hipattn, synth, pool16, nq, nkv, hd, ctxs, layers, replicas)
+    try:
+        max_abs, rel_l2 = w.check(oracle)
+        ok = max_abs <= 2e-3 and rel_l2 <= 1e-3
+        ms = w.time_steps(steps, warmup)
+        kern_ms = w.time_kernel(min(steps, 256))
+        gbs = w.bytes_per_step / (kern_ms * 1e-3) / 1e9
+        return {"workload": name, "shape": "%d/%d/%d" % (nq, nkv, hd), "sessions": len(ctxs),
+                "ctx": ctxs[0] if len(set(ctxs)) == 1 else [min(ctxs), max(ctxs)],
+                "bytes_per_launch": w.bytes_per_step, "kernel_us": round(kern_ms * 1e3, 2),
+                "GB/s": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
+                "wall_us_per_step": round(ms * 1e3, 2),
+                "working_set_MB": round(w.bytes_per_step * layers * replicas / 1e6, 1),
+                "check_session0": {"max_abs": max_abs, "rel_l2": rel_l2, "ok": ok}}
+    finally:
+        w.close()
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -76,14 +203,16 @@ def main() -> None:
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-proj", action="store_true")
     ap.add_argument("--no-e2e", action="store_true")
+    ap.add_argument("--no-decode-configs", action="store_true")
     ap.add_argument("--keys-per-wg", type=int, default=0)
     ap.add_argument("--workload", default="headline",
                     choices=["headline", "ragged16", "long16", "long16-hd256", "batch1"],
-                    help="headline: 16 sessions x --ctx, 32/8/128 (the metric's configuration); "
+                    help="headline: 16 sessions x --ctx, 32/8/128 (the metric's configuration), with "
+                         "the other decode workloads as secondary keys; "
                          "ragged16: 16 sessions with contexts drawn from [256, 4096]; "
                          "long16 / long16-hd256: 16 sessions x 32768 at 32/8/128 / 8/4/256; "
                          "batch1: one session, 16/8/128, --ctx keys.  Other than headline they "
-                         "report the decode figures only")
+                         "run that one workload as the timed steps and report the decode figures only")
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -95,7 +224,7 @@ def main() -> None:
 
     hipattn.init(0)
     nq, nkv, hd = 32, 8, 128
-    S, ctx, L = args.sessions, args.ctx, args.layers
+    S, ctx, L, R = args.sessions, args.ctx, args.layers, 1
     ctxs = None
     if args.workload == "ragged16":
         S = 16
@@ -105,90 +234,45 @@ def main() -> None:
         if args.workload == "long16-hd256":
             nq, nkv, hd = 8, 4, 256
     elif args.workload == "batch1":
-        nq, S, L = 16, 1, max(L, 16)
+        nq, S = 16, 1
+        L, R = batch1_rotation(ctx)
     if ctxs is None:
         ctxs = [ctx] * S
     secondary = args.workload != "headline"
     if secondary:
-        args.no_prefill = args.no_proj = args.no_e2e = True
+        args.no_prefill = args.no_proj = args.no_e2e = args.no_decode_configs = True
         args.cpu_seconds = 0.0
-    row = nkv * hd
 
     t0 = time.time()
     pool16 = synth.f32_to_f16_trunc(synth.normal(synth.config_seed(3, 0), (1 << 24,)))
-    caches = []
-    host_kv = {}                                    # (session) -> (k16, v16) of layer 0, for checks
-    for s in range(S):
-        c = ctxs[s]
-        kv = hipattn.KVCache(L, hd, nkv, c)
-        for layer in range(L):
-            k16 = pooled16(pool16, 1 + 2 * (s * L + layer), c * row)
-            v16 = pooled16(pool16, 2 + 2 * (s * L + layer), c * row)
-            k16 = k16.reshape(c, nkv, hd)
-            v16 = v16.reshape(c, nkv, hd)
-            kv.write_f16(layer, 0, k16, v16)
-            if layer == 0 and s == 0:
-                host_kv[s] = (k16, v16)
-            elif layer == 0 and not secondary:
-                host_kv[s] = (k16, v16)
-        caches.append(kv)
-    q_host = synth.normal(synth.config_seed(3, 1), (L, S, nq, hd))
-    q_dev = hipattn.DeviceBuffer.from_host(q_host)
-    out_dev = hipattn.DeviceBuffer(S * nq * hd * 4)
-    seq_k = list(ctxs)
-    step_q_bytes = S * nq * hd * 4
+    work = DecodeWorkload(hipattn, synth, pool16, nq, nkv, hd, ctxs, L, R,
+                          keep_host="first" if secondary else "all")
+    caches, host_kv, q_host = work.caches[0], work.host_kv, work.q_host
     setup_s = time.time() - t0
 
     if args.keys_per_wg:
         hipattn.set_tuning(args.keys_per_wg, False)
 
-    class _Off:                                     # device pointer at an offset
-        def __init__(self, p):
-            self.p = p
-
-    def step(i: int) -> None:
-        layer = i % L
-        hipattn.decode_batched_dev(caches, layer, seq_k, _Off(q_dev.p + layer * step_q_bytes),
-                                   out_dev, nq)
-
     # ---- correctness of what is being timed: session 0, layer 0 vs the oracle
     import oracle
     oracle.set_attn_max_seq(1 << 20)
-    step(0)
-    hipattn.sync()
-    got = out_dev.to_host((S, nq, hd))
-    want0 = oracle.attention(q_host[0, 0][None], host_kv[0][0], host_kv[0][1])[0]
-    max_abs = float(np.max(np.abs(got[0] - want0)))
-    rel_l2 = float(np.linalg.norm(got[0] - want0) / np.linalg.norm(want0))
+    max_abs, rel_l2 = work.check(oracle)
     if not (max_abs <= 2e-3 and rel_l2 <= 1e-3):
         print("bench.py: device output outside tolerance: max_abs=%g rel_l2=%g" % (max_abs, rel_l2),
               file=sys.stderr)
         sys.exit(1)
 
     # ---- timed region
-    for i in range(args.warmup):
-        step(i)
-    hipattn.sync()
-    t = time.perf_counter()
-    for i in range(args.steps):
-        step(i)
-    hipattn.sync()
-    wall = time.perf_counter() - t
-    ms_per_step = wall * 1e3 / args.steps
-    bytes_per_step = 2 * 2 * nkv * hd * sum(ctxs)            # K and V, two bytes each
+    ms_per_step = work.time_steps(args.steps, args.warmup)
+    bytes_per_step = work.bytes_per_step
     value = bytes_per_step / (ms_per_step * 1e-3) / 1e9
 
     # ---- dominant kernel alone, per-launch events
-    n_prof = min(args.steps, 512)
-    hipattn.profile_begin(n_prof)
-    for i in range(n_prof):
-        step(i)
-    kern_ms, n_timed = hipattn.profile_end()
-    kern_avg_ms = kern_ms / max(n_timed, 1)
+    kern_avg_ms = work.time_kernel(min(max(args.steps, 100), 512))
     achieved = bytes_per_step / (kern_avg_ms * 1e-3) / 1e9
     roofline = {"bound": "hbm", "kernel": "decode_mfma_kernel<%d>" % hd, "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                "traffic": PMC_TRAFFIC_BYTES.get((S, ctx)) if not secondary else None,
+                "traffic": pmc_traffic_bytes(S, ctx) if not secondary and len(set(ctxs)) == 1 else None,
                 "kernel_avg_us": round(kern_avg_ms * 1e3, 2),
                 "bytes_per_launch": bytes_per_step}
 
@@ -364,6 +448,28 @@ def main() -> None:
                                     "sample": "%d threads x %d calls, %.1f s" % (n_thr, rounds, t_par)},
                "host": "%s, %d cpus visible" % (cpu_model, os.cpu_count() or 0)}
 
+    # ---- the other decode workloads (secondary figures): same timing code as the
+    # headline, fewer steps; each checks session 0 against the oracle first
+    decode_configs = None
+    if not args.no_decode_configs:
+        work.close()
+        caches = []
+        decode_configs = []
+        sec_steps, sec_warm = 60, 10
+        ragged = [int(c) for c in synth.ragged_contexts(synth.config_seed(3, 0), 16, 256, 4096)]
+        specs = [("ragged16", 32, 8, 128, ragged, 8, 1),
+                 ("long16", 32, 8, 128, [32768] * 16, 2, 1),
+                 ("long16-hd256", 8, 4, 256, [32768] * 16, 2, 1)]
+        for c1 in (128, 512, 2048, 8192):
+            l1, r1 = batch1_rotation(c1)
+            specs.append(("batch1-ctx%d" % c1, 16, 8, 128, [c1], l1, r1))
+        for name, cnq, cnkv, chd, cctx, cl, cr in specs:
+            try:
+                decode_configs.append(decode_config(hipattn, synth, oracle, pool16, name, cnq, cnkv, chd,
+                                                    cctx, cl, cr, sec_steps, sec_warm))
+            except Exception as exc:                  # reported, not fatal to the headline line
+                decode_configs.append({"workload": name, "error": repr(exc)[:200]})
+
     # ---- the host engine end to end on a random-init Qwen3-0.6B-shaped model
     # (secondary figures): a child process, so this process's device state and
     # the engine's do not meet.  A failure is reported, not fatal.
@@ -393,14 +499,15 @@ def main() -> None:
                                                       args.workload, L)),
                    "sessions": S, "ctx": ctx if len(set(ctxs)) == 1 else ctxs, "layers": L},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
-        "roofline": roofline, "cpu_baseline": cpu, "prefill": prefill, "projection": proj,
+        "roofline": roofline, "cpu_baseline": cpu, "prefill": prefill, "decode_configs": decode_configs,
+        "projection": proj,
         "end_to_end": e2e,
         "check": {"max_abs": max_abs, "rel_l2": rel_l2},
         "device": hipattn.device_name(), "setup_s": round(setup_s, 1),
     }
     print(json.dumps(line), flush=True)
-    for kv in caches:
-        kv.close()
+    if caches:
+        work.close()
 
 
 if __name__ == "__main__":

@@ -23,6 +23,19 @@ struct wr_hip_kv {
 
 static int g_inited;
 static uint64_t g_calls;
+/* Test hook: the k-th attention call from now (1 = the next one) does its work
+ * and then reports WR_HIP_ERR_INTERNAL, the way the device library reports a
+ * kernel that gave up a bounded wait: found at the wait that ends the call,
+ * after the outputs have been written with data that cannot be trusted. */
+static int g_late_error_in;
+
+void wr_hip_attn_debug_late_error_in(int k) { g_late_error_in = k; }
+
+static int late_error(void)
+{
+    if (g_late_error_in > 0 && --g_late_error_in == 0) return WR_HIP_ERR_INTERNAL;
+    return WR_HIP_OK;
+}
 
 int wr_hip_attn_init(int device)
 {
@@ -169,12 +182,12 @@ int wr_hip_attn_decode(wr_hip_kv *kv, uint32_t layer, uint32_t seq_k, const floa
 {
     if (!g_inited) return WR_HIP_ERR_STATE;
     if (!kv || !q || !out) return WR_HIP_ERR_INVAL;
+    g_calls++;                 /* counted before the shape checks (src/core/kernels.c:1423) */
     int rc = check_decode(kv, layer, seq_k, nq);
     if (rc) return rc;
     wro_attention_f16kv(q, kv->k[layer], kv->v[layer], out, 1, nq, kv->nkv, kv->hd[layer], seq_k,
                         scale_override, window);
-    g_calls++;
-    return WR_HIP_OK;
+    return late_error();
 }
 
 int wr_hip_attn_decode_batched(uint32_t n, wr_hip_kv *const *kv, uint32_t layer,
@@ -184,32 +197,34 @@ int wr_hip_attn_decode_batched(uint32_t n, wr_hip_kv *const *kv, uint32_t layer,
     if (!g_inited) return WR_HIP_ERR_STATE;
     if (!kv || !seq_k || !q || !out) return WR_HIP_ERR_INVAL;
     if (n == 0 || n > WR_HIP_BATCH_MAX) return WR_HIP_ERR_LIMIT;
+    for (uint32_t i = 0; i < n; i++)
+        if (!kv[i]) return WR_HIP_ERR_INVAL;
+    g_calls += n;
     for (uint32_t i = 0; i < n; i++) {
         int rc = check_decode(kv[i], layer, seq_k[i], nq);
         if (rc) return rc;
         for (uint32_t j = 0; j < i; j++)
             if (kv[i] == kv[j]) return WR_HIP_ERR_INVAL;
     }
-    for (uint32_t i = 0; i < n; i++) {
+    for (uint32_t i = 0; i < n; i++)
         wro_attention_f16kv(q[i], kv[i]->k[layer], kv[i]->v[layer], out[i], 1, nq, kv[i]->nkv,
                             kv[i]->hd[layer], seq_k[i], scale_override, window);
-        g_calls++;
-    }
-    return WR_HIP_OK;
+    return late_error();
 }
 
 int wr_hip_attn_prefill(wr_hip_kv *kv, uint32_t layer, uint32_t p0, uint32_t T, const float *q,
                         float *out, uint32_t nq, float scale_override, uint32_t window)
 {
     if (!g_inited) return WR_HIP_ERR_STATE;
-    if (!layer_ok(kv, layer) || !q || !out || T == 0) return WR_HIP_ERR_INVAL;
+    if (!kv || !q || !out) return WR_HIP_ERR_INVAL;
+    g_calls += T;
+    if (!layer_ok(kv, layer) || T == 0) return WR_HIP_ERR_INVAL;
     if (nq == 0 || nq % kv->nkv) return WR_HIP_ERR_INVAL;
     if ((uint64_t)p0 + T > WR_HIP_ATTN_MAX_SEQ) return WR_HIP_ERR_LIMIT;
     if ((uint64_t)p0 + T > kv->max_ctx) return WR_HIP_ERR_INVAL;
     wro_causal_prefill(q, kv->k[layer], kv->v[layer], out, p0, T, nq, kv->nkv, kv->hd[layer],
                        scale_override, window);
-    g_calls += T;
-    return WR_HIP_OK;
+    return late_error();
 }
 
 /* ---- not offered by the test double -----------------------------------------

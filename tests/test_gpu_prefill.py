@@ -136,6 +136,28 @@ def test_prefill_workload_sizes_after_rope_sampled_rows(nq, nkv, theta, T, hd):
     kv.close()
 
 
+@pytest.mark.parametrize("nq,nkv,theta,T", [
+    (32, 8, 5e5, 2048),             # Llama-3: the paired-block launch form
+    (16, 8, 1e6, 2048),             # Qwen3: the one-block-per-workgroup form
+    (16, 8, 1e6, 4096),             # Qwen3 at the longest chunk of the workload
+])
+def test_prefill_workload_sizes_after_rope_every_row(nq, nkv, theta, T):
+    # the prefill workload at full size with EVERY row checked against the serial
+    # stepping oracle (rows spread over 16 host threads): a wrong row anywhere in
+    # either launch form cannot hide between samples
+    hd = 128
+    print("prefill workload, all rows", nq, nkv, T, flush=True)
+    kv, q, k16, v16 = _setup(nq, nkv, hd, 0, T, seed=synth.config_seed(4, 50 + nq + T % 97), theta=theta)
+    got = kv.prefill(0, 0, q)
+    assert not np.isnan(got).any()
+    want = oracle.causal_prefill(q, k16, v16, threads=16)
+    print("  errors over all rows", util.assert_close(got, want), flush=True)
+    # per row as well: one bad row must not drown in the aggregate norm
+    err = np.max(np.abs(got - want).reshape(T, -1), axis=1)
+    assert float(err.max()) <= util.MAX_ABS, (int(err.argmax()), float(err.max()))
+    kv.close()
+
+
 @pytest.mark.parametrize("nq,nkv,hd,p0,T,win", [
     (32, 8, 128, 100, 2048, 500),   # a long and a short block per workgroup, behind a non-empty cache, windowed
     (32, 8, 64, 37, 2048, 0),
@@ -165,7 +187,13 @@ def test_prefill_error_contract():
     assert pre(0, 0) == hipattn.ERR_INVAL
     assert pre(62, 4) == hipattn.ERR_INVAL                 # runs past the allocation
     assert pre(hipattn.ATTN_MAX_SEQ, 4) == hipattn.ERR_LIMIT
+    calls = lib.wr_hip_attn_calls()
     assert pre(0, 4, nq=12) == hipattn.ERR_INVAL
+    # refused for its shape, yet counted: the reference counts each of the four
+    # calls before it looks at shapes (kernels.c:1418-1423)
+    assert lib.wr_hip_attn_calls() == calls + 4
+    assert lib.wr_hip_attn_prefill(kv.h, 0, 0, 4, None, out.ctypes.data, 16, 0.0, 0) == hipattn.ERR_INVAL
+    assert lib.wr_hip_attn_calls() == calls + 4            # a null pointer is refused before the count
     calls = lib.wr_hip_attn_calls()
     assert pre(0, 4) == hipattn.OK
     assert lib.wr_hip_attn_calls() == calls + 4            # one per token, as the serial loop counts

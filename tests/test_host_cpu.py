@@ -3,6 +3,7 @@ the C11 host engine linked against an oracle-backed stand-in for the device
 library).  Covers what needs no GPU: the GGUF loader, the greedy token stream of
 a toy model against the compiled reference's golden stream, context limits,
 all-or-nothing rollback, batched == serial, and the error contract."""
+import ctypes as C
 import os
 import struct
 
@@ -116,6 +117,37 @@ def test_injected_attention_failure_rolls_back(eng, model):
     assert twin.prefill([2, 6]) == 2 and s.prefill([2, 6]) == 2
     assert np.array_equal(s.step(1), twin.step(1))
     s.close(); twin.close()
+
+
+def test_device_error_found_after_the_work_rolls_back(eng, model):
+    # The device library finds a kernel's expired bounded wait only at the wait
+    # that ends a call: the outputs are already written (with data that cannot be
+    # trusted) when the call returns WR_HIP_ERR_INTERNAL.  The test double plays
+    # that: the k-th attention call from now does its work, then fails.  The
+    # session must consume nothing, report WR_ERR_INTERNAL, and a retry must
+    # equal an undisturbed twin, for a step, a prefill and a batched step.
+    late = eng.lib.wr_hip_attn_debug_late_error_in
+    late.argtypes, late.restype = [C.c_int], None
+    s, twin = model.session(32), model.session(32)
+    for sess in (s, twin):
+        assert sess.prefill([3, 1, 4, 1, 5]) == 5
+    late(TINY.n_layers)                                         # the last layer's call of this step
+    assert s.step(9) is None
+    assert s.status == E.WR_ERR_INTERNAL and s.pos == 5
+    assert np.array_equal(s.step(9), twin.step(9))
+    late(1)                                                     # the first layer's call of a prefill
+    assert s.prefill([2, 6, 7]) == E.WR_ERR_INTERNAL and s.pos == 6
+    assert twin.prefill([2, 6, 7]) == 3 and s.prefill([2, 6, 7]) == 3
+    other, other_twin = model.session(16), model.session(16)
+    late(2)                                                     # second layer of a batched step
+    assert E.batch_step([s, other], [1, 2])[0] == E.WR_ERR_INTERNAL
+    assert (s.pos, other.pos) == (9, 0)
+    n, logits = E.batch_step([s, other], [1, 2])
+    assert n == 2
+    assert np.array_equal(logits[0], twin.step(1)) and np.array_equal(logits[1], other_twin.step(2))
+    late(0)
+    for x in (s, twin, other, other_twin):
+        x.close()
 
 
 def test_batched_step_equals_serial_steps_bit_for_bit(model):

@@ -113,6 +113,9 @@ static_assert(sizeof(DecodeArgs::items) == kBatchMax * kMaxSplits * sizeof(uint1
 // s_waitcnt vmcnt(0)) and a workgroup barrier before one thread takes the
 // ticket.  A device-wide release fence instead would write back the whole L2
 // (buffer_wbl2) from every workgroup: measured at 5-10x the kernel's run time.
+#if defined(__HIP_DEVICE_COMPILE__) && !defined(__gfx950__)
+#error "the cross-workgroup exchange below relies on how gfx950 executes agent-scope relaxed atomics (sc1 write-through stores, L2-coherent loads); it has not been argued for any other target"
+#endif
 __device__ __forceinline__ float part_load(const float* p)
 {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

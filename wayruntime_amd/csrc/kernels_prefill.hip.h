@@ -19,7 +19,14 @@ struct PrefillArgs {
     uint32_t p0, T, nq, nkv, group, hd, ctx_pad, window;
     float qscale;            // softmax scale * log2(e)
     uint32_t single;         // MFMA kernels: one position block per workgroup (grid = blocks) instead of a pair
+    uint32_t* err;           // error word (host memory the device can write); see set_barrier
+    uint32_t err_code;       // what to store there: kDevErrWaitExpired | layer
 };
+
+// Layout of the error word a kernel leaves for the host when it gives up a
+// bounded wait: bit 31 set, the layer in the low bits.
+constexpr uint32_t kDevErrWaitExpired = 0x80000000u;
+constexpr uint32_t kDevErrLayerMask = 0x0000FFFFu;
 
 // Any head_dim / group: one workgroup per (row, head), vector ALU only.
 __global__ __launch_bounds__(kDecodeThreads) void prefill_generic_kernel(const PrefillArgs a)
@@ -551,20 +558,27 @@ __device__ __forceinline__ void split_move(const SplitCtx<HD>& cx, uint32_t j, i
 // Barrier among the four waves of one set: every wave adds one to the set's
 // counter in LDS and waits until it has reached `target` (4 x the number of
 // barriers so far; the counter is never reset inside a block).  The wait is
-// bounded: should a wave never arrive, the others go on (with wrong data)
-// instead of hanging the device.
+// bounded: should a wave never arrive, the others go on instead of hanging the
+// device, with wrong data, and say so: lane 0 stores `err_code` in the error
+// word, which the host finds at its next wait for the stream and turns into an
+// error status for the caller.
 __device__ __forceinline__ void set_barrier(unsigned char* smem, uint32_t cnt_off, uint32_t target,
-                                            int lane)
+                                            int lane, uint32_t* err, uint32_t err_code)
 {
     uint32_t* cnt = reinterpret_cast<uint32_t*>(smem + cnt_off);
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     if (lane == 0) __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    bool arrived = false;
     for (uint32_t spins = 0; spins < (1u << 22); spins++) {
         const uint32_t seen = (uint32_t)__builtin_amdgcn_readfirstlane(
             __hip_atomic_load(cnt, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP));
-        if ((int32_t)(seen - target) >= 0) break;
+        if ((int32_t)(seen - target) >= 0) {
+            arrived = true;
+            break;
+        }
         __builtin_amdgcn_s_sleep(1);
     }
+    if (!arrived && lane == 0) *err = err_code;
     asm volatile("" ::: "memory");
 }
 
@@ -879,12 +893,12 @@ __device__ __forceinline__ void split_block(const PrefillArgs& a, unsigned char*
     for (uint32_t j = 0;; j += 2) {
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * L::NL) : "memory");
         split_patch_tail<HD>(smem, cx, j, sub, lane);
-        set_barrier(smem, cx.cnt, 4 * (j + 1), lane);
+        set_barrier(smem, cx.cnt, 4 * (j + 1), lane, a.err, a.err_code);
         split_wave_step<HD>(R, negm, s0, s1, smem, cx, j, wave, g);
         if (j + 1 >= nsteps) break;
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * L::NL) : "memory");
         split_patch_tail<HD>(smem, cx, j + 1, sub, lane);
-        set_barrier(smem, cx.cnt, 4 * (j + 2), lane);
+        set_barrier(smem, cx.cnt, 4 * (j + 2), lane, a.err, a.err_code);
         split_wave_step<HD>(R, negm, s1, s0, smem, cx, j + 1, wave, g);
         if (j + 2 >= nsteps) break;
     }

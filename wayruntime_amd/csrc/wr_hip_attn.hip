@@ -74,6 +74,7 @@ struct Lib {
     std::mutex mu;               // serialises submissions and workspace growth
     bool inited = false;
     int device = -1;
+    uint32_t n_cus = 256;        // compute units of the device in use
     hipStream_t stream = nullptr;
     char name[320] = "uninitialised";
     Buffer d_stage;              // device staging for host-pointer entry points
@@ -81,6 +82,11 @@ struct Lib {
     Buffer d_proj;               // projection operand fragments and row scales
     uint32_t* d_counters = nullptr;   // split-K tickets, zero whenever no launch is in flight
     unsigned char* noalloc_ws[kMaxDevices] = {};   // device address of `scratch`, per device
+    // Error word: page-locked host memory that kernels can write.  A kernel whose
+    // bounded wait expires stores kDevErrWaitExpired | layer there; the host reads
+    // it after every wait for the stream (no copy, no extra latency).
+    volatile uint32_t* err_host = nullptr;
+    uint32_t* err_dev = nullptr;
     Buffer h_pin;                // pinned host staging
     std::atomic<uint64_t> calls{0};
     wr_hip_log_fn log_fn = nullptr;
@@ -148,6 +154,42 @@ int ensure_pinned(Buffer& b, size_t need)
     return WR_HIP_OK;
 }
 
+// Puts the split-K tickets back to zero.  They return to zero by themselves at
+// the end of every launch that completes; after a launch or a wait has failed
+// nothing is known about them, and a non-zero ticket would make the next launch
+// merge partial rows that were never written.
+void reset_tickets()
+{
+    if (!g.d_counters) return;
+    const size_t cb = (size_t)WR_HIP_BATCH_MAX * kMaxHeads * sizeof(uint32_t);
+    if (hipMemsetAsync(g.d_counters, 0, cb, g.stream) == hipSuccess) (void)hipStreamSynchronize(g.stream);
+    (void)hipGetLastError();
+}
+
+// Waits for the library stream, then looks at the error word.  Every entry point
+// that promises results on return waits through here, so a kernel that gave up a
+// bounded wait (and went on with wrong data) turns into WR_HIP_ERR_INTERNAL on the
+// first call that could hand those results to the caller, logged with the layer
+// (as the reference reports op failures, src/core/session.c:170-174).
+int sync_checked(const char* what, uint32_t layer)
+{
+    const hipError_t e = hipStreamSynchronize(g.stream);
+    if (e != hipSuccess) {
+        const int rc = hip_fail(e, what, layer);
+        reset_tickets();
+        return rc;
+    }
+    const uint32_t w = g.err_host ? *g.err_host : 0u;
+    if (w != 0) {
+        *g.err_host = 0;
+        logmsg(0, "device: a kernel's bounded wait expired at layer %u (error word 0x%08x, seen at: %s); "
+                  "results produced since the previous wait are invalid", w & kDevErrLayerMask, w, what);
+        reset_tickets();
+        return WR_HIP_ERR_INTERNAL;
+    }
+    return WR_HIP_OK;
+}
+
 // Host -> device / device -> host on the library stream.  Small transfers go
 // through pinned staging (predictable latency); large ones are handed to the
 // runtime directly.  Both leave the stream synchronised for the host buffer.
@@ -168,17 +210,18 @@ int copy_up(void* dst_dev, const void* src_host, size_t bytes, size_t pin_off)
 
 int copy_down_sync(void* dst_host, const void* src_dev, size_t bytes)
 {
-    if (bytes == 0) return hipStreamSynchronize(g.stream) == hipSuccess ? WR_HIP_OK
-                                                                         : WR_HIP_ERR_INTERNAL;
+    if (bytes == 0) return sync_checked("sync", 0);
     if (bytes <= g.h_pin.cap && bytes <= kPinSmall) {
         HIP_TRY(hipMemcpyAsync(g.h_pin.p, src_dev, bytes, hipMemcpyDeviceToHost, g.stream),
                 "d2h", 0);
-        HIP_TRY(hipStreamSynchronize(g.stream), "d2h sync", 0);
+        int rc = sync_checked("d2h sync", 0);
+        if (rc) return rc;
         memcpy(dst_host, g.h_pin.p, bytes);
     } else {
         HIP_TRY(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, g.stream),
                 "d2h", 0);
-        HIP_TRY(hipStreamSynchronize(g.stream), "d2h sync", 0);
+        int rc = sync_checked("d2h sync", 0);
+        if (rc) return rc;
     }
     return WR_HIP_OK;
 }
@@ -398,8 +441,14 @@ int decode_locked(uint32_t n, wr_hip_kv* const* kv, uint32_t layer, const uint32
     } else {
         launch_main(decode_generic_kernel, dim3(nq, a.n_items), dim3(kDecodeThreads), a);
     }
-    HIP_TRY(hipGetLastError(), "decode launch", layer);
-    g.calls.fetch_add(n, std::memory_order_relaxed);
+    {
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess) {
+            const int rc = hip_fail(e, "decode launch", layer);
+            reset_tickets();
+            return rc;
+        }
+    }
     return WR_HIP_OK;
 }
 
@@ -409,6 +458,12 @@ int check_decode(uint32_t n, wr_hip_kv* const* kv, uint32_t layer, const uint32_
     if (!g.inited) return WR_HIP_ERR_STATE;
     if (!kv || !seq_k || !q || !out) return WR_HIP_ERR_INVAL;
     if (n == 0 || n > WR_HIP_BATCH_MAX) return WR_HIP_ERR_LIMIT;
+    for (uint32_t i = 0; i < n; i++)
+        if (!kv[i]) return WR_HIP_ERR_INVAL;
+    // The reference counts an attention call once its pointer checks have passed
+    // and before it looks at any shape (src/core/kernels.c:1418-1423), so calls
+    // refused for their shapes count too: one per session here.
+    g.calls.fetch_add(n, std::memory_order_relaxed);
     for (uint32_t i = 0; i < n; i++) {
         int rc = check_layer(kv[i], layer);
         if (rc) return rc;
@@ -445,6 +500,8 @@ int prefill_locked(wr_hip_kv* kv, uint32_t layer, uint32_t p0, uint32_t T, const
     a.hd = hd;
     a.ctx_pad = kv->ctx_pad;
     a.window = window;
+    a.err = g.err_dev;
+    a.err_code = kDevErrWaitExpired | (layer & kDevErrLayerMask);
     const float scale = (scale_override > 0.0f) ? scale_override : 1.0f / sqrtf((float)hd);
     a.qscale = scale * kLog2e;
     const uint32_t G = a.group;
@@ -460,7 +517,7 @@ int prefill_locked(wr_hip_kv* kv, uint32_t layer, uint32_t p0, uint32_t T, const
         // not even give every CU a workgroup, one block per workgroup finishes
         // with the longest block instead of with a pair's sum plus a second
         // prologue and epilogue.
-        a.single = ((nblk + 1) / 2) * ny < 256 ? 1 : 0;
+        a.single = ((nblk + 1) / 2) * ny < g.n_cus ? 1 : 0;
         const uint32_t nwg = a.single ? nblk : (nblk + 1) / 2;
         if (hd == 64)
             launch_main(prefill_split_kernel<64>, dim3(ny, nwg), dim3(kSplitThreads), a,
@@ -474,7 +531,6 @@ int prefill_locked(wr_hip_kv* kv, uint32_t layer, uint32_t p0, uint32_t T, const
         launch_main(prefill_generic_kernel, dim3(T, nq), dim3(kDecodeThreads), a);
     }
     HIP_TRY(hipGetLastError(), "prefill launch", layer);
-    g.calls.fetch_add(T, std::memory_order_relaxed);
     return WR_HIP_OK;
 }
 
@@ -482,9 +538,13 @@ int check_prefill(const wr_hip_kv* kv, uint32_t layer, uint32_t p0, uint32_t T, 
                   const void* out, uint32_t nq)
 {
     if (!g.inited) return WR_HIP_ERR_STATE;
+    if (!kv || !q || !out) return WR_HIP_ERR_INVAL;
+    // one count per row: prefill stands for T attention calls of the reference,
+    // each counted after its pointer checks and before its shape checks
+    // (src/core/kernels.c:1418-1423)
+    g.calls.fetch_add(T, std::memory_order_relaxed);
     int rc = check_layer(kv, layer);
     if (rc) return rc;
-    if (!q || !out) return WR_HIP_ERR_INVAL;
     if (T == 0) return WR_HIP_ERR_INVAL;
     if (nq == 0 || nq % kv->nkv != 0) return WR_HIP_ERR_INVAL;
     if ((uint64_t)p0 + T > WR_HIP_ATTN_MAX_SEQ) return WR_HIP_ERR_LIMIT;
@@ -721,6 +781,7 @@ int wr_hip_attn_init(int device)
     }
     HIP_TRY(hipStreamCreateWithFlags(&g.stream, hipStreamNonBlocking), "stream create", 0);
     g.device = device;
+    g.n_cus = prop.multiProcessorCount > 0 ? (uint32_t)prop.multiProcessorCount : 256u;
     snprintf(g.name, sizeof g.name, "%s %s, %d CUs, %.1f GiB", prop.gcnArchName, prop.name,
              prop.multiProcessorCount, (double)prop.totalGlobalMem / (1024.0 * 1024.0 * 1024.0));
     g.inited = true;
@@ -733,6 +794,20 @@ int wr_hip_attn_init(int device)
         if (e == hipSuccess) e = hipMemsetAsync(g.d_counters, 0, cb, g.stream);
         if (e == hipSuccess) e = hipStreamSynchronize(g.stream);
         if (e != hipSuccess) rc = hip_fail(e, "ticket array", 0);
+    }
+    if (rc == WR_HIP_OK) {
+        void* hp = nullptr;
+        void* dp = nullptr;
+        hipError_t e = hipHostMalloc(&hp, 64, hipHostMallocMapped);
+        if (e == hipSuccess) e = hipHostGetDevicePointer(&dp, hp, 0);
+        if (e != hipSuccess) {
+            rc = hip_fail(e, "error word", 0);
+            if (hp) (void)hipHostFree(hp);
+        } else {
+            memset(hp, 0, 64);
+            g.err_host = reinterpret_cast<volatile uint32_t*>(hp);
+            g.err_dev = reinterpret_cast<uint32_t*>(dp);
+        }
     }
     if (rc == WR_HIP_OK) {
         // device address of the no-alloc entry point's scratch array, once per
@@ -771,6 +846,9 @@ int wr_hip_attn_init(int device)
     }
     if (rc != WR_HIP_OK) {
         g.inited = false;
+        if (g.err_host) (void)hipHostFree((void*)g.err_host);
+        g.err_host = nullptr;
+        g.err_dev = nullptr;
         (void)hipStreamDestroy(g.stream);
         g.stream = nullptr;
     }
@@ -792,6 +870,9 @@ void wr_hip_attn_shutdown(void)
     if (g.d_counters) (void)hipFree(g.d_counters);
     g.d_counters = nullptr;
     if (g.h_pin.p) (void)hipHostFree(g.h_pin.p);
+    if (g.err_host) (void)hipHostFree((void*)g.err_host);
+    g.err_host = nullptr;
+    g.err_dev = nullptr;
     if (g.d_proj.p) (void)hipFree(g.d_proj.p);
     g.d_proj = Buffer();
     g.d_stage = Buffer();
@@ -1107,7 +1188,8 @@ int wr_hip_attn_decode_batched(uint32_t n, wr_hip_kv* const* kv, uint32_t layer,
     if (rc) return rc;
     HIP_TRY(hipMemcpyAsync(g.h_pin.p, dout, n * row, hipMemcpyDeviceToHost, g.stream), "out d2h",
             layer);
-    HIP_TRY(hipStreamSynchronize(g.stream), "decode sync", layer);
+    rc = sync_checked("decode sync", layer);
+    if (rc) return rc;
     for (uint32_t i = 0; i < n; i++) memcpy(out[i], (uint8_t*)g.h_pin.p + i * row, row);
     return WR_HIP_OK;
 }
@@ -1204,16 +1286,14 @@ int wr_hip_attn_d2h(void* dst_host, const void* src_dev, size_t bytes)
     if (!dst_host || !src_dev) return WR_HIP_ERR_INVAL;
     Locked lk;
     HIP_TRY(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, g.stream), "d2h", 0);
-    HIP_TRY(hipStreamSynchronize(g.stream), "d2h sync", 0);
-    return WR_HIP_OK;
+    return sync_checked("d2h sync", 0);
 }
 
 int wr_hip_attn_sync(void)
 {
     if (!g.inited) return WR_HIP_ERR_STATE;
     Locked lk;
-    HIP_TRY(hipStreamSynchronize(g.stream), "sync", 0);
-    return WR_HIP_OK;
+    return sync_checked("sync", 0);
 }
 
 void* wr_hip_attn_stream(void) { return g.inited ? (void*)g.stream : nullptr; }
