@@ -1,0 +1,631 @@
+// Causal prefill attention on the matrix cores, two waves per SIMD in lock step.
+//
+// Same semantics as kernels_prefill.hip.h (reference: the prefill loop
+// src/core/session.c:615-625 over src/core/kernels.c:1475-1523), same workgroup
+// shape, LDS image, data movement and arithmetic as prefill_split_kernel there:
+// 8 waves = one KV head x 4 (head, 32-row block) pairs x 2 key sets (even / odd
+// 32-key tiles), tiles copied from global memory straight into a per-set ring of
+// three LDS slots, Q^T held in registers, S^T = K.Q^T and O^T += Vt.P^T on
+// v_mfma_f32_32x32x16_f16, lazy softmax reference, partials of the two sets
+// merged through LDS.
+//
+// What differs is when the two waves that share a SIMD do what.  A wave issues
+// at most one instruction every four clocks, whatever its kind, and a
+// 32x32x16 MFMA keeps the matrix pipe busy for 32: a wave that runs sixteen
+// MFMAs and the two hundred other instructions of a step in one stream cannot
+// keep the pipe busy, and two such waves drifting freely ask for the pipe at
+// the same time about as often as not.  Here a step is two blocks:
+//
+//   matrix block:  S(j+1) = K(j+1).Q^T and O^T += Vt(j).P(j)^T: sixteen MFMAs
+//                  back to back, every operand already in registers;
+//   vector block:  the operand reads of the next matrix block (K of tile j+2,
+//                  Vt of tile j+1), the softmax of S(j+1), the step's copies
+//                  from global memory into LDS;
+//
+// and the two key sets alternate: while the waves of one set run their matrix
+// block, their SIMD neighbours of the other set run their vector block in its
+// shadow.  The workgroup's hardware barrier, twice per step, keeps the sets in
+// that phase; it also publishes a set's copies to its four waves and frees the
+// ring slot the step overwrites.  Every wave executes the same number of
+// barriers whatever its set or rows.  For the matrix pipe to stay busy the
+// vector block has to fit the matrix block's 512 clocks, i.e. ~120 instructions:
+// the loop is unrolled over the ring (slot offsets become immediates), operand
+// addresses are loop-invariant registers, and the rare paths (masks at the
+// diagonal and the window edge, a moving softmax reference, the tail of the
+// appended rows) are wave-uniform branches.
+#pragma once
+
+#include "kernels_prefill.hip.h"
+
+namespace wr {
+
+#ifdef WR_PP_PROF
+// Measurement build only: cycle stamps of one workgroup's waves 0 and 4, summed
+// per phase, left in a global array that a debug export reads back.
+__device__ unsigned long long wr_pp_prof[2][8];
+#define PP_T(var) const unsigned long long var = clock64()
+#define PP_ADD(slot, t1, t0) prof_acc[slot] += (t1) - (t0)
+#else
+#define PP_T(var)
+#define PP_ADD(slot, t1, t0)
+#endif
+
+#ifndef WR_PP_PRIO
+#define WR_PP_PRIO 1
+#endif
+constexpr bool kPpPrio = WR_PP_PRIO != 0;
+
+template <int HD>
+struct PpCtx {
+    // wave-uniform
+    const unsigned char* kbase;       // this KV head's K / Vt, bytes
+    const unsigned char* vtbase;
+    uint32_t m0k, m0v;                // LDS byte address of this wave's first K / Vt copy in ring slot 0
+    uint32_t t0, nt, t_last;          // the set's first tile and tile count, the block's last tile
+    uint32_t tail_tile;               // tiles from this one on reach past the appended rows
+    uint32_t jt_lo, jt_hi;            // set-local tile indices this wave's rows take part in (empty: lo > hi)
+    uint32_t pl_lo, pl_hi;            // ... of which these are plain: every (row, key) pair visible
+    uint32_t ring;                    // byte offset of the set's ring in the kernel's LDS
+    // per lane
+    uint32_t gk_off, gv_off;          // offset inside a K tile / Vt block of this lane's 16 bytes
+    const unsigned char* kop[HD / 16];   // K operand read of contraction step i, ring slot 0
+    const unsigned char* vop[2];         // Vt operand read of half t, dimension block 0, ring slot 0
+    float thr;                        // a row maximum above this moves the softmax reference
+};
+
+// The set's tile with index jt, clamped to the block's last tile (copies past a
+// set's range land in ring slots nobody reads, so the number in flight is fixed).
+template <int HD>
+__device__ __forceinline__ uint32_t pp_tile(const PpCtx<HD>& cx, uint32_t jt)
+{
+    return min(cx.t0 + 2 * jt, cx.t_last);
+}
+
+// One of this wave's NL copies of the set's K tile jt / Vt block jt into ring slot SLOT.
+template <int HD, int SLOT>
+__device__ __forceinline__ void pp_issue_k1(const PpCtx<HD>& cx, uint32_t jt, int u)
+{
+    using L = SplitLds<HD>;
+    const unsigned char* src = cx.kbase + (size_t)pp_tile(cx, jt) * L::KTILE;
+    lds_direct_load(cx.m0k + SLOT * L::KTILE + u * 4096, src + u * 128, cx.gk_off);
+}
+
+template <int HD, int SLOT>
+__device__ __forceinline__ void pp_issue_v1(const PpCtx<HD>& cx, uint32_t jt, int u)
+{
+    using L = SplitLds<HD>;
+    const unsigned char* src = cx.vtbase + (size_t)pp_tile(cx, jt) * L::VTILE;
+    lds_direct_load(cx.m0v + SLOT * L::VTILE + u * 4096, src + u * 4096, cx.gv_off);
+}
+
+template <int HD, int SLOT>
+__device__ __forceinline__ void pp_issue_k(const PpCtx<HD>& cx, uint32_t jt)
+{
+#pragma unroll
+    for (int u = 0; u < SplitLds<HD>::NL; u++) pp_issue_k1<HD, SLOT>(cx, jt, u);
+}
+
+template <int HD, int SLOT>
+__device__ __forceinline__ void pp_issue_v(const PpCtx<HD>& cx, uint32_t jt)
+{
+#pragma unroll
+    for (int u = 0; u < SplitLds<HD>::NL; u++) pp_issue_v1<HD, SLOT>(cx, jt, u);
+}
+
+// Zeroes, in the staged Vt of the set's tile jt (ring slot SLOT), the positions
+// that were never appended: they may hold anything, and 0 * garbage must not
+// reach the accumulator.  Every lane patches the chunks its own copies
+// delivered, so only this wave's copies have to have landed.
+template <int HD, int SLOT>
+__device__ __forceinline__ void pp_patch_tail(unsigned char* smem, const PpCtx<HD>& cx, uint32_t jt,
+                                              int sub, int lane, uint32_t kv_valid)
+{
+    using L = SplitLds<HD>;
+    const uint32_t tile = pp_tile(cx, jt);
+    if (tile < cx.tail_tile) return;
+#pragma unroll
+    for (int u = 0; u < L::NL; u++) {
+        const int q = sub + 4 * u;
+        const int row = q * 16 + lane / 4;                // Vt row (dimension)
+        const int c = (lane & 3) ^ L::fv(row);            // key chunk this slot holds
+        const uint32_t key0 = tile * kTileKeys + c * 8;
+        u32x4* at = reinterpret_cast<u32x4*>(smem + cx.ring + L::V_IN_SET + SLOT * L::VTILE + q * 1024 +
+                                             lane * 16);
+        u32x4 v = *at;
+        uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            if (key0 + 2 * e >= kv_valid) w[e] &= 0xFFFF0000u;
+            if (key0 + 2 * e + 1 >= kv_valid) w[e] &= 0x0000FFFFu;
+        }
+        *at = u32x4{w[0], w[1], w[2], w[3]};
+    }
+}
+
+__device__ __forceinline__ void pp_barrier()
+{
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+// Row maximum of the sixteen scores a lane holds, in one block of instructions
+// (v_max3 without the canonicalising self-maximum a compiler-made maximum gets
+// per operand, and without a hazard nop after every statement).
+__device__ __forceinline__ float pp_max16(const f32x16& c)
+{
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3\n\t"
+        "v_max3_f32 %0, %0, %4, %5\n\t"
+        "v_max3_f32 %0, %0, %6, %7\n\t"
+        "v_max3_f32 %0, %0, %8, %9\n\t"
+        "v_max3_f32 %0, %0, %10, %11\n\t"
+        "v_max3_f32 %0, %0, %12, %13\n\t"
+        "v_max3_f32 %0, %0, %14, %15\n\t"
+        "v_max_f32 %0, %0, %16"
+        : "=&v"(r)
+        : "v"(c[0]), "v"(c[1]), "v"(c[2]), "v"(c[3]), "v"(c[4]), "v"(c[5]), "v"(c[6]), "v"(c[7]), "v"(c[8]),
+          "v"(c[9]), "v"(c[10]), "v"(c[11]), "v"(c[12]), "v"(c[13]), "v"(c[14]), "v"(c[15]));
+    return r;
+}
+
+// Masks of a tile that is not plain for this wave (rare, wave-uniform branch).
+// Both masks write the score registers in place, instruction by instruction:
+// written as ordinary assignments they give the masked scores new registers,
+// and the path that skips the masks (the one that matters) pays sixteen copies.
+template <int HD>
+__device__ __forceinline__ void pp_mask_special(const PrefillRows<HD>& R, const PpCtx<HD>& cx, f32x16& c,
+                                                uint32_t tile, uint32_t jt, int g)
+{
+    const float ninf = -INFINITY;
+    if (jt < cx.jt_lo || jt > cx.jt_hi) {
+        // this wave's rows do not see the tile at all: probabilities of zero
+#pragma unroll
+        for (int r = 0; r < 16; r++) asm volatile("v_mov_b32 %0, %1" : "+v"(c[r]) : "v"(ninf));
+    } else {
+        // register r of this lane: key kb + 16*(r/8) + 8*g + r%8, row n; some
+        // (row, key) pair of the tile is above the diagonal or below the window
+        const uint32_t kb = tile * kTileKeys;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const uint32_t key = kb + 16 * (r >> 3) + 8 * g + (r & 7);
+            const uint64_t hide = __builtin_amdgcn_ballot_w64(key > R.pos || key < R.row_lo);
+            asm volatile("v_cndmask_b32 %0, %0, %1, %2" : "+v"(c[r]) : "v"(ninf), "s"(hide));
+        }
+    }
+}
+
+// The softmax reference of a row moves (rare, wave-uniform branch): this tile's
+// scores are shifted, the accumulators rescaled and the block of -m rewritten.
+template <int HD>
+__device__ __forceinline__ void pp_move_reference(PrefillRows<HD>& R, PpCtx<HD>& cx, f32x16& negm,
+                                                  f32x16& c, float tmax, bool jump)
+{
+    const bool unset = (R.m_run == -INFINITY);
+    const float delta = jump ? tmax : 0.f;
+    const float alpha = jump ? (unset ? 0.f : fast_exp2(-delta)) : 1.0f;
+    R.l_run *= alpha;
+#pragma unroll
+    for (int dt = 0; dt < HD / 32; dt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) R.o[dt][r] *= alpha;
+    // updated in place with the instructions spelled out: left to itself the
+    // compiler gives the updated values new registers and pays with 32 copies
+    // on the path that skips this branch, which is the one that matters
+#pragma unroll
+    for (int r = 0; r < 16; r++) asm volatile("v_sub_f32 %0, %0, %1" : "+v"(c[r]) : "v"(delta));
+    if (jump) R.m_run = (unset ? 0.f : R.m_run) + delta;
+    const bool still = (R.m_run == -INFINITY);
+    const float nm = still ? 0.f : -R.m_run;
+#pragma unroll
+    for (int r = 0; r < 16; r++) asm volatile("v_mov_b32 %0, %1" : "+v"(negm[r]) : "v"(nm));
+    asm volatile("v_mov_b32 %0, %1" : "+v"(cx.thr) : "v"(still ? -INFINITY : kLazyLog2));
+}
+
+// Matrix block of the step that ends with vector block jt (P == jt % kRing):
+// the score chain of the set's tile jt with this wave's copies for later steps
+// between its links, then P.V of tile jt-1 with the row maximum of the new
+// scores in its shadow.  The scores come out of the chain with the row's
+// reference already subtracted (the chain starts from the block of -m); the
+// reference moves only when a row's maximum exceeds it by more than kLazyLog2
+// or is the row's first finite score.
+template <int HD, int P>
+__device__ __forceinline__ void pp_matrix_block(PrefillRows<HD>& R, PpCtx<HD>& cx, f32x16& negm, f32x16& s,
+                                                const u32x4 (&pop)[2], const half8 (&kf)[HD / 16],
+                                                const half8 (&vf)[HD / 16], uint32_t jt, int g)
+{
+    using L = SplitLds<HD>;
+    constexpr int NS = HD / 16, ND = HD / 32;
+    static_assert(NS >= 2 * L::NL, "a copy between every two links of the chain");
+    if (kPpPrio) __builtin_amdgcn_s_setprio(1);
+    // K of the set's tile jt+3 and Vt of tile jt+2 replace K of tile jt and Vt of
+    // tile jt-1, both read for the last time in the previous vector block
+#pragma unroll
+    for (int i = 0; i < NS; i++) {
+        if (i == 0)
+            s = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[0], R.qop[0], negm, 0, 0, 0);
+        else
+            s = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[i], R.qop[i], s, 0, 0, 0);
+        if (i < L::NL) pp_issue_k1<HD, P>(cx, jt + 3, i);
+        else if (i < 2 * L::NL) pp_issue_v1<HD, (P + 2) % 3>(cx, jt + 2, i - L::NL);
+    }
+    const uint32_t tile = cx.t0 + 2 * jt;
+    if (jt < cx.pl_lo || jt > cx.pl_hi) pp_mask_special<HD>(R, cx, s, tile, jt, g);
+#pragma unroll
+    for (int i = 0; i < NS; i++) {
+        const int t = i / ND, dt = i % ND;
+        R.o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[t * ND + dt], __builtin_bit_cast(half8, pop[t]),
+                                                           R.o[dt], 0, 0, 0);
+    }
+    float tmax = pp_max16(s);
+    {
+        const uint32_t u = __float_as_uint(tmax);
+        const auto sw = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+        tmax = max3_raw(__uint_as_float(sw[0]), __uint_as_float(sw[1]), tmax);   // same in both lanes of a row
+    }
+    const bool jump = tmax > cx.thr;                      // thr: -inf until the row has a reference, then kLazyLog2
+    if (__builtin_amdgcn_ballot_w64(jump) != 0) pp_move_reference<HD>(R, cx, negm, s, tmax, jump);
+    if (kPpPrio) __builtin_amdgcn_s_setprio(0);
+}
+
+// jt: set-local index of the tile whose scores are in `s`; P == jt % kRing.
+template <int HD, int P>
+__device__ __forceinline__ void pp_vector_block(PrefillRows<HD>& R, PpCtx<HD>& cx, f32x16& negm,
+                                                f32x16& s, u32x4 (&pop)[2], half8 (&kf)[HD / 16],
+                                                half8 (&vf)[HD / 16], unsigned char* smem, uint32_t jt,
+                                                int sub, int lane, int g, uint32_t kv_valid
+#ifdef WR_PP_PROF
+                                                , unsigned long long (&stamp)[5]
+// (the compiler's own counter read, so that its wait for the value is tracked: a
+// hand-written s_memtime returns into registers the compiler believes are free)
+#define PP_STAMP(i)                                 \
+    do {                                            \
+        __builtin_amdgcn_sched_barrier(0);          \
+        stamp[i] = __builtin_readcyclecounter();    \
+        __builtin_amdgcn_sched_barrier(0);          \
+    } while (0)
+#else
+#define PP_STAMP(i)
+#endif
+                                                )
+{
+    using L = SplitLds<HD>;
+    constexpr int NS = HD / 16, ND = HD / 32;
+    static_assert(kRing == 3, "slot arithmetic below is for a ring of three");
+    PP_STAMP(0);
+    constexpr int KS = (P + 1) % 3;       // slot of K of tile jt+1
+    constexpr int VS = P;                 // slot of Vt of tile jt
+    // All copies but the ones the matrix block before this one issued have had a
+    // whole step to land: K of tile jt+2 and Vt of tile jt+1, which the next vector
+    // block reads once the barrier that ends this one has published them.
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * L::NL) : "memory");
+    pp_patch_tail<HD, KS>(smem, cx, jt + 1, sub, lane, kv_valid);
+    PP_STAMP(1);
+    // operands of the next matrix block: their LDS latency runs under the softmax
+#ifndef WR_PP_WHATIF_NOLDS
+#pragma unroll
+    for (int i = 0; i < NS; i++)
+        kf[i] = *reinterpret_cast<const half8*>(cx.kop[i] + KS * L::KTILE);
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int dt = 0; dt < ND; dt++)
+            vf[t * ND + dt] = *reinterpret_cast<const half8*>(cx.vop[t] + VS * L::VTILE + dt * 2048);
+#endif
+
+    PP_STAMP(2);
+    PP_STAMP(3);
+    float psum = 0.f;
+    const half2v ones = {(_Float16)1.0f, (_Float16)1.0f};
+#ifdef WR_PP_WHATIF_NOEXP
+    pop[0] = pop[1] = u32x4{0x3c003c00u, 0x3c003c00u, 0x3c003c00u, 0x3c003c00u};
+    if (false)
+#endif
+#pragma unroll
+    for (int r = 0; r < 16; r += 2) {
+        // two exp2, one pack to F16, one dot product with (1, 1): the normaliser is
+        // the sum of exactly the rounded values P.V multiplies.  The pair stays one
+        // 32-bit word all the way into the matrix instruction's operand.
+        const half2v ph = {(_Float16)fast_exp2(s[r]), (_Float16)fast_exp2(s[r + 1])};
+        psum = __builtin_amdgcn_fdot2(ph, ones, psum, false);
+        pop[r >> 3][(r & 7) >> 1] = __builtin_bit_cast(uint32_t, ph);
+    }
+    R.l_run += psum;
+    PP_STAMP(4);
+}
+
+template <int HD>
+__device__ __forceinline__ void pp_block(const PrefillArgs& a, unsigned char* smem, uint32_t pb,
+                                         uint32_t kvh, uint32_t hc)
+{
+    using L = SplitLds<HD>;
+    static_assert(L::NL == 1 || L::NL == 2, "one or two copies per wave, tile and operand");
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // in a scalar register
+    const int n = lane & 31, g = lane >> 5;
+    const int kg = wave >> 2, sub = wave & 3;             // key set (tile parity), rows served
+    const uint32_t G = a.group;
+    const uint32_t Gw = G < 4 ? G : 4;
+    const uint32_t BP = 32 * (4 / Gw);                    // positions per block
+    const uint32_t head = kvh * G + hc * Gw + (sub % Gw);
+    const uint32_t row0 = pb * BP + (sub / Gw) * 32;      // first chunk row of this wave
+    const uint32_t kv_valid = a.p0 + a.T;                 // rows of the cache that hold data
+    uint32_t t_first, t_last;
+    prefill_block_tiles(a, pb, BP, t_first, t_last);
+
+    PrefillRows<HD> R;
+    prefill_rows_init<HD, false>(R, a, row0, head, n, g);
+
+    PpCtx<HD> cx;
+    cx.t0 = t_first + kg;                                 // this set's tiles: t0, t0 + 2, ...
+    cx.nt = (cx.t0 <= t_last) ? (t_last - cx.t0) / 2 + 1 : 0;
+    cx.t_last = t_last;
+    cx.tail_tile = kv_valid / kTileKeys;
+    cx.kbase = uniform_ptr(reinterpret_cast<const unsigned char*>(a.k + (size_t)kvh * a.ctx_pad * HD));
+    cx.vtbase = uniform_ptr(reinterpret_cast<const unsigned char*>(
+        a.vt + (size_t)kvh * (a.ctx_pad / kVBlock) * HD * kVBlock));
+    cx.ring = kg * L::SET_BYTES;
+    {
+        // low half of a generic LDS pointer = LDS byte address
+        const uint32_t lds0 = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)smem);
+        cx.m0k = lds0 + cx.ring + sub * 1024;
+        cx.m0v = lds0 + cx.ring + L::V_IN_SET + sub * 1024;
+        // set-local tile indices this wave's rows take part in
+        const uint32_t lo_t = max(R.wt_first, cx.t0), hi_t = min(R.wt_last, t_last);
+        if (R.wave_ok && cx.nt > 0 && lo_t <= hi_t && (lo_t - cx.t0 + 1) / 2 <= (hi_t - cx.t0) / 2) {
+            cx.jt_lo = (lo_t - cx.t0 + 1) / 2;
+            cx.jt_hi = (hi_t - cx.t0) / 2;
+        } else {
+            cx.jt_lo = 1;
+            cx.jt_hi = 0;
+        }
+        // Tile kb holds an invisible (row, key) pair if kb + 31 > the first row's
+        // position (diagonal), i.e. from tile edge_hi on, or kb < the last row's
+        // window floor, i.e. below tile edge_lo.  The others are plain.
+        const uint32_t edge_hi = (R.w_first_pos + 1) / kTileKeys;
+        const uint32_t edge_lo = (R.w_hi_lo + kTileKeys - 1) / kTileKeys;
+        cx.pl_lo = 1;
+        cx.pl_hi = 0;
+        if (cx.jt_lo <= cx.jt_hi && edge_hi >= 1 && edge_hi - 1 >= cx.t0) {
+            const uint32_t lo = edge_lo > cx.t0 ? max(cx.jt_lo, (edge_lo - cx.t0 + 1) / 2) : cx.jt_lo;
+            const uint32_t hi = min(cx.jt_hi, (edge_hi - 1 - cx.t0) / 2);
+            if (lo <= hi) {
+                cx.pl_lo = lo;
+                cx.pl_hi = hi;
+            }
+        }
+        cx.jt_lo = (uint32_t)__builtin_amdgcn_readfirstlane(cx.jt_lo);
+        cx.jt_hi = (uint32_t)__builtin_amdgcn_readfirstlane(cx.jt_hi);
+        cx.pl_lo = (uint32_t)__builtin_amdgcn_readfirstlane(cx.pl_lo);
+        cx.pl_hi = (uint32_t)__builtin_amdgcn_readfirstlane(cx.pl_hi);
+    }
+    {
+        // K: lane -> (row of the tile, slot); fetch the chunk that belongs in that slot
+        const int row = sub * (1024 / L::RB) + lane / L::CPR;
+        const int chunk = (lane % L::CPR) ^ L::fk(row);
+        cx.gk_off = ((k_tile_half(row) * L::CPR + chunk) * 16 + k_tile_slot(row)) * 16;
+        // Vt: rows of 64 bytes, four slots each
+        const int vrow = sub * 16 + lane / 4;
+        cx.gv_off = vrow * 64 + ((lane & 3) ^ L::fv(vrow)) * 16;
+        static_assert(L::NL == 1 || (4 * (1024 / L::RB) == 16 && L::fk(16) == L::fk(0) && L::fv(64) == L::fv(0)),
+                      "the second copy is 16 K rows (128 bytes in the cache) / 64 Vt rows (4 KiB) further");
+        const int krow = prefill_key_perm(n);             // tile row this lane feeds to MFMA row n
+        const uint32_t kread = krow * L::RB + ((g ^ L::fk(krow)) * 16);
+        const uint32_t vread = n * 64 + ((g ^ L::fv(n)) * 16);
+#pragma unroll
+        for (int i = 0; i < HD / 16; i++) cx.kop[i] = smem + ((cx.ring + kread) ^ (i * 32));
+#pragma unroll
+        for (int t = 0; t < 2; t++) cx.vop[t] = smem + cx.ring + L::V_IN_SET + (vread ^ (t * 32));
+    }
+    cx.thr = -INFINITY;
+    // steps of the loop: the even set's tile count (the odd set has as many or one
+    // fewer and spends its last step on probabilities of zero); the same in every wave
+    const uint32_t nsteps = (t_last - t_first) / 2 + 1;
+
+    // everything the first two vector blocks read, in order of need
+    pp_issue_k<HD, 0>(cx, 0);
+    pp_issue_k<HD, 1>(cx, 1);
+    pp_issue_v<HD, 0>(cx, 0);
+    pp_issue_k<HD, 2>(cx, 2);
+    pp_issue_v<HD, 1>(cx, 1);
+
+    // Q: every row is 4*HD contiguous bytes in global memory, so it is read with
+    // whole-row coalesced loads (the two waves serving a sub-block take 16 rows
+    // each), converted to pre-scaled F16 and turned into the per-lane operand
+    // layout through LDS.
+    _Float16 (*qs)[32][HD + 8] = reinterpret_cast<_Float16 (*)[32][HD + 8]>(smem + L::Q_OFF);
+    {
+        constexpr int LPR = HD / 4;                       // lanes per row (one float4 each)
+        constexpr int RPI = 64 / LPR;                     // rows per load instruction
+#pragma unroll
+        for (int j = 0; j < 16 / RPI; j++) {
+            const int r = kg * 16 + j * RPI + lane / LPR;
+            const uint32_t row = min(row0 + r, a.T - 1);  // idle rows re-read the last one
+            const float4 x = *reinterpret_cast<const float4*>(
+                a.q + ((size_t)row * a.nq + head) * HD + (lane % LPR) * 4);
+            half4 h;
+            h[0] = (_Float16)(x.x * a.qscale);
+            h[1] = (_Float16)(x.y * a.qscale);
+            h[2] = (_Float16)(x.z * a.qscale);
+            h[3] = (_Float16)(x.w * a.qscale);
+            *reinterpret_cast<half4*>(&qs[sub][r][(lane % LPR) * 4]) = h;
+        }
+    }
+    f32x16 s, negm;
+    u32x4 pop[2];
+    half8 kf[HD / 16], vf[HD / 16];
+#pragma unroll
+    for (int r = 0; r < 16; r++) s[r] = negm[r] = 0.f;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    pp_patch_tail<HD, 0>(smem, cx, 0, sub, lane, kv_valid);
+    pp_barrier();                                         // first tiles and Q visible to all
+#pragma unroll
+    for (int i = 0; i < HD / 16; i++)
+        R.qop[i] = *reinterpret_cast<const half8*>(&qs[sub][n][i * 16 + g * 8]);
+    // The set's first tile goes through a matrix block of its own, with nothing to
+    // add to the outputs yet (probabilities of zero against operands of zero).
+#pragma unroll
+    for (int i = 0; i < HD / 16; i++) kf[i] = *reinterpret_cast<const half8*>(cx.kop[i]);
+#pragma unroll
+    for (int i = 0; i < HD / 16; i++)
+#pragma unroll
+        for (int e = 0; e < 8; e++) vf[i][e] = (_Float16)0.0f;
+    pop[0] = pop[1] = u32x4{0u, 0u, 0u, 0u};
+    pp_barrier();                                         // slot 0 of K has been read by all: the block refills it
+    pp_matrix_block<HD, 0>(R, cx, negm, s, pop, kf, vf, 0, g);
+#ifdef WR_PP_PROF
+    unsigned long long stamp[5];
+    unsigned long long seg[4] = {0, 0, 0, 0};
+    pp_vector_block<HD, 0>(R, cx, negm, s, pop, kf, vf, smem, 0, sub, lane, g, kv_valid, stamp);
+#else
+    pp_vector_block<HD, 0>(R, cx, negm, s, pop, kf, vf, smem, 0, sub, lane, g, kv_valid);
+#endif
+    pp_barrier();
+
+    // The odd set runs half a step behind the even one: one barrier more before
+    // the loop, one fewer after it.
+#ifndef WR_PP_WHATIF_INPHASE
+    if (kg == 1) pp_barrier();
+#endif
+#ifdef WR_PP_PROF
+    unsigned long long prof_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#endif
+    PP_T(t_loop0);
+#ifdef WR_PP_PROF
+#define PP_VEC(PHASE) pp_vector_block<HD, PHASE>(R, cx, negm, s, pop, kf, vf, smem, j + 1, sub, lane, g, kv_valid, stamp);
+#define PP_SEG for (int q = 0; q < 4; q++) seg[q] += stamp[q + 1] - stamp[q];
+#else
+#define PP_VEC(PHASE) pp_vector_block<HD, PHASE>(R, cx, negm, s, pop, kf, vf, smem, j + 1, sub, lane, g, kv_valid);
+#define PP_SEG
+#endif
+#define WR_PP_STEP(PHASE)                                                                          \
+    {                                                                                              \
+        PP_T(t0);                                                                                  \
+        pp_matrix_block<HD, PHASE>(R, cx, negm, s, pop, kf, vf, j + 1, g);                         \
+        __builtin_amdgcn_sched_barrier(0);                                                         \
+        PP_T(t1);                                                                                  \
+        pp_barrier();                                                                              \
+        PP_T(t2);                                                                                  \
+        PP_VEC(PHASE)                                                                              \
+        __builtin_amdgcn_sched_barrier(0);                                                         \
+        PP_T(t3);                                                                                  \
+        pp_barrier();                                                                              \
+        PP_T(t4);                                                                                  \
+        PP_SEG                                                                                     \
+        PP_ADD(0, t1, t0);                                                                         \
+        PP_ADD(1, t2, t1);                                                                         \
+        PP_ADD(2, t3, t2);                                                                         \
+        PP_ADD(3, t4, t3);                                                                         \
+    }
+#pragma unroll 1
+    for (uint32_t j = 0;;) {
+        WR_PP_STEP(1)
+        if (++j >= nsteps) break;
+        WR_PP_STEP(2)
+        if (++j >= nsteps) break;
+        WR_PP_STEP(0)
+        if (++j >= nsteps) break;
+    }
+#undef WR_PP_STEP
+#ifndef WR_PP_WHATIF_INPHASE
+    if (kg == 0) pp_barrier();
+#endif
+#ifdef WR_PP_PROF
+    if (blockIdx.x == 0 && blockIdx.y == 0 && lane == 0 && sub == 0) {
+        prof_acc[4] = seg[0] | (seg[1] << 32);       // vector block: wait + tail check | reads + copies issued
+        prof_acc[5] = seg[2] | (seg[3] << 32);       // masks, maximum, reference | exponentials, sums
+        prof_acc[6] = nsteps;
+        for (int i = 0; i < 8; i++) wr_pp_prof[kg][i] += prof_acc[i];
+    }
+#endif
+
+    // merge the odd-tile partials into the even-tile waves; the ring must be
+    // quiet first (the last steps' copies still target it)
+    constexpr int NREG = HD / 2;
+    float* mg = reinterpret_cast<float*>(smem) + (size_t)sub * (NREG + 2) * 64;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (kg == 1) {
+#pragma unroll
+        for (int dt = 0; dt < HD / 32; dt++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) mg[(dt * 16 + r) * 64 + lane] = R.o[dt][r];
+        mg[NREG * 64 + lane] = R.m_run;
+        mg[(NREG + 1) * 64 + lane] = R.l_run;
+    }
+    __syncthreads();
+    // rows leave through LDS as well: the merged tile is written row-major into
+    // the sub-block's own scratch, then both of its waves store whole rows
+    float (*os)[HD + 4] = reinterpret_cast<float (*)[HD + 4]>(mg);
+    static_assert((size_t)32 * (HD + 4) <= (size_t)(NREG + 2) * 64, "row-major tile fits the merge scratch");
+    if (kg == 0) {
+        const float m1 = mg[NREG * 64 + lane], l1 = mg[(NREG + 1) * 64 + lane];
+        const float m = fmaxf(R.m_run, m1);
+        const float f0m = (R.m_run == -INFINITY) ? 0.f : fast_exp2(R.m_run - m);
+        const float f1m = (m1 == -INFINITY) ? 0.f : fast_exp2(m1 - m);
+        const float l_tot = wave_pair32_sum(R.l_run * f0m + l1 * f1m);
+        const float inv = (l_tot > 0.f) ? 1.0f / l_tot : 0.f;
+        const float w0 = f0m * inv, w1 = f1m * inv;
+#pragma unroll
+        for (int dt = 0; dt < HD / 32; dt++)
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+                R.o[dt][r] = R.o[dt][r] * w0 + mg[(dt * 16 + r) * 64 + lane] * w1;
+        // the scratch has been read into registers; the same wave now reuses it
+#pragma unroll
+        for (int dt = 0; dt < HD / 32; dt++)
+#pragma unroll
+            for (int q4 = 0; q4 < 4; q4++) {
+                float4 v;
+                v.x = R.o[dt][4 * q4 + 0];
+                v.y = R.o[dt][4 * q4 + 1];
+                v.z = R.o[dt][4 * q4 + 2];
+                v.w = R.o[dt][4 * q4 + 3];
+                *reinterpret_cast<float4*>(&os[n][dt * 32 + 8 * q4 + 4 * g]) = v;
+            }
+    }
+    __syncthreads();
+    {
+        constexpr int LPR = HD / 4;                       // lanes per row (one float4 each)
+        constexpr int RPI = 64 / LPR;                     // rows per store instruction
+#pragma unroll
+        for (int j = 0; j < 16 / RPI; j++) {
+            const int r = kg * 16 + j * RPI + lane / LPR;
+            const float4 v = *reinterpret_cast<const float4*>(&os[r][(lane % LPR) * 4]);
+            if (row0 + r < a.T)
+                *reinterpret_cast<float4*>(a.out + ((size_t)(row0 + r) * a.nq + head) * HD +
+                                           (lane % LPR) * 4) = v;
+        }
+    }
+}
+
+// grid = (KV heads x head chunks, ceil(blocks / 2)): consecutive workgroups (which
+// the dispatcher deals round-robin to the XCDs) differ in KV head, so one XCD's
+// L2 keeps seeing the same few heads' K / Vt.  Workgroup y takes position block
+// (blocks-1-y) and then block y: a long block and a short one, so every
+// workgroup streams the same number of tiles despite the causal triangle.
+// a.single: grid.y = blocks, one block per workgroup, long blocks first.
+template <int HD>
+__global__ __launch_bounds__(kSplitThreads, 1) void prefill_pp_kernel(const PrefillArgs a)
+{
+    extern __shared__ __attribute__((aligned(16))) unsigned char prefill_smem_raw[];
+    const uint32_t G = a.group;
+    const uint32_t Gw = G < 4 ? G : 4;
+    const uint32_t chunks = G / Gw;
+    const uint32_t kvh = blockIdx.x / chunks, hc = blockIdx.x % chunks;
+    const uint32_t BP = 32 * (4 / Gw);
+    const uint32_t nblk = (a.T + BP - 1) / BP;
+    const uint32_t lo = blockIdx.y, hi = nblk - 1 - blockIdx.y;
+    const int passes = a.single ? 1 : 2;
+#pragma unroll 1
+    for (int pass = 0; pass < passes; pass++) {
+        if (pass) {
+            if (hi == lo) break;
+            __syncthreads();                              // LDS changes hands
+        }
+        pp_block<HD>(a, prefill_smem_raw, pass ? lo : hi, kvh, hc);
+    }
+}
+
+}  // namespace wr

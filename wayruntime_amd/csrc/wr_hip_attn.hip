@@ -23,6 +23,7 @@
 #include "kernels_append.hip.h"
 #include "kernels_decode.hip.h"
 #include "kernels_prefill.hip.h"
+#include "kernels_prefill_pp.hip.h"
 #include "kernels_proj.hip.h"
 #include "kernels_rows.hip.h"
 
@@ -252,7 +253,7 @@ void launch_main(Kern kernel, dim3 grid, dim3 block, const Args& args, size_t ld
 
 bool mfma_shape(uint32_t hd, uint32_t group)
 {
-    return !g.force_generic && (hd == 64 || hd == 128 || hd == 256) && group <= kMaxGroupMfma;
+    return g.force_generic != 1 && (hd == 64 || hd == 128 || hd == 256) && group <= kMaxGroupMfma;
 }
 
 int check_layer(const wr_hip_kv* kv, uint32_t layer)
@@ -505,7 +506,7 @@ int prefill_locked(wr_hip_kv* kv, uint32_t layer, uint32_t p0, uint32_t T, const
     const float scale = (scale_override > 0.0f) ? scale_override : 1.0f / sqrtf((float)hd);
     a.qscale = scale * kLog2e;
     const uint32_t G = a.group;
-    const bool mfma = !g.force_generic && (hd == 64 || hd == 128 || hd == 256) &&
+    const bool mfma = g.force_generic != 1 && (hd == 64 || hd == 128 || hd == 256) &&
                       (G == 1 || G == 2 || G == 4 || G == 8);
     if (mfma) {
         const uint32_t Gw = G < 4 ? G : 4;
@@ -519,11 +520,18 @@ int prefill_locked(wr_hip_kv* kv, uint32_t layer, uint32_t p0, uint32_t T, const
         // prologue and epilogue.
         a.single = ((nblk + 1) / 2) * ny < g.n_cus ? 1 : 0;
         const uint32_t nwg = a.single ? nblk : (nblk + 1) / 2;
-        if (hd == 64)
+        const bool drift = g.force_generic == 2;           // measurement: the free-running kernel
+        if (hd == 64 && drift)
             launch_main(prefill_split_kernel<64>, dim3(ny, nwg), dim3(kSplitThreads), a,
                         split_smem_bytes<64>());
-        else if (hd == 128)
+        else if (hd == 128 && drift)
             launch_main(prefill_split_kernel<128>, dim3(ny, nwg), dim3(kSplitThreads), a,
+                        split_smem_bytes<128>());
+        else if (hd == 64)
+            launch_main(prefill_pp_kernel<64>, dim3(ny, nwg), dim3(kSplitThreads), a,
+                        split_smem_bytes<64>());
+        else if (hd == 128)
+            launch_main(prefill_pp_kernel<128>, dim3(ny, nwg), dim3(kSplitThreads), a,
                         split_smem_bytes<128>());
         else   // 256: one wave per SIMD (the accumulators alone need 256 registers)
             launch_main(prefill_mfma_kernel<256>, dim3(nwg, ny), dim3(kPrefillThreads), a);
@@ -831,6 +839,14 @@ int wr_hip_attn_init(int device)
                                            (int)split_smem_bytes<64>());
         if (e == hipSuccess)
             e = hipFuncSetAttribute(reinterpret_cast<const void*>(prefill_split_kernel<128>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)split_smem_bytes<128>());
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute(reinterpret_cast<const void*>(prefill_pp_kernel<64>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)split_smem_bytes<64>());
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute(reinterpret_cast<const void*>(prefill_pp_kernel<128>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize,
                                     (int)split_smem_bytes<128>());
         if (e == hipSuccess)
@@ -1616,5 +1632,19 @@ int wr_hip_attn_profile_end(double* total_ms, uint32_t* n_launches)
     g.ev_used = 0;
     return WR_HIP_OK;
 }
+
+#ifdef WR_PP_PROF
+// measurement build only: reads and clears the prefill kernel's phase counters
+int wr_hip_debug_pp_prof(unsigned long long* out16)
+{
+    Locked lk;
+    (void)hipStreamSynchronize(g.stream);
+    if (hipMemcpyFromSymbol(out16, HIP_SYMBOL(wr_pp_prof), 16 * sizeof(unsigned long long)) != hipSuccess)
+        return WR_HIP_ERR_INTERNAL;
+    unsigned long long z[16] = {};
+    (void)hipMemcpyToSymbol(HIP_SYMBOL(wr_pp_prof), z, sizeof z);
+    return WR_HIP_OK;
+}
+#endif
 
 }  // extern "C"
