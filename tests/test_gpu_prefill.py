@@ -177,6 +177,29 @@ def test_prefill_paired_blocks_with_offset_and_window_sampled_rows(nq, nkv, hd, 
     kv.close()
 
 
+@pytest.mark.parametrize("nq,nkv,hd", [(4, 2, 64), (32, 8, 128), (16, 8, 128), (8, 4, 256)])
+def test_prefill_is_bit_identical_from_launch_to_launch(nq, nkv, hd):
+    # The same chunk through caches at different addresses and launch after launch
+    # must give the same bits: the batched step equals serial steps only if it does
+    # (src/core/batch.c:15-19), and a kernel whose result depends on timing (a
+    # result read before it is complete, a slot refilled while still being read)
+    # shows up here long before it leaves the tolerance.
+    for T in (39, 65, 130, 300, 2048):
+        print("prefill determinism", nq, nkv, hd, T, flush=True)
+        k32 = synth.normal(1, (T, nkv, hd))
+        v32 = synth.normal(2, (T, nkv, hd))
+        q = synth.normal(3, (T, nq, hd))
+        kvs = [hipattn.KVCache(1, hd, nkv, T + 17 * i) for i in range(3)]
+        for kv in kvs:
+            assert kv.append(0, 0, k32, v32) == hipattn.OK
+        first = kvs[0].prefill(0, 0, q)
+        for rep in range(1, 7):
+            again = kvs[rep % 3].prefill(0, 0, q)
+            assert np.array_equal(first, again), f"T={T}: launch {rep} differs from the first"
+        for kv in kvs:
+            kv.close()
+
+
 def test_prefill_error_contract():
     lib = hipattn.lib()
     kv = hipattn.KVCache(1, 128, 8, 64)

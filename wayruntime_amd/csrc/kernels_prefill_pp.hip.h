@@ -140,6 +140,7 @@ __device__ __forceinline__ void pp_patch_tail(unsigned char* smem, const PpCtx<H
         }
         *at = u32x4{w[0], w[1], w[2], w[3]};
     }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");    // the patch is in LDS before the barrier that follows
 }
 
 __device__ __forceinline__ void pp_barrier()
@@ -152,8 +153,16 @@ __device__ __forceinline__ void pp_barrier()
 // Row maximum of the sixteen scores a lane holds, in one block of instructions
 // (v_max3 without the canonicalising self-maximum a compiler-made maximum gets
 // per operand, and without a hazard nop after every statement).
+//
+// The scores are the result of a matrix instruction, and the hardware does not
+// hold back a vector instruction that reads such a result too early: the wait
+// states are the compiler's job, and it does not look inside inline assembly.
+// So the first instruction to touch the scores is one the compiler sees (an add
+// of zero), and the block of maxima depends on its result; every other
+// hand-written instruction on the scores is ordered behind this maximum.
 __device__ __forceinline__ float pp_max16(const f32x16& c)
 {
+    const float c0 = c[0] + 0.0f;
     float r;
     asm("v_max3_f32 %0, %1, %2, %3\n\t"
         "v_max3_f32 %0, %0, %4, %5\n\t"
@@ -164,7 +173,7 @@ __device__ __forceinline__ float pp_max16(const f32x16& c)
         "v_max3_f32 %0, %0, %14, %15\n\t"
         "v_max_f32 %0, %0, %16"
         : "=&v"(r)
-        : "v"(c[0]), "v"(c[1]), "v"(c[2]), "v"(c[3]), "v"(c[4]), "v"(c[5]), "v"(c[6]), "v"(c[7]), "v"(c[8]),
+        : "v"(c0), "v"(c[1]), "v"(c[2]), "v"(c[3]), "v"(c[4]), "v"(c[5]), "v"(c[6]), "v"(c[7]), "v"(c[8]),
           "v"(c[9]), "v"(c[10]), "v"(c[11]), "v"(c[12]), "v"(c[13]), "v"(c[14]), "v"(c[15]));
     return r;
 }
@@ -173,15 +182,19 @@ __device__ __forceinline__ float pp_max16(const f32x16& c)
 // Both masks write the score registers in place, instruction by instruction:
 // written as ordinary assignments they give the masked scores new registers,
 // and the path that skips the masks (the one that matters) pays sixteen copies.
+// `after`: the row maximum taken of `c` before (pp_max16); naming it as an input
+// keeps these hand-written instructions behind the first compiler-visible read
+// of the matrix instruction's result.
 template <int HD>
 __device__ __forceinline__ void pp_mask_special(const PrefillRows<HD>& R, const PpCtx<HD>& cx, f32x16& c,
-                                                uint32_t tile, uint32_t jt, int g)
+                                                uint32_t tile, uint32_t jt, int g, float after)
 {
     const float ninf = -INFINITY;
+    asm volatile("" ::"v"(after));
     if (jt < cx.jt_lo || jt > cx.jt_hi) {
         // this wave's rows do not see the tile at all: probabilities of zero
 #pragma unroll
-        for (int r = 0; r < 16; r++) asm volatile("v_mov_b32 %0, %1" : "+v"(c[r]) : "v"(ninf));
+        for (int r = 0; r < 16; r++) asm volatile("v_mov_b32 %0, %1" : "+v"(c[r]) : "v"(ninf), "v"(after));
     } else {
         // register r of this lane: key kb + 16*(r/8) + 8*g + r%8, row n; some
         // (row, key) pair of the tile is above the diagonal or below the window
@@ -190,7 +203,7 @@ __device__ __forceinline__ void pp_mask_special(const PrefillRows<HD>& R, const 
         for (int r = 0; r < 16; r++) {
             const uint32_t key = kb + 16 * (r >> 3) + 8 * g + (r & 7);
             const uint64_t hide = __builtin_amdgcn_ballot_w64(key > R.pos || key < R.row_lo);
-            asm volatile("v_cndmask_b32 %0, %0, %1, %2" : "+v"(c[r]) : "v"(ninf), "s"(hide));
+            asm volatile("v_cndmask_b32 %0, %0, %1, %2" : "+v"(c[r]) : "v"(ninf), "s"(hide), "v"(after));
         }
     }
 }
@@ -231,13 +244,14 @@ __device__ __forceinline__ void pp_move_reference(PrefillRows<HD>& R, PpCtx<HD>&
 // or is the row's first finite score.
 template <int HD, int P>
 __device__ __forceinline__ void pp_matrix_block(PrefillRows<HD>& R, PpCtx<HD>& cx, f32x16& negm, f32x16& s,
-                                                const u32x4 (&pop)[2], const half8 (&kf)[HD / 16],
+                                                const u32x4 (&pop)[2], half8 (&kf)[HD / 16],
                                                 const half8 (&vf)[HD / 16], uint32_t jt, int g)
 {
     using L = SplitLds<HD>;
     constexpr int NS = HD / 16, ND = HD / 32;
+    constexpr int KS = (P + 1) % 3;       // slot of K of tile jt+1
     static_assert(NS >= 2 * L::NL, "a copy between every two links of the chain");
-    if (kPpPrio) __builtin_amdgcn_s_setprio(1);
+    if (kPpPrio) __builtin_amdgcn_s_setprio(WR_PP_PRIO == 2 ? 0 : 1);
     // K of the set's tile jt+3 and Vt of tile jt+2 replace K of tile jt and Vt of
     // tile jt-1, both read for the last time in the previous vector block
 #pragma unroll
@@ -249,15 +263,24 @@ __device__ __forceinline__ void pp_matrix_block(PrefillRows<HD>& R, PpCtx<HD>& c
         if (i < L::NL) pp_issue_k1<HD, P>(cx, jt + 3, i);
         else if (i < 2 * L::NL) pp_issue_v1<HD, (P + 2) % 3>(cx, jt + 2, i - L::NL);
     }
-    const uint32_t tile = cx.t0 + 2 * jt;
-    if (jt < cx.pl_lo || jt > cx.pl_hi) pp_mask_special<HD>(R, cx, s, tile, jt, g);
+    // The chain has consumed its K operands: the next step's (K of tile jt+1, landed
+    // and published a step ago) are read here, between the P.V products, so that
+    // the vector block is left with the Vt operands only.
 #pragma unroll
     for (int i = 0; i < NS; i++) {
         const int t = i / ND, dt = i % ND;
         R.o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[t * ND + dt], __builtin_bit_cast(half8, pop[t]),
                                                            R.o[dt], 0, 0, 0);
+        kf[i] = *reinterpret_cast<const half8*>(cx.kop[i] + KS * L::KTILE);
     }
+    // The row maximum runs in the products' shadow as if the tile were plain; a tile
+    // with invisible (row, key) pairs is masked afterwards and its maximum taken
+    // again (rare, wave-uniform).
     float tmax = pp_max16(s);
+    if (jt < cx.pl_lo || jt > cx.pl_hi) {
+        pp_mask_special<HD>(R, cx, s, cx.t0 + 2 * jt, jt, g, tmax);
+        tmax = pp_max16(s);
+    }
     {
         const uint32_t u = __float_as_uint(tmax);
         const auto sw = __builtin_amdgcn_permlane32_swap(u, u, false, false);
@@ -265,7 +288,7 @@ __device__ __forceinline__ void pp_matrix_block(PrefillRows<HD>& R, PpCtx<HD>& c
     }
     const bool jump = tmax > cx.thr;                      // thr: -inf until the row has a reference, then kLazyLog2
     if (__builtin_amdgcn_ballot_w64(jump) != 0) pp_move_reference<HD>(R, cx, negm, s, tmax, jump);
-    if (kPpPrio) __builtin_amdgcn_s_setprio(0);
+    if (kPpPrio) __builtin_amdgcn_s_setprio(WR_PP_PRIO == 2 ? 1 : 0);
 }
 
 // jt: set-local index of the tile whose scores are in `s`; P == jt % kRing.
@@ -303,9 +326,6 @@ __device__ __forceinline__ void pp_vector_block(PrefillRows<HD>& R, PpCtx<HD>& c
     PP_STAMP(1);
     // operands of the next matrix block: their LDS latency runs under the softmax
 #ifndef WR_PP_WHATIF_NOLDS
-#pragma unroll
-    for (int i = 0; i < NS; i++)
-        kf[i] = *reinterpret_cast<const half8*>(cx.kop[i] + KS * L::KTILE);
 #pragma unroll
     for (int t = 0; t < 2; t++)
 #pragma unroll

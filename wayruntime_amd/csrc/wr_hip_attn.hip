@@ -24,6 +24,7 @@
 #include "kernels_decode.hip.h"
 #include "kernels_prefill.hip.h"
 #include "kernels_prefill_pp.hip.h"
+#include "kernels_prefill_il.hip.h"
 #include "kernels_proj.hip.h"
 #include "kernels_rows.hip.h"
 
@@ -527,11 +528,17 @@ int prefill_locked(wr_hip_kv* kv, uint32_t layer, uint32_t p0, uint32_t T, const
         else if (hd == 128 && drift)
             launch_main(prefill_split_kernel<128>, dim3(ny, nwg), dim3(kSplitThreads), a,
                         split_smem_bytes<128>());
-        else if (hd == 64)
+        else if (hd == 64 && g.force_generic == 3)
             launch_main(prefill_pp_kernel<64>, dim3(ny, nwg), dim3(kSplitThreads), a,
                         split_smem_bytes<64>());
-        else if (hd == 128)
+        else if (hd == 128 && g.force_generic == 3)
             launch_main(prefill_pp_kernel<128>, dim3(ny, nwg), dim3(kSplitThreads), a,
+                        split_smem_bytes<128>());
+        else if (hd == 64)
+            launch_main(prefill_il_kernel<64>, dim3(ny, nwg), dim3(kSplitThreads), a,
+                        split_smem_bytes<64>());
+        else if (hd == 128)
+            launch_main(prefill_il_kernel<128>, dim3(ny, nwg), dim3(kSplitThreads), a,
                         split_smem_bytes<128>());
         else   // 256: one wave per SIMD (the accumulators alone need 256 registers)
             launch_main(prefill_mfma_kernel<256>, dim3(nwg, ny), dim3(kPrefillThreads), a);
@@ -839,6 +846,14 @@ int wr_hip_attn_init(int device)
                                            (int)split_smem_bytes<64>());
         if (e == hipSuccess)
             e = hipFuncSetAttribute(reinterpret_cast<const void*>(prefill_split_kernel<128>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)split_smem_bytes<128>());
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute(reinterpret_cast<const void*>(prefill_il_kernel<64>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)split_smem_bytes<64>());
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute(reinterpret_cast<const void*>(prefill_il_kernel<128>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize,
                                     (int)split_smem_bytes<128>());
         if (e == hipSuccess)
@@ -1642,6 +1657,7 @@ int wr_hip_debug_pp_prof(unsigned long long* out16)
     if (hipMemcpyFromSymbol(out16, HIP_SYMBOL(wr_pp_prof), 16 * sizeof(unsigned long long)) != hipSuccess)
         return WR_HIP_ERR_INTERNAL;
     unsigned long long z[16] = {};
+    z[8 + 4] = ~0ull;                                     // slot that takes a minimum
     (void)hipMemcpyToSymbol(HIP_SYMBOL(wr_pp_prof), z, sizeof z);
     return WR_HIP_OK;
 }
