@@ -1,19 +1,49 @@
-// Causal prefill attention on the matrix cores: both key sets of a workgroup in
-// phase, every wave's matrix instructions spread evenly through its step.
+// Causal prefill attention on the matrix cores for head dims up to 128
+// (v_mfma_f32_32x32x16_f16, F32 accumulate).  MFMA-bound: 4 * nq * hd flops per
+// (query row, visible key).
 //
-// Same semantics, workgroup shape, LDS image and arithmetic as
-// kernels_prefill_pp.hip.h (8 waves = one KV head x 4 (head, 32-row block) pairs
-// x 2 key sets, ring of three tile slots per set, lazy softmax reference, the
-// sets' partials merged through LDS).  What differs is the shape of a step.  A
-// wave issues in order; what it issues right behind a matrix instruction runs
-// in that instruction's shadow (about six instructions per 32x32x16 MFMA), and
-// two waves of a SIMD that both keep a matrix instruction ready share the
-// matrix pipe without leaving it idle.  So every step is one stream in which
-// each MFMA is followed by its share of the step's other work:
+// Semantics: kernels_prefill.hip.h (reference: the prefill loop
+// src/core/session.c:615-625 over src/core/kernels.c:1475-1523).
 //
-//   first half:   the score chain S(j+1) = K(j+1).Q^T, and between its links the
-//                 Vt operand reads of tile j and the exponentials, packs and
-//                 row sums of S(j) (two score buffers alternate);
+// Workgroup = 8 waves = one KV head x 4 (head, 32-row block) pairs x 2 key sets:
+// waves 0-3 take the even 32-key tiles of the block's key range, waves 4-7 the
+// odd ones (split-K inside the workgroup, the two partial (m, l, O) triples merged
+// through LDS at the end), two waves per SIMD at <= 256 registers each.  Per wave
+// and tile, with the query row as the MFMA COLUMN (lane % 32):
+//   S^T[key][row]  = K[key][:] . Q^T[:][row]          HD/16 MFMAs, a dependent chain
+//   online softmax on the 16 scores a lane holds (+ one exchange with lane^32)
+//   O^T[dim][row] += Vt[dim][key] . P^T[key][row]     HD/16 MFMAs
+// K rows enter the first MFMA permuted so that the scores a lane ends up with are
+// 8 consecutive keys per contraction step: P^T is then already the second MFMA's
+// operand, and the matching Vt operand is one 16-byte read of the block-transposed
+// V.  Q is rounded to F16 once, P per tile.  The softmax reference is lazy: it
+// moves only when a row's maximum exceeds it by more than 2^kLazyLog2 (with 32
+// independent rows per wave an eager maximum moves in most tiles and costs a
+// 64-register rescale each time), and the score chain starts from a block of -m,
+// so the scores come out with the reference already subtracted.
+//
+// Data movement: tiles travel from global memory straight into LDS
+// (global_load_lds_dwordx4: no staging registers, no LDS store instructions), each
+// set into its own ring of three tile slots, issued one step before the barrier
+// that publishes them.  Such a copy writes a wave's 64 x 16 bytes to consecutive
+// LDS addresses, so rows cannot be padded; the 16-byte chunks of a row are permuted
+// instead (chunk c of row r sits at slot c ^ f(r)), on the global side where any
+// permutation inside a row keeps the access coalesced; f is chosen so that the
+// sixteen rows a 128-bit LDS read touches per cycle fall into sixteen different
+// slots of the 256-byte bank row.  Copies are issued unconditionally (tile indices
+// clamped to the block's last tile; duplicates land in slots nobody reads) so the
+// number in flight is the same at every wait.
+//
+// Shape of a step.  A wave issues in order; what it issues right behind a matrix
+// instruction runs in that instruction's shadow (about six instructions per
+// 32x32x16 MFMA), and two waves of a SIMD that both keep a matrix instruction
+// ready share the matrix pipe without leaving it idle.  So both key sets run in
+// phase and every step is one stream in which each MFMA is followed by its share
+// of the step's other work:
+//
+//   first half:   the score chain S(j+1) = K(j+1).Q^T, and behind each link one
+//                 Vt operand read of tile j and a share of the exponentials and
+//                 packs of S(j) (two score buffers alternate);
 //   second half:  O^T += Vt(j).P(j)^T, and between the products the K operand
 //                 reads of tile j+2 (the chain has consumed its own), the step's
 //                 copies from global memory into LDS and the row maximum of
@@ -22,17 +52,246 @@
 //   frees the ring slots the next step overwrites.
 //
 // The loop is unrolled over the ring and the two score buffers (six step
-// variants), so slot offsets are immediates and nothing is copied between steps.
+// variants): slot offsets are immediates, operand addresses loop-invariant
+// registers, and nothing is copied between steps.  Rare paths (masks at the
+// diagonal and the window edge, a moving reference, the tail of the appended
+// rows) are wave-uniform branches that update registers in place.
+//
+// A result of a matrix instruction must not be read by a vector instruction too
+// early, and the hardware does not hold the reader back: the wait states are the
+// compiler's job, and it does not look inside inline assembly.  Every
+// hand-written instruction that touches scores is therefore ordered behind a
+// compiler-visible read of them (il_max16).
 #pragma once
 
-#include "kernels_prefill_pp.hip.h"
+#include "kernels_prefill.hip.h"
 
 namespace wr {
+
+constexpr int kSplitThreads = 512;
+constexpr int kRing = 3;
+
+template <int HD>
+struct SplitLds {
+    static constexpr int RB = 2 * HD;                     // bytes per K row
+    static constexpr int CPR = HD / 8;                    // 16-byte chunks per K row
+    static constexpr int RPB = 256 / RB > 0 ? 256 / RB : 1;   // K rows per 256-byte bank row
+    static constexpr int KTILE = kTileKeys * RB;          // bytes of one tile's K
+    static constexpr int VTILE = HD * kVBlock * 2;        // bytes of one tile's Vt block
+    static constexpr int NL = KTILE / 1024 / 4;           // loads per wave and tile, each of K and Vt
+    static constexpr int SET_BYTES = kRing * (KTILE + VTILE);   // one wave set's ring
+    static constexpr int V_IN_SET = kRing * KTILE;        // Vt slots follow the K slots
+    static constexpr int Q_OFF = 2 * SET_BYTES;           // Q staging, [4][32][HD + 8] halves
+    static constexpr int Q_BYTES = 4 * 32 * (HD + 8) * 2;
+    static constexpr int MERGE_BYTES = 4 * (HD / 2 + 2) * 64 * 4;   // laid over the rings
+    static constexpr int TOTAL = Q_OFF + Q_BYTES;
+    static_assert(MERGE_BYTES <= Q_OFF, "merge scratch fits the rings");
+    static_assert(KTILE == VTILE && NL >= 1, "one chunk schedule serves K and Vt");
+    // slot permutation of K rows / Vt rows
+    __device__ static constexpr int fk(int row) { return (row / RPB) & (CPR - 1); }
+    __device__ static constexpr int fv(int row) { return (row >> 2) & 3; }
+};
+
+template <int HD>
+constexpr size_t split_smem_bytes()
+{
+    return SplitLds<HD>::TOTAL;
+}
+
+// max of three without the canonicalising self-maximum the compiler puts in
+// front of every fmaxf operand (the operands here are never signalling NaNs
+// that anyone would want quieted)
+__device__ __forceinline__ float max3_raw(float a, float b, float c)
+{
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
+template <int HD>
+struct IlCtx {
+    // wave-uniform
+    const unsigned char* kbase;       // this KV head's K / Vt, bytes
+    const unsigned char* vtbase;
+    uint32_t m0k, m0v;                // LDS byte address of this wave's first K / Vt copy in ring slot 0
+    uint32_t t0, nt, t_last;          // the set's first tile and tile count, the block's last tile
+    uint32_t tail_tile;               // tiles from this one on reach past the appended rows
+    uint32_t jt_lo, jt_hi;            // set-local tile indices this wave's rows take part in (empty: lo > hi)
+    uint32_t pl_lo, pl_hi;            // ... of which these are plain: every (row, key) pair visible
+    uint32_t ring;                    // byte offset of the set's ring in the kernel's LDS
+    // per lane
+    uint32_t gk_off, gv_off;          // offset inside a K tile / Vt block of this lane's 16 bytes
+    const unsigned char* kop[HD / 16];   // K operand read of contraction step i, ring slot 0
+    const unsigned char* vop[2];         // Vt operand read of half t, dimension block 0, ring slot 0
+    float thr;                        // a row maximum above this moves the softmax reference
+};
+
+// The set's tile with index jt, clamped to the block's last tile (copies past a
+// set's range land in ring slots nobody reads, so the number in flight is fixed).
+template <int HD>
+__device__ __forceinline__ uint32_t il_tile(const IlCtx<HD>& cx, uint32_t jt)
+{
+    return min(cx.t0 + 2 * jt, cx.t_last);
+}
+
+// One of this wave's NL copies of the set's K tile jt / Vt block jt into ring slot SLOT.
+template <int HD, int SLOT>
+__device__ __forceinline__ void il_issue_k1(const IlCtx<HD>& cx, uint32_t jt, int u)
+{
+    using L = SplitLds<HD>;
+    const unsigned char* src = cx.kbase + (size_t)il_tile(cx, jt) * L::KTILE;
+    lds_direct_load(cx.m0k + SLOT * L::KTILE + u * 4096, src + u * 128, cx.gk_off);
+}
+
+template <int HD, int SLOT>
+__device__ __forceinline__ void il_issue_v1(const IlCtx<HD>& cx, uint32_t jt, int u)
+{
+    using L = SplitLds<HD>;
+    const unsigned char* src = cx.vtbase + (size_t)il_tile(cx, jt) * L::VTILE;
+    lds_direct_load(cx.m0v + SLOT * L::VTILE + u * 4096, src + u * 4096, cx.gv_off);
+}
+
+template <int HD, int SLOT>
+__device__ __forceinline__ void il_issue_k(const IlCtx<HD>& cx, uint32_t jt)
+{
+#pragma unroll
+    for (int u = 0; u < SplitLds<HD>::NL; u++) il_issue_k1<HD, SLOT>(cx, jt, u);
+}
+
+template <int HD, int SLOT>
+__device__ __forceinline__ void il_issue_v(const IlCtx<HD>& cx, uint32_t jt)
+{
+#pragma unroll
+    for (int u = 0; u < SplitLds<HD>::NL; u++) il_issue_v1<HD, SLOT>(cx, jt, u);
+}
+
+// Zeroes, in the staged Vt of the set's tile jt (ring slot SLOT), the positions
+// that were never appended: they may hold anything, and 0 * garbage must not
+// reach the accumulator.  Every lane patches the chunks its own copies
+// delivered, so only this wave's copies have to have landed.
+template <int HD, int SLOT>
+__device__ __forceinline__ void il_patch_tail(unsigned char* smem, const IlCtx<HD>& cx, uint32_t jt,
+                                              int sub, int lane, uint32_t kv_valid)
+{
+    using L = SplitLds<HD>;
+    const uint32_t tile = il_tile(cx, jt);
+    if (tile < cx.tail_tile) return;
+#pragma unroll
+    for (int u = 0; u < L::NL; u++) {
+        const int q = sub + 4 * u;
+        const int row = q * 16 + lane / 4;                // Vt row (dimension)
+        const int c = (lane & 3) ^ L::fv(row);            // key chunk this slot holds
+        const uint32_t key0 = tile * kTileKeys + c * 8;
+        u32x4* at = reinterpret_cast<u32x4*>(smem + cx.ring + L::V_IN_SET + SLOT * L::VTILE + q * 1024 +
+                                             lane * 16);
+        u32x4 v = *at;
+        uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            if (key0 + 2 * e >= kv_valid) w[e] &= 0xFFFF0000u;
+            if (key0 + 2 * e + 1 >= kv_valid) w[e] &= 0x0000FFFFu;
+        }
+        *at = u32x4{w[0], w[1], w[2], w[3]};
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");    // the patch is in LDS before the barrier that follows
+}
+
+__device__ __forceinline__ void il_barrier()
+{
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+// Row maximum of the sixteen scores a lane holds, in one block of instructions
+// (v_max3 without the canonicalising self-maximum a compiler-made maximum gets
+// per operand, and without a hazard nop after every statement).
+//
+// The scores are the result of a matrix instruction, and the hardware does not
+// hold back a vector instruction that reads such a result too early: the wait
+// states are the compiler's job, and it does not look inside inline assembly.
+// So the first instruction to touch the scores is one the compiler sees (an add
+// of zero), and the block of maxima depends on its result; every other
+// hand-written instruction on the scores is ordered behind this maximum.
+__device__ __forceinline__ float il_max16(const f32x16& c)
+{
+    const float c0 = c[0] + 0.0f;
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3\n\t"
+        "v_max3_f32 %0, %0, %4, %5\n\t"
+        "v_max3_f32 %0, %0, %6, %7\n\t"
+        "v_max3_f32 %0, %0, %8, %9\n\t"
+        "v_max3_f32 %0, %0, %10, %11\n\t"
+        "v_max3_f32 %0, %0, %12, %13\n\t"
+        "v_max3_f32 %0, %0, %14, %15\n\t"
+        "v_max_f32 %0, %0, %16"
+        : "=&v"(r)
+        : "v"(c0), "v"(c[1]), "v"(c[2]), "v"(c[3]), "v"(c[4]), "v"(c[5]), "v"(c[6]), "v"(c[7]), "v"(c[8]),
+          "v"(c[9]), "v"(c[10]), "v"(c[11]), "v"(c[12]), "v"(c[13]), "v"(c[14]), "v"(c[15]));
+    return r;
+}
+
+// Masks of a tile that is not plain for this wave (rare, wave-uniform branch).
+// Both masks write the score registers in place, instruction by instruction:
+// written as ordinary assignments they give the masked scores new registers,
+// and the path that skips the masks (the one that matters) pays sixteen copies.
+// `after`: the row maximum taken of `c` before (il_max16); naming it as an input
+// keeps these hand-written instructions behind the first compiler-visible read
+// of the matrix instruction's result.
+template <int HD>
+__device__ __forceinline__ void il_mask_special(const PrefillRows<HD>& R, const IlCtx<HD>& cx, f32x16& c,
+                                                uint32_t tile, uint32_t jt, int g, float after)
+{
+    const float ninf = -INFINITY;
+    asm volatile("" ::"v"(after));
+    if (jt < cx.jt_lo || jt > cx.jt_hi) {
+        // this wave's rows do not see the tile at all: probabilities of zero
+#pragma unroll
+        for (int r = 0; r < 16; r++) asm volatile("v_mov_b32 %0, %1" : "+v"(c[r]) : "v"(ninf), "v"(after));
+    } else {
+        // register r of this lane: key kb + 16*(r/8) + 8*g + r%8, row n; some
+        // (row, key) pair of the tile is above the diagonal or below the window
+        const uint32_t kb = tile * kTileKeys;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const uint32_t key = kb + 16 * (r >> 3) + 8 * g + (r & 7);
+            const uint64_t hide = __builtin_amdgcn_ballot_w64(key > R.pos || key < R.row_lo);
+            asm volatile("v_cndmask_b32 %0, %0, %1, %2" : "+v"(c[r]) : "v"(ninf), "s"(hide), "v"(after));
+        }
+    }
+}
+
+// The softmax reference of a row moves (rare, wave-uniform branch): this tile's
+// scores are shifted, the accumulators rescaled and the block of -m rewritten.
+template <int HD>
+__device__ __forceinline__ void il_move_reference(PrefillRows<HD>& R, IlCtx<HD>& cx, f32x16& negm,
+                                                  f32x16& c, float tmax, bool jump)
+{
+    const bool unset = (R.m_run == -INFINITY);
+    const float delta = jump ? tmax : 0.f;
+    const float alpha = jump ? (unset ? 0.f : fast_exp2(-delta)) : 1.0f;
+    R.l_run *= alpha;
+#pragma unroll
+    for (int dt = 0; dt < HD / 32; dt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) R.o[dt][r] *= alpha;
+    // updated in place with the instructions spelled out: left to itself the
+    // compiler gives the updated values new registers and pays with 32 copies
+    // on the path that skips this branch, which is the one that matters
+#pragma unroll
+    for (int r = 0; r < 16; r++) asm volatile("v_sub_f32 %0, %0, %1" : "+v"(c[r]) : "v"(delta));
+    if (jump) R.m_run = (unset ? 0.f : R.m_run) + delta;
+    const bool still = (R.m_run == -INFINITY);
+    const float nm = still ? 0.f : -R.m_run;
+#pragma unroll
+    for (int r = 0; r < 16; r++) asm volatile("v_mov_b32 %0, %1" : "+v"(negm[r]) : "v"(nm));
+    asm volatile("v_mov_b32 %0, %1" : "+v"(cx.thr) : "v"(still ? -INFINITY : kLazyLog2));
+}
 
 // The row maximum of the scores in `c` joined across the two lanes of a row and,
 // rarely, a move of the row's reference.
 template <int HD>
-__device__ __forceinline__ void il_settle(PrefillRows<HD>& R, PpCtx<HD>& cx, f32x16& negm, f32x16& c, float tmax)
+__device__ __forceinline__ void il_settle(PrefillRows<HD>& R, IlCtx<HD>& cx, f32x16& negm, f32x16& c, float tmax)
 {
     {
         const uint32_t u = __float_as_uint(tmax);
@@ -40,14 +299,14 @@ __device__ __forceinline__ void il_settle(PrefillRows<HD>& R, PpCtx<HD>& cx, f32
         tmax = max3_raw(__uint_as_float(sw[0]), __uint_as_float(sw[1]), tmax);   // same in both lanes of a row
     }
     const bool jump = tmax > cx.thr;                      // thr: -inf until the row has a reference, then kLazyLog2
-    if (__builtin_amdgcn_ballot_w64(jump) != 0) pp_move_reference<HD>(R, cx, negm, c, tmax, jump);
+    if (__builtin_amdgcn_ballot_w64(jump) != 0) il_move_reference<HD>(R, cx, negm, c, tmax, jump);
 }
 
 // Step j of a wave (P == j % kRing).  On entry `cur` holds the scores of the set's
 // tile j (masked, reference settled), kf the K operands of tile j+1; on exit `nxt`
 // holds the scores of tile j+1 in the same state and kf the operands of tile j+2.
 template <int HD, int P>
-__device__ __forceinline__ void il_step(PrefillRows<HD>& R, PpCtx<HD>& cx, f32x16& negm, const f32x16& cur,
+__device__ __forceinline__ void il_step(PrefillRows<HD>& R, IlCtx<HD>& cx, f32x16& negm, const f32x16& cur,
                                         f32x16& nxt, u32x4 (&pop)[2], half8 (&kf)[HD / 16],
                                         half8 (&vf)[HD / 16], unsigned char* smem, uint32_t j, int sub,
                                         int lane, int g, uint32_t kv_valid)
@@ -80,41 +339,36 @@ __device__ __forceinline__ void il_step(PrefillRows<HD>& R, PpCtx<HD>& cx, f32x1
             psum = __builtin_amdgcn_fdot2(ph, ones, psum, false);
             pop[r >> 3][(r & 7) >> 1] = __builtin_bit_cast(uint32_t, ph);
         }
+        // every link keeps its own share of the vector work behind it (left to
+        // itself the scheduler bunches the exponentials behind the first links,
+        // and both waves of a SIMD then leave the matrix pipe idle together)
+        __builtin_amdgcn_sched_barrier(0);
     }
     R.l_run += psum;
-    // requested order of the first half: each link of the chain, one operand read,
-    // then its share of the exponentials, packs and sums (masks: 0x8 MFMA, 0x100
-    // LDS read, 0x2 vector ALU)
-#pragma unroll
-    for (int i = 0; i < NS; i++) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x002, 4 * PAIRS, 0);
-    }
 #pragma unroll
     for (int i = 0; i < NS; i++) {
         const int t = i / ND, dt = i % ND;
         R.o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[i], __builtin_bit_cast(half8, pop[t]), R.o[dt], 0, 0,
                                                            0);
         kf[i] = *reinterpret_cast<const half8*>(cx.kop[i] + KS * L::KTILE);
-        if (i < L::NL) pp_issue_k1<HD, KC>(cx, j + 4, i);
-        else if (i < 2 * L::NL) pp_issue_v1<HD, VC>(cx, j + 2, i - L::NL);
+        if (i < L::NL) il_issue_k1<HD, KC>(cx, j + 4, i);
+        else if (i < 2 * L::NL) il_issue_v1<HD, VC>(cx, j + 2, i - L::NL);
     }
     // The row maximum runs in the products' shadow as if the tile were plain; a
     // tile with invisible (row, key) pairs is masked afterwards and its maximum
     // taken again (rare, wave-uniform).  Kept behind the products so that the
     // whole step up to here is one block the scheduler can interleave.
-    float tmax = pp_max16(nxt);
+    float tmax = il_max16(nxt);
     const uint32_t jt = j + 1;
     if (jt < cx.pl_lo || jt > cx.pl_hi) {
-        pp_mask_special<HD>(R, cx, nxt, cx.t0 + 2 * jt, jt, g, tmax);
-        tmax = pp_max16(nxt);
+        il_mask_special<HD>(R, cx, nxt, cx.t0 + 2 * jt, jt, g, tmax);
+        tmax = il_max16(nxt);
     }
     il_settle<HD>(R, cx, negm, nxt, tmax);
     // all copies but this step's have landed: K of tile j+3 and Vt of tile j+1,
     // which the next step reads once the barrier has published them
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * L::NL) : "memory");
-    pp_patch_tail<HD, TS>(smem, cx, j + 1, sub, lane, kv_valid);
+    il_patch_tail<HD, TS>(smem, cx, j + 1, sub, lane, kv_valid);
     // (no wait for this step's K operand reads here: their slot is not overwritten
     // before the step after next, long after the next chain has consumed them)
     __builtin_amdgcn_sched_barrier(0);
@@ -128,11 +382,6 @@ __device__ __forceinline__ void il_block(const PrefillArgs& a, unsigned char* sm
 {
     using L = SplitLds<HD>;
     static_assert(L::NL == 1 || L::NL == 2, "one or two copies per wave, tile and operand");
-#ifdef WR_PP_PROF
-    __builtin_amdgcn_sched_barrier(0);
-    const unsigned long long il_ta = clock64();
-    __builtin_amdgcn_sched_barrier(0);
-#endif
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // in a scalar register
@@ -150,7 +399,7 @@ __device__ __forceinline__ void il_block(const PrefillArgs& a, unsigned char* sm
     PrefillRows<HD> R;
     prefill_rows_init<HD, false>(R, a, row0, head, n, g);
 
-    PpCtx<HD> cx;
+    IlCtx<HD> cx;
     cx.t0 = t_first + kg;                                 // this set's tiles: t0, t0 + 2, ...
     cx.nt = (cx.t0 <= t_last) ? (t_last - cx.t0) / 2 + 1 : 0;
     cx.t_last = t_last;
@@ -216,17 +465,12 @@ __device__ __forceinline__ void il_block(const PrefillArgs& a, unsigned char* sm
     // fewer and spends its last step on probabilities of zero); the same in every wave
     const uint32_t nsteps = (t_last - t_first) / 2 + 1;
 
-#ifdef WR_PP_PROF
-    __builtin_amdgcn_sched_barrier(0);
-    const unsigned long long il_tb = clock64();
-    __builtin_amdgcn_sched_barrier(0);
-#endif
     // everything the first two vector blocks read, in order of need
-    pp_issue_k<HD, 0>(cx, 0);
-    pp_issue_k<HD, 1>(cx, 1);
-    pp_issue_v<HD, 0>(cx, 0);
-    pp_issue_k<HD, 2>(cx, 2);
-    pp_issue_v<HD, 1>(cx, 1);
+    il_issue_k<HD, 0>(cx, 0);
+    il_issue_k<HD, 1>(cx, 1);
+    il_issue_v<HD, 0>(cx, 0);
+    il_issue_k<HD, 2>(cx, 2);
+    il_issue_v<HD, 1>(cx, 1);
 
     // Q: every row is 4*HD contiguous bytes in global memory, so it is read with
     // whole-row coalesced loads (the two waves serving a sub-block take 16 rows
@@ -250,17 +494,14 @@ __device__ __forceinline__ void il_block(const PrefillArgs& a, unsigned char* sm
             *reinterpret_cast<half4*>(&qs[sub][r][(lane % LPR) * 4]) = h;
         }
     }
-#ifdef WR_PP_PROF
-    const unsigned long long il_t0 = clock64();
-#endif
     f32x16 sa, sb, negm;
     u32x4 pop[2];
     half8 kf[HD / 16], vf[HD / 16];
 #pragma unroll
     for (int r = 0; r < 16; r++) sa[r] = sb[r] = negm[r] = 0.f;
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    pp_patch_tail<HD, 0>(smem, cx, 0, sub, lane, kv_valid);
-    pp_barrier();                                         // first tiles and Q visible to all
+    il_patch_tail<HD, 0>(smem, cx, 0, sub, lane, kv_valid);
+    il_barrier();                                         // first tiles and Q visible to all
 #pragma unroll
     for (int i = 0; i < HD / 16; i++)
         R.qop[i] = *reinterpret_cast<const half8*>(&qs[sub][n][i * 16 + g * 8]);
@@ -270,26 +511,23 @@ __device__ __forceinline__ void il_block(const PrefillArgs& a, unsigned char* sm
 #pragma unroll
     for (int i = 0; i < HD / 16; i++)
         sa = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[i], R.qop[i], sa, 0, 0, 0);
-    pp_barrier();                                         // slot 0 of K has been read by all: it is refilled
-    pp_issue_k<HD, 0>(cx, 3);
+    il_barrier();                                         // slot 0 of K has been read by all: it is refilled
+    il_issue_k<HD, 0>(cx, 3);
 #pragma unroll
     for (int i = 0; i < HD / 16; i++) kf[i] = *reinterpret_cast<const half8*>(cx.kop[i] + L::KTILE);
     {
-        float tmax0 = pp_max16(sa);
+        float tmax0 = il_max16(sa);
         if (0 < cx.pl_lo || 0 > cx.pl_hi) {
-            pp_mask_special<HD>(R, cx, sa, cx.t0, 0, g, tmax0);
-            tmax0 = pp_max16(sa);
+            il_mask_special<HD>(R, cx, sa, cx.t0, 0, g, tmax0);
+            tmax0 = il_max16(sa);
         }
         il_settle<HD>(R, cx, negm, sa, tmax0);
     }
-    pp_barrier();                                         // slot 1 of K has been read by all: step 0 refills it
+    il_barrier();                                         // slot 1 of K has been read by all: step 0 refills it
 
     // steps of the loop: the even set's tile count (the odd set has as many or one
     // fewer and spends its last step on probabilities of zero); the same in every
     // wave, and every step ends with the workgroup's barrier
-#ifdef WR_PP_PROF
-    const unsigned long long il_t1 = clock64();
-#endif
 #define WR_IL_STEP(PHASE, CUR, NXT)                                                          \
     il_step<HD, PHASE>(R, cx, negm, CUR, NXT, pop, kf, vf, smem, j, sub, lane, g, kv_valid); \
     if (++j >= nsteps) break;
@@ -303,9 +541,6 @@ __device__ __forceinline__ void il_block(const PrefillArgs& a, unsigned char* sm
         WR_IL_STEP(2, sb, sa)
     }
 #undef WR_IL_STEP
-#ifdef WR_PP_PROF
-    const unsigned long long il_t2 = clock64();
-#endif
 
     // merge the odd-tile partials into the even-tile waves; the ring must be
     // quiet first (the last steps' copies still target it)
@@ -365,28 +600,18 @@ __device__ __forceinline__ void il_block(const PrefillArgs& a, unsigned char* sm
                                            (lane % LPR) * 4) = v;
         }
     }
-#ifdef WR_PP_PROF
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    if (blockIdx.x == 0 && blockIdx.y == 0 && lane == 0 && sub == 0) {
-        const unsigned long long il_t3 = clock64();
-        wr_pp_prof[kg][0] += il_t1 - il_t0;      // prologue (from the first copies to the loop)
-        wr_pp_prof[kg][4] += il_tb - il_ta;      // setup
-        wr_pp_prof[kg][5] += il_t0 - il_tb;      // first copies issued, Q loaded and staged
-        wr_pp_prof[kg][1] += il_t2 - il_t1;      // loop
-        wr_pp_prof[kg][2] += il_t3 - il_t2;      // merge and store
-        wr_pp_prof[kg][6] += nsteps;
-    }
-#endif
 }
 
-// grid and block pairing as prefill_pp_kernel
+// grid = (KV heads x head chunks, ceil(blocks / 2)): consecutive workgroups (which
+// the dispatcher deals round-robin to the XCDs) differ in KV head, so one XCD's
+// L2 keeps seeing the same few heads' K / Vt.  Workgroup y takes position block
+// (blocks-1-y) and then block y: a long block and a short one, so every
+// workgroup streams the same number of tiles despite the causal triangle.
+// a.single: grid.y = blocks, one block per workgroup, long blocks first.
 template <int HD>
 __global__ __launch_bounds__(kSplitThreads, 1) void prefill_il_kernel(const PrefillArgs a)
 {
     extern __shared__ __attribute__((aligned(16))) unsigned char prefill_smem_raw[];
-#ifdef WR_PP_PROF
-    const unsigned long long k_t0 = clock64();
-#endif
     const uint32_t G = a.group;
     const uint32_t Gw = G < 4 ? G : 4;
     const uint32_t chunks = G / Gw;
@@ -403,15 +628,6 @@ __global__ __launch_bounds__(kSplitThreads, 1) void prefill_il_kernel(const Pref
         }
         il_block<HD>(a, prefill_smem_raw, pass ? lo : hi, kvh, hc);
     }
-#ifdef WR_PP_PROF
-    if (threadIdx.x == 0) {
-        const unsigned long long k_t1 = clock64();
-        atomicMax(&wr_pp_prof[1][3], k_t1 - k_t0);               // longest workgroup
-        atomicMin(&wr_pp_prof[1][4], k_t0);                       // first entry (array cleared to ~0 by the reader)
-        atomicMax(&wr_pp_prof[1][5], k_t1);                       // last exit
-        if (blockIdx.x == 0 && blockIdx.y == 0) wr_pp_prof[0][3] = k_t1 - k_t0;
-    }
-#endif
 }
 
 }  // namespace wr

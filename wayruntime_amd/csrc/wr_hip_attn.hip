@@ -23,7 +23,6 @@
 #include "kernels_append.hip.h"
 #include "kernels_decode.hip.h"
 #include "kernels_prefill.hip.h"
-#include "kernels_prefill_pp.hip.h"
 #include "kernels_prefill_il.hip.h"
 #include "kernels_proj.hip.h"
 #include "kernels_rows.hip.h"
@@ -84,9 +83,12 @@ struct Lib {
     Buffer d_proj;               // projection operand fragments and row scales
     uint32_t* d_counters = nullptr;   // split-K tickets, zero whenever no launch is in flight
     unsigned char* noalloc_ws[kMaxDevices] = {};   // device address of `scratch`, per device
-    // Error word: page-locked host memory that kernels can write.  A kernel whose
-    // bounded wait expires stores kDevErrWaitExpired | layer there; the host reads
-    // it after every wait for the stream (no copy, no extra latency).
+    // Error word: page-locked host memory that kernels can write.  A kernel that
+    // gives up a bounded wait (and so goes on with data it cannot vouch for) stores
+    // (bit 31 | layer) there; the host reads it after every wait for the
+    // stream (no copy, no extra latency).  None of the present kernels waits on
+    // anything but the hardware barrier, so nothing writes it today; a kernel that
+    // spins on a flag must bound the spin and report here.
     volatile uint32_t* err_host = nullptr;
     uint32_t* err_dev = nullptr;
     Buffer h_pin;                // pinned host staging
@@ -100,6 +102,7 @@ struct Lib {
     bool profiling = false;
 } g;
 
+constexpr uint32_t kDevErrLayerMask = 0x0000FFFFu;     // error word: bit 31 set (kDevErrWaitExpired), the layer in the low bits
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr uint32_t kDefaultTilesPerWg = 32;  // split-K decode: 1024 keys per workgroup
 constexpr uint32_t kMaxHeads = 4096;        // query heads per session the ticket array is sized for
@@ -254,7 +257,7 @@ void launch_main(Kern kernel, dim3 grid, dim3 block, const Args& args, size_t ld
 
 bool mfma_shape(uint32_t hd, uint32_t group)
 {
-    return g.force_generic != 1 && (hd == 64 || hd == 128 || hd == 256) && group <= kMaxGroupMfma;
+    return !g.force_generic && (hd == 64 || hd == 128 || hd == 256) && group <= kMaxGroupMfma;
 }
 
 int check_layer(const wr_hip_kv* kv, uint32_t layer)
@@ -502,12 +505,10 @@ int prefill_locked(wr_hip_kv* kv, uint32_t layer, uint32_t p0, uint32_t T, const
     a.hd = hd;
     a.ctx_pad = kv->ctx_pad;
     a.window = window;
-    a.err = g.err_dev;
-    a.err_code = kDevErrWaitExpired | (layer & kDevErrLayerMask);
     const float scale = (scale_override > 0.0f) ? scale_override : 1.0f / sqrtf((float)hd);
     a.qscale = scale * kLog2e;
     const uint32_t G = a.group;
-    const bool mfma = g.force_generic != 1 && (hd == 64 || hd == 128 || hd == 256) &&
+    const bool mfma = !g.force_generic && (hd == 64 || hd == 128 || hd == 256) &&
                       (G == 1 || G == 2 || G == 4 || G == 8);
     if (mfma) {
         const uint32_t Gw = G < 4 ? G : 4;
@@ -521,20 +522,7 @@ int prefill_locked(wr_hip_kv* kv, uint32_t layer, uint32_t p0, uint32_t T, const
         // prologue and epilogue.
         a.single = ((nblk + 1) / 2) * ny < g.n_cus ? 1 : 0;
         const uint32_t nwg = a.single ? nblk : (nblk + 1) / 2;
-        const bool drift = g.force_generic == 2;           // measurement: the free-running kernel
-        if (hd == 64 && drift)
-            launch_main(prefill_split_kernel<64>, dim3(ny, nwg), dim3(kSplitThreads), a,
-                        split_smem_bytes<64>());
-        else if (hd == 128 && drift)
-            launch_main(prefill_split_kernel<128>, dim3(ny, nwg), dim3(kSplitThreads), a,
-                        split_smem_bytes<128>());
-        else if (hd == 64 && g.force_generic == 3)
-            launch_main(prefill_pp_kernel<64>, dim3(ny, nwg), dim3(kSplitThreads), a,
-                        split_smem_bytes<64>());
-        else if (hd == 128 && g.force_generic == 3)
-            launch_main(prefill_pp_kernel<128>, dim3(ny, nwg), dim3(kSplitThreads), a,
-                        split_smem_bytes<128>());
-        else if (hd == 64)
+        if (hd == 64)
             launch_main(prefill_il_kernel<64>, dim3(ny, nwg), dim3(kSplitThreads), a,
                         split_smem_bytes<64>());
         else if (hd == 128)
@@ -841,27 +829,11 @@ int wr_hip_attn_init(int device)
     if (rc == WR_HIP_OK) {
         // the two-waves-per-SIMD prefill kernels stage more than the 64 KiB a
         // kernel may use without asking
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(prefill_split_kernel<64>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(prefill_il_kernel<64>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize,
                                            (int)split_smem_bytes<64>());
         if (e == hipSuccess)
-            e = hipFuncSetAttribute(reinterpret_cast<const void*>(prefill_split_kernel<128>),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    (int)split_smem_bytes<128>());
-        if (e == hipSuccess)
-            e = hipFuncSetAttribute(reinterpret_cast<const void*>(prefill_il_kernel<64>),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    (int)split_smem_bytes<64>());
-        if (e == hipSuccess)
             e = hipFuncSetAttribute(reinterpret_cast<const void*>(prefill_il_kernel<128>),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    (int)split_smem_bytes<128>());
-        if (e == hipSuccess)
-            e = hipFuncSetAttribute(reinterpret_cast<const void*>(prefill_pp_kernel<64>),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    (int)split_smem_bytes<64>());
-        if (e == hipSuccess)
-            e = hipFuncSetAttribute(reinterpret_cast<const void*>(prefill_pp_kernel<128>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize,
                                     (int)split_smem_bytes<128>());
         if (e == hipSuccess)
@@ -1647,20 +1619,5 @@ int wr_hip_attn_profile_end(double* total_ms, uint32_t* n_launches)
     g.ev_used = 0;
     return WR_HIP_OK;
 }
-
-#ifdef WR_PP_PROF
-// measurement build only: reads and clears the prefill kernel's phase counters
-int wr_hip_debug_pp_prof(unsigned long long* out16)
-{
-    Locked lk;
-    (void)hipStreamSynchronize(g.stream);
-    if (hipMemcpyFromSymbol(out16, HIP_SYMBOL(wr_pp_prof), 16 * sizeof(unsigned long long)) != hipSuccess)
-        return WR_HIP_ERR_INTERNAL;
-    unsigned long long z[16] = {};
-    z[8 + 4] = ~0ull;                                     // slot that takes a minimum
-    (void)hipMemcpyToSymbol(HIP_SYMBOL(wr_pp_prof), z, sizeof z);
-    return WR_HIP_OK;
-}
-#endif
 
 }  // extern "C"
