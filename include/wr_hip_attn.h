@@ -189,6 +189,18 @@ int wr_hip_attn_append_batched_dev(uint32_t n, wr_hip_kv *const *kv,
  * the library's stream like the other *_dev calls. */
 int wr_hip_attn_rope_dev(void *x_dev, const void *cos_sin_dev, uint32_t rows,
                          uint32_t heads, uint32_t hd, uint32_t n_rot);
+/* The table that rotation takes, made on the device: cos_sin_dev, device F32
+ * [rows, n_rot, 2], receives (cos, sin) of position / base^(2j/hd) for row r's
+ * position (pos[r] when pos, a host array of rows <= WR_HIP_BATCH_MAX entries,
+ * is not NULL; pos0 + r otherwise) and pair j < n_rot, where n_rot is
+ * n_rot_pairs when that is in [1, hd/2) and hd/2 otherwise, and a base below 1
+ * stands for 10000 (the angle of wri_op_rope, src/core/kernels.c:1384-1404,
+ * through the polynomials and the range reduction of src/core/mathx.c:37-57,
+ * :72-86 and :112-147 operation for operation: the bytes equal what the
+ * reference computes per element).  Asynchronous on the library's stream. */
+int wr_hip_attn_rope_table_dev(float *cos_sin_dev, uint32_t rows, uint32_t pos0,
+                               const uint32_t *pos, uint32_t hd,
+                               float theta_base, uint32_t n_rot_pairs);
 int wr_hip_attn_decode_batched_dev(uint32_t n, wr_hip_kv *const *kv,
                                    uint32_t layer, const uint32_t *seq_k,
                                    const float *q_dev, float *out_dev,

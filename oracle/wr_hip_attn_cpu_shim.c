@@ -257,6 +257,12 @@ int wr_hip_attn_decode_batched_dev(uint32_t n, wr_hip_kv *const *kv, uint32_t la
     (void)window;
     return WR_HIP_ERR_STATE;
 }
+int wr_hip_attn_rope_table_dev(float *cos_sin, uint32_t rows, uint32_t pos0, const uint32_t *pos,
+                               uint32_t hd, float theta_base, uint32_t n_rot_pairs)
+{
+    (void)cos_sin; (void)rows; (void)pos0; (void)pos; (void)hd; (void)theta_base; (void)n_rot_pairs;
+    return WR_HIP_ERR_STATE;
+}
 int wr_hip_attn_prefill_dev(wr_hip_kv *kv, uint32_t layer, uint32_t p0, uint32_t T, const float *q,
                             float *out, uint32_t nq, float scale_override, uint32_t window)
 {

@@ -281,3 +281,41 @@ def test_qkv_append_gemma_flags(hd):
         c.close()
     for b in bufs + [qx]:
         b.free()
+
+
+# The table the rotation takes, made on the device.  The reference reduces an
+# angle by one subtraction of 2*pi per turn, each rounded, and evaluates its own
+# polynomials (kernels.c:1384-1404, mathx.c:37-57, :72-86, :112-147); the device
+# restates them operation for operation, so the BYTES must be equal: every
+# position a 32768-token context can hold, for the bases of the three families
+# (Llama 5e5, Qwen3 1e6, Gemma's sliding-window layers 1e4) and a partial
+# rotation.
+@pytest.mark.parametrize("hd,theta,rot_pairs", [(128, 1e6, 0), (128, 5e5, 0), (256, 1e4, 0),
+                                                (64, 1e6, 0), (128, 1e6, 24), (96, 0.5, 0)])
+def test_rope_table_on_device_is_the_oracles_bytes(hd, theta, rot_pairs):
+    print("rope table", hd, theta, rot_pairs, flush=True)
+    n = 32768
+    want = oracle.rope_table(n, hd, 0, theta, rot_pairs)
+    got = hipattn.rope_table_dev(n, hd, theta, rot_pairs, pos0=0)
+    assert got.shape == want.shape
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    # a window that does not start at zero, and a ragged row count
+    got = hipattn.rope_table_dev(77, hd, theta, rot_pairs, pos0=31000)
+    assert np.array_equal(got.view(np.uint32), want[31000:31077].view(np.uint32))
+
+
+def test_rope_table_on_device_listed_positions():
+    positions = [0, 32767, 5, 4096, 4095, 1, 77, 20000, 31, 32, 33, 9999, 16384, 2, 3, 12345]
+    for n in (1, 7, 16):
+        got = hipattn.rope_table_dev(n, 128, 1e6, 0, pos=positions[:n])
+        want = np.concatenate([oracle.rope_table(1, 128, p, 1e6, 0) for p in positions[:n]])
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    lib = hipattn.lib()
+    buf = hipattn.DeviceBuffer(17 * 64 * 8)
+    import ctypes as C
+    plist = (C.c_uint32 * 17)(*range(17))
+    assert lib.wr_hip_attn_rope_table_dev(buf.p, 17, 0, plist, 128, 1e6, 0) == hipattn.ERR_INVAL
+    assert lib.wr_hip_attn_rope_table_dev(buf.p, 1, 0, None, 127, 1e6, 0) == hipattn.ERR_INVAL
+    assert lib.wr_hip_attn_rope_table_dev(None, 1, 0, None, 128, 1e6, 0) == hipattn.ERR_INVAL
+    assert lib.wr_hip_attn_rope_table_dev(buf.p, 0, 0, None, 128, 1e6, 0) == hipattn.ERR_INVAL
+    buf.free()

@@ -80,12 +80,10 @@ __global__ __launch_bounds__(256) void append_v_kernel(const Src* __restrict__ s
 // pairing (element j with element j + hd/2, j < n_rot), as the reference
 // applies it before the append (reference: src/core/kernels.c:1356-1412):
 //   r[j] = x0*c - x1*s,  r[j + hd/2] = x0*s + x1*c
-// with c = cs[row][j][0], s = cs[row][j][1].  The angles come from the caller:
-// the reference reduces them with a loop of single subtractions of 2*pi whose
-// rounding only the same loop reproduces, thousands of dependent steps at long
-// positions, which one CPU core runs faster than one GPU lane.  The products
-// and the sum are rounded separately (no fused multiply-add), so the rotated
-// values, and with them the cache bits, equal the reference's bit for bit.
+// with c = cs[row][j][0], s = cs[row][j][1], the table rope_table_kernel below
+// (or the caller) makes.  The products and the sum are rounded separately (no
+// fused multiply-add), so the rotated values, and with them the cache bits,
+// equal the reference's bit for bit.
 __global__ __launch_bounds__(256) void rope_rows_kernel(float* __restrict__ x,
                                                         const float* __restrict__ cs,
                                                         uint32_t rows, uint32_t heads,
@@ -108,6 +106,83 @@ __global__ __launch_bounds__(256) void rope_rows_kernel(float* __restrict__ x,
     const float a0 = x0 * c, b0 = x1 * sn, a1 = x0 * sn, b1 = x1 * c;
     row[j] = a0 - b0;
     row[j + half] = a1 + b1;
+}
+
+// ---- rotary angles ---------------------------------------------------------
+// (cos, sin) of angle(p, j) = p / base^(2j/hd) for `rows` positions and n_rot
+// pairs, out [rows][n_rot][2], through the reference's own scalar forms
+// operation for operation (reference: src/core/kernels.c:1384-1404 for the
+// angle, src/core/mathx.c:37-57 exp, :72-86 log, :112-147 range reduction, sine
+// and cosine), every operator rounded by itself, division and int conversion
+// as C has them: the table's bytes equal the reference's.
+//
+// The reference folds an angle into [-pi, pi] by subtracting 2*pi once per
+// turn, and each subtraction rounds: only the same loop gives the same bits,
+// thousands of dependent steps for the low pairs of a late position.  The
+// lanes of a wave therefore take 64 consecutive ROWS of one pair: their angles
+// differ by at most 63 / base^(2j/hd), so all 64 leave the loop within a few
+// turns of each other and a wave costs what its slowest lane costs; a launch
+// has (rows / 64) x n_rot such waves, and the higher pairs (the angle shrinks
+// geometrically with j) finish early and free their slots.
+struct RopeTableArgs {
+    float* out;
+    uint32_t rows, hd, n_rot;
+    float theta;
+    uint32_t pos0;
+    uint32_t listed;          // rows <= 16 positions given one by one
+    uint32_t pos[16];
+};
+
+__device__ __forceinline__ float ref_exp(float x)
+{
+#pragma clang fp contract(off)
+    if (x < -88.0f) return 0.0f;
+    if (x > 88.0f) return 1e38f;
+    const float ln2 = 0.6931471805599453f;
+    const int k = (int)(x / ln2 + (x >= 0 ? 0.5f : -0.5f));
+    const float r = x - (float)k * ln2;
+    const float r2 = r * r;
+    float e = 1.0f + r + r2 * 0.5f + r2 * r * (1.0f / 6.0f) + r2 * r2 * (1.0f / 24.0f) +
+              r2 * r2 * r * (1.0f / 120.0f);
+    if (k >= -126 && k <= 127) e = __uint_as_float(__float_as_uint(e) + ((uint32_t)k << 23));
+    return e;
+}
+
+__device__ __forceinline__ float ref_log(float x)
+{
+#pragma clang fp contract(off)
+    if (x <= 0.0f) return -1e38f;
+    const uint32_t u = __float_as_uint(x);
+    const int e = (int)((u >> 23) & 0xFF) - 127;
+    const float m = __uint_as_float((u & 0x007FFFFFu) | 0x3F800000u);
+    const float t = (m - 1.0f) / (m + 1.0f);
+    const float t2 = t * t;
+    const float lnm =
+        2.0f * t * (1.0f + t2 * (1.0f / 3.0f + t2 * (1.0f / 5.0f + t2 * (1.0f / 7.0f))));
+    return lnm + (float)e * 0.6931471805599453f;
+}
+
+__global__ __launch_bounds__(64) void rope_table_kernel(const RopeTableArgs a)
+{
+#pragma clang fp contract(off)
+    const uint32_t r = blockIdx.x * 64u + threadIdx.x;
+    const uint32_t j = blockIdx.y;
+    if (r >= a.rows) return;
+    const uint32_t p = a.listed ? a.pos[r & 15u] : a.pos0 + r;
+    const float lnb = ref_log(a.theta);
+    const float exponent = (float)(2u * j) / (float)a.hd;
+    const float powv = ref_exp(exponent * lnb);
+    float x = (float)p / powv;
+    const float pi = 3.14159265358979f, two_pi = 6.28318530717958f;
+    while (x > pi) x -= two_pi;
+    while (x < -pi) x += two_pi;
+    const float x2 = x * x;
+    const float x3 = x2 * x, x5 = x3 * x2, x7 = x5 * x2;
+    const float sn = x - x3 * (1.0f / 6.0f) + x5 * (1.0f / 120.0f) - x7 * (1.0f / 5040.0f);
+    const float x4 = x2 * x2, x6 = x4 * x2;
+    const float cs = 1.0f - x2 * 0.5f + x4 * (1.0f / 24.0f) - x6 * (1.0f / 720.0f);
+    float2* o = reinterpret_cast<float2*>(a.out) + ((size_t)r * a.n_rot + j);
+    *o = make_float2(cs, sn);
 }
 
 // One new row for each of up to 16 sessions in one launch (the batched decode

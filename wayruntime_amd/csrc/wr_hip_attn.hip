@@ -1037,6 +1037,30 @@ int wr_hip_attn_rope_dev(void* x_dev, const void* cos_sin_dev, uint32_t rows, ui
     return WR_HIP_OK;
 }
 
+int wr_hip_attn_rope_table_dev(float* cos_sin_dev, uint32_t rows, uint32_t pos0,
+                               const uint32_t* pos, uint32_t hd, float theta_base,
+                               uint32_t n_rot_pairs)
+{
+    if (!g.inited) return WR_HIP_ERR_STATE;
+    if (!cos_sin_dev || rows == 0) return WR_HIP_ERR_INVAL;
+    if (hd < 2 || (hd & 1)) return WR_HIP_ERR_INVAL;
+    if (pos && rows > WR_HIP_BATCH_MAX) return WR_HIP_ERR_INVAL;
+    if (!pos && (uint64_t)pos0 + rows > (1ull << 32)) return WR_HIP_ERR_INVAL;
+    RopeTableArgs a{};
+    a.out = cos_sin_dev;
+    a.rows = rows;
+    a.hd = hd;
+    a.n_rot = (n_rot_pairs >= 1 && n_rot_pairs < hd / 2) ? n_rot_pairs : hd / 2;
+    a.theta = theta_base < 1.0f ? 10000.0f : theta_base;
+    a.pos0 = pos0;
+    a.listed = pos ? 1u : 0u;
+    for (uint32_t i = 0; pos && i < rows; i++) a.pos[i] = pos[i];
+    Locked lk;
+    hipLaunchKernelGGL(rope_table_kernel, dim3((rows + 63u) / 64u, a.n_rot), dim3(64), 0, g.stream, a);
+    HIP_TRY(hipGetLastError(), "rotary table launch", 0);
+    return WR_HIP_OK;
+}
+
 int wr_hip_attn_append_rope(wr_hip_kv* kv, uint32_t layer, uint32_t pos, uint32_t n_rows,
                             const float* k_f32, const float* v_f32, const float* cos_sin,
                             uint32_t n_rot)

@@ -64,6 +64,8 @@ def load() -> C.CDLL:
                                                      _vp, _vp]),
         "wr_hip_attn_append_rope": (C.c_int, [_vp, _u32, _u32, _u32, _vp, _vp, _vp, _u32]),
         "wr_hip_attn_rope_dev": (C.c_int, [_vp, _vp, _u32, _u32, _u32, _u32]),
+        "wr_hip_attn_rope_table_dev": (C.c_int, [_vp, _u32, _u32, C.POINTER(_u32), _u32, C.c_float,
+                                                 _u32]),
         "wr_hip_attn_decode_batched_dev": (C.c_int, [_u32, C.POINTER(_vp), _u32, C.POINTER(_u32),
                                                      _vp, _vp, _u32, C.c_float, _u32]),
         "wr_hip_attn_decode_batched_dev_noalloc": (C.c_int, [_u32, C.POINTER(_vp), _u32,
@@ -307,6 +309,24 @@ def append_dev(cache: KVCache, layer: int, pos: int, n_rows: int, k_dev: DeviceB
 def rope_dev(x_dev: DeviceBuffer, cos_sin_dev: DeviceBuffer, rows: int, heads: int, hd: int,
              n_rot: int) -> None:
     _check(lib().wr_hip_attn_rope_dev(x_dev.p, cos_sin_dev.p, rows, heads, hd, n_rot), "rope_dev")
+
+
+def rope_table_dev(rows: int, hd: int, theta: float, n_rot_pairs: int = 0, pos0: int = 0,
+                   pos=None) -> np.ndarray:
+    """The rotary table made on the device (wr_hip_attn_rope_table_dev), brought
+    down: float32 [rows, n_rot, 2] of (cos, sin) for positions pos0 + r, or the
+    listed ones."""
+    n_rot = n_rot_pairs if 1 <= n_rot_pairs < hd // 2 else hd // 2
+    buf = DeviceBuffer(rows * n_rot * 8)
+    try:
+        plist = None
+        if pos is not None:
+            plist = (_u32 * len(pos))(*[int(p) for p in pos])
+        _check(lib().wr_hip_attn_rope_table_dev(buf.p, rows, pos0, plist, hd, theta, n_rot_pairs),
+               "rope_table_dev")
+        return buf.to_host((rows, n_rot, 2))
+    finally:
+        buf.free()
 
 
 class Weight:

@@ -275,20 +275,12 @@ static wr_status dev_fail(wr_engine *e, const char *what, uint32_t layer, int rc
         if (rc != WR_HIP_OK) return dev_fail(e, what, L, rc);  \
     } while (0)
 
-/* Host part of a pass: embedding rows and rotary angles of R tokens into the
- * host workspace, rows in parallel (the angles go through the reference's
- * scalar polynomials: four microseconds a position on one core). */
-static wr_status stage_rows(wr_model *m, wrh_workspace *hs, uint32_t R, wr_session *const *ss,
-                            const uint32_t *tokens, uint32_t pos0, int batch)
+/* Host part of a pass: the embedding rows of R tokens into the host workspace,
+ * rows in parallel.  (The rotary angles are made on the device, where the
+ * cache lives: wr_hip_attn_rope_table_dev.) */
+static wr_status stage_rows(wr_model *m, wrh_workspace *hs, uint32_t R, const uint32_t *tokens)
 {
-    const uint32_t hidden = m->hidden, hd = m->head_dim;
-    const uint32_t n_rot = (m->n_rot_pairs >= 1 && m->n_rot_pairs < hd / 2) ? m->n_rot_pairs : hd / 2;
-    const size_t ts = (size_t)2 * n_rot;
-    /* Gemma: scaled embeddings, and a second table for the sliding-window
-     * layers (their own head_dim and base, full rotation; session.c:262-283) */
-    const uint32_t hd_s = m->head_dim_swa ? m->head_dim_swa : hd;
-    const size_t ts_s = hd_s;                             /* hd_s / 2 pairs of two */
-    const int swa = m->is_gemma && m->has_swa;
+    const uint32_t hidden = m->hidden;
     const wr_engine *e = m->engine;
     const int threads = (e && e->n_threads > 0) ? e->n_threads : 1;
     int bad = WR_OK;
@@ -297,10 +289,8 @@ static wr_status stage_rows(wr_model *m, wrh_workspace *hs, uint32_t R, wr_sessi
         float *row = hs->residual + (size_t)r * hidden;
         const int rc = wrh_embed(&m->embed, tokens[r], row);
         if (rc != WR_OK) __atomic_store_n(&bad, rc, __ATOMIC_RELAXED);
+        /* Gemma: scaled embeddings (session.c:262-283) */
         if (m->is_gemma && m->embed_scale != 0.0f) wrh_scale(row, hidden, m->embed_scale);
-        const uint32_t p = batch ? ss[r]->pos : pos0 + r;
-        (void)wrh_rope_table(hs->rope + r * ts, hd, p, m->rope_base, m->n_rot_pairs);
-        if (swa) (void)wrh_rope_table(hs->rope_swa + r * ts_s, hd_s, p, m->rope_base_swa, 0);
     }
     return (wr_status)bad;
 }
@@ -312,7 +302,7 @@ void wrh_stage_next_rows(wr_model *m, wrh_workspace *hs, uint32_t R, const uint3
                          uint32_t pos0)
 {
     hs->staged_rows = 0;
-    if (stage_rows(m, hs, R, NULL, tokens, pos0, 0) != WR_OK) return;   /* the pass itself reports it */
+    if (stage_rows(m, hs, R, tokens) != WR_OK) return;   /* the pass itself reports it */
     hs->staged_tokens = tokens;
     hs->staged_rows = R;
     hs->staged_pos0 = pos0;
@@ -333,22 +323,30 @@ wr_status wrh_forward_rows_device(wr_model *m, wrh_workspace *hs, wrh_devspace *
     const uint32_t hidden = m->hidden, hd = m->head_dim, nq = m->n_q, nkv = m->n_kv;
     const uint32_t ffn = m->ffn;
     const uint32_t n_rot = (m->n_rot_pairs >= 1 && m->n_rot_pairs < hd / 2) ? m->n_rot_pairs : hd / 2;
-    const size_t ts = (size_t)2 * n_rot;
     uint32_t L = 0;
     int rc;
 
     const int staged = !batch && hs->staged_rows == R && hs->staged_tokens == tokens && hs->staged_pos0 == pos0;
     hs->staged_rows = 0;
     if (!staged) {
-        rc = stage_rows(m, hs, R, ss, tokens, pos0, batch);
+        rc = stage_rows(m, hs, R, tokens);
         if (rc != WR_OK) return dev_fail(e, "embed", 0, rc);
     }
     TRY(wr_hip_attn_h2d(ds->resid, hs->residual, (size_t)R * hidden * sizeof(float)), "rows up");
-    TRY(wr_hip_attn_h2d(ds->rope, hs->rope, (size_t)R * ts * sizeof(float)), "angles up");
+    /* rotary tables of the rows' positions; Gemma's sliding-window layers have
+     * their own head_dim and base and rotate fully (session.c:262-283) */
+    uint32_t plist[WR_HIP_BATCH_MAX];
+    if (batch) {
+        if (R > WR_HIP_BATCH_MAX) return dev_fail(e, "angles", 0, WR_HIP_ERR_INVAL);
+        for (uint32_t r = 0; r < R; r++) plist[r] = ss[r]->pos;
+    }
+    TRY(wr_hip_attn_rope_table_dev(ds->rope, R, pos0, batch ? plist : NULL, hd, m->rope_base,
+                                   m->n_rot_pairs), "angles");
     const int gemma = m->is_gemma;
     const uint32_t hd_s = m->head_dim_swa ? m->head_dim_swa : hd;
     if (gemma && m->has_swa)
-        TRY(wr_hip_attn_h2d(ds->rope_swa, hs->rope_swa, (size_t)R * hd_s * sizeof(float)), "angles up");
+        TRY(wr_hip_attn_rope_table_dev(ds->rope_swa, R, pos0, batch ? plist : NULL, hd_s,
+                                       m->rope_base_swa, 0), "angles");
     const float scale = gemma ? m->attn_scale : 0.0f;
 
     for (L = 0; L < m->n_layers; L++) {
