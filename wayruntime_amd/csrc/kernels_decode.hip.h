@@ -102,6 +102,7 @@ __device__ __forceinline__ TileRange split_tiles(const DecodeSession& S, uint32_
 // heads (log-sum-exp over the split maxima, one normalisation), writes the
 // final rows and puts the counter back to zero for the next launch.
 constexpr int kMaxSplits = 64;        // key splits per session (host picks tiles_per_wg to respect it)
+constexpr int kMergeInRegs = 8;       // up to this many partials a merge holds in registers
 static_assert(kTileKeys == kKTile, "decode tiles are the cache's K tiles");
 static_assert(sizeof(DecodeArgs::items) == kBatchMax * kMaxSplits * sizeof(uint16_t), "work list size");
 
@@ -145,6 +146,43 @@ __device__ __forceinline__ void publish_and_merge(const DecodeArgs& a, uint32_t 
     if (s_ticket != n_splits - 1) return;
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
 
+    const uint32_t hd = a.hd;
+    if (n_splits <= kMergeInRegs) {
+        // Few partials: every thread asks for all it needs at once, its output
+        // element's n_splits partial values and the head's (m, l) pairs, and
+        // works the weights out for itself; one trip to memory instead of two
+        // dependent ones, at the end of the launch where nothing hides them.
+        for (uint32_t idx = threadIdx.x; idx < nh * hd; idx += blockDim.x) {
+            const uint32_t h = idx / hd, d = idx % hd;
+            const size_t p0 = ((size_t)sess * a.nq + head0 + h) * a.max_splits;
+            float v[kMergeInRegs], m[kMergeInRegs], l[kMergeInRegs];
+#pragma unroll
+            for (uint32_t i = 0; i < (uint32_t)kMergeInRegs; i++) {
+                const uint32_t ii = i < n_splits ? i : 0;
+                v[i] = part_load(a.part_o + (p0 + ii) * hd + d);
+                m[i] = part_load(&a.part_ml[(p0 + ii) * 2]);
+                l[i] = part_load(&a.part_ml[(p0 + ii) * 2 + 1]);
+            }
+            float M = -INFINITY;
+#pragma unroll
+            for (uint32_t i = 0; i < (uint32_t)kMergeInRegs; i++)
+                if (i < n_splits) M = fmaxf(M, m[i]);
+            float L = 0.f;
+#pragma unroll
+            for (uint32_t i = 0; i < (uint32_t)kMergeInRegs; i++) {
+                m[i] = (i < n_splits) ? fast_exp2(m[i] - M) : 0.f;
+                L += l[i] * m[i];
+            }
+            const float inv = (L > 0.f) ? 1.0f / L : 0.f;
+            float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (uint32_t i = 0; i < (uint32_t)kMergeInRegs; i++) acc[i & 3] += v[i] * (m[i] * inv);
+            a.out[((size_t)sess * a.nq + head0 + h) * hd + d] = (acc[0] + acc[1]) + (acc[2] + acc[3]);
+        }
+        if (threadIdx.x == 0) a.counters[counter_idx] = 0;
+        return;
+    }
+
     float* s_m = scratch;                       // [nh][kMaxSplits]
     float* s_l = scratch + nh * kMaxSplits;
     float* s_w = scratch + 2 * nh * kMaxSplits;
@@ -170,7 +208,6 @@ __device__ __forceinline__ void publish_and_merge(const DecodeArgs& a, uint32_t 
     }
     __syncthreads();
 
-    const uint32_t hd = a.hd;
     for (uint32_t idx = threadIdx.x; idx < nh * hd; idx += blockDim.x) {
         const uint32_t h = idx / hd, d = idx % hd;
         const float* po = a.part_o + (((size_t)sess * a.nq + head0 + h) * a.max_splits) * hd + d;
@@ -388,30 +425,51 @@ void decode_mfma_kernel(const DecodeArgs a)
     const uint16_t* kbase = S.k + (size_t)kvh * S.ctx_pad * HD;
     const uint16_t* vtbase = S.vt + (size_t)kvh * (S.ctx_pad / kVBlock) * HD * kVBlock;
 
-    // The first tile's loads go out before anything else: the HBM latency
-    // then overlaps the staging of Q.
+    // Loads go out in the order they are needed back: the group's Q rows (a few
+    // KB), then this wave's first tile, then (where a wave holds two tiles) its
+    // second.  Memory channels serve requests roughly in arrival order and every
+    // workgroup of the launch starts at once, so a Q request issued after the
+    // tiles waits behind the whole launch's first tiles (5 us at 16 x 4096), and
+    // no workgroup can ask for a second tile until then: the queue runs dry once.
+    constexpr bool kSingle = decode_single_buffered<HD>();
+    constexpr int kQPerThread = kMaxGroupMfma * HD / kDecodeThreads;
+    const float* qg = a.q + ((size_t)sess * a.nq + kvh * G) * HD;     // G contiguous rows
+    float qreg[kQPerThread];
+#pragma unroll
+    for (int i = 0; i < kQPerThread; i++) {
+        const int idx = threadIdx.x + i * kDecodeThreads;
+        qreg[i] = (idx < G * HD) ? qg[idx] : 0.f;
+    }
+    // Both loads are unconditional (a wave with fewer tiles re-reads the
+    // workgroup's last one and ignores it): the compiler places its waits by
+    // counting the loads issued since the one it needs, and a load that is only
+    // sometimes issued makes it assume the smaller count everywhere downstream,
+    // which turns "wait for this tile" into "wait for the prefetched tile too".
     DecodeFrag<HD> fa, fb;
     uint32_t t = tr.t_begin + wave;
-    if (t < tr.t_end) load_frag<HD>(fa, kbase, vtbase, t, lane);
+    load_frag<HD>(fa, kbase, vtbase, min(t, tr.t_end - 1), lane);
+    if constexpr (!kSingle) load_frag<HD>(fb, kbase, vtbase, min(t + kDecodeWaves, tr.t_end - 1), lane);
 
     // Q^T operand through LDS: row c of lds_q is MFMA column c.  Columns
     // 0..G-1 hold the hi terms of the group's heads, G..2G-1 the lo terms,
     // the rest zero; values are pre-multiplied by scale*log2(e).
     __shared__ __attribute__((aligned(16))) _Float16 lds_q[16][HD + 8];
     {
-        const float* qg = a.q + ((size_t)sess * a.nq + kvh * G) * HD;     // G contiguous rows
-        for (int idx = threadIdx.x; idx < G * HD; idx += kDecodeThreads) {
-            const int h = idx / HD, d = idx % HD;
-            const float x = qg[idx] * a.qscale;
-            const _Float16 hi = (_Float16)x;
-            lds_q[h][d] = hi;
-            lds_q[h + G][d] = (_Float16)(x - (float)hi);
+#pragma unroll
+        for (int i = 0; i < kQPerThread; i++) {
+            const int idx = threadIdx.x + i * kDecodeThreads;
+            if (idx < G * HD) {
+                const int h = idx / HD, d = idx % HD;
+                const float x = qreg[i] * a.qscale;
+                const _Float16 hi = (_Float16)x;
+                lds_q[h][d] = hi;
+                lds_q[h + G][d] = (_Float16)(x - (float)hi);
+            }
         }
         for (int idx = threadIdx.x; idx < (16 - 2 * G) * HD; idx += kDecodeThreads)
             lds_q[2 * G + idx / HD][idx % HD] = (_Float16)0.0f;
     }
     __syncthreads();
-    constexpr bool kSingle = decode_single_buffered<HD>();
     half8 qop[kSingle ? 1 : HD / 32];
     if constexpr (!kSingle) {
 #pragma unroll
@@ -429,11 +487,8 @@ void decode_mfma_kernel(const DecodeArgs a)
     st.m = -INFINITY;
     st.l = 0.f;
 
-    // Loads inside the loops below are unconditional, and the last one or two
-    // tiles are peeled off: the compiler places its waits by counting loads
-    // issued since the one it needs, and a load that is only sometimes issued
-    // makes it assume the smaller count, which turns "wait for this tile" into
-    // "wait for the prefetched tile as well".
+    // Loads inside the loops below are unconditional too, and the last tiles
+    // are peeled off, for the same reason.
     if constexpr (kSingle) {
         const _Float16* qrow = &lds_q[n][g * 8];
         if (t < tr.t_end) {
@@ -452,21 +507,27 @@ void decode_mfma_kernel(const DecodeArgs a)
             tile_update<HD>(st, fa, c, t, S.key_lo, S.seq_k, lane, partner_addr, col_kind);
         }
     } else if (t < tr.t_end) {
-        while (t + 2 * kDecodeWaves < tr.t_end) {
-            load_frag<HD>(fb, kbase, vtbase, t + kDecodeWaves, lane);
+        // fa holds tile t, fb tile t + W (both asked for above); each tile's
+        // buffer is refilled with the tile two rounds on as soon as it is used
+        while (t + 3 * kDecodeWaves < tr.t_end) {
             process_tile<HD>(st, fa, qop, t, S.key_lo, S.seq_k, lane, partner_addr, col_kind);
             load_frag<HD>(fa, kbase, vtbase, t + 2 * kDecodeWaves, lane);
             process_tile<HD>(st, fb, qop, t + kDecodeWaves, S.key_lo, S.seq_k, lane, partner_addr,
                              col_kind);
+            load_frag<HD>(fb, kbase, vtbase, t + 3 * kDecodeWaves, lane);
             t += 2 * kDecodeWaves;
         }
-        if (t + kDecodeWaves < tr.t_end) {
-            load_frag<HD>(fb, kbase, vtbase, t + kDecodeWaves, lane);
-            process_tile<HD>(st, fa, qop, t, S.key_lo, S.seq_k, lane, partner_addr, col_kind);
+        // one, two or three tiles left; the first two are in flight
+        process_tile<HD>(st, fa, qop, t, S.key_lo, S.seq_k, lane, partner_addr, col_kind);
+        if (t + 2 * kDecodeWaves < tr.t_end) {
+            load_frag<HD>(fa, kbase, vtbase, t + 2 * kDecodeWaves, lane);
             process_tile<HD>(st, fb, qop, t + kDecodeWaves, S.key_lo, S.seq_k, lane, partner_addr,
                              col_kind);
-        } else {
-            process_tile<HD>(st, fa, qop, t, S.key_lo, S.seq_k, lane, partner_addr, col_kind);
+            process_tile<HD>(st, fa, qop, t + 2 * kDecodeWaves, S.key_lo, S.seq_k, lane, partner_addr,
+                             col_kind);
+        } else if (t + kDecodeWaves < tr.t_end) {
+            process_tile<HD>(st, fb, qop, t + kDecodeWaves, S.key_lo, S.seq_k, lane, partner_addr,
+                             col_kind);
         }
     }
     // denominator: add the four lane groups' shares
