@@ -18,11 +18,20 @@
  *     rollback is "reset the cursor"; rows above it are never read;
  *   - host-pointer entry points are synchronous: results are in the caller's
  *     buffer on return.  `_dev` entry points take device pointers, enqueue on
- *     the library stream and return without waiting;
+ *     the calling thread's stream and return without waiting;
  *   - thread safety: calls on DIFFERENT wr_hip_kv objects may run concurrently
  *     from different threads (reference threading contract,
  *     include/wayruntime/wayruntime.h:29-40); calls on one object must be
- *     serialised by the caller (the session lock does that).
+ *     serialised by the caller (the session lock does that);
+ *   - streams: every calling thread has a stream of its own in the library
+ *     (made on the thread's first call, handed on to a later thread when the
+ *     thread ends), with its own staging, split-K tickets and partial rows, so
+ *     work submitted from different threads overlaps on the device.  "The
+ *     stream" below is always the calling thread's: `_dev` calls made by one
+ *     thread run in the order made, wr_hip_attn_sync and the synchronous
+ *     entry points wait for the calling thread's work only.  Device memory
+ *     written by one thread's `_dev` calls may be used from another thread
+ *     once the first has waited (wr_hip_attn_sync or any synchronous call).
  */
 #ifndef WR_HIP_ATTN_H
 #define WR_HIP_ATTN_H
@@ -154,7 +163,7 @@ int wr_hip_attn_prefill(wr_hip_kv *kv, uint32_t layer, uint32_t p0,
 
 /* ---- device-resident forms (measurement, device-side callers) ------------
  * Same semantics, but q / out / k_f32 / v_f32 are DEVICE pointers obtained
- * from wr_hip_attn_dev_alloc, the work is enqueued on the library stream and
+ * from wr_hip_attn_dev_alloc, the work is enqueued on the calling thread's stream and
  * the call returns without waiting; wr_hip_attn_sync waits.  For the batched
  * form q_dev and out_dev are [n, nq, hd] contiguous. */
 void *wr_hip_attn_dev_alloc(size_t bytes);
@@ -167,7 +176,7 @@ void  wr_hip_attn_host_free(void *p);
 int   wr_hip_attn_h2d(void *dst_dev, const void *src_host, size_t bytes);
 int   wr_hip_attn_d2h(void *dst_host, const void *src_dev, size_t bytes);
 int   wr_hip_attn_sync(void);
-void *wr_hip_attn_stream(void);          /* hipStream_t of the library */
+void *wr_hip_attn_stream(void);          /* hipStream_t of the calling thread */
 
 int wr_hip_attn_append_dev(wr_hip_kv *kv, uint32_t layer, uint32_t pos,
                            uint32_t n_rows, const float *k_f32_dev,
@@ -186,7 +195,7 @@ int wr_hip_attn_append_batched_dev(uint32_t n, wr_hip_kv *const *kv,
 /* The same rotation alone, in place on device F32 rows [rows, heads, hd]
  * (wri_op_rope, src/core/kernels.c:1356-1412, for callers that keep Q or K on
  * the device); cos_sin_dev is device F32 [rows, n_rot, 2].  Asynchronous on
- * the library's stream like the other *_dev calls. */
+ * the stream like the other *_dev calls. */
 int wr_hip_attn_rope_dev(void *x_dev, const void *cos_sin_dev, uint32_t rows,
                          uint32_t heads, uint32_t hd, uint32_t n_rot);
 /* The table that rotation takes, made on the device: cos_sin_dev, device F32
@@ -197,7 +206,7 @@ int wr_hip_attn_rope_dev(void *x_dev, const void *cos_sin_dev, uint32_t rows,
  * stands for 10000 (the angle of wri_op_rope, src/core/kernels.c:1384-1404,
  * through the polynomials and the range reduction of src/core/mathx.c:37-57,
  * :72-86 and :112-147 operation for operation: the bytes equal what the
- * reference computes per element).  Asynchronous on the library's stream. */
+ * reference computes per element).  Asynchronous on the stream. */
 int wr_hip_attn_rope_table_dev(float *cos_sin_dev, uint32_t rows, uint32_t pos0,
                                const uint32_t *pos, uint32_t hd,
                                float theta_base, uint32_t n_rot_pairs);
@@ -224,9 +233,11 @@ int wr_hip_attn_prefill_dev(wr_hip_kv *kv, uint32_t layer, uint32_t p0,
  * behind its first 64 KiB (with the automatic split rule a session has at most
  * 8 key splits: 16 sessions of 32 heads x 128 need 2.1 MB); beyond either,
  * WR_HIP_ERR_LIMIT and nothing is launched.  All calls on one device share the
- * array: the library's stream runs them one after the other, but a caller must
- * not let two of them overlap on one device by other means (two processes'
- * worth of streams replaying captured launches, say): they would race. */
+ * array: the library runs them one after the other, also when they come from
+ * different threads (each launch waits for an event the previous one
+ * recorded), but a caller must not let two of them overlap on one device by
+ * other means (two processes' worth of streams replaying captured launches,
+ * say): they would race. */
 #define WR_HIP_NOALLOC_SCRATCH_BYTES (20u * 1024u * 1024u)
 #define WR_HIP_NOALLOC_MAX_HEADS     1024u
 int wr_hip_attn_decode_batched_dev_noalloc(uint32_t n, wr_hip_kv *const *kv,
@@ -266,7 +277,7 @@ uint32_t wr_hip_proj_weight_cols(const wr_hip_weight *w);
 /* y[rows][n_out] = x[rows][n_in] . W^T, host F32 in and out, synchronous. */
 int wr_hip_proj_rows(const wr_hip_weight *w, uint32_t rows, const float *x,
                      float *y);
-/* Device-resident form, asynchronous on the library stream: row strides ldx >=
+/* Device-resident form, asynchronous on the stream: row strides ldx >=
  * n_in and ldy >= n_out (ldy a multiple of 4, y_dev 16-byte aligned);
  * add_dev, if not NULL, is [rows][ldy] and is added to the product (the
  * residual add that follows wo, src/core/session.c:505-506). */
@@ -300,7 +311,7 @@ int wr_hip_proj_rows_geglu_dev(const wr_hip_weight *w, uint32_t rows,
 /* ---- row steps between the projections and the attention path --------------
  * For callers that keep a layer's activations on the device.  All arguments
  * are device pointers (wr_hip_attn_dev_alloc), all calls are asynchronous on
- * the library stream.  Sums over a row are tree reductions here and
+ * the stream.  Sums over a row are tree reductions here and
  * sequential loops in the reference, so results agree to F32 rounding.
  *
  * rmsnorm: out[r][j] = x[r][j] / sqrt(mean_j x[r][j]^2 + eps) * w[j % wn], or

@@ -221,3 +221,74 @@ def test_concurrent_calls_on_one_model(eng, tmp_path, walk):
         ta.start(); tb.start(); ta.join(); tb.join()
         assert a and b and a[0] == serial[0] and b[0] == serial[1]
     m.close()
+
+
+def test_eight_threads_then_a_batch_beside_a_single_session(eng, tmp_path, walk):
+    # The reference's concurrency case (test/sdk_gen.c:799-904): four prompts,
+    # their greedy chains computed one after another as the reference; then
+    # eight threads each run one of the chains on a session of their own, and
+    # every step's logits must equal the sequential ones byte for byte; then a
+    # batched step over two sessions runs while a third session steps in
+    # another thread, same bar.  Each thread submits through its own stream in
+    # the device library, so the launches of different sessions overlap.
+    import threading
+    p = str(tmp_path / "small16.gguf")
+    gw.write_model(p, SMALL16)
+    m = eng.load(p)
+    shape = gw.ModelShape(vocab=m.vocab)
+    prompts = [workload(shape, n) for n in (5, 11, 23, 40)]
+    STEPS = 6
+
+    def chain(prompt, ref=None):
+        """logits bytes of STEPS greedy steps after the prompt; with ref, the count of steps that differ"""
+        s = m.session(len(prompt) + STEPS)
+        assert s.prefill(prompt[:-1]) == len(prompt) - 1
+        tok, out, bad = int(prompt[-1]), [], 0
+        for k in range(STEPS):
+            lg = s.step(tok)
+            assert lg is not None, s.status
+            out.append(lg.tobytes())
+            bad += ref is not None and out[-1] != ref[k]
+            tok = int(np.argmax(lg))
+        s.close()
+        return out, bad
+
+    refs = [chain(pr)[0] for pr in prompts]
+
+    results = [None] * 8
+    def job(t):
+        try:
+            results[t] = chain(prompts[t % 4], refs[t % 4])[1]
+        except Exception as e:                    # an assert in a thread would otherwise pass silently
+            results[t] = repr(e)
+    threads = [threading.Thread(target=job, args=(t,)) for t in range(8)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert results == [0] * 8, results
+
+    side = [None]
+    def side_job():
+        try:
+            side[0] = chain(prompts[2], refs[2])[1]
+        except Exception as e:
+            side[0] = repr(e)
+    st = threading.Thread(target=side_job)
+    st.start()
+    ab = [m.session(len(prompts[i]) + STEPS) for i in range(2)]
+    for i in range(2):
+        assert ab[i].prefill(prompts[i][:-1]) == len(prompts[i]) - 1
+    cur = [int(prompts[0][-1]), int(prompts[1][-1])]
+    mism = 0
+    for k in range(STEPS):
+        rc, lo = E.batch_step(ab, cur)
+        assert rc == 2
+        for i in range(2):
+            mism += lo[i].tobytes() != refs[i][k]
+            cur[i] = int(np.argmax(lo[i]))
+    st.join()
+    for s in ab:
+        s.close()
+    assert mism == 0 and side[0] == 0, (mism, side[0])
+    m.close()

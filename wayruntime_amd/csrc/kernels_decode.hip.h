@@ -126,6 +126,46 @@ __device__ __forceinline__ void part_store(float* p, float v)
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// Merge of up to N partials per head, everything a thread needs asked for at
+// once: its output element's partial values and the head's (m, l) pairs; the
+// thread works the weights out for itself.  One trip to memory instead of two
+// dependent ones, at the end of the launch where nothing hides them.  (Slots
+// past n_splits re-read partial 0 with weight zero; which N serves a session
+// depends on its split count alone.)
+template <int N>
+__device__ __forceinline__ void merge_in_regs(const DecodeArgs& a, uint32_t sess, uint32_t head0,
+                                              uint32_t nh, uint32_t n_splits)
+{
+    const uint32_t hd = a.hd;
+    for (uint32_t idx = threadIdx.x; idx < nh * hd; idx += blockDim.x) {
+        const uint32_t h = idx / hd, d = idx % hd;
+        const size_t p0 = ((size_t)sess * a.nq + head0 + h) * a.max_splits;
+        float v[N], m[N], l[N];
+#pragma unroll
+        for (uint32_t i = 0; i < (uint32_t)N; i++) {
+            const uint32_t ii = i < n_splits ? i : 0;
+            v[i] = part_load(a.part_o + (p0 + ii) * hd + d);
+            m[i] = part_load(&a.part_ml[(p0 + ii) * 2]);
+            l[i] = part_load(&a.part_ml[(p0 + ii) * 2 + 1]);
+        }
+        float M = -INFINITY;
+#pragma unroll
+        for (uint32_t i = 0; i < (uint32_t)N; i++)
+            if (i < n_splits) M = fmaxf(M, m[i]);
+        float L = 0.f;
+#pragma unroll
+        for (uint32_t i = 0; i < (uint32_t)N; i++) {
+            m[i] = (i < n_splits) ? fast_exp2(m[i] - M) : 0.f;
+            L += l[i] * m[i];
+        }
+        const float inv = (L > 0.f) ? 1.0f / L : 0.f;
+        float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (uint32_t i = 0; i < (uint32_t)N; i++) acc[i & 3] += v[i] * (m[i] * inv);
+        a.out[((size_t)sess * a.nq + head0 + h) * hd + d] = (acc[0] + acc[1]) + (acc[2] + acc[3]);
+    }
+}
+
 // Called by every thread of a workgroup after it has stored its partial rows
 // for heads [head0, head0 + nh) of `sess` at its split index.  The workgroup
 // that draws the last of the n_splits tickets merges the partials of those
@@ -148,37 +188,10 @@ __device__ __forceinline__ void publish_and_merge(const DecodeArgs& a, uint32_t 
 
     const uint32_t hd = a.hd;
     if (n_splits <= kMergeInRegs) {
-        // Few partials: every thread asks for all it needs at once, its output
-        // element's n_splits partial values and the head's (m, l) pairs, and
-        // works the weights out for itself; one trip to memory instead of two
-        // dependent ones, at the end of the launch where nothing hides them.
-        for (uint32_t idx = threadIdx.x; idx < nh * hd; idx += blockDim.x) {
-            const uint32_t h = idx / hd, d = idx % hd;
-            const size_t p0 = ((size_t)sess * a.nq + head0 + h) * a.max_splits;
-            float v[kMergeInRegs], m[kMergeInRegs], l[kMergeInRegs];
-#pragma unroll
-            for (uint32_t i = 0; i < (uint32_t)kMergeInRegs; i++) {
-                const uint32_t ii = i < n_splits ? i : 0;
-                v[i] = part_load(a.part_o + (p0 + ii) * hd + d);
-                m[i] = part_load(&a.part_ml[(p0 + ii) * 2]);
-                l[i] = part_load(&a.part_ml[(p0 + ii) * 2 + 1]);
-            }
-            float M = -INFINITY;
-#pragma unroll
-            for (uint32_t i = 0; i < (uint32_t)kMergeInRegs; i++)
-                if (i < n_splits) M = fmaxf(M, m[i]);
-            float L = 0.f;
-#pragma unroll
-            for (uint32_t i = 0; i < (uint32_t)kMergeInRegs; i++) {
-                m[i] = (i < n_splits) ? fast_exp2(m[i] - M) : 0.f;
-                L += l[i] * m[i];
-            }
-            const float inv = (L > 0.f) ? 1.0f / L : 0.f;
-            float acc[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (uint32_t i = 0; i < (uint32_t)kMergeInRegs; i++) acc[i & 3] += v[i] * (m[i] * inv);
-            a.out[((size_t)sess * a.nq + head0 + h) * hd + d] = (acc[0] + acc[1]) + (acc[2] + acc[3]);
-        }
+        if (n_splits <= 4)
+            merge_in_regs<4>(a, sess, head0, nh, n_splits);
+        else
+            merge_in_regs<kMergeInRegs>(a, sess, head0, nh, n_splits);
         if (threadIdx.x == 0) a.counters[counter_idx] = 0;
         return;
     }

@@ -71,18 +71,16 @@ struct Buffer {
     size_t cap = 0;
 };
 
-struct Lib {
-    std::mutex mu;               // serialises submissions and workspace growth
-    bool inited = false;
-    int device = -1;
-    uint32_t n_cus = 256;        // compute units of the device in use
+// What one calling thread submits through: its own stream, so that sessions
+// driven from different threads overlap on the device (the reference lets
+// independent sessions run concurrently, include/wayruntime.h:29-40), and the
+// buffers whose contents belong to the launches on that stream.
+struct Ctx {
     hipStream_t stream = nullptr;
-    char name[320] = "uninitialised";
     Buffer d_stage;              // device staging for host-pointer entry points
     Buffer d_part;               // split-K partials
     Buffer d_proj;               // projection operand fragments and row scales
     uint32_t* d_counters = nullptr;   // split-K tickets, zero whenever no launch is in flight
-    unsigned char* noalloc_ws[kMaxDevices] = {};   // device address of `scratch`, per device
     // Error word: page-locked host memory that kernels can write.  A kernel that
     // gives up a bounded wait (and so goes on with data it cannot vouch for) stores
     // (bit 31 | layer) there; the host reads it after every wait for the
@@ -92,15 +90,36 @@ struct Lib {
     volatile uint32_t* err_host = nullptr;
     uint32_t* err_dev = nullptr;
     Buffer h_pin;                // pinned host staging
+    std::vector<hipEvent_t> ev;  // kernel timing (profile_begin / profile_end of this thread)
+    uint32_t ev_used = 0;
+    bool profiling = false;
+};
+
+struct Lib {
+    std::mutex mu;               // init / shutdown, the set of thread contexts, the knobs
+    bool inited = false;
+    int device = -1;
+    uint32_t n_cus = 256;        // compute units of the device in use
+    uint64_t generation = 0;     // bumped by every init: contexts of an earlier one are gone
+    std::vector<Ctx*> ctxs;      // every context of this generation
+    std::vector<Ctx*> idle;      // contexts whose thread has ended, for the next new thread
+    char name[320] = "uninitialised";
+    unsigned char* noalloc_ws[kMaxDevices] = {};   // device address of `scratch`, per device
+    // The fixed scratch array is one per device: launches that use it are
+    // chained across threads' streams through this event (recorded after each,
+    // waited for before the next), under its own lock.
+    std::mutex noalloc_mu;
+    hipEvent_t noalloc_done = nullptr;
+    bool noalloc_recorded = false;
     std::atomic<uint64_t> calls{0};
     wr_hip_log_fn log_fn = nullptr;
     void* log_user = nullptr;
-    uint32_t tune_keys_per_wg = 0;
-    int force_generic = 0;
-    std::vector<hipEvent_t> ev;
-    uint32_t ev_used = 0;
-    bool profiling = false;
+    std::atomic<uint32_t> tune_keys_per_wg{0};
+    std::atomic<int> force_generic{0};
 } g;
+
+// The calling thread's context (set by Entered, below).
+thread_local Ctx* cx = nullptr;
 
 constexpr uint32_t kDevErrLayerMask = 0x0000FFFFu;     // error word: bit 31 set (kDevErrWaitExpired), the layer in the low bits
 constexpr float kLog2e = 1.4426950408889634f;
@@ -136,7 +155,7 @@ int hip_fail(hipError_t e, const char* what, uint32_t layer)
 int ensure_device(Buffer& b, size_t need)
 {
     if (need <= b.cap) return WR_HIP_OK;
-    HIP_TRY(hipStreamSynchronize(g.stream), "sync before workspace growth", 0);
+    HIP_TRY(hipStreamSynchronize(cx->stream), "sync before workspace growth", 0);
     if (b.p) (void)hipFree(b.p);
     b.p = nullptr;
     b.cap = 0;
@@ -149,7 +168,7 @@ int ensure_device(Buffer& b, size_t need)
 int ensure_pinned(Buffer& b, size_t need)
 {
     if (need <= b.cap) return WR_HIP_OK;
-    HIP_TRY(hipStreamSynchronize(g.stream), "sync before pinned growth", 0);
+    HIP_TRY(hipStreamSynchronize(cx->stream), "sync before pinned growth", 0);
     if (b.p) (void)hipHostFree(b.p);
     b.p = nullptr;
     b.cap = 0;
@@ -165,28 +184,28 @@ int ensure_pinned(Buffer& b, size_t need)
 // merge partial rows that were never written.
 void reset_tickets()
 {
-    if (!g.d_counters) return;
+    if (!cx->d_counters) return;
     const size_t cb = (size_t)WR_HIP_BATCH_MAX * kMaxHeads * sizeof(uint32_t);
-    if (hipMemsetAsync(g.d_counters, 0, cb, g.stream) == hipSuccess) (void)hipStreamSynchronize(g.stream);
+    if (hipMemsetAsync(cx->d_counters, 0, cb, cx->stream) == hipSuccess) (void)hipStreamSynchronize(cx->stream);
     (void)hipGetLastError();
 }
 
-// Waits for the library stream, then looks at the error word.  Every entry point
+// Waits for the calling thread's stream, then looks at the error word.  Every entry point
 // that promises results on return waits through here, so a kernel that gave up a
 // bounded wait (and went on with wrong data) turns into WR_HIP_ERR_INTERNAL on the
 // first call that could hand those results to the caller, logged with the layer
 // (as the reference reports op failures, src/core/session.c:170-174).
 int sync_checked(const char* what, uint32_t layer)
 {
-    const hipError_t e = hipStreamSynchronize(g.stream);
+    const hipError_t e = hipStreamSynchronize(cx->stream);
     if (e != hipSuccess) {
         const int rc = hip_fail(e, what, layer);
         reset_tickets();
         return rc;
     }
-    const uint32_t w = g.err_host ? *g.err_host : 0u;
+    const uint32_t w = cx->err_host ? *cx->err_host : 0u;
     if (w != 0) {
-        *g.err_host = 0;
+        *cx->err_host = 0;
         logmsg(0, "device: a kernel's bounded wait expired at layer %u (error word 0x%08x, seen at: %s); "
                   "results produced since the previous wait are invalid", w & kDevErrLayerMask, w, what);
         reset_tickets();
@@ -195,20 +214,20 @@ int sync_checked(const char* what, uint32_t layer)
     return WR_HIP_OK;
 }
 
-// Host -> device / device -> host on the library stream.  Small transfers go
+// Host -> device / device -> host on the stream.  Small transfers go
 // through pinned staging (predictable latency); large ones are handed to the
 // runtime directly.  Both leave the stream synchronised for the host buffer.
 int copy_up(void* dst_dev, const void* src_host, size_t bytes, size_t pin_off)
 {
     if (bytes == 0) return WR_HIP_OK;
-    if (pin_off + bytes <= g.h_pin.cap && bytes <= kPinSmall) {
-        memcpy((uint8_t*)g.h_pin.p + pin_off, src_host, bytes);
-        HIP_TRY(hipMemcpyAsync(dst_dev, (uint8_t*)g.h_pin.p + pin_off, bytes,
-                               hipMemcpyHostToDevice, g.stream), "h2d", 0);
+    if (pin_off + bytes <= cx->h_pin.cap && bytes <= kPinSmall) {
+        memcpy((uint8_t*)cx->h_pin.p + pin_off, src_host, bytes);
+        HIP_TRY(hipMemcpyAsync(dst_dev, (uint8_t*)cx->h_pin.p + pin_off, bytes,
+                               hipMemcpyHostToDevice, cx->stream), "h2d", 0);
     } else {
-        HIP_TRY(hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, g.stream),
+        HIP_TRY(hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, cx->stream),
                 "h2d", 0);
-        HIP_TRY(hipStreamSynchronize(g.stream), "h2d sync", 0);
+        HIP_TRY(hipStreamSynchronize(cx->stream), "h2d sync", 0);
     }
     return WR_HIP_OK;
 }
@@ -216,14 +235,14 @@ int copy_up(void* dst_dev, const void* src_host, size_t bytes, size_t pin_off)
 int copy_down_sync(void* dst_host, const void* src_dev, size_t bytes)
 {
     if (bytes == 0) return sync_checked("sync", 0);
-    if (bytes <= g.h_pin.cap && bytes <= kPinSmall) {
-        HIP_TRY(hipMemcpyAsync(g.h_pin.p, src_dev, bytes, hipMemcpyDeviceToHost, g.stream),
+    if (bytes <= cx->h_pin.cap && bytes <= kPinSmall) {
+        HIP_TRY(hipMemcpyAsync(cx->h_pin.p, src_dev, bytes, hipMemcpyDeviceToHost, cx->stream),
                 "d2h", 0);
         int rc = sync_checked("d2h sync", 0);
         if (rc) return rc;
-        memcpy(dst_host, g.h_pin.p, bytes);
+        memcpy(dst_host, cx->h_pin.p, bytes);
     } else {
-        HIP_TRY(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, g.stream),
+        HIP_TRY(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, cx->stream),
                 "d2h", 0);
         int rc = sync_checked("d2h sync", 0);
         if (rc) return rc;
@@ -234,24 +253,24 @@ int copy_down_sync(void* dst_host, const void* src_dev, size_t bytes)
 template <typename Kern, typename A0, typename A1>
 void launch_main(Kern kernel, dim3 grid, dim3 block, const A0& a0, const A1& a1, size_t lds_bytes)
 {
-    if (g.profiling && g.ev_used + 2 <= g.ev.size()) {
-        hipExtLaunchKernelGGL(kernel, grid, block, lds_bytes, g.stream, g.ev[g.ev_used],
-                              g.ev[g.ev_used + 1], 0, a0, a1);
-        g.ev_used += 2;
+    if (cx->profiling && cx->ev_used + 2 <= cx->ev.size()) {
+        hipExtLaunchKernelGGL(kernel, grid, block, lds_bytes, cx->stream, cx->ev[cx->ev_used],
+                              cx->ev[cx->ev_used + 1], 0, a0, a1);
+        cx->ev_used += 2;
     } else {
-        hipLaunchKernelGGL(kernel, grid, block, lds_bytes, g.stream, a0, a1);
+        hipLaunchKernelGGL(kernel, grid, block, lds_bytes, cx->stream, a0, a1);
     }
 }
 
 template <typename Kern, typename Args>
 void launch_main(Kern kernel, dim3 grid, dim3 block, const Args& args, size_t lds_bytes = 0)
 {
-    if (g.profiling && g.ev_used + 2 <= g.ev.size()) {
-        hipExtLaunchKernelGGL(kernel, grid, block, lds_bytes, g.stream, g.ev[g.ev_used],
-                              g.ev[g.ev_used + 1], 0, args);
-        g.ev_used += 2;
+    if (cx->profiling && cx->ev_used + 2 <= cx->ev.size()) {
+        hipExtLaunchKernelGGL(kernel, grid, block, lds_bytes, cx->stream, cx->ev[cx->ev_used],
+                              cx->ev[cx->ev_used + 1], 0, args);
+        cx->ev_used += 2;
     } else {
-        hipLaunchKernelGGL(kernel, grid, block, lds_bytes, g.stream, args);
+        hipLaunchKernelGGL(kernel, grid, block, lds_bytes, cx->stream, args);
     }
 }
 
@@ -273,7 +292,7 @@ uint32_t key_lo_for(uint32_t window, uint32_t seq_k)
 }
 
 // ------------------------------------------------------------------------
-// Unlocked bodies (caller holds g.mu and has set the device).
+// Bodies (the caller has entered: device current, cx set).
 
 template <typename Src>
 int append_rows_locked(wr_hip_kv* kv, uint32_t layer, uint32_t pos, uint32_t n_rows,
@@ -284,11 +303,11 @@ int append_rows_locked(wr_hip_kv* kv, uint32_t layer, uint32_t pos, uint32_t n_r
     uint16_t* vbase = reinterpret_cast<uint16_t*>(kv->slab + kv->vt_off[layer]);
     const size_t total = (size_t)n_rows * nkv * hd;
     const uint32_t blocks = (uint32_t)((total + 255) / 256);
-    hipLaunchKernelGGL(HIP_KERNEL_NAME(append_k_kernel<Src>), dim3(blocks), dim3(256), 0, g.stream,
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(append_k_kernel<Src>), dim3(blocks), dim3(256), 0, cx->stream,
                        k_dev, kbase, pos, n_rows, nkv, hd, kv->ctx_pad);
     const uint32_t nblk = (pos + n_rows - 1) / kVBlock - pos / kVBlock + 1;
     hipLaunchKernelGGL(HIP_KERNEL_NAME(append_v_kernel<Src>), dim3((hd + 63) / 64, nkv, nblk),
-                       dim3(256), 0, g.stream, v_dev, vbase, pos, n_rows, nkv, hd, kv->ctx_pad);
+                       dim3(256), 0, cx->stream, v_dev, vbase, pos, n_rows, nkv, hd, kv->ctx_pad);
     HIP_TRY(hipGetLastError(), "append launch", layer);
     return WR_HIP_OK;
 }
@@ -352,10 +371,11 @@ int decode_locked(uint32_t n, wr_hip_kv* const* kv, uint32_t layer, const uint32
     // one session at a time can lower the figure with wr_hip_attn_set_tuning.
     (void)tiles_total;
     uint32_t max_splits = 1;
+    const uint32_t tune = g.tune_keys_per_wg.load(std::memory_order_relaxed);
     for (uint32_t i = 0; i < n; i++) {
         uint32_t tpw;
-        if (g.tune_keys_per_wg) {
-            tpw = g.tune_keys_per_wg / kTileKeys;
+        if (tune) {
+            tpw = tune / kTileKeys;
             if (tpw == 0) tpw = 1;
         } else {
             uint32_t cap = kDefaultTilesPerWg * 128u / (hd < 32 ? 32 : hd);
@@ -403,7 +423,7 @@ int decode_locked(uint32_t n, wr_hip_kv* const* kv, uint32_t layer, const uint32
     a.group = group;
     a.hd = hd;
     a.max_splits = max_splits;
-    a.counters = fixed.ws ? reinterpret_cast<uint32_t*>(fixed.ws) : g.d_counters;
+    a.counters = fixed.ws ? reinterpret_cast<uint32_t*>(fixed.ws) : cx->d_counters;
     const float scale = (scale_override > 0.0f) ? scale_override : 1.0f / sqrtf((float)hd);
     a.qscale = scale * kLog2e;
 
@@ -420,9 +440,9 @@ int decode_locked(uint32_t n, wr_hip_kv* const* kv, uint32_t layer, const uint32
             }
             base = fixed.ws + fixed.ticket_bytes;
         } else {
-            int rc = ensure_device(g.d_part, po + pml);
+            int rc = ensure_device(cx->d_part, po + pml);
             if (rc) return rc;
-            base = reinterpret_cast<uint8_t*>(g.d_part.p);
+            base = reinterpret_cast<uint8_t*>(cx->d_part.p);
         }
         a.part_o = reinterpret_cast<float*>(base);
         a.part_ml = reinterpret_cast<float*>(base + po);
@@ -430,7 +450,7 @@ int decode_locked(uint32_t n, wr_hip_kv* const* kv, uint32_t layer, const uint32
             // the array keeps the last call's contents: the tickets this launch
             // uses must start at zero
             const uint32_t words = n * (use_mfma ? nkv : nq);
-            hipLaunchKernelGGL(fill_u32_kernel, dim3((words + 255) / 256), dim3(256), 0, g.stream,
+            hipLaunchKernelGGL(fill_u32_kernel, dim3((words + 255) / 256), dim3(256), 0, cx->stream,
                                a.counters, words, 0u);
         }
     }
@@ -555,17 +575,117 @@ int check_prefill(const wr_hip_kv* kv, uint32_t layer, uint32_t p0, uint32_t T, 
     return WR_HIP_OK;
 }
 
-struct Locked {
-    std::lock_guard<std::mutex> lk;
-    Locked() : lk(g.mu)
+// ---- thread contexts -------------------------------------------------------
+
+void ctx_destroy(Ctx* c)
+{
+    if (!c) return;
+    if (c->stream) (void)hipStreamSynchronize(c->stream);
+    for (hipEvent_t e : c->ev) (void)hipEventDestroy(e);
+    if (c->d_stage.p) (void)hipFree(c->d_stage.p);
+    if (c->d_part.p) (void)hipFree(c->d_part.p);
+    if (c->d_proj.p) (void)hipFree(c->d_proj.p);
+    if (c->d_counters) (void)hipFree(c->d_counters);
+    if (c->h_pin.p) (void)hipHostFree(c->h_pin.p);
+    if (c->err_host) (void)hipHostFree((void*)c->err_host);
+    if (c->stream) (void)hipStreamDestroy(c->stream);
+    delete c;
+}
+
+// A new context: stream (default priority), staging, zeroed tickets, error word.
+// Caller holds g.mu and has set the device.
+Ctx* ctx_create()
+{
+    Ctx* c = new (std::nothrow) Ctx();
+    if (!c) return nullptr;
+    Ctx* const saved = cx;
+    cx = c;                                  // the helpers below work on the current context
+    int rc = WR_HIP_OK;
+    hipError_t e = hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking);
+    if (e != hipSuccess) rc = hip_fail(e, "stream create", 0);
+    if (rc == WR_HIP_OK) rc = ensure_pinned(c->h_pin, 2 * kPinSmall);
+    if (rc == WR_HIP_OK) rc = ensure_device(c->d_stage, 2 * kPinSmall);
+    if (rc == WR_HIP_OK) {
+        const size_t cb = (size_t)WR_HIP_BATCH_MAX * kMaxHeads * sizeof(uint32_t);
+        e = hipMalloc((void**)&c->d_counters, cb);
+        if (e == hipSuccess) e = hipMemsetAsync(c->d_counters, 0, cb, c->stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(c->stream);
+        if (e != hipSuccess) rc = hip_fail(e, "ticket array", 0);
+    }
+    if (rc == WR_HIP_OK) {
+        void* hp = nullptr;
+        void* dp = nullptr;
+        e = hipHostMalloc(&hp, 64, hipHostMallocMapped);
+        if (e == hipSuccess) e = hipHostGetDevicePointer(&dp, hp, 0);
+        if (e != hipSuccess) {
+            rc = hip_fail(e, "error word", 0);
+            if (hp) (void)hipHostFree(hp);
+        } else {
+            memset(hp, 0, 64);
+            c->err_host = reinterpret_cast<volatile uint32_t*>(hp);
+            c->err_dev = reinterpret_cast<uint32_t*>(dp);
+        }
+    }
+    cx = saved;
+    if (rc != WR_HIP_OK) {
+        ctx_destroy(c);
+        return nullptr;
+    }
+    return c;
+}
+
+// Hands a thread's context back when the thread ends, for the next new thread
+// (threads of a pool come and go; their streams and staging need not).
+struct ThreadSlot {
+    Ctx* c = nullptr;
+    uint64_t generation = 0;
+    ~ThreadSlot()
     {
-        if (g.inited) (void)hipSetDevice(g.device);
+        if (!c) return;
+        std::lock_guard<std::mutex> lk(g.mu);
+        if (g.inited && generation == g.generation) g.idle.push_back(c);
     }
 };
+thread_local ThreadSlot t_slot;
+
+// Every entry point that touches the device starts here: the device is made
+// current for the calling thread and `cx` is the thread's context, created on
+// the thread's first call.  ok() is false when that failed (out of memory) or
+// the library is not initialised.  No lock is held afterwards: calls from
+// different threads run side by side, each on its own stream.
+struct Entered {
+    bool good = false;
+    Entered()
+    {
+        if (!g.inited) return;
+        (void)hipSetDevice(g.device);
+        if (!t_slot.c || t_slot.generation != g.generation) {
+            std::lock_guard<std::mutex> lk(g.mu);
+            if (!g.inited) return;
+            Ctx* c = nullptr;
+            if (!g.idle.empty()) {
+                c = g.idle.back();
+                g.idle.pop_back();
+            } else {
+                c = ctx_create();
+                if (c) g.ctxs.push_back(c);
+            }
+            t_slot.c = c;
+            t_slot.generation = g.generation;
+        }
+        cx = t_slot.c;
+        good = cx != nullptr;
+    }
+    bool ok() const { return good; }
+};
+
+#define ENTER()                                   \
+    Entered entered_;                             \
+    if (!entered_.ok()) return g.inited ? WR_HIP_ERR_NOMEM : WR_HIP_ERR_STATE
 
 }  // namespace
 
-// projections: launch helpers (caller holds g.mu)
+// projections: launch helpers (the caller has entered)
 namespace {
 
 template <int GROUPS, int NT>
@@ -634,7 +754,7 @@ struct ProjSource {
 };
 
 // y_dev[rows][ldy] = source(x_dev)[rows][n_in] . W^T (+ add_dev), rows <= kProjMaxRows.
-// Caller holds g.mu.
+// The caller has entered.
 int proj_chunk_locked(const wr_hip_weight* w, uint32_t rows, const float* x_dev, uint32_t ldx,
                       const ProjSource& src, const float* add_dev, float* y_dev, uint32_t ldy)
 {
@@ -646,10 +766,10 @@ int proj_chunk_locked(const wr_hip_weight* w, uint32_t rows, const float* x_dev,
     // one row: the fragment step runs inside the product's kernel (4 bytes of LDS per input)
     const bool row1 = rows == 1 && (size_t)w->n_in * 4 <= kProjRow1MaxLds;
     const size_t frag_bytes = (size_t)groups * ktiles * 1024;
-    int rc = ensure_device(g.d_proj, frag_bytes + kProjMaxRows * sizeof(float));
+    int rc = ensure_device(cx->d_proj, frag_bytes + kProjMaxRows * sizeof(float));
     if (rc) return rc;
-    half8* frag = reinterpret_cast<half8*>(g.d_proj.p);
-    float* scales = reinterpret_cast<float*>((uint8_t*)g.d_proj.p + frag_bytes);
+    half8* frag = reinterpret_cast<half8*>(cx->d_proj.p);
+    float* scales = reinterpret_cast<float*>((uint8_t*)cx->d_proj.p + frag_bytes);
     ProjPrepArgs pa;
     pa.x = x_dev;
     pa.norm_w = src.norm_w;
@@ -667,7 +787,7 @@ int proj_chunk_locked(const wr_hip_weight* w, uint32_t rows, const float* x_dev,
                           ((uintptr_t)src.norm_w & 15) == 0;
     const uint32_t kin = w->n_in;
 #define WR_LAUNCH_PREP_GROUP(SRC, CH) \
-    hipLaunchKernelGGL(HIP_KERNEL_NAME(proj_prep_group_kernel<SRC, CH>), dim3(groups), pblock, 0, g.stream, pa)
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(proj_prep_group_kernel<SRC, CH>), dim3(groups), pblock, 0, cx->stream, pa)
 #define WR_LAUNCH_PREP(SRC)                                                                          \
     do {                                                                                             \
         if (by_group && kin <= 1024)                                                                 \
@@ -679,9 +799,9 @@ int proj_chunk_locked(const wr_hip_weight* w, uint32_t rows, const float* x_dev,
         else if (by_group)                                                                           \
             WR_LAUNCH_PREP_GROUP(SRC, 0);                                                            \
         else if (in_regs)                                                                            \
-            hipLaunchKernelGGL(HIP_KERNEL_NAME(proj_prep_kernel<SRC, 2>), pgrid, pblock, 0, g.stream, pa); \
+            hipLaunchKernelGGL(HIP_KERNEL_NAME(proj_prep_kernel<SRC, 2>), pgrid, pblock, 0, cx->stream, pa); \
         else                                                                                         \
-            hipLaunchKernelGGL(HIP_KERNEL_NAME(proj_prep_kernel<SRC, 0>), pgrid, pblock, 0, g.stream, pa); \
+            hipLaunchKernelGGL(HIP_KERNEL_NAME(proj_prep_kernel<SRC, 0>), pgrid, pblock, 0, cx->stream, pa); \
     } while (0)
     if (row1)
         ;                                           // no fragment launch
@@ -782,35 +902,18 @@ int wr_hip_attn_init(int device)
                prop.gcnArchName);
         return WR_HIP_ERR_UNSUPPORTED;
     }
-    HIP_TRY(hipStreamCreateWithFlags(&g.stream, hipStreamNonBlocking), "stream create", 0);
     g.device = device;
     g.n_cus = prop.multiProcessorCount > 0 ? (uint32_t)prop.multiProcessorCount : 256u;
     snprintf(g.name, sizeof g.name, "%s %s, %d CUs, %.1f GiB", prop.gcnArchName, prop.name,
              prop.multiProcessorCount, (double)prop.totalGlobalMem / (1024.0 * 1024.0 * 1024.0));
     g.inited = true;
     g.calls.store(0);
-    int rc = ensure_pinned(g.h_pin, 2 * kPinSmall);
-    if (rc == WR_HIP_OK) rc = ensure_device(g.d_stage, 2 * kPinSmall);
-    if (rc == WR_HIP_OK) {
-        const size_t cb = (size_t)WR_HIP_BATCH_MAX * kMaxHeads * sizeof(uint32_t);
-        hipError_t e = hipMalloc((void**)&g.d_counters, cb);
-        if (e == hipSuccess) e = hipMemsetAsync(g.d_counters, 0, cb, g.stream);
-        if (e == hipSuccess) e = hipStreamSynchronize(g.stream);
-        if (e != hipSuccess) rc = hip_fail(e, "ticket array", 0);
-    }
-    if (rc == WR_HIP_OK) {
-        void* hp = nullptr;
-        void* dp = nullptr;
-        hipError_t e = hipHostMalloc(&hp, 64, hipHostMallocMapped);
-        if (e == hipSuccess) e = hipHostGetDevicePointer(&dp, hp, 0);
-        if (e != hipSuccess) {
-            rc = hip_fail(e, "error word", 0);
-            if (hp) (void)hipHostFree(hp);
-        } else {
-            memset(hp, 0, 64);
-            g.err_host = reinterpret_cast<volatile uint32_t*>(hp);
-            g.err_dev = reinterpret_cast<uint32_t*>(dp);
-        }
+    g.generation++;
+    int rc = WR_HIP_OK;
+    {
+        const hipError_t e = hipEventCreateWithFlags(&g.noalloc_done, hipEventDisableTiming);
+        if (e != hipSuccess) rc = hip_fail(e, "event create", 0);
+        g.noalloc_recorded = false;
     }
     if (rc == WR_HIP_OK) {
         // device address of the no-alloc entry point's scratch array, once per
@@ -849,11 +952,8 @@ int wr_hip_attn_init(int device)
     }
     if (rc != WR_HIP_OK) {
         g.inited = false;
-        if (g.err_host) (void)hipHostFree((void*)g.err_host);
-        g.err_host = nullptr;
-        g.err_dev = nullptr;
-        (void)hipStreamDestroy(g.stream);
-        g.stream = nullptr;
+        if (g.noalloc_done) (void)hipEventDestroy(g.noalloc_done);
+        g.noalloc_done = nullptr;
     }
     return rc;
 }
@@ -863,26 +963,12 @@ void wr_hip_attn_shutdown(void)
     std::lock_guard<std::mutex> lk(g.mu);
     if (!g.inited) return;
     (void)hipSetDevice(g.device);
-    (void)hipStreamSynchronize(g.stream);
-    for (hipEvent_t e : g.ev) (void)hipEventDestroy(e);
-    g.ev.clear();
-    g.ev_used = 0;
-    g.profiling = false;
-    if (g.d_stage.p) (void)hipFree(g.d_stage.p);
-    if (g.d_part.p) (void)hipFree(g.d_part.p);
-    if (g.d_counters) (void)hipFree(g.d_counters);
-    g.d_counters = nullptr;
-    if (g.h_pin.p) (void)hipHostFree(g.h_pin.p);
-    if (g.err_host) (void)hipHostFree((void*)g.err_host);
-    g.err_host = nullptr;
-    g.err_dev = nullptr;
-    if (g.d_proj.p) (void)hipFree(g.d_proj.p);
-    g.d_proj = Buffer();
-    g.d_stage = Buffer();
-    g.d_part = Buffer();
-    g.h_pin = Buffer();
-    (void)hipStreamDestroy(g.stream);
-    g.stream = nullptr;
+    for (Ctx* c : g.ctxs) ctx_destroy(c);      // waits for each stream first
+    g.ctxs.clear();
+    g.idle.clear();
+    cx = nullptr;
+    if (g.noalloc_done) (void)hipEventDestroy(g.noalloc_done);
+    g.noalloc_done = nullptr;
     g.inited = false;
     g.device = -1;
     g.tune_keys_per_wg = 0;
@@ -948,15 +1034,15 @@ int wr_hip_attn_kv_create(uint32_t n_layers, const uint32_t* hd_per_layer, uint3
     }
     kv->bytes = cur;
 
-    Locked lk;
+    ENTER();
     hipError_t e = hipMalloc((void**)&kv->slab, cur);
     if (e != hipSuccess) {
         logmsg(0, "session: device slab alloc failed (%zu bytes): %s", cur, hipGetErrorString(e));
         delete kv;
         return WR_HIP_ERR_NOMEM;
     }
-    e = hipMemsetAsync(kv->slab, 0, cur, g.stream);
-    if (e == hipSuccess) e = hipStreamSynchronize(g.stream);
+    e = hipMemsetAsync(kv->slab, 0, cur, cx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(cx->stream);
     if (e != hipSuccess) {
         (void)hipFree(kv->slab);
         delete kv;
@@ -970,9 +1056,9 @@ void wr_hip_attn_kv_destroy(wr_hip_kv* kv)
 {
     if (!kv) return;
     if (g.inited) {
-        Locked lk;
-        (void)hipStreamSynchronize(g.stream);
-        if (kv->slab) (void)hipFree(kv->slab);
+        Entered entered_;
+        if (entered_.ok()) (void)hipStreamSynchronize(cx->stream);
+        if (kv->slab) (void)hipFree(kv->slab);     // (waits for the device's other streams by itself)
     }
     delete kv;
 }
@@ -986,7 +1072,7 @@ int wr_hip_attn_append_dev(wr_hip_kv* kv, uint32_t layer, uint32_t pos, uint32_t
 {
     int rc = check_append(kv, layer, pos, n_rows, k_f32_dev, v_f32_dev);
     if (rc || n_rows == 0) return rc;
-    Locked lk;
+    ENTER();
     return append_rows_locked<float>(kv, layer, pos, n_rows, k_f32_dev, v_f32_dev);
 }
 
@@ -1015,8 +1101,8 @@ int wr_hip_attn_append_batched_dev(uint32_t n, wr_hip_kv* const* kv, uint32_t la
     a.v_src = v_f32_dev;
     a.nkv = kv[0]->nkv;
     a.hd = kv[0]->hd[layer];
-    Locked lk;
-    hipLaunchKernelGGL(append_batch_kernel, dim3(n), dim3(256), 0, g.stream, a);
+    ENTER();
+    hipLaunchKernelGGL(append_batch_kernel, dim3(n), dim3(256), 0, cx->stream, a);
     HIP_TRY(hipGetLastError(), "batched append launch", layer);
     return WR_HIP_OK;
 }
@@ -1028,10 +1114,10 @@ int wr_hip_attn_rope_dev(void* x_dev, const void* cos_sin_dev, uint32_t rows, ui
     if (!x_dev || !cos_sin_dev) return WR_HIP_ERR_INVAL;
     if (hd < 2 || (hd & 1) || heads == 0 || n_rot > hd / 2) return WR_HIP_ERR_INVAL;
     if (rows == 0 || n_rot == 0) return WR_HIP_OK;
-    Locked lk;
+    ENTER();
     const size_t total = (size_t)rows * heads * n_rot;
     hipLaunchKernelGGL(rope_rows_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
-                       g.stream, reinterpret_cast<float*>(x_dev),
+                       cx->stream, reinterpret_cast<float*>(x_dev),
                        reinterpret_cast<const float*>(cos_sin_dev), rows, heads, hd, n_rot);
     HIP_TRY(hipGetLastError(), "rope launch", 0);
     return WR_HIP_OK;
@@ -1055,8 +1141,8 @@ int wr_hip_attn_rope_table_dev(float* cos_sin_dev, uint32_t rows, uint32_t pos0,
     a.pos0 = pos0;
     a.listed = pos ? 1u : 0u;
     for (uint32_t i = 0; pos && i < rows; i++) a.pos[i] = pos[i];
-    Locked lk;
-    hipLaunchKernelGGL(rope_table_kernel, dim3((rows + 63u) / 64u, a.n_rot), dim3(64), 0, g.stream, a);
+    ENTER();
+    hipLaunchKernelGGL(rope_table_kernel, dim3((rows + 63u) / 64u, a.n_rot), dim3(64), 0, cx->stream, a);
     HIP_TRY(hipGetLastError(), "rotary table launch", 0);
     return WR_HIP_OK;
 }
@@ -1073,24 +1159,24 @@ int wr_hip_attn_append_rope(wr_hip_kv* kv, uint32_t layer, uint32_t pos, uint32_
     const uint32_t hd = kv->hd[layer], nkv = kv->nkv;
     const size_t bytes = (size_t)n_rows * nkv * hd * sizeof(float);
     const size_t tbytes = (size_t)n_rows * n_rot * 2 * sizeof(float);
-    Locked lk;
-    rc = ensure_device(g.d_stage, 2 * bytes + tbytes);
+    ENTER();
+    rc = ensure_device(cx->d_stage, 2 * bytes + tbytes);
     if (rc) return rc;
-    float* dk = reinterpret_cast<float*>(g.d_stage.p);
-    float* dv = reinterpret_cast<float*>((uint8_t*)g.d_stage.p + bytes);
-    float* dt = reinterpret_cast<float*>((uint8_t*)g.d_stage.p + 2 * bytes);
+    float* dk = reinterpret_cast<float*>(cx->d_stage.p);
+    float* dv = reinterpret_cast<float*>((uint8_t*)cx->d_stage.p + bytes);
+    float* dt = reinterpret_cast<float*>((uint8_t*)cx->d_stage.p + 2 * bytes);
     rc = copy_up(dk, k_f32, bytes, 0);
     if (rc == WR_HIP_OK) rc = copy_up(dv, v_f32, bytes, bytes);
     if (rc == WR_HIP_OK) rc = copy_up(dt, cos_sin, tbytes, 2 * bytes);
     if (rc == WR_HIP_OK && n_rot > 0) {
         const size_t total = (size_t)n_rows * nkv * n_rot;
         hipLaunchKernelGGL(rope_rows_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
-                           g.stream, dk, dt, n_rows, nkv, hd, n_rot);
+                           cx->stream, dk, dt, n_rows, nkv, hd, n_rot);
         HIP_TRY(hipGetLastError(), "rope launch", layer);
     }
     if (rc == WR_HIP_OK) rc = append_rows_locked<float>(kv, layer, pos, n_rows, dk, dv);
     // the staging buffers are reused by the next call: wait for the kernels
-    if (rc == WR_HIP_OK) HIP_TRY(hipStreamSynchronize(g.stream), "append sync", layer);
+    if (rc == WR_HIP_OK) HIP_TRY(hipStreamSynchronize(cx->stream), "append sync", layer);
     return rc;
 }
 
@@ -1100,16 +1186,16 @@ int wr_hip_attn_append(wr_hip_kv* kv, uint32_t layer, uint32_t pos, uint32_t n_r
     int rc = check_append(kv, layer, pos, n_rows, k_f32, v_f32);
     if (rc || n_rows == 0) return rc;
     const size_t bytes = (size_t)n_rows * kv->nkv * kv->hd[layer] * sizeof(float);
-    Locked lk;
-    rc = ensure_device(g.d_stage, 2 * bytes);
+    ENTER();
+    rc = ensure_device(cx->d_stage, 2 * bytes);
     if (rc) return rc;
-    float* dk = reinterpret_cast<float*>(g.d_stage.p);
-    float* dv = reinterpret_cast<float*>((uint8_t*)g.d_stage.p + bytes);
+    float* dk = reinterpret_cast<float*>(cx->d_stage.p);
+    float* dv = reinterpret_cast<float*>((uint8_t*)cx->d_stage.p + bytes);
     rc = copy_up(dk, k_f32, bytes, 0);
     if (rc == WR_HIP_OK) rc = copy_up(dv, v_f32, bytes, bytes);
     if (rc == WR_HIP_OK) rc = append_rows_locked<float>(kv, layer, pos, n_rows, dk, dv);
     // the staging buffers are reused by the next call: wait for the kernels
-    if (rc == WR_HIP_OK) HIP_TRY(hipStreamSynchronize(g.stream), "append sync", layer);
+    if (rc == WR_HIP_OK) HIP_TRY(hipStreamSynchronize(cx->stream), "append sync", layer);
     return rc;
 }
 
@@ -1119,15 +1205,15 @@ int wr_hip_attn_kv_write(wr_hip_kv* kv, uint32_t layer, uint32_t pos, uint32_t n
     int rc = check_append(kv, layer, pos, n_rows, k_f16, v_f16);
     if (rc || n_rows == 0) return rc;
     const size_t bytes = (size_t)n_rows * kv->nkv * kv->hd[layer] * sizeof(uint16_t);
-    Locked lk;
-    rc = ensure_device(g.d_stage, 2 * bytes);
+    ENTER();
+    rc = ensure_device(cx->d_stage, 2 * bytes);
     if (rc) return rc;
-    uint16_t* dk = reinterpret_cast<uint16_t*>(g.d_stage.p);
-    uint16_t* dv = reinterpret_cast<uint16_t*>((uint8_t*)g.d_stage.p + bytes);
+    uint16_t* dk = reinterpret_cast<uint16_t*>(cx->d_stage.p);
+    uint16_t* dv = reinterpret_cast<uint16_t*>((uint8_t*)cx->d_stage.p + bytes);
     rc = copy_up(dk, k_f16, bytes, 0);
     if (rc == WR_HIP_OK) rc = copy_up(dv, v_f16, bytes, bytes);
     if (rc == WR_HIP_OK) rc = append_rows_locked<uint16_t>(kv, layer, pos, n_rows, dk, dv);
-    if (rc == WR_HIP_OK) HIP_TRY(hipStreamSynchronize(g.stream), "kv_write sync", layer);
+    if (rc == WR_HIP_OK) HIP_TRY(hipStreamSynchronize(cx->stream), "kv_write sync", layer);
     return rc;
 }
 
@@ -1143,13 +1229,13 @@ int wr_hip_attn_kv_read(wr_hip_kv* kv, uint32_t layer, uint32_t pos, uint32_t n_
     const uint32_t hd = kv->hd[layer], nkv = kv->nkv;
     const size_t total = (size_t)n_rows * nkv * hd;
     const size_t bytes = total * sizeof(uint16_t);
-    Locked lk;
-    rc = ensure_device(g.d_stage, 2 * bytes);
+    ENTER();
+    rc = ensure_device(cx->d_stage, 2 * bytes);
     if (rc) return rc;
-    uint16_t* dk = reinterpret_cast<uint16_t*>(g.d_stage.p);
-    uint16_t* dv = reinterpret_cast<uint16_t*>((uint8_t*)g.d_stage.p + bytes);
+    uint16_t* dk = reinterpret_cast<uint16_t*>(cx->d_stage.p);
+    uint16_t* dv = reinterpret_cast<uint16_t*>((uint8_t*)cx->d_stage.p + bytes);
     hipLaunchKernelGGL(export_kv_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0,
-                       g.stream,
+                       cx->stream,
                        reinterpret_cast<const uint16_t*>(kv->slab + kv->k_off[layer]),
                        reinterpret_cast<const uint16_t*>(kv->slab + kv->vt_off[layer]), dk, dv, pos,
                        n_rows, nkv, hd, kv->ctx_pad);
@@ -1167,7 +1253,7 @@ int wr_hip_attn_decode_batched_dev(uint32_t n, wr_hip_kv* const* kv, uint32_t la
 {
     int rc = check_decode(n, kv, layer, seq_k, q_dev, out_dev, nq);
     if (rc) return rc;
-    Locked lk;
+    ENTER();
     return decode_locked(n, kv, layer, seq_k, q_dev, out_dev, nq, scale_override, window);
 }
 
@@ -1183,13 +1269,21 @@ int wr_hip_attn_decode_batched_dev_noalloc(uint32_t n, wr_hip_kv* const* kv, uin
                nq, kNoAllocMaxHeads);
         return WR_HIP_ERR_LIMIT;
     }
-    Locked lk;
+    ENTER();
     DecodeWorkspace fixed;
     fixed.ws = g.noalloc_ws[g.device];
     fixed.ticket_bytes = kNoAllocTicketBytes;
     fixed.bytes = kNoAllocScratchBytes;
     if (!fixed.ws) return WR_HIP_ERR_STATE;
-    return decode_locked(n, kv, layer, seq_k, q_dev, out_dev, nq, scale_override, window, fixed);
+    // One array per device, whatever thread calls: this launch waits for the
+    // previous one that used it (on whichever stream that was), and leaves its
+    // own mark for the next.  Event waits and records allocate nothing.
+    std::lock_guard<std::mutex> chain(g.noalloc_mu);
+    if (g.noalloc_recorded)
+        HIP_TRY(hipStreamWaitEvent(cx->stream, g.noalloc_done, 0), "wait for the scratch array", layer);
+    rc = decode_locked(n, kv, layer, seq_k, q_dev, out_dev, nq, scale_override, window, fixed);
+    if (hipEventRecord(g.noalloc_done, cx->stream) == hipSuccess) g.noalloc_recorded = true;
+    return rc;
 }
 
 int wr_hip_attn_decode_batched(uint32_t n, wr_hip_kv* const* kv, uint32_t layer,
@@ -1201,23 +1295,23 @@ int wr_hip_attn_decode_batched(uint32_t n, wr_hip_kv* const* kv, uint32_t layer,
     for (uint32_t i = 0; i < n; i++)
         if (!q[i] || !out[i]) return WR_HIP_ERR_INVAL;
     const size_t row = (size_t)nq * kv[0]->hd[layer] * sizeof(float);
-    Locked lk;
-    rc = ensure_device(g.d_stage, 2 * n * row);
+    ENTER();
+    rc = ensure_device(cx->d_stage, 2 * n * row);
     if (rc) return rc;
-    rc = ensure_pinned(g.h_pin, n * row);
+    rc = ensure_pinned(cx->h_pin, n * row);
     if (rc) return rc;
-    float* dq = reinterpret_cast<float*>(g.d_stage.p);
-    float* dout = reinterpret_cast<float*>((uint8_t*)g.d_stage.p + n * row);
-    for (uint32_t i = 0; i < n; i++) memcpy((uint8_t*)g.h_pin.p + i * row, q[i], row);
-    HIP_TRY(hipMemcpyAsync(dq, g.h_pin.p, n * row, hipMemcpyHostToDevice, g.stream), "q h2d",
+    float* dq = reinterpret_cast<float*>(cx->d_stage.p);
+    float* dout = reinterpret_cast<float*>((uint8_t*)cx->d_stage.p + n * row);
+    for (uint32_t i = 0; i < n; i++) memcpy((uint8_t*)cx->h_pin.p + i * row, q[i], row);
+    HIP_TRY(hipMemcpyAsync(dq, cx->h_pin.p, n * row, hipMemcpyHostToDevice, cx->stream), "q h2d",
             layer);
     rc = decode_locked(n, kv, layer, seq_k, dq, dout, nq, scale_override, window);
     if (rc) return rc;
-    HIP_TRY(hipMemcpyAsync(g.h_pin.p, dout, n * row, hipMemcpyDeviceToHost, g.stream), "out d2h",
+    HIP_TRY(hipMemcpyAsync(cx->h_pin.p, dout, n * row, hipMemcpyDeviceToHost, cx->stream), "out d2h",
             layer);
     rc = sync_checked("decode sync", layer);
     if (rc) return rc;
-    for (uint32_t i = 0; i < n; i++) memcpy(out[i], (uint8_t*)g.h_pin.p + i * row, row);
+    for (uint32_t i = 0; i < n; i++) memcpy(out[i], (uint8_t*)cx->h_pin.p + i * row, row);
     return WR_HIP_OK;
 }
 
@@ -1239,7 +1333,7 @@ int wr_hip_attn_prefill_dev(wr_hip_kv* kv, uint32_t layer, uint32_t p0, uint32_t
 {
     int rc = check_prefill(kv, layer, p0, T, q_dev, out_dev, nq);
     if (rc) return rc;
-    Locked lk;
+    ENTER();
     return prefill_locked(kv, layer, p0, T, q_dev, out_dev, nq, scale_override, window);
 }
 
@@ -1249,11 +1343,11 @@ int wr_hip_attn_prefill(wr_hip_kv* kv, uint32_t layer, uint32_t p0, uint32_t T, 
     int rc = check_prefill(kv, layer, p0, T, q, out, nq);
     if (rc) return rc;
     const size_t bytes = (size_t)T * nq * kv->hd[layer] * sizeof(float);
-    Locked lk;
-    rc = ensure_device(g.d_stage, 2 * bytes);
+    ENTER();
+    rc = ensure_device(cx->d_stage, 2 * bytes);
     if (rc) return rc;
-    float* dq = reinterpret_cast<float*>(g.d_stage.p);
-    float* dout = reinterpret_cast<float*>((uint8_t*)g.d_stage.p + bytes);
+    float* dq = reinterpret_cast<float*>(cx->d_stage.p);
+    float* dout = reinterpret_cast<float*>((uint8_t*)cx->d_stage.p + bytes);
     rc = copy_up(dq, q, bytes, 0);
     if (rc == WR_HIP_OK)
         rc = prefill_locked(kv, layer, p0, T, dq, dout, nq, scale_override, window);
@@ -1266,7 +1360,8 @@ int wr_hip_attn_prefill(wr_hip_kv* kv, uint32_t layer, uint32_t p0, uint32_t T, 
 void* wr_hip_attn_dev_alloc(size_t bytes)
 {
     if (!g.inited || bytes == 0) return nullptr;
-    Locked lk;
+    Entered entered_;
+    if (!entered_.ok()) return nullptr;
     void* p = nullptr;
     if (hipMalloc(&p, bytes) != hipSuccess) return nullptr;
     return p;
@@ -1275,15 +1370,17 @@ void* wr_hip_attn_dev_alloc(size_t bytes)
 void wr_hip_attn_dev_free(void* p)
 {
     if (!g.inited || !p) return;
-    Locked lk;
-    (void)hipStreamSynchronize(g.stream);
+    Entered entered_;
+    if (!entered_.ok()) return;
+    (void)hipStreamSynchronize(cx->stream);
     (void)hipFree(p);
 }
 
 void* wr_hip_attn_host_alloc(size_t bytes)
 {
     if (!g.inited || bytes == 0) return nullptr;
-    Locked lk;
+    Entered entered_;
+    if (!entered_.ok()) return nullptr;
     void* p = nullptr;
     if (hipHostMalloc(&p, bytes, hipHostMallocDefault) != hipSuccess) return nullptr;
     return p;
@@ -1292,8 +1389,9 @@ void* wr_hip_attn_host_alloc(size_t bytes)
 void wr_hip_attn_host_free(void* p)
 {
     if (!g.inited || !p) return;
-    Locked lk;
-    (void)hipStreamSynchronize(g.stream);
+    Entered entered_;
+    if (!entered_.ok()) return;
+    (void)hipStreamSynchronize(cx->stream);
     (void)hipHostFree(p);
 }
 
@@ -1301,9 +1399,9 @@ int wr_hip_attn_h2d(void* dst_dev, const void* src_host, size_t bytes)
 {
     if (!g.inited) return WR_HIP_ERR_STATE;
     if (!dst_dev || !src_host) return WR_HIP_ERR_INVAL;
-    Locked lk;
-    HIP_TRY(hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, g.stream), "h2d", 0);
-    HIP_TRY(hipStreamSynchronize(g.stream), "h2d sync", 0);
+    ENTER();
+    HIP_TRY(hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, cx->stream), "h2d", 0);
+    HIP_TRY(hipStreamSynchronize(cx->stream), "h2d sync", 0);
     return WR_HIP_OK;
 }
 
@@ -1311,19 +1409,19 @@ int wr_hip_attn_d2h(void* dst_host, const void* src_dev, size_t bytes)
 {
     if (!g.inited) return WR_HIP_ERR_STATE;
     if (!dst_host || !src_dev) return WR_HIP_ERR_INVAL;
-    Locked lk;
-    HIP_TRY(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, g.stream), "d2h", 0);
+    ENTER();
+    HIP_TRY(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, cx->stream), "d2h", 0);
     return sync_checked("d2h sync", 0);
 }
 
 int wr_hip_attn_sync(void)
 {
     if (!g.inited) return WR_HIP_ERR_STATE;
-    Locked lk;
+    ENTER();
     return sync_checked("sync", 0);
 }
 
-void* wr_hip_attn_stream(void) { return g.inited ? (void*)g.stream : nullptr; }
+void* wr_hip_attn_stream(void) { return g.inited ? (void*)cx->stream : nullptr; }
 
 // ------------------------------------------------------------ projections --
 
@@ -1348,7 +1446,7 @@ int wr_hip_proj_weight_create(uint32_t n_parts, const uint16_t* const* parts_f16
     w->bytes = (size_t)n_out * n_in * 2;
     w->tiles = nullptr;
 
-    Locked lk;
+    ENTER();
     void* rowmajor = nullptr;
     hipError_t e = hipMalloc(&w->tiles, w->bytes);
     if (e == hipSuccess) e = hipMalloc(&rowmajor, w->bytes);
@@ -1362,17 +1460,17 @@ int wr_hip_proj_weight_create(uint32_t n_parts, const uint16_t* const* parts_f16
     size_t off = 0;
     for (uint32_t i = 0; i < n_parts && e == hipSuccess; i++) {
         const size_t nb = (size_t)rows_per_part[i] * n_in * 2;
-        e = hipMemcpyAsync((uint8_t*)rowmajor + off, parts_f16[i], nb, hipMemcpyHostToDevice, g.stream);
-        if (e == hipSuccess) e = hipStreamSynchronize(g.stream);     // pageable source
+        e = hipMemcpyAsync((uint8_t*)rowmajor + off, parts_f16[i], nb, hipMemcpyHostToDevice, cx->stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(cx->stream);     // pageable source
         off += nb;
     }
     if (e == hipSuccess) {
         const size_t units = w->bytes / 16;
         hipLaunchKernelGGL(proj_pack_weights_kernel, dim3((uint32_t)((units + 255) / 256)), dim3(256),
-                           0, g.stream, reinterpret_cast<const uint16_t*>(rowmajor),
+                           0, cx->stream, reinterpret_cast<const uint16_t*>(rowmajor),
                            reinterpret_cast<u32x4*>(w->tiles), w->n_out, w->n_in);
         e = hipGetLastError();
-        if (e == hipSuccess) e = hipStreamSynchronize(g.stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(cx->stream);
     }
     (void)hipFree(rowmajor);
     if (e != hipSuccess) {
@@ -1388,8 +1486,8 @@ void wr_hip_proj_weight_destroy(wr_hip_weight* w)
 {
     if (!w) return;
     if (g.inited) {
-        Locked lk;
-        (void)hipStreamSynchronize(g.stream);
+        Entered entered_;
+        if (entered_.ok()) (void)hipStreamSynchronize(cx->stream);
         (void)hipFree(w->tiles);
     }
     delete w;
@@ -1412,7 +1510,7 @@ static int proj_dev_common(const wr_hip_weight* w, uint32_t rows, const float* x
     int rc = check_proj(w, rows, x_dev, ldx, min_ldx, y_dev, ldy);
     if (rc || rows == 0) return rc;
     if (((uintptr_t)y_dev & 15) || (add_dev && ((uintptr_t)add_dev & 15))) return WR_HIP_ERR_INVAL;
-    Locked lk;
+    ENTER();
     return proj_locked(w, rows, x_dev, ldx, src, add_dev, y_dev, ldy);
 }
 
@@ -1457,11 +1555,11 @@ int wr_hip_proj_rows(const wr_hip_weight* w, uint32_t rows, const float* x, floa
     if (rc || rows == 0) return rc;
     const size_t xb = ((size_t)rows * w->n_in * sizeof(float) + 255) & ~(size_t)255;
     const size_t yb = (size_t)rows * w->n_out * sizeof(float);
-    Locked lk;
-    rc = ensure_device(g.d_stage, xb + yb);
+    ENTER();
+    rc = ensure_device(cx->d_stage, xb + yb);
     if (rc) return rc;
-    float* dx = reinterpret_cast<float*>(g.d_stage.p);
-    float* dy = reinterpret_cast<float*>((uint8_t*)g.d_stage.p + xb);
+    float* dx = reinterpret_cast<float*>(cx->d_stage.p);
+    float* dy = reinterpret_cast<float*>((uint8_t*)cx->d_stage.p + xb);
     rc = copy_up(dx, x, (size_t)rows * w->n_in * sizeof(float), 0);
     if (rc == WR_HIP_OK) rc = proj_locked(w, rows, dx, w->n_in, ProjSource(), nullptr, dy, w->n_out);
     if (rc == WR_HIP_OK) rc = copy_down_sync(y, dy, yb);
@@ -1477,8 +1575,8 @@ int wr_hip_rows_rmsnorm_dev(const float* x_dev, uint32_t ldx, const float* w_dev
     if (!x_dev || !out_dev || dim == 0 || ldx < dim || ldo < dim) return WR_HIP_ERR_INVAL;
     if (wn > 0 && !w_dev) return WR_HIP_ERR_INVAL;
     if (rows == 0) return WR_HIP_OK;
-    Locked lk;
-    hipLaunchKernelGGL(rmsnorm_rows_kernel, dim3(rows), dim3(256), 0, g.stream, x_dev, ldx, w_dev, wn,
+    ENTER();
+    hipLaunchKernelGGL(rmsnorm_rows_kernel, dim3(rows), dim3(256), 0, cx->stream, x_dev, ldx, w_dev, wn,
                        out_dev, ldo, dim, eps, 0);
     HIP_TRY(hipGetLastError(), "rmsnorm launch", 0);
     return WR_HIP_OK;
@@ -1491,8 +1589,8 @@ int wr_hip_rows_rmsnorm_add_dev(const float* x_dev, uint32_t ldx, const float* w
     if (!x_dev || !acc_dev || dim == 0 || ldx < dim || lda < dim) return WR_HIP_ERR_INVAL;
     if (wn > 0 && !w_dev) return WR_HIP_ERR_INVAL;
     if (rows == 0) return WR_HIP_OK;
-    Locked lk;
-    hipLaunchKernelGGL(rmsnorm_rows_kernel, dim3(rows), dim3(256), 0, g.stream, x_dev, ldx, w_dev, wn,
+    ENTER();
+    hipLaunchKernelGGL(rmsnorm_rows_kernel, dim3(rows), dim3(256), 0, cx->stream, x_dev, ldx, w_dev, wn,
                        acc_dev, lda, dim, eps, 1);
     HIP_TRY(hipGetLastError(), "rmsnorm + add launch", 0);
     return WR_HIP_OK;
@@ -1524,8 +1622,8 @@ int wr_hip_rows_qkv_prep_dev(const float* qkv_dev, uint32_t ld, uint32_t rows, u
     a.hd = hd;
     a.n_rot = n_rot;
     a.eps = eps;
-    Locked lk;
-    hipLaunchKernelGGL(qkv_prep_kernel, dim3(rows, nq + 2 * nkv), dim3(64), 0, g.stream, a);
+    ENTER();
+    hipLaunchKernelGGL(qkv_prep_kernel, dim3(rows, nq + 2 * nkv), dim3(64), 0, cx->stream, a);
     HIP_TRY(hipGetLastError(), "qkv prep launch", 0);
     return WR_HIP_OK;
 }
@@ -1587,8 +1685,8 @@ int wr_hip_rows_qkv_append_dev(const float* qkv_dev, uint32_t ld, uint32_t rows,
     }
     const uint32_t gx = a.per_session ? rows : (pos[0] + rows - 1) / kVBlock - pos[0] / kVBlock + 1;
     const size_t lds = std::max((size_t)4 * hd * sizeof(float), (size_t)hd * (kVBlock + 2) * sizeof(uint16_t));
-    Locked lk;
-    hipLaunchKernelGGL(qkv_append_kernel, dim3(gx, nq + (q_only ? 0 : 2 * nkv)), dim3(256), lds, g.stream, a);
+    ENTER();
+    hipLaunchKernelGGL(qkv_append_kernel, dim3(gx, nq + (q_only ? 0 : 2 * nkv)), dim3(256), lds, cx->stream, a);
     HIP_TRY(hipGetLastError(), "qkv append launch", layer);
     return WR_HIP_OK;
 }
@@ -1600,10 +1698,10 @@ int wr_hip_rows_swiglu_dev(const float* gate_up_dev, uint32_t ld, float* act_dev
     if (!gate_up_dev || !act_dev || ffn == 0 || (uint64_t)ld < 2ull * ffn || ldo < ffn)
         return WR_HIP_ERR_INVAL;
     if (rows == 0) return WR_HIP_OK;
-    Locked lk;
+    ENTER();
     const size_t total = (size_t)rows * ffn;
     hipLaunchKernelGGL(swiglu_rows_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0,
-                       g.stream, gate_up_dev, ld, act_dev, ldo, rows, ffn);
+                       cx->stream, gate_up_dev, ld, act_dev, ldo, rows, ffn);
     HIP_TRY(hipGetLastError(), "swiglu launch", 0);
     return WR_HIP_OK;
 }
@@ -1614,33 +1712,33 @@ uint32_t wr_hip_proj_weight_cols(const wr_hip_weight* w) { return w ? w->n_in : 
 int wr_hip_attn_profile_begin(uint32_t max_launches)
 {
     if (!g.inited) return WR_HIP_ERR_STATE;
-    Locked lk;
-    HIP_TRY(hipStreamSynchronize(g.stream), "sync", 0);
-    while (g.ev.size() < 2 * (size_t)max_launches) {
+    ENTER();
+    HIP_TRY(hipStreamSynchronize(cx->stream), "sync", 0);
+    while (cx->ev.size() < 2 * (size_t)max_launches) {
         hipEvent_t e;
         HIP_TRY(hipEventCreate(&e), "event create", 0);
-        g.ev.push_back(e);
+        cx->ev.push_back(e);
     }
-    g.ev_used = 0;
-    g.profiling = true;
+    cx->ev_used = 0;
+    cx->profiling = true;
     return WR_HIP_OK;
 }
 
 int wr_hip_attn_profile_end(double* total_ms, uint32_t* n_launches)
 {
     if (!g.inited) return WR_HIP_ERR_STATE;
-    Locked lk;
-    HIP_TRY(hipStreamSynchronize(g.stream), "sync", 0);
+    ENTER();
+    HIP_TRY(hipStreamSynchronize(cx->stream), "sync", 0);
     double sum = 0.0;
-    for (uint32_t i = 0; i + 1 < g.ev_used; i += 2) {
+    for (uint32_t i = 0; i + 1 < cx->ev_used; i += 2) {
         float ms = 0.f;
-        HIP_TRY(hipEventElapsedTime(&ms, g.ev[i], g.ev[i + 1]), "event elapsed", 0);
+        HIP_TRY(hipEventElapsedTime(&ms, cx->ev[i], cx->ev[i + 1]), "event elapsed", 0);
         sum += ms;
     }
     if (total_ms) *total_ms = sum;
-    if (n_launches) *n_launches = g.ev_used / 2;
-    g.profiling = false;
-    g.ev_used = 0;
+    if (n_launches) *n_launches = cx->ev_used / 2;
+    cx->profiling = false;
+    cx->ev_used = 0;
     return WR_HIP_OK;
 }
 

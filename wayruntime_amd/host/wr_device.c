@@ -134,6 +134,8 @@ wr_status wrh_device_model_init(wr_model *m)
         if (rc == WR_HIP_OK) rc = stack(&d->L[l].wdown, &m->w_down[l], NULL, NULL);
     }
     if (rc == WR_HIP_OK) rc = stack(&d->lm_head, &m->lm_head, NULL, NULL);
+    /* the uploads ran on this thread's stream; sessions may step on others */
+    if (rc == WR_HIP_OK) rc = wr_hip_attn_sync();
     if (rc != WR_HIP_OK) {
         wrh_logf(m->engine, 0, "device layers: weight upload failed (rc=%d)", rc);
         wrh_device_model_free(m);
