@@ -83,9 +83,18 @@ struct SplitLds {
     static constexpr int V_IN_SET = kRing * KTILE;        // Vt slots follow the K slots
     static constexpr int Q_OFF = 2 * SET_BYTES;           // Q staging, [4][32][HD + 8] halves
     static constexpr int Q_BYTES = 4 * 32 * (HD + 8) * 2;
-    static constexpr int MERGE_BYTES = 4 * (HD / 2 + 2) * 64 * 4;   // laid over the rings
-    static constexpr int TOTAL = Q_OFF + Q_BYTES;
-    static_assert(MERGE_BYTES <= Q_OFF, "merge scratch fits the rings");
+    // Merge scratch (end of a block): at the end of the kernel's LDS, over the Q
+    // staging (Q is in registers by then) and, where 160 KiB are not enough for
+    // everything, over the tail of the odd set's last Vt slot.  It stays clear of
+    // every slot the first copies of a block go to, so the next block's first
+    // tiles can be on their way while this block is merged and stored.
+    static constexpr int MERGE_BYTES = 4 * (HD / 2 + 2) * 64 * 4;
+    static constexpr int LDS_MAX = 160 * 1024;
+    static constexpr int MERGE_OFF = (Q_OFF + Q_BYTES + MERGE_BYTES <= LDS_MAX) ? Q_OFF + Q_BYTES
+                                                                                : LDS_MAX - MERGE_BYTES;
+    static constexpr int TOTAL = MERGE_OFF + MERGE_BYTES;
+    static_assert(MERGE_OFF >= SET_BYTES + V_IN_SET + 2 * VTILE,
+                  "merge scratch may overlap the odd set's third Vt slot only (no copy of a block's prologue lands there)");
     static_assert(KTILE == VTILE && NL >= 1, "one chunk schedule serves K and Vt");
     // slot permutation of K rows / Vt rows
     __device__ static constexpr int fk(int row) { return (row / RPB) & (CPR - 1); }
@@ -376,9 +385,73 @@ __device__ __forceinline__ void il_step(PrefillRows<HD>& R, IlCtx<HD>& cx, f32x1
     __builtin_amdgcn_sched_barrier(0);
 }
 
+// The lane's index, computed where it is asked for.  The step loop runs at the
+// register limit; whatever the code after it derives from a lane index that
+// was computed before it would have to live through the loop (or be spilled,
+// and a reload waits for every load in flight, the next block's first tiles
+// included).
+__device__ __forceinline__ int il_fresh_lane()
+{
+    int l;
+    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(l));
+    return l;
+}
+
+// Q rows of one wave (16 of the sub-block's 32), as read from global memory:
+// every row is 4*HD contiguous bytes, read with whole-row coalesced loads.
+template <int HD>
+struct IlQRows {
+    static constexpr int LPR = HD / 4;                    // lanes per row (one float4 each)
+    static constexpr int RPI = 64 / LPR;                  // rows per load instruction
+    float4 x[16 / RPI];
+};
+
+template <int HD>
+__device__ __forceinline__ void il_load_q(IlQRows<HD>& q, const PrefillArgs& a, uint32_t row0, uint32_t head,
+                                          int kg, int lane)
+{
+    using Q = IlQRows<HD>;
+#pragma unroll
+    for (int j = 0; j < 16 / Q::RPI; j++) {
+        const int r = kg * 16 + j * Q::RPI + lane / Q::LPR;
+        const uint32_t row = min(row0 + r, a.T - 1);      // idle rows re-read the last one
+        q.x[j] = *reinterpret_cast<const float4*>(a.q + ((size_t)row * a.nq + head) * HD + (lane % Q::LPR) * 4);
+    }
+}
+
+// The tile range of position block pb for key set kg, into the context.
+template <int HD>
+__device__ __forceinline__ void il_ctx_tiles(IlCtx<HD>& cx, const PrefillArgs& a, uint32_t pb, uint32_t BP,
+                                             int kg, uint32_t& t_first, uint32_t& t_last)
+{
+    prefill_block_tiles(a, pb, BP, t_first, t_last);
+    cx.t0 = t_first + kg;                                 // this set's tiles: t0, t0 + 2, ...
+    cx.nt = (cx.t0 <= t_last) ? (t_last - cx.t0) / 2 + 1 : 0;
+    cx.t_last = t_last;
+}
+
+// The copies and loads a block starts with: the first three K tiles and two Vt
+// blocks of the set into their ring slots, in order of need, and the wave's Q rows.
+template <int HD>
+__device__ __forceinline__ void il_first_loads(const IlCtx<HD>& cx, IlQRows<HD>& q, const PrefillArgs& a,
+                                               uint32_t row0, uint32_t head, int kg, int lane)
+{
+    il_load_q<HD>(q, a, row0, head, kg, lane);
+    il_issue_k<HD, 0>(cx, 0);
+    il_issue_k<HD, 1>(cx, 1);
+    il_issue_v<HD, 0>(cx, 0);
+    il_issue_k<HD, 2>(cx, 2);
+    il_issue_v<HD, 1>(cx, 1);
+}
+
+// One position block.  started: the block's first loads are already on their way
+// (q holds its Q rows).  next_pb >= 0: once this block's loop is over, the first
+// loads of block next_pb are issued, before the merge and the stores, and q
+// returns its Q rows.
 template <int HD>
 __device__ __forceinline__ void il_block(const PrefillArgs& a, unsigned char* smem, uint32_t pb,
-                                         uint32_t kvh, uint32_t hc)
+                                         uint32_t kvh, uint32_t hc, const unsigned char* kbase, const unsigned char* vtbase,
+                                         bool started, IlQRows<HD>& q, int next_pb)
 {
     using L = SplitLds<HD>;
     static_assert(L::NL == 1 || L::NL == 2, "one or two copies per wave, tile and operand");
@@ -390,23 +463,23 @@ __device__ __forceinline__ void il_block(const PrefillArgs& a, unsigned char* sm
     const uint32_t G = a.group;
     const uint32_t Gw = G < 4 ? G : 4;
     const uint32_t BP = 32 * (4 / Gw);                    // positions per block
-    const uint32_t head = kvh * G + hc * Gw + (sub % Gw);
-    const uint32_t row0 = pb * BP + (sub / Gw) * 32;      // first chunk row of this wave
+    // wave-uniform, and pinned to scalar registers: integer division runs on the
+    // vector unit, and a quotient left there costs a vector register for the
+    // whole block (or a spill)
+    const uint32_t head = (uint32_t)__builtin_amdgcn_readfirstlane(kvh * G + hc * Gw + (sub % Gw));
+    const uint32_t sub_rows = (uint32_t)__builtin_amdgcn_readfirstlane((sub / Gw) * 32);
+    const uint32_t row0 = pb * BP + sub_rows;             // first chunk row of this wave
     const uint32_t kv_valid = a.p0 + a.T;                 // rows of the cache that hold data
     uint32_t t_first, t_last;
-    prefill_block_tiles(a, pb, BP, t_first, t_last);
 
     PrefillRows<HD> R;
     prefill_rows_init<HD, false>(R, a, row0, head, n, g);
 
     IlCtx<HD> cx;
-    cx.t0 = t_first + kg;                                 // this set's tiles: t0, t0 + 2, ...
-    cx.nt = (cx.t0 <= t_last) ? (t_last - cx.t0) / 2 + 1 : 0;
-    cx.t_last = t_last;
+    il_ctx_tiles<HD>(cx, a, pb, BP, kg, t_first, t_last);
     cx.tail_tile = kv_valid / kTileKeys;
-    cx.kbase = uniform_ptr(reinterpret_cast<const unsigned char*>(a.k + (size_t)kvh * a.ctx_pad * HD));
-    cx.vtbase = uniform_ptr(reinterpret_cast<const unsigned char*>(
-        a.vt + (size_t)kvh * (a.ctx_pad / kVBlock) * HD * kVBlock));
+    cx.kbase = kbase;
+    cx.vtbase = vtbase;
     cx.ring = kg * L::SET_BYTES;
     {
         // low half of a generic LDS pointer = LDS byte address
@@ -465,33 +538,24 @@ __device__ __forceinline__ void il_block(const PrefillArgs& a, unsigned char* sm
     // fewer and spends its last step on probabilities of zero); the same in every wave
     const uint32_t nsteps = (t_last - t_first) / 2 + 1;
 
-    // everything the first two vector blocks read, in order of need
-    il_issue_k<HD, 0>(cx, 0);
-    il_issue_k<HD, 1>(cx, 1);
-    il_issue_v<HD, 0>(cx, 0);
-    il_issue_k<HD, 2>(cx, 2);
-    il_issue_v<HD, 1>(cx, 1);
+    // everything the first two vector blocks read, in order of need, and Q
+    if (!started) il_first_loads<HD>(cx, q, a, row0, head, kg, lane);
 
-    // Q: every row is 4*HD contiguous bytes in global memory, so it is read with
-    // whole-row coalesced loads (the two waves serving a sub-block take 16 rows
-    // each), converted to pre-scaled F16 and turned into the per-lane operand
-    // layout through LDS.
+    // Q is converted to pre-scaled F16 and turned into the per-lane operand
+    // layout through LDS (the two waves serving a sub-block take 16 rows each).
     _Float16 (*qs)[32][HD + 8] = reinterpret_cast<_Float16 (*)[32][HD + 8]>(smem + L::Q_OFF);
     {
-        constexpr int LPR = HD / 4;                       // lanes per row (one float4 each)
-        constexpr int RPI = 64 / LPR;                     // rows per load instruction
+        using Q = IlQRows<HD>;
 #pragma unroll
-        for (int j = 0; j < 16 / RPI; j++) {
-            const int r = kg * 16 + j * RPI + lane / LPR;
-            const uint32_t row = min(row0 + r, a.T - 1);  // idle rows re-read the last one
-            const float4 x = *reinterpret_cast<const float4*>(
-                a.q + ((size_t)row * a.nq + head) * HD + (lane % LPR) * 4);
+        for (int j = 0; j < 16 / Q::RPI; j++) {
+            const int r = kg * 16 + j * Q::RPI + lane / Q::LPR;
+            const float4 x = q.x[j];
             half4 h;
             h[0] = (_Float16)(x.x * a.qscale);
             h[1] = (_Float16)(x.y * a.qscale);
             h[2] = (_Float16)(x.z * a.qscale);
             h[3] = (_Float16)(x.w * a.qscale);
-            *reinterpret_cast<half4*>(&qs[sub][r][(lane % LPR) * 4]) = h;
+            *reinterpret_cast<half4*>(&qs[sub][r][(lane % Q::LPR) * 4]) = h;
         }
     }
     f32x16 sa, sb, negm;
@@ -545,16 +609,27 @@ __device__ __forceinline__ void il_block(const PrefillArgs& a, unsigned char* sm
     // merge the odd-tile partials into the even-tile waves; the ring must be
     // quiet first (the last steps' copies still target it)
     constexpr int NREG = HD / 2;
-    float* mg = reinterpret_cast<float*>(smem) + (size_t)sub * (NREG + 2) * 64;
+    float* mg = reinterpret_cast<float*>(smem + L::MERGE_OFF) + (size_t)sub * (NREG + 2) * 64;
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
+    const int lane_e = il_fresh_lane();                   // lane, n, g again, for the code after the loop
+    const int n_e = lane_e & 31, g_e = lane_e >> 5;
+    if (next_pb >= 0) {
+        // the rings are quiet and the merge below does not touch the slots these
+        // go to: the next block's first tiles and Q rows travel while this block
+        // is merged and stored
+        IlCtx<HD> cn = cx;
+        uint32_t nf, nl;
+        il_ctx_tiles<HD>(cn, a, (uint32_t)next_pb, BP, kg, nf, nl);
+        il_first_loads<HD>(cn, q, a, (uint32_t)next_pb * BP + sub_rows, head, kg, lane_e);
+    }
     if (kg == 1) {
 #pragma unroll
         for (int dt = 0; dt < HD / 32; dt++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) mg[(dt * 16 + r) * 64 + lane] = R.o[dt][r];
-        mg[NREG * 64 + lane] = R.m_run;
-        mg[(NREG + 1) * 64 + lane] = R.l_run;
+            for (int r = 0; r < 16; r++) mg[(dt * 16 + r) * 64 + lane_e] = R.o[dt][r];
+        mg[NREG * 64 + lane_e] = R.m_run;
+        mg[(NREG + 1) * 64 + lane_e] = R.l_run;
     }
     __syncthreads();
     // rows leave through LDS as well: the merged tile is written row-major into
@@ -562,7 +637,7 @@ __device__ __forceinline__ void il_block(const PrefillArgs& a, unsigned char* sm
     float (*os)[HD + 4] = reinterpret_cast<float (*)[HD + 4]>(mg);
     static_assert((size_t)32 * (HD + 4) <= (size_t)(NREG + 2) * 64, "row-major tile fits the merge scratch");
     if (kg == 0) {
-        const float m1 = mg[NREG * 64 + lane], l1 = mg[(NREG + 1) * 64 + lane];
+        const float m1 = mg[NREG * 64 + lane_e], l1 = mg[(NREG + 1) * 64 + lane_e];
         const float m = fmaxf(R.m_run, m1);
         const float f0m = (R.m_run == -INFINITY) ? 0.f : fast_exp2(R.m_run - m);
         const float f1m = (m1 == -INFINITY) ? 0.f : fast_exp2(m1 - m);
@@ -573,7 +648,7 @@ __device__ __forceinline__ void il_block(const PrefillArgs& a, unsigned char* sm
         for (int dt = 0; dt < HD / 32; dt++)
 #pragma unroll
             for (int r = 0; r < 16; r++)
-                R.o[dt][r] = R.o[dt][r] * w0 + mg[(dt * 16 + r) * 64 + lane] * w1;
+                R.o[dt][r] = R.o[dt][r] * w0 + mg[(dt * 16 + r) * 64 + lane_e] * w1;
         // the scratch has been read into registers; the same wave now reuses it
 #pragma unroll
         for (int dt = 0; dt < HD / 32; dt++)
@@ -584,7 +659,7 @@ __device__ __forceinline__ void il_block(const PrefillArgs& a, unsigned char* sm
                 v.y = R.o[dt][4 * q4 + 1];
                 v.z = R.o[dt][4 * q4 + 2];
                 v.w = R.o[dt][4 * q4 + 3];
-                *reinterpret_cast<float4*>(&os[n][dt * 32 + 8 * q4 + 4 * g]) = v;
+                *reinterpret_cast<float4*>(&os[n_e][dt * 32 + 8 * q4 + 4 * g_e]) = v;
             }
     }
     __syncthreads();
@@ -593,11 +668,11 @@ __device__ __forceinline__ void il_block(const PrefillArgs& a, unsigned char* sm
         constexpr int RPI = 64 / LPR;                     // rows per store instruction
 #pragma unroll
         for (int j = 0; j < 16 / RPI; j++) {
-            const int r = kg * 16 + j * RPI + lane / LPR;
-            const float4 v = *reinterpret_cast<const float4*>(&os[r][(lane % LPR) * 4]);
+            const int r = kg * 16 + j * RPI + lane_e / LPR;
+            const float4 v = *reinterpret_cast<const float4*>(&os[r][(lane_e % LPR) * 4]);
             if (row0 + r < a.T)
                 *reinterpret_cast<float4*>(a.out + ((size_t)(row0 + r) * a.nq + head) * HD +
-                                           (lane % LPR) * 4) = v;
+                                           (lane_e % LPR) * 4) = v;
         }
     }
 }
@@ -615,18 +690,23 @@ __global__ __launch_bounds__(kSplitThreads, 1) void prefill_il_kernel(const Pref
     const uint32_t G = a.group;
     const uint32_t Gw = G < 4 ? G : 4;
     const uint32_t chunks = G / Gw;
-    const uint32_t kvh = blockIdx.x / chunks, hc = blockIdx.x % chunks;
+    const uint32_t kvh = (uint32_t)__builtin_amdgcn_readfirstlane(blockIdx.x / chunks);
+    const uint32_t hc = (uint32_t)__builtin_amdgcn_readfirstlane(blockIdx.x % chunks);
     const uint32_t BP = 32 * (4 / Gw);
-    const uint32_t nblk = (a.T + BP - 1) / BP;
+    const uint32_t nblk = (uint32_t)__builtin_amdgcn_readfirstlane((a.T + BP - 1) / BP);
     const uint32_t lo = blockIdx.y, hi = nblk - 1 - blockIdx.y;
-    const int passes = a.single ? 1 : 2;
-#pragma unroll 1
-    for (int pass = 0; pass < passes; pass++) {
-        if (pass) {
-            if (hi == lo) break;
-            __syncthreads();                              // LDS changes hands
-        }
-        il_block<HD>(a, prefill_smem_raw, pass ? lo : hi, kvh, hc);
+    // this KV head's K / Vt, in scalar registers for both blocks
+    const unsigned char* kbase =
+        uniform_ptr(reinterpret_cast<const unsigned char*>(a.k + (size_t)kvh * a.ctx_pad * HD));
+    const unsigned char* vtbase = uniform_ptr(reinterpret_cast<const unsigned char*>(
+        a.vt + (size_t)kvh * (a.ctx_pad / kVBlock) * HD * kVBlock));
+    IlQRows<HD> q;
+    if (a.single || hi == lo) {
+        il_block<HD>(a, prefill_smem_raw, hi, kvh, hc, kbase, vtbase, false, q, -1);
+    } else {
+        il_block<HD>(a, prefill_smem_raw, hi, kvh, hc, kbase, vtbase, false, q, (int)lo);
+        __syncthreads();                                  // LDS changes hands
+        il_block<HD>(a, prefill_smem_raw, lo, kvh, hc, kbase, vtbase, true, q, -1);
     }
 }
 
