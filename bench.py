@@ -470,6 +470,27 @@ def main() -> None:
             except Exception as exc:                  # reported, not fatal to the headline line
                 decode_configs.append({"workload": name, "error": repr(exc)[:200]})
 
+    # ---- what a kernel that only reads gets out of HBM on this device, for the
+    # decode kernel's access pattern and for the friendliest one (secondary
+    # figure: the roofline above stays priced against the published peak)
+    read_probe = None
+    probe_exe = os.path.join(ROOT, "wayruntime_amd", "calib_read")
+    if not args.no_decode_configs and os.path.exists(probe_exe):
+        import subprocess
+        try:
+            res = subprocess.run([probe_exe, "256", "24"], capture_output=True, text=True, timeout=120)
+            read_probe = []
+            for ln in res.stdout.splitlines():
+                if " avg " in ln and "GB/s" in ln:
+                    f = ln.split()
+                    read_probe.append({"pattern": ln.split("  grid")[0].strip(), "workgroups": int(f[f.index("grid") + 1]),
+                                       "kernel_us": float(f[f.index("avg") + 1]),
+                                       "GB/s": float(f[f.index("GB/s") - 1])})
+            if res.returncode != 0 or not read_probe:
+                read_probe = {"error": "exit %d: %s" % (res.returncode, (res.stderr or res.stdout)[-200:])}
+        except Exception as exc:
+            read_probe = {"error": repr(exc)[:200]}
+
     # ---- the host engine end to end on a random-init Qwen3-0.6B-shaped model
     # (secondary figures): a child process, so this process's device state and
     # the engine's do not meet.  A failure is reported, not fatal.
@@ -500,6 +521,7 @@ def main() -> None:
                    "sessions": S, "ctx": ctx if len(set(ctxs)) == 1 else ctxs, "layers": L},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
         "roofline": roofline, "cpu_baseline": cpu, "prefill": prefill, "decode_configs": decode_configs,
+        "hbm_read_probe": read_probe,
         "projection": proj,
         "end_to_end": e2e,
         "check": {"max_abs": max_abs, "rel_l2": rel_l2},

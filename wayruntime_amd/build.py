@@ -61,16 +61,20 @@ def build_host() -> str:
     return HOST_SO
 
 
+CALIB_BINS = {"calib_copy": "calib_copy.hip", "calib_read": "calib_read.hip"}
 CALIB_BIN = os.path.join(PKG, "calib_copy")
 
 
 def build_calib() -> str:
-    """Counter-calibration copy program (measurement aid, see csrc/calib_copy.hip)."""
-    res = subprocess.run(["hipcc", "-O3", "--offload-arch=gfx950", "-o", CALIB_BIN,
-                          os.path.join(PKG, "csrc", "calib_copy.hip")], capture_output=True, text=True)
-    if res.returncode != 0:
-        sys.stderr.write(res.stderr)
-        raise RuntimeError("hipcc failed building " + CALIB_BIN)
+    """Measurement aids: the counter-calibration copy program and the read-only
+    bandwidth probe (see csrc/calib_copy.hip, csrc/calib_read.hip)."""
+    for name, src in CALIB_BINS.items():
+        out = os.path.join(PKG, name)
+        res = subprocess.run(["hipcc", "-O3", "--offload-arch=gfx950", "-o", out,
+                              os.path.join(PKG, "csrc", src)], capture_output=True, text=True)
+        if res.returncode != 0:
+            sys.stderr.write(res.stderr)
+            raise RuntimeError("hipcc failed building " + out)
     return CALIB_BIN
 
 

@@ -456,7 +456,7 @@ __device__ __forceinline__ void il_block(const PrefillArgs& a, unsigned char* sm
     using L = SplitLds<HD>;
     static_assert(L::NL == 1 || L::NL == 2, "one or two copies per wave, tile and operand");
     const int tid = threadIdx.x;
-    const int lane = tid & 63;
+    const int lane = il_fresh_lane();                     // per call: nothing lane-derived is shared between the blocks of a workgroup
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // in a scalar register
     const int n = lane & 31, g = lane >> 5;
     const int kg = wave >> 2, sub = wave & 3;             // key set (tile parity), rows served
