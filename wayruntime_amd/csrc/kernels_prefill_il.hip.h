@@ -556,6 +556,7 @@ __device__ __forceinline__ void il_block(const PrefillArgs& a, unsigned char* sm
             h[2] = (_Float16)(x.z * a.qscale);
             h[3] = (_Float16)(x.w * a.qscale);
             *reinterpret_cast<half4*>(&qs[sub][r][(lane % Q::LPR) * 4]) = h;
+            q.x[j] = make_float4(0.f, 0.f, 0.f, 0.f);      // consumed: nothing of it has to outlive the step loop
         }
     }
     f32x16 sa, sb, negm;
