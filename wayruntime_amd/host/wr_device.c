@@ -4,10 +4,11 @@
  * walks on the host).  Used when the device library offers projections
  * (WR_HIP_CAP_PROJ) and every matrix of the model is F16 with dimensions the
  * projection kernel takes; WAYRT_HOST_LAYERS=1 in the environment keeps the
- * host walk.  Per call the host embeds the rows and works out the rotary
- * angles (the reference's polynomial sin / cos and range reduction stay on the
- * host), sends both up once, runs the layers without coming back, and brings
- * down the logits (wr_step, wr_batch_step) or nothing (wr_prefill).  The Gemma
+ * host walk.  Per call the host embeds the rows and sends them up once; the
+ * rotary angles of their positions are made on the device (the reference's
+ * polynomial sin / cos and range reduction restated there bit for bit:
+ * wr_hip_attn_rope_table_dev); the layers run without coming back, and the
+ * logits come down (wr_step, wr_batch_step) or nothing does (wr_prefill).  The Gemma
  * family's block (session.c:251-437) takes the same walk with its own steps:
  * per-layer head_dim, two rotary tables, layers that read another layer's
  * cache, the weightless V norm, sandwich norms, GeGLU, attention scale 1.

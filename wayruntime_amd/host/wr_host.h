@@ -102,8 +102,8 @@ typedef struct wrh_workspace {
     float *rope;                         /* [R][hd/2][2] (cos, sin) of the rows' angles */
     float *rope_swa;                     /* the same for Gemma's sliding-window layers */
     void  *block;
-    /* device walk: `residual` and `rope` already hold the embedded rows and
-     * angles of these tokens (staged while the device worked on the rows before) */
+    /* device walk: `residual` already holds the embedded rows of these tokens
+     * (staged while the device worked on the rows before) */
     const uint32_t *staged_tokens;
     uint32_t staged_rows, staged_pos0;
 } wrh_workspace;
@@ -133,7 +133,7 @@ typedef struct wrh_devspace {
 
 /* Everything a multi-row call of the device walk needs besides the model. */
 struct wrh_scratch {
-    wrh_workspace ws;                    /* host rows (embedding, angles) */
+    wrh_workspace ws;                    /* host rows (embedding) */
     wrh_devspace  ds;
     float        *logits_host;           /* page-locked, [logit_rows][vocab]; NULL when logit_rows == 0 */
     uint32_t      rows, logit_rows;
