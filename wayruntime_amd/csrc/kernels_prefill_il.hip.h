@@ -632,7 +632,7 @@ __device__ __forceinline__ void il_block(const PrefillArgs& a, unsigned char* sm
         mg[NREG * 64 + lane_e] = R.m_run;
         mg[(NREG + 1) * 64 + lane_e] = R.l_run;
     }
-    __syncthreads();
+    lds_barrier();                                        // LDS traffic only: the next block's loads stay in flight
     // rows leave through LDS as well: the merged tile is written row-major into
     // the sub-block's own scratch, then both of its waves store whole rows
     float (*os)[HD + 4] = reinterpret_cast<float (*)[HD + 4]>(mg);
@@ -663,7 +663,7 @@ __device__ __forceinline__ void il_block(const PrefillArgs& a, unsigned char* sm
                 *reinterpret_cast<float4*>(&os[n_e][dt * 32 + 8 * q4 + 4 * g_e]) = v;
             }
     }
-    __syncthreads();
+    lds_barrier();
     {
         constexpr int LPR = HD / 4;                       // lanes per row (one float4 each)
         constexpr int RPI = 64 / LPR;                     // rows per store instruction
@@ -706,7 +706,7 @@ __global__ __launch_bounds__(kSplitThreads, 1) void prefill_il_kernel(const Pref
         il_block<HD>(a, prefill_smem_raw, hi, kvh, hc, kbase, vtbase, false, q, -1);
     } else {
         il_block<HD>(a, prefill_smem_raw, hi, kvh, hc, kbase, vtbase, false, q, (int)lo);
-        __syncthreads();                                  // LDS changes hands
+        lds_barrier();                                    // LDS changes hands
         il_block<HD>(a, prefill_smem_raw, lo, kvh, hc, kbase, vtbase, true, q, -1);
     }
 }
