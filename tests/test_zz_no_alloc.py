@@ -135,3 +135,52 @@ def test_no_alloc_decode_refuses_what_does_not_fit():
         hipattn.set_tuning(0, False)
         for kv in caches:
             kv.close()
+
+
+def test_no_alloc_decode_from_several_threads_shares_the_one_array():
+    # Every calling thread has its own stream in the library, but the scratch
+    # array is one per device: launches that use it are chained by an event
+    # whatever thread they come from.  Four threads each step their own
+    # sessions twenty times through the no-alloc entry point; every output must
+    # equal the ordinary entry point's (which uses per-thread partial buffers).
+    import threading
+    nq, nkv, hd = 32, 8, 128
+    ctx_sets = [[3000, 1500, 2600], [4096, 2049], [1300, 3500, 2200, 2900], [2500]]
+    groups = [_sessions(7700 + 40 * t, ctxs, nkv, hd) for t, ctxs in enumerate(ctx_sets)]
+    qs = [synth.normal(7800 + t, (len(ctxs), nq, hd)) for t, ctxs in enumerate(ctx_sets)]
+    # reference outputs, one thread, ordinary entry point
+    want = []
+    for t, ctxs in enumerate(ctx_sets):
+        q_dev = hipattn.DeviceBuffer.from_host(qs[t])
+        o = hipattn.DeviceBuffer(qs[t].nbytes)
+        hipattn.decode_batched_dev(groups[t][0], 0, ctxs, q_dev, o, nq)
+        hipattn.sync()
+        want.append(o.to_host(qs[t].shape))
+        q_dev.free(); o.free()
+    bad = [None] * 4
+
+    def job(t):
+        try:
+            ctxs = ctx_sets[t]
+            q_dev = hipattn.DeviceBuffer.from_host(qs[t])
+            o = hipattn.DeviceBuffer(qs[t].nbytes)
+            wrong = 0
+            for _ in range(20):
+                assert hipattn.decode_batched_dev_noalloc(groups[t][0], 0, ctxs, q_dev, o, nq) == hipattn.OK
+                hipattn.sync()
+                wrong += not np.array_equal(o.to_host(qs[t].shape), want[t])
+            q_dev.free(); o.free()
+            bad[t] = wrong
+        except Exception as e:
+            bad[t] = repr(e)
+    threads = [threading.Thread(target=job, args=(t,)) for t in range(4)]
+    try:
+        for th in threads:
+            th.start()
+        for th in threads:
+            th.join()
+        assert bad == [0] * 4, bad
+    finally:
+        for caches, _ in groups:
+            for kv in caches:
+                kv.close()
