@@ -641,14 +641,20 @@ __global__ __launch_bounds__(kProjThreads) void proj_row1_kernel(const ProjArgs 
     const uint32_t k_begin = part * kper, k_end = k_begin + kper;
     const half8* wp = a.w + (size_t)(live ? nt0 : ntiles - 1) * ktiles * 64 + lane;
 
-    // the first batch of weights leaves before the row is touched
-    half8 wa[KB], wb[KB];
+    // Up to three batches of weights leave before the row is touched (24 k-steps:
+    // the whole share of a wave for inputs up to 3072 at four waves per tile), so
+    // that they arrive while the row's terms are being made; a launch of this
+    // kernel is a chain of latencies, not of bytes.
+    half8 wa[KB], wb[KB], wc[KB];
     uint32_t kt = k_begin;
-    const uint32_t full_end = k_begin + kper / KB * KB;
-    if (kt < full_end) {
+    const uint32_t nb = kper / KB;                               // whole batches of this wave
+    auto load_batch = [&](half8 (&w)[KB], uint32_t b) {
 #pragma unroll
-        for (int u = 0; u < KB; u++) wa[u] = __builtin_nontemporal_load(&wp[(size_t)(kt + u) * 64]);
-    }
+        for (int u = 0; u < KB; u++) w[u] = __builtin_nontemporal_load(&wp[(size_t)(k_begin + b * KB + u) * 64]);
+    };
+    if (nb > 0) load_batch(wa, 0);
+    if (nb > 1) load_batch(wb, 1);
+    if (nb > 2) load_batch(wc, 2);
 
     // the row's terms, as proj_prep_kernel forms them
     const float* xr = p.x;
@@ -690,21 +696,30 @@ __global__ __launch_bounds__(kProjThreads) void proj_row1_kernel(const ProjArgs 
         const half8 xb = has ? my[(size_t)k * 8] : zero;
         acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(wv, xb, acc, 0, 0, 0);
     };
-    if (kt < full_end) {
-        while (kt + 2 * KB <= full_end) {
+    // k-steps in ascending order, whatever buffer holds them (the order of the sum
+    // is that of proj_rows_kernel<1, 1>)
+    auto steps = [&](const half8 (&w)[KB], uint32_t b) {
 #pragma unroll
-            for (int u = 0; u < KB; u++) wb[u] = __builtin_nontemporal_load(&wp[(size_t)(kt + KB + u) * 64]);
-#pragma unroll
-            for (int u = 0; u < KB; u++) step(wa[u], kt + u);
-#pragma unroll
-            for (int u = 0; u < KB; u++) wa[u] = wb[u];
-            kt += KB;
+        for (int u = 0; u < KB; u++) step(w[u], k_begin + b * KB + u);
+    };
+    if (nb > 0) {
+        steps(wa, 0);
+        if (nb > 3) load_batch(wa, 3);
+        if (nb > 1) {
+            steps(wb, 1);
+            if (nb > 4) load_batch(wb, 4);
         }
-#pragma unroll
-        for (int u = 0; u < KB; u++) step(wa[u], kt + u);
-        kt += KB;
+        if (nb > 2) steps(wc, 2);
+        for (uint32_t b = 3; b < nb; b += 2) {                   // wa holds batch b, wb batch b + 1
+            steps(wa, b);
+            if (b + 2 < nb) load_batch(wa, b + 2);
+            if (b + 1 < nb) {
+                steps(wb, b + 1);
+                if (b + 3 < nb) load_batch(wb, b + 3);
+            }
+        }
     }
-    for (; kt < k_end; kt++) step(__builtin_nontemporal_load(&wp[(size_t)kt * 64]), kt);
+    for (kt = k_begin + nb * KB; kt < k_end; kt++) step(__builtin_nontemporal_load(&wp[(size_t)kt * 64]), kt);
 
     if (S > 1) {                                                 // uniform over the workgroup
         if (part > 0) s_part[(slot * (S - 1) + (part - 1)) * 64 + lane] = acc;
