@@ -388,3 +388,42 @@ def test_work_list_at_its_largest():
     hipattn.set_tuning(0, False)
     for kv in caches:
         kv.close()
+
+
+def test_threads_that_come_and_go_get_a_working_stream():
+    # Every calling thread submits through a stream of its own in the library;
+    # a thread that ends hands its stream and buffers on to the next new thread.
+    # Thirty threads one after another, then eight at once, each attend the
+    # same session: all must produce the main thread's bits.
+    import threading
+    nq, nkv, hd, ctx = 32, 8, 128, 3000
+    _a, _b, k16, v16 = util.make_kv(9100, ctx, nkv, hd)
+    kvs = []
+    for _ in range(8):                            # one cache per concurrent thread (a cache is not shared)
+        kv = hipattn.KVCache(1, hd, nkv, ctx)
+        kv.write_f16(0, 0, k16, v16)
+        kvs.append(kv)
+    q = synth.normal(9101, (nq, hd))
+    want = kvs[0].decode(0, ctx, q)
+    util.assert_close(want, util.oracle_decode(q, k16, v16, ctx), "main thread")
+    bad = []
+
+    def job(i):
+        try:
+            got = kvs[i % 8].decode(0, ctx, q)
+            if not np.array_equal(got, want):
+                bad.append(i)
+        except Exception as e:
+            bad.append(repr(e))
+    for i in range(30):
+        th = threading.Thread(target=job, args=(i,))
+        th.start()
+        th.join()
+    ths = [threading.Thread(target=job, args=(100 + i,)) for i in range(8)]
+    for th in ths:
+        th.start()
+    for th in ths:
+        th.join()
+    for kv in kvs:
+        kv.close()
+    assert not bad, bad

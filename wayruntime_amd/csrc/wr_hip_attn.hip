@@ -666,6 +666,8 @@ struct Entered {
             if (!g.idle.empty()) {
                 c = g.idle.back();
                 g.idle.pop_back();
+                c->profiling = false;            // the thread that had it before may have ended mid-measurement
+                c->ev_used = 0;
             } else {
                 c = ctx_create();
                 if (c) g.ctxs.push_back(c);
@@ -1421,7 +1423,11 @@ int wr_hip_attn_sync(void)
     return sync_checked("sync", 0);
 }
 
-void* wr_hip_attn_stream(void) { return g.inited ? (void*)cx->stream : nullptr; }
+void* wr_hip_attn_stream(void)
+{
+    Entered entered_;
+    return entered_.ok() ? (void*)cx->stream : nullptr;
+}
 
 // ------------------------------------------------------------ projections --
 
