@@ -658,22 +658,11 @@ __global__ __launch_bounds__(kProjThreads) void proj_row1_kernel(const ProjArgs 
 
     // the row's terms, as proj_prep_kernel forms them
     const float* xr = p.x;
-    float inv_rms = 1.0f;
-    if constexpr (SRC == kProjSrcRmsNorm)
-        inv_rms = 1.0f / sqrtf(row_sumsq_256(xr, a.K, s4) / (float)a.K + p.eps);
-    float mx = 0.f;
-    for (uint32_t k = t; k < a.K; k += 256) mx = fmaxf(mx, fabsf(proj_src_value<SRC>(p, xr, k, inv_rms)));
-    mx = block_max_256(mx, s4);
-    uint32_t ex = (__float_as_uint(mx) >> 23) & 0xFFu;
-    if (ex == 0 || ex == 0xFF) ex = 127;
-    if (ex > 253) ex = 253;
-    if (t == 0) s_scale = __uint_as_float(ex << 23);
-    const float inv = __uint_as_float((254u - ex) << 23);
-    for (uint32_t q = t; q < nchunks; q += 256) {
+    auto put_chunk = [&](uint32_t q, const float (&v)[8], float inv) {
         half8 hi, lo;
 #pragma unroll
         for (int j = 0; j < 8; j++) {
-            const float sv = proj_src_value<SRC>(p, xr, q * 8 + j, inv_rms) * inv;
+            const float sv = v[j] * inv;
             _Float16 h = (_Float16)sv;
             if (fabsf((float)h) < 6.103515625e-05f) h = (_Float16)0.0f;      // 2^-14
             hi[j] = h;
@@ -681,6 +670,97 @@ __global__ __launch_bounds__(kProjThreads) void proj_row1_kernel(const ProjArgs 
         }
         sfrag[q * 2] = hi;
         sfrag[q * 2 + 1] = lo;
+    };
+    constexpr int CH = 2;                                        // chunks of eight inputs a thread can hold
+    if (a.K <= 2048u * CH) {
+        // One read of the row: its values stay in registers between the passes
+        // (sum of squares, largest magnitude, terms).  Every pass over memory is a
+        // round trip, and a launch of this kernel is little else.  Same values,
+        // same order of the sum as the passes below (thread t takes the chunks t,
+        // t + 256, ... in order).
+        float v[CH][8];
+        float ss = 0.f;
+#pragma unroll
+        for (int i = 0; i < CH; i++) {
+            const uint32_t q = t + 256u * i;
+            if (q < nchunks) {
+                const f32x4 lo4 = *reinterpret_cast<const f32x4*>(xr + q * 8),
+                            hi4 = *reinterpret_cast<const f32x4*>(xr + q * 8 + 4);
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    v[i][j] = lo4[j];
+                    v[i][4 + j] = hi4[j];
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; j++) v[i][j] = 0.f;
+            }
+            if constexpr (SRC == kProjSrcRmsNorm) {
+#pragma unroll
+                for (int j = 0; j < 8; j++) ss = fmaf(v[i][j], v[i][j], ss);
+            }
+        }
+        if constexpr (SRC == kProjSrcRmsNorm) {
+            const float inv_rms = 1.0f / sqrtf(block_sum_256(ss, s4) / (float)a.K + p.eps);
+#pragma unroll
+            for (int i = 0; i < CH; i++) {
+                const uint32_t q = t + 256u * i;
+                if (q < nchunks) {
+                    const f32x4 wl = *reinterpret_cast<const f32x4*>(p.norm_w + q * 8),
+                                wh = *reinterpret_cast<const f32x4*>(p.norm_w + q * 8 + 4);
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        v[i][j] = v[i][j] * inv_rms * wl[j];
+                        v[i][4 + j] = v[i][4 + j] * inv_rms * wh[j];
+                    }
+                }
+            }
+        } else if constexpr (SRC == kProjSrcSwiglu || SRC == kProjSrcGeglu) {
+#pragma unroll
+            for (int i = 0; i < CH; i++) {
+                const uint32_t q = t + 256u * i;
+                if (q < nchunks) {
+                    const f32x4 ul = *reinterpret_cast<const f32x4*>(xr + a.K + q * 8),
+                                uh = *reinterpret_cast<const f32x4*>(xr + a.K + q * 8 + 4);
+#pragma unroll
+                    for (int j = 0; j < 8; j++) v[i][j] = proj_gated<SRC>(v[i][j], j < 4 ? ul[j] : uh[j - 4]);
+                }
+            }
+        }
+        float mx = 0.f;
+#pragma unroll
+        for (int i = 0; i < CH; i++)
+#pragma unroll
+            for (int j = 0; j < 8; j++) mx = fmaxf(mx, fabsf(v[i][j]));
+        mx = block_max_256(mx, s4);
+        uint32_t ex = (__float_as_uint(mx) >> 23) & 0xFFu;
+        if (ex == 0 || ex == 0xFF) ex = 127;
+        if (ex > 253) ex = 253;
+        if (t == 0) s_scale = __uint_as_float(ex << 23);
+        const float inv = __uint_as_float((254u - ex) << 23);
+#pragma unroll
+        for (int i = 0; i < CH; i++) {
+            const uint32_t q = t + 256u * i;
+            if (q < nchunks) put_chunk(q, v[i], inv);
+        }
+    } else {
+        float inv_rms = 1.0f;
+        if constexpr (SRC == kProjSrcRmsNorm)
+            inv_rms = 1.0f / sqrtf(row_sumsq_256(xr, a.K, s4) / (float)a.K + p.eps);
+        float mx = 0.f;
+        for (uint32_t k = t; k < a.K; k += 256) mx = fmaxf(mx, fabsf(proj_src_value<SRC>(p, xr, k, inv_rms)));
+        mx = block_max_256(mx, s4);
+        uint32_t ex = (__float_as_uint(mx) >> 23) & 0xFFu;
+        if (ex == 0 || ex == 0xFF) ex = 127;
+        if (ex > 253) ex = 253;
+        if (t == 0) s_scale = __uint_as_float(ex << 23);
+        const float inv = __uint_as_float((254u - ex) << 23);
+        for (uint32_t q = t; q < nchunks; q += 256) {
+            float v[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) v[j] = proj_src_value<SRC>(p, xr, q * 8 + j, inv_rms);
+            put_chunk(q, v, inv);
+        }
     }
     __syncthreads();
 
