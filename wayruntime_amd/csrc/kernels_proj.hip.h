@@ -92,14 +92,17 @@ struct ProjPrepArgs {
     float eps;
 };
 
+// (The barriers in these two wait for LDS traffic only: __syncthreads() would
+// also wait for every global load in flight, and the one-row product has its
+// weights on the way while it reduces.)
 __device__ __forceinline__ float block_sum_256(float v, float* s4)
 {
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) v += wave_xor_f32(v, off);
     if ((threadIdx.x & 63) == 0) s4[threadIdx.x >> 6] = v;
-    __syncthreads();
+    lds_barrier();
     const float t = (s4[0] + s4[1]) + (s4[2] + s4[3]);
-    __syncthreads();
+    lds_barrier();
     return t;
 }
 
@@ -108,9 +111,9 @@ __device__ __forceinline__ float block_max_256(float v, float* s4)
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, wave_xor_f32(v, off));
     if ((threadIdx.x & 63) == 0) s4[threadIdx.x >> 6] = v;
-    __syncthreads();
+    lds_barrier();
     const float t = fmaxf(fmaxf(s4[0], s4[1]), fmaxf(s4[2], s4[3]));
-    __syncthreads();
+    lds_barrier();
     return t;
 }
 
@@ -762,7 +765,7 @@ __global__ __launch_bounds__(kProjThreads) void proj_row1_kernel(const ProjArgs 
             put_chunk(q, v, inv);
         }
     }
-    __syncthreads();
+    lds_barrier();                                              // the terms are in LDS (the weights may still be on their way)
 
     // B operand of k-step kt: column 0 = hi, column 8 = lo of row 0, the rest zero
     const int c = lane & 15, g = lane >> 4;
