@@ -12,6 +12,7 @@
 
 #include "common.hip.h"
 #include "kernels_proj.hip.h"      // row_sumsq_256: the one summation order of every row norm
+#include "row8.hip.h"              // a head's norm and rotation with eight lanes per position
 
 namespace wr {
 
@@ -135,22 +136,6 @@ struct QkvAppendArgs {
     float eps;
 };
 
-// wave_sum_f32 over a row whose 64 partial sums sit eight to a lane in eight
-// neighbouring lanes (lane `part` of the eight holds partial sums 8 part ..
-// 8 part + 7).  The wave sum pairs partial sums 32, 16, 8, 4, 2, 1 apart, in
-// that order: the first three are the lanes 4, 2, 1 away, the last three are
-// in the lane.  The same additions, hence the same bits.
-__device__ __forceinline__ float row8_sum_f32(float (&s)[8])
-{
-#pragma unroll
-    for (int m = 4; m >= 1; m >>= 1)
-#pragma unroll
-        for (int e = 0; e < 8; e++) s[e] += wave_xor_f32(s[e], m);
-    const float b0 = s[0] + s[4], b1 = s[1] + s[5], b2 = s[2] + s[6], b3 = s[3] + s[7];
-    const float c0 = b0 + b2, c1 = b1 + b3;
-    return c0 + c1;
-}
-
 // One workgroup's share of qkv_append_kernel for head dims of 128 and 256
 // (NJ = hd / 64) with everything 16-byte aligned: eight lanes per position, all
 // 32 positions of the block at once.  Lane `part` of a position holds the
@@ -170,48 +155,10 @@ __device__ __forceinline__ void qkv_append_row8(const QkvAppendArgs& a, unsigned
     const bool live = i < np;
     const uint32_t r = row0 + (live ? i : 0);
     const float* src = a.qkv + (size_t)r * a.ld + (size_t)h * HD + part * 8;
-    float x[NJ][8];
-#pragma unroll
-    for (int c = 0; c < NJ; c++) {
-        f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = lo;
-        if (live) {
-            lo = *reinterpret_cast<const f32x4*>(src + c * 64);
-            hi = *reinterpret_cast<const f32x4*>(src + c * 64 + 4);
-        }
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-            x[c][e] = lo[e];
-            x[c][4 + e] = hi[e];
-        }
-    }
     const bool is_v = h >= a.nq + a.nkv, is_q = h < a.nq;
-    const float* nw = is_v ? nullptr : (is_q ? a.q_norm : a.k_norm);
-    if (is_v ? a.v_norm != 0 : nw != nullptr) {           // workgroup-uniform
-        float s[8];
-#pragma unroll
-        for (int e = 0; e < 8; e++) {
-            float ss = 0.f;
-#pragma unroll
-            for (int c = 0; c < NJ; c++) ss += x[c][e] * x[c][e];
-            s[e] = ss;
-        }
-        const float inv_rms = 1.0f / sqrtf(row8_sum_f32(s) / (float)HD + a.eps);
-#pragma unroll
-        for (int c = 0; c < NJ; c++) {
-            if (is_v) {
-#pragma unroll
-                for (int e = 0; e < 8; e++) x[c][e] = x[c][e] * inv_rms;
-            } else {
-                const f32x4 wl = *reinterpret_cast<const f32x4*>(nw + c * 64 + part * 8);
-                const f32x4 wh = *reinterpret_cast<const f32x4*>(nw + c * 64 + part * 8 + 4);
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    x[c][e] = x[c][e] * inv_rms * wl[e];
-                    x[c][4 + e] = x[c][4 + e] * inv_rms * wh[e];
-                }
-            }
-        }
-    }
+    float x[NJ][8];
+    row8_head_values<NJ>(x, src, live, is_v ? nullptr : (is_q ? a.q_norm : a.k_norm), is_v && a.v_norm != 0,
+                         a.eps, part, is_v ? nullptr : a.cos_sin + (size_t)r * a.n_rot * 2, a.n_rot);
 
     if (is_v) {
         const uint32_t kvh = h - a.nq - a.nkv;
@@ -231,26 +178,6 @@ __device__ __forceinline__ void qkv_append_row8(const QkvAppendArgs& a, unsigned
         return;
     }
 
-    // rotation of the pairs (j, j + hd/2), j = 64 c + 8 part + e for c < NJ / 2
-    const float* cs = a.cos_sin + (size_t)r * a.n_rot * 2;
-#pragma unroll
-    for (int c = 0; c < NJ / 2; c++) {
-        const uint32_t j0 = c * 64 + part * 8;
-        if (live && j0 < a.n_rot) {                       // n_rot is a multiple of eight here
-#pragma unroll
-            for (int q = 0; q < 4; q++) {
-                const f32x4 t = *reinterpret_cast<const f32x4*>(cs + 2 * j0 + 4 * q);
-#pragma unroll
-                for (int u = 0; u < 2; u++) {
-                    const float co = t[2 * u], sn = t[2 * u + 1];
-                    const float x0 = x[c][2 * q + u], x1 = x[c + NJ / 2][2 * q + u];
-                    const float a0 = x0 * co, b0 = x1 * sn, a1 = x0 * sn, b1 = x1 * co;
-                    x[c][2 * q + u] = a0 - b0;
-                    x[c + NJ / 2][2 * q + u] = a1 + b1;
-                }
-            }
-        }
-    }
     if (!live) return;
     if (is_q) {
         float* dst = a.q_out + ((size_t)r * a.nq + h) * HD + part * 8;
