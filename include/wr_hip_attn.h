@@ -220,6 +220,28 @@ int wr_hip_attn_prefill_dev(wr_hip_kv *kv, uint32_t layer, uint32_t p0,
                             uint32_t nq, float scale_override,
                             uint32_t window);
 
+/* A decode step's row work and attention in one launch: row i of qkv_dev
+ * [n][ld] is session i's stacked projection (nq Q heads, then nkv K heads, then
+ * nkv V heads, hd wide each).  Every head gets its per-head RMSNorm when the two
+ * weight vectors are given (src/core/session.c:459-474), Q and K the rotation of
+ * cos_sin_dev's row i (:475-478); K and V are truncated to F16 and appended at
+ * pos[i] (kv_append_row, :483-486), and the nq heads attend over keys
+ * 0 .. pos[i] (wri_op_gqa_attention, :488-496) into out_dev [n][nq][hd].  Q, the
+ * cache bytes and the output are those of wr_hip_rows_qkv_append_dev followed by
+ * wr_hip_attn_decode_batched_dev with seq_k = pos + 1, bit for bit; the point is
+ * one dependent launch less per layer of a decode step.  Takes head dim 128 with
+ * 16-byte aligned operands, ld a multiple of 4 and n_rot of 8; anything else is
+ * WR_HIP_ERR_UNSUPPORTED with nothing written or counted, and the caller makes
+ * the two calls.  pos[i] >= max_ctx is WR_HIP_ERR_CTX_FULL, nothing written. */
+int wr_hip_attn_append_decode_batched_dev(uint32_t n, wr_hip_kv *const *kv,
+                                          uint32_t layer, const uint32_t *pos,
+                                          const float *qkv_dev, uint32_t ld,
+                                          uint32_t nq, const float *q_norm_dev,
+                                          const float *k_norm_dev, float eps,
+                                          const float *cos_sin_dev, uint32_t n_rot,
+                                          float *out_dev, float scale_override,
+                                          uint32_t window);
+
 /* wr_hip_attn_decode_batched_dev for callers that cannot allocate device
  * memory (code under HIP graph capture, tight serving loops, harnesses that
  * forbid hipMalloc).  It has no counterpart in the reference.  Same arguments,

@@ -257,6 +257,16 @@ int wr_hip_attn_decode_batched_dev(uint32_t n, wr_hip_kv *const *kv, uint32_t la
     (void)window;
     return WR_HIP_ERR_STATE;
 }
+int wr_hip_attn_append_decode_batched_dev(uint32_t n, wr_hip_kv *const *kv, uint32_t layer,
+                                          const uint32_t *pos, const float *qkv, uint32_t ld, uint32_t nq,
+                                          const float *q_norm, const float *k_norm, float eps,
+                                          const float *cos_sin, uint32_t n_rot, float *out,
+                                          float scale_override, uint32_t window)
+{
+    (void)n; (void)kv; (void)layer; (void)pos; (void)qkv; (void)ld; (void)nq; (void)q_norm; (void)k_norm;
+    (void)eps; (void)cos_sin; (void)n_rot; (void)out; (void)scale_override; (void)window;
+    return WR_HIP_ERR_STATE;
+}
 int wr_hip_attn_rope_table_dev(float *cos_sin, uint32_t rows, uint32_t pos0, const uint32_t *pos,
                                uint32_t hd, float theta_base, uint32_t n_rot_pairs)
 {

@@ -427,3 +427,93 @@ def test_threads_that_come_and_go_get_a_working_stream():
     for kv in kvs:
         kv.close()
     assert not bad, bad
+
+
+# ---------------------------------------------- row step inside the attention launch --
+
+@pytest.mark.parametrize("nq,nkv,norm,rot_pairs,window,kpw", [
+    (16, 8, True, 0, 0, 0),          # Qwen3: per-head norms, full rotation
+    (32, 8, False, 0, 0, 0),         # Llama: no norms
+    (32, 8, True, 24, 0, 0),         # partial rotation
+    (16, 8, True, 0, 300, 0),        # sliding window
+    (16, 8, True, 0, 0, 64),         # forced fine key splits: the new row's tile is the last split's
+])
+def test_append_and_decode_in_one_launch_equals_the_two_calls(nq, nkv, norm, rot_pairs, window, kpw):
+    # wr_hip_attn_append_decode_batched_dev against wr_hip_rows_qkv_append_dev +
+    # wr_hip_attn_decode_batched_dev on twin caches: the same output bits and
+    # the same cache bytes, for one session and for a ragged batch, at positions
+    # on every side of a 32-key tile edge; both also against the oracle.
+    import ctypes as C
+    hd, eps, theta = 128, 1e-6, 1e6
+    lib = hipattn.lib()
+    positions = [0, 1, 31, 32, 33, 63, 64, 500, 1023, 1024, 2047, 2500, 95, 96, 1999, 7]
+    cap = 2600
+    n_rot = rot_pairs if rot_pairs else hd // 2
+    width = (nq + 2 * nkv) * hd
+    qw = synth.normal(9300, (hd,), std=1.0) if norm else None
+    kw = synth.normal(9301, (hd,), std=1.0) if norm else None
+    qwd = hipattn.DeviceBuffer.from_host(qw) if norm else None
+    kwd = hipattn.DeviceBuffer.from_host(kw) if norm else None
+    for n in (1, 16):
+        pos = positions[:n] if n > 1 else [777]
+        print("fused step", nq, nkv, norm, rot_pairs, window, kpw, "n", n, flush=True)
+        twins = []
+        for i in range(n):
+            _a, _b, k16, v16 = util.make_kv(9400 + 2 * i, cap, nkv, hd)
+            pair = []
+            for _ in range(2):
+                kv = hipattn.KVCache(1, hd, nkv, cap)
+                kv.write_f16(0, 0, k16, v16)          # rows at and above pos hold other data: they must not matter
+                pair.append(kv)
+            twins.append(pair)
+        x = synth.normal(9500 + n, (n, width), std=1.5)
+        xd = hipattn.DeviceBuffer.from_host(x)
+        tab = np.concatenate([oracle.rope_table(1, hd, p, theta, rot_pairs) for p in pos])
+        td = hipattn.DeviceBuffer.from_host(tab)
+        pp = (C.c_uint32 * n)(*pos)
+        sk = (C.c_uint32 * n)(*[p + 1 for p in pos])
+        qn = qwd.p if norm else None
+        kn = kwd.p if norm else None
+        hipattn.set_tuning(kpw, False)
+        # two calls, on the first twin of every session
+        kv_a = (C.c_void_p * n)(*[t[0].h for t in twins])
+        q_dev = hipattn.DeviceBuffer(n * nq * hd * 4)
+        o_a = hipattn.DeviceBuffer.from_host(np.full((n, nq, hd), 3.0, dtype=np.float32))
+        assert lib.wr_hip_rows_qkv_append_dev(xd.p, width, n, nq, qn, kn, eps, td.p, n_rot, n, kv_a, 0, pp,
+                                              q_dev.p, 0) == hipattn.OK
+        assert lib.wr_hip_attn_decode_batched_dev(n, kv_a, 0, sk, q_dev.p, o_a.p, nq, 0.0, window) == hipattn.OK
+        # one call, on the second twin
+        kv_b = (C.c_void_p * n)(*[t[1].h for t in twins])
+        o_b = hipattn.DeviceBuffer.from_host(np.full((n, nq, hd), -4.0, dtype=np.float32))
+        calls = int(hipattn.lib().wr_hip_attn_calls())
+        assert lib.wr_hip_attn_append_decode_batched_dev(n, kv_b, 0, pp, xd.p, width, nq, qn, kn, eps, td.p, n_rot,
+                                                         o_b.p, 0.0, window) == hipattn.OK
+        assert int(hipattn.lib().wr_hip_attn_calls()) == calls + n
+        hipattn.sync()
+        hipattn.set_tuning(0, False)
+        got_a, got_b = o_a.to_host((n, nq, hd)), o_b.to_host((n, nq, hd))
+        assert np.array_equal(got_a, got_b), "outputs differ from the two-call path"
+        for i in range(n):
+            ka, va = twins[i][0].read_f16(0, 0, pos[i] + 1)
+            kb, vb = twins[i][1].read_f16(0, 0, pos[i] + 1)
+            assert np.array_equal(ka, kb) and np.array_equal(va, vb), f"cache of session {i} differs"
+            util.assert_close(got_b[i], util.oracle_decode(q_dev.to_host((n, nq, hd))[i], ka, va, pos[i] + 1, 0.0, window),
+                              f"session {i}")
+        # refusals: a full cache (nothing written), a shape the one-launch form does not take
+        full = (C.c_uint32 * n)(*([cap] + list(pos[1:])))
+        assert lib.wr_hip_attn_append_decode_batched_dev(n, kv_b, 0, full, xd.p, width, nq, qn, kn, eps, td.p, n_rot,
+                                                         o_b.p, 0.0, window) == hipattn.ERR_CTX_FULL
+        calls = int(hipattn.lib().wr_hip_attn_calls())
+        assert lib.wr_hip_attn_append_decode_batched_dev(n, kv_b, 0, pp, xd.p, width + 2, nq, qn, kn, eps, td.p, n_rot,
+                                                         o_b.p, 0.0, window) == hipattn.ERR_UNSUPPORTED
+        assert int(hipattn.lib().wr_hip_attn_calls()) == calls
+        hipattn.sync()
+        assert np.array_equal(o_b.to_host((n, nq, hd)), got_b)
+        for b in (xd, td, q_dev, o_a, o_b):
+            b.free()
+        for pair in twins:
+            for kv in pair:
+                kv.close()
+    for b in (qwd, kwd):
+        if b is not None:
+            b.free()

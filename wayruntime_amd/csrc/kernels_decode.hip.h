@@ -41,6 +41,7 @@
 #pragma once
 
 #include "common.hip.h"
+#include "row8.hip.h"
 
 namespace wr {
 
@@ -79,6 +80,32 @@ struct DecodeArgs {
     // the same share of a ragged batch.
     uint32_t n_items;
     uint16_t items[kBatchMax * 64];
+};
+
+// The decode step's new row made inside the attention launch (FUSED form of the
+// MFMA kernel, head dim 128): row i of qkv is session i's stacked projection
+// [nq Q heads | nkv K heads | nkv V heads]; the heads get their per-head RMSNorm
+// (when the weights are given) and the rotation of the row's position, Q goes
+// straight into the kernel's Q^T operand, and the workgroup whose key range
+// holds the new position (seq_k - 1) truncates K and V to F16, writes them into
+// the cache for later steps and puts them into its own copy of that tile, which
+// was read before the row existed.  The arithmetic is qkv_append_kernel's
+// (row8.hip.h), so Q, the cache and the output are the bits of the two launches
+// this replaces (reference: src/core/session.c:459-496).
+struct DecodeFusedArgs {
+    const float* qkv;        // [n][ld]
+    const float* q_norm;     // [hd] or null
+    const float* k_norm;
+    const float* cos_sin;    // [n][n_rot][2], or null when n_rot == 0
+    uint32_t ld, n_rot;
+    float eps;
+    uint32_t pad_;
+};
+
+template <int HD>
+struct DecodeNewRow {        // the new position's K and V as the cache holds them
+    uint16_t k[HD];
+    uint16_t v[HD];
 };
 
 struct TileRange {
@@ -400,12 +427,46 @@ __device__ __forceinline__ void tile_update(DecodeState<HD>& st, DecodeFrag<HD>&
     }
 }
 
+// Position p (0..31) of a tile held in registers replaced by the new row: its K
+// row is slot k_tile_slot(p) of half k_tile_half(p) (the lanes 16 g + slot hold
+// its chunks 4 s + g), its V values are element p % 8 of the lanes of group p / 8.
+template <int HD>
+__device__ __forceinline__ void patch_new_row(DecodeFrag<HD>& f, const DecodeNewRow<HD>& nr, uint32_t p,
+                                              int lane)
+{
+    const uint32_t m = lane & 15, g = lane >> 4;
+    if (m == k_tile_slot(p)) {
+        const bool upper = k_tile_half(p) != 0;
+#pragma unroll
+        for (int s = 0; s < HD / 32; s++) {
+            const half8 kv = *reinterpret_cast<const half8*>(&nr.k[(4 * s + g) * 8]);
+            if (upper)
+                f.k[1][s] = kv;
+            else
+                f.k[0][s] = kv;
+        }
+    }
+    if (g == (p >> 3)) {
+        const uint32_t e = p & 7;
+#pragma unroll
+        for (int dt = 0; dt < HD / 16; dt++) {
+            const uint16_t bits = nr.v[dt * 16 + m];
+            const _Float16 val = *reinterpret_cast<const _Float16*>(&bits);
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+                if ((uint32_t)j == e) f.v[dt][j] = val;
+        }
+    }
+}
+
 template <int HD>
 __device__ __forceinline__ void process_tile(DecodeState<HD>& st, DecodeFrag<HD>& f,
                                              const half8 (&qop)[HD / 32], uint32_t tile,
                                              uint32_t key_lo, uint32_t seq_k, int lane,
-                                             int partner_addr, int col_kind)
+                                             int partner_addr, int col_kind,
+                                             const DecodeNewRow<HD>* nr = nullptr, uint32_t patch_tile = 0xFFFFFFFFu)
 {
+    if (nr != nullptr && tile == patch_tile) patch_new_row<HD>(f, *nr, (seq_k - 1) % kTileKeys, lane);
     f32x4 c[2];
     tile_scores<HD>(c, f, qop);
     tile_update<HD>(st, f, c, tile, key_lo, seq_k, lane, partner_addr, col_kind);
@@ -421,10 +482,11 @@ __device__ __forceinline__ void process_tile(DecodeState<HD>& st, DecodeFrag<HD>
 template <int HD>
 constexpr bool decode_single_buffered() { return HD >= 256; }
 
-template <int HD>
+template <int HD, bool FUSED = false>
 __global__ __launch_bounds__(kDecodeThreads, 2)
-void decode_mfma_kernel(const DecodeArgs a)
+void decode_mfma_kernel(const DecodeArgs a, const DecodeFusedArgs fz)
 {
+    static_assert(!FUSED || HD == 128, "the fused form is built for head dim 128");
     const uint32_t kvh = blockIdx.x;
     const uint32_t item = a.items[blockIdx.y];
     const uint32_t sess = item >> 8, split = item & 0xFFu;
@@ -446,12 +508,33 @@ void decode_mfma_kernel(const DecodeArgs a)
     // no workgroup can ask for a second tile until then: the queue runs dry once.
     constexpr bool kSingle = decode_single_buffered<HD>();
     constexpr int kQPerThread = kMaxGroupMfma * HD / kDecodeThreads;
-    const float* qg = a.q + ((size_t)sess * a.nq + kvh * G) * HD;     // G contiguous rows
+    constexpr int kNJ = FUSED ? HD / 64 : 1;
     float qreg[kQPerThread];
+    float xrow[kNJ][8];                                   // FUSED: this lane's share of one head of the new row
+    // FUSED: the new position's tile, whether this workgroup's range holds it,
+    // and the wave that has it (its last tile)
+    const uint32_t new_pos = S.seq_k - 1, new_tile = new_pos / kTileKeys;
+    const bool owner = FUSED && new_tile >= tr.t_begin && new_tile < tr.t_end;
+    const uint32_t patch_tile =
+        (owner && (new_tile - tr.t_begin) % kDecodeWaves == (uint32_t)wave) ? new_tile : 0xFFFFFFFFu;
+    const uint32_t hslot = threadIdx.x >> 3, part = threadIdx.x & 7;   // FUSED: head slot (Q heads, K, V), lane of eight
+    if constexpr (FUSED) {
+        if (hslot < (uint32_t)G + (owner ? 2u : 0u)) {
+            const bool is_q = hslot < (uint32_t)G, is_k = hslot == (uint32_t)G;
+            const uint32_t head = is_q ? kvh * G + hslot : (is_k ? a.nq + kvh : a.nq + a.nkv + kvh);
+            const float* src = fz.qkv + (size_t)sess * fz.ld + (size_t)head * HD + part * 8;
+            row8_head_values<kNJ>(xrow, src, true, is_q ? fz.q_norm : (is_k ? fz.k_norm : nullptr), false, fz.eps,
+                                  part, (hslot <= (uint32_t)G && fz.cos_sin) ? fz.cos_sin + (size_t)sess * fz.n_rot * 2
+                                                                              : nullptr,
+                                  fz.n_rot);
+        }
+    } else {
+        const float* qg = a.q + ((size_t)sess * a.nq + kvh * G) * HD;     // G contiguous rows
 #pragma unroll
-    for (int i = 0; i < kQPerThread; i++) {
-        const int idx = threadIdx.x + i * kDecodeThreads;
-        qreg[i] = (idx < G * HD) ? qg[idx] : 0.f;
+        for (int i = 0; i < kQPerThread; i++) {
+            const int idx = threadIdx.x + i * kDecodeThreads;
+            qreg[i] = (idx < G * HD) ? qg[idx] : 0.f;
+        }
     }
     // Both loads are unconditional (a wave with fewer tiles re-reads the
     // workgroup's last one and ignores it): the compiler places its waits by
@@ -467,7 +550,50 @@ void decode_mfma_kernel(const DecodeArgs a)
     // 0..G-1 hold the hi terms of the group's heads, G..2G-1 the lo terms,
     // the rest zero; values are pre-multiplied by scale*log2(e).
     __shared__ __attribute__((aligned(16))) _Float16 lds_q[16][HD + 8];
-    {
+    __shared__ __attribute__((aligned(16))) DecodeNewRow<FUSED ? HD : 8> new_row;
+    if constexpr (FUSED) {
+        if (hslot < (uint32_t)G) {
+            // a Q head: element 64 c + 8 part + e of MFMA columns hslot (hi) and hslot + G (lo)
+#pragma unroll
+            for (int c = 0; c < kNJ; c++)
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const int d = c * 64 + (int)part * 8 + e;
+                    const float x = xrow[c][e] * a.qscale;
+                    const _Float16 hi = (_Float16)x;
+                    lds_q[hslot][d] = hi;
+                    lds_q[hslot + G][d] = (_Float16)(x - (float)hi);
+                }
+        } else if (owner && hslot == (uint32_t)G) {
+            // the K head: truncated to F16, into the cache and into the workgroup's copy
+            uint16_t* kw = const_cast<uint16_t*>(S.k);
+#pragma unroll
+            for (int c = 0; c < kNJ; c++) {
+                uint32_t w[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    w[e] = (uint32_t)f32_to_f16_trunc(xrow[c][2 * e]) |
+                           ((uint32_t)f32_to_f16_trunc(xrow[c][2 * e + 1]) << 16);
+                const u32x4 packed = u32x4{w[0], w[1], w[2], w[3]};
+                *reinterpret_cast<u32x4*>(kw + k_offset(kvh, S.ctx_pad, new_pos, c * 64 + part * 8, HD)) = packed;
+                *reinterpret_cast<u32x4*>(&new_row.k[c * 64 + part * 8]) = packed;
+            }
+        } else if (owner && hslot == (uint32_t)G + 1) {
+            // the V head: truncated, into the block-transposed Vt and the workgroup's copy
+            uint16_t* vw = const_cast<uint16_t*>(S.vt);
+#pragma unroll
+            for (int c = 0; c < kNJ; c++)
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const uint32_t d = c * 64 + part * 8 + e;
+                    const uint16_t bits = f32_to_f16_trunc(xrow[c][e]);
+                    vw[vt_offset(kvh, S.ctx_pad, new_pos, d, HD)] = bits;
+                    new_row.v[d] = bits;
+                }
+        }
+        for (int idx = threadIdx.x; idx < (16 - 2 * G) * HD; idx += kDecodeThreads)
+            lds_q[2 * G + idx / HD][idx % HD] = (_Float16)0.0f;
+    } else {
 #pragma unroll
         for (int i = 0; i < kQPerThread; i++) {
             const int idx = threadIdx.x + i * kDecodeThreads;
@@ -483,6 +609,8 @@ void decode_mfma_kernel(const DecodeArgs a)
             lds_q[2 * G + idx / HD][idx % HD] = (_Float16)0.0f;
     }
     __syncthreads();
+    const DecodeNewRow<HD>* nrp = nullptr;
+    if constexpr (FUSED) nrp = reinterpret_cast<const DecodeNewRow<HD>*>(&new_row);
     half8 qop[kSingle ? 1 : HD / 32];
     if constexpr (!kSingle) {
 #pragma unroll
@@ -523,24 +651,24 @@ void decode_mfma_kernel(const DecodeArgs a)
         // fa holds tile t, fb tile t + W (both asked for above); each tile's
         // buffer is refilled with the tile two rounds on as soon as it is used
         while (t + 3 * kDecodeWaves < tr.t_end) {
-            process_tile<HD>(st, fa, qop, t, S.key_lo, S.seq_k, lane, partner_addr, col_kind);
+            process_tile<HD>(st, fa, qop, t, S.key_lo, S.seq_k, lane, partner_addr, col_kind, nrp, patch_tile);
             load_frag<HD>(fa, kbase, vtbase, t + 2 * kDecodeWaves, lane);
             process_tile<HD>(st, fb, qop, t + kDecodeWaves, S.key_lo, S.seq_k, lane, partner_addr,
-                             col_kind);
+                             col_kind, nrp, patch_tile);
             load_frag<HD>(fb, kbase, vtbase, t + 3 * kDecodeWaves, lane);
             t += 2 * kDecodeWaves;
         }
         // one, two or three tiles left; the first two are in flight
-        process_tile<HD>(st, fa, qop, t, S.key_lo, S.seq_k, lane, partner_addr, col_kind);
+        process_tile<HD>(st, fa, qop, t, S.key_lo, S.seq_k, lane, partner_addr, col_kind, nrp, patch_tile);
         if (t + 2 * kDecodeWaves < tr.t_end) {
             load_frag<HD>(fa, kbase, vtbase, t + 2 * kDecodeWaves, lane);
             process_tile<HD>(st, fb, qop, t + kDecodeWaves, S.key_lo, S.seq_k, lane, partner_addr,
-                             col_kind);
+                             col_kind, nrp, patch_tile);
             process_tile<HD>(st, fa, qop, t + 2 * kDecodeWaves, S.key_lo, S.seq_k, lane, partner_addr,
-                             col_kind);
+                             col_kind, nrp, patch_tile);
         } else if (t + kDecodeWaves < tr.t_end) {
             process_tile<HD>(st, fb, qop, t + kDecodeWaves, S.key_lo, S.seq_k, lane, partner_addr,
-                             col_kind);
+                             col_kind, nrp, patch_tile);
         }
     }
     // denominator: add the four lane groups' shares

@@ -334,7 +334,8 @@ struct DecodeWorkspace {
 
 int decode_locked(uint32_t n, wr_hip_kv* const* kv, uint32_t layer, const uint32_t* seq_k,
                   const float* q_dev, float* out_dev, uint32_t nq, float scale_override,
-                  uint32_t window, const DecodeWorkspace& fixed = DecodeWorkspace())
+                  uint32_t window, const DecodeWorkspace& fixed = DecodeWorkspace(),
+                  const DecodeFusedArgs* fused = nullptr)
 {
     const uint32_t hd = kv[0]->hd[layer], nkv = kv[0]->nkv;
     const uint32_t group = nq / nkv;
@@ -455,14 +456,19 @@ int decode_locked(uint32_t n, wr_hip_kv* const* kv, uint32_t layer, const uint32
         }
     }
 
+    if (fused && !(use_mfma && hd == 128)) return WR_HIP_ERR_UNSUPPORTED;
     if (use_mfma) {
         const dim3 grid(nkv, a.n_items), block(kDecodeThreads);
-        if (hd == 64)
-            launch_main(decode_mfma_kernel<64>, grid, block, a);
+        DecodeFusedArgs none;
+        memset(&none, 0, sizeof none);
+        if (fused)
+            launch_main(decode_mfma_kernel<128, true>, grid, block, a, *fused, 0);
+        else if (hd == 64)
+            launch_main(decode_mfma_kernel<64>, grid, block, a, none, 0);
         else if (hd == 128)
-            launch_main(decode_mfma_kernel<128>, grid, block, a);
+            launch_main(decode_mfma_kernel<128>, grid, block, a, none, 0);
         else
-            launch_main(decode_mfma_kernel<256>, grid, block, a);
+            launch_main(decode_mfma_kernel<256>, grid, block, a, none, 0);
     } else {
         launch_main(decode_generic_kernel, dim3(nq, a.n_items), dim3(kDecodeThreads), a);
     }
@@ -1286,6 +1292,51 @@ int wr_hip_attn_decode_batched_dev_noalloc(uint32_t n, wr_hip_kv* const* kv, uin
     rc = decode_locked(n, kv, layer, seq_k, q_dev, out_dev, nq, scale_override, window, fixed);
     if (hipEventRecord(g.noalloc_done, cx->stream) == hipSuccess) g.noalloc_recorded = true;
     return rc;
+}
+
+int wr_hip_attn_append_decode_batched_dev(uint32_t n, wr_hip_kv* const* kv, uint32_t layer,
+                                          const uint32_t* pos, const float* qkv_dev, uint32_t ld,
+                                          uint32_t nq, const float* q_norm_dev, const float* k_norm_dev,
+                                          float eps, const float* cos_sin_dev, uint32_t n_rot,
+                                          float* out_dev, float scale_override, uint32_t window)
+{
+    if (!g.inited) return WR_HIP_ERR_STATE;
+    if (!kv || !pos || !qkv_dev || !out_dev) return WR_HIP_ERR_INVAL;
+    if (n == 0 || n > WR_HIP_BATCH_MAX) return WR_HIP_ERR_LIMIT;
+    for (uint32_t i = 0; i < n; i++) {
+        if (!kv[i]) return WR_HIP_ERR_INVAL;
+        int rc = check_layer(kv[i], layer);
+        if (rc) return rc;
+    }
+    const uint32_t hd = kv[0]->hd[layer], nkv = kv[0]->nkv;
+    if (nq == 0 || nq % nkv != 0) return WR_HIP_ERR_INVAL;
+    if ((q_norm_dev == nullptr) != (k_norm_dev == nullptr)) return WR_HIP_ERR_INVAL;
+    if (n_rot > hd / 2 || (n_rot > 0 && !cos_sin_dev)) return WR_HIP_ERR_INVAL;
+    if ((uint64_t)ld < (uint64_t)(nq + 2 * nkv) * hd) return WR_HIP_ERR_INVAL;
+    // What the in-kernel form of the row step takes; for anything else the caller
+    // keeps the two separate calls (nothing has been counted or written yet).
+    const uintptr_t addrs = (uintptr_t)qkv_dev | (uintptr_t)cos_sin_dev | (uintptr_t)q_norm_dev |
+                            (uintptr_t)k_norm_dev;
+    if (hd != 128 || !mfma_shape(hd, nq / nkv) || n_rot % 8 != 0 || ld % 4 != 0 || addrs % 16 != 0)
+        return WR_HIP_ERR_UNSUPPORTED;
+    uint32_t seq_k[WR_HIP_BATCH_MAX];
+    for (uint32_t i = 0; i < n; i++) {
+        if (pos[i] >= kv[i]->max_ctx) return WR_HIP_ERR_CTX_FULL;          // as the append: nothing is written
+        seq_k[i] = pos[i] + 1;
+    }
+    int rc = check_decode(n, kv, layer, seq_k, qkv_dev, out_dev, nq);      // the attention's own checks, the call counter
+    if (rc) return rc;
+    DecodeFusedArgs fz;
+    memset(&fz, 0, sizeof fz);
+    fz.qkv = qkv_dev;
+    fz.q_norm = q_norm_dev;
+    fz.k_norm = k_norm_dev;
+    fz.cos_sin = n_rot ? cos_sin_dev : nullptr;
+    fz.ld = ld;
+    fz.n_rot = n_rot;
+    fz.eps = eps;
+    ENTER();
+    return decode_locked(n, kv, layer, seq_k, nullptr, out_dev, nq, scale_override, window, DecodeWorkspace(), &fz);
 }
 
 int wr_hip_attn_decode_batched(uint32_t n, wr_hip_kv* const* kv, uint32_t layer,

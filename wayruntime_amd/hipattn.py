@@ -71,6 +71,9 @@ def load() -> C.CDLL:
         "wr_hip_attn_decode_batched_dev_noalloc": (C.c_int, [_u32, C.POINTER(_vp), _u32,
                                                              C.POINTER(_u32), _vp, _vp, _u32,
                                                              C.c_float, _u32]),
+        "wr_hip_attn_append_decode_batched_dev": (C.c_int, [_u32, C.POINTER(_vp), _u32, C.POINTER(_u32),
+                                                            _vp, _u32, _u32, _vp, _vp, C.c_float, _vp,
+                                                            _u32, _vp, C.c_float, _u32]),
         "wr_hip_attn_prefill_dev": (C.c_int, [_vp, _u32, _u32, _u32, _vp, _vp, _u32, C.c_float,
                                               _u32]),
         "wr_hip_proj_weight_create": (C.c_int, [_u32, C.POINTER(_vp), C.POINTER(_u32), _u32,

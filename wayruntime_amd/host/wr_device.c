@@ -4,7 +4,8 @@
  * walks on the host).  Used when the device library offers projections
  * (WR_HIP_CAP_PROJ) and every matrix of the model is F16 with dimensions the
  * projection kernel takes; WAYRT_HOST_LAYERS=1 in the environment keeps the
- * host walk.  Per call the host embeds the rows and sends them up once; the
+ * host walk, WAYRT_STEP_TWO_LAUNCHES=1 keeps a decode step's row step and its
+ * attention as two launches.  Per call the host embeds the rows and sends them up once; the
  * rotary angles of their positions are made on the device (the reference's
  * polynomial sin / cos and range reduction restated there bit for bit:
  * wr_hip_attn_rope_table_dev); the layers run without coming back, and the
@@ -35,6 +36,11 @@ struct wrh_dev_model {
     wr_hip_weight *lm_head;
     float         *vecs;                                       /* one device block for all norm vectors */
     const float   *final_norm;
+    /* decode steps: does the library take the row step (split, norms, rotation,
+     * append) inside the attention launch for this model?  0 = not asked yet,
+     * 1 = yes, -1 = no (the two calls are made).  Read and written atomically:
+     * sessions step from several threads. */
+    int            step_in_one_launch;
 };
 
 static int proj_dims_ok(const wrh_weight *w)
@@ -93,6 +99,9 @@ wr_status wrh_device_model_init(wr_model *m)
     struct wrh_dev_model *d = calloc(1, sizeof *d);
     if (!d) return WR_ERR_NOMEM;
     m->dev = d;
+    /* WAYRT_STEP_TWO_LAUNCHES=1: a decode step's row step and attention stay two calls */
+    env = getenv("WAYRT_STEP_TWO_LAUNCHES");
+    if (env && env[0] == '1') d->step_in_one_launch = -1;
     int rc = WR_HIP_OK;
     /* norm vectors: [final | per layer: attn, ffn, (q, k), (post-attn, post-ffn)] */
     size_t n_vec = m->hidden;
@@ -369,7 +378,32 @@ wr_status wrh_forward_rows_device(wr_model *m, wrh_workspace *hs, wrh_devspace *
                                       ds->qkv, width), "attn norm + qkv projection");
         /* Q/K/V split, per-head norms, rotation and the cache append in one launch */
         if (fail_layer == (int)L) return dev_fail(e, "gqa (injected)", L, WR_ERR_INTERNAL);
-        if (batch) {
+        /* A decode step of the plain block (one row per session): the row step and
+         * the attention in ONE launch where the library takes the shape -- the
+         * same bits as the two calls below, one dependent launch less per layer. */
+        int fused_done = 0;
+        if (!prefill && !gemma && !shared && (batch || R == 1) &&
+            __atomic_load_n(&m->dev->step_in_one_launch, __ATOMIC_RELAXED) >= 0) {
+            wr_hip_kv *kvs[WR_BATCH_MAX];
+            uint32_t at[WR_BATCH_MAX];
+            for (uint32_t r = 0; r < R; r++) {
+                kvs[r] = batch ? ss[r]->kv : ss[0]->kv;
+                at[r] = batch ? ss[r]->pos : pos0;
+            }
+            rc = wr_hip_attn_append_decode_batched_dev(R, kvs, ksrc, at, ds->qkv, width, nq, dl->q_norm, dl->k_norm,
+                                                       m->rms_eps, tab, nr, ds->attn, scale, window);
+            if (rc == WR_HIP_ERR_UNSUPPORTED) {
+                __atomic_store_n(&m->dev->step_in_one_launch, -1, __ATOMIC_RELAXED);
+            } else {
+                if (rc != WR_HIP_OK) return dev_fail(e, "kv append + gqa", L, rc);
+                __atomic_store_n(&m->dev->step_in_one_launch, 1, __ATOMIC_RELAXED);
+                for (uint32_t r = 0; r < R; r++) (batch ? ss[r] : ss[0])->kv_rows[L] = at[r] + 1;
+                fused_done = 1;
+            }
+        }
+        if (fused_done) {
+            /* nothing left to do for the attention of this layer */
+        } else if (batch) {
             wr_hip_kv *kvs[WR_BATCH_MAX];
             uint32_t seq_k[WR_BATCH_MAX];
             uint32_t at[WR_BATCH_MAX];
