@@ -137,6 +137,44 @@ def test_no_alloc_decode_refuses_what_does_not_fit():
             kv.close()
 
 
+def test_partials_of_one_launch_are_never_read_from_the_launch_before():
+    # Two batches of different shape take turns on the one scratch array, back
+    # to back without a host wait in between, so the partial rows a launch
+    # finds there belong to the other batch: a workgroup that merged before
+    # every partial of its own launch had landed would write a row that is
+    # wrong, not merely old.  (A workgroup draws its ticket only after its own
+    # partial stores have been acknowledged.)
+    nq, nkv, hd = 32, 8, 128
+    ctx_sets = [[1300, 3500, 2200, 2900], [4096, 2049, 600]]
+    groups = [_sessions(7900 + 40 * t, ctxs, nkv, hd) for t, ctxs in enumerate(ctx_sets)]
+    qs = [synth.normal(7950 + t, (len(ctxs), nq, hd)) for t, ctxs in enumerate(ctx_sets)]
+    try:
+        want, q_dev, outs = [], [], []
+        for t, ctxs in enumerate(ctx_sets):
+            q_dev.append(hipattn.DeviceBuffer.from_host(qs[t]))
+            o = hipattn.DeviceBuffer(qs[t].nbytes)
+            hipattn.decode_batched_dev(groups[t][0], 0, ctxs, q_dev[t], o, nq)
+            hipattn.sync()
+            want.append(o.to_host(qs[t].shape))
+            o.free()
+        rounds = 40
+        for t in range(2):
+            outs.append([hipattn.DeviceBuffer(qs[t].nbytes) for _ in range(rounds)])
+        for r in range(rounds):
+            for t, ctxs in enumerate(ctx_sets):
+                assert hipattn.decode_batched_dev_noalloc(groups[t][0], 0, ctxs, q_dev[t], outs[t][r], nq) == hipattn.OK
+        hipattn.sync()
+        wrong = [(t, r) for t in range(2) for r in range(rounds)
+                 if not np.array_equal(outs[t][r].to_host(qs[t].shape), want[t])]
+        assert wrong == []
+        for b in q_dev + outs[0] + outs[1]:
+            b.free()
+    finally:
+        for caches, _ in groups:
+            for kv in caches:
+                kv.close()
+
+
 def test_no_alloc_decode_from_several_threads_shares_the_one_array():
     # Every calling thread has its own stream in the library, but the scratch
     # array is one per device: launches that use it are chained by an event
@@ -164,13 +202,16 @@ def test_no_alloc_decode_from_several_threads_shares_the_one_array():
             ctxs = ctx_sets[t]
             q_dev = hipattn.DeviceBuffer.from_host(qs[t])
             o = hipattn.DeviceBuffer(qs[t].nbytes)
-            wrong = 0
-            for _ in range(20):
+            wrong = []
+            for it in range(20):
                 assert hipattn.decode_batched_dev_noalloc(groups[t][0], 0, ctxs, q_dev, o, nq) == hipattn.OK
                 hipattn.sync()
-                wrong += not np.array_equal(o.to_host(qs[t].shape), want[t])
+                got = o.to_host(qs[t].shape)
+                if not np.array_equal(got, want[t]):
+                    d = np.abs(got - want[t]).max(axis=2)              # [session][head]
+                    wrong.append((it, [(int(a), int(b), float(d[a, b])) for a, b in np.argwhere(d > 0)][:8]))
             q_dev.free(); o.free()
-            bad[t] = wrong
+            bad[t] = wrong or 0
         except Exception as e:
             bad[t] = repr(e)
     threads = [threading.Thread(target=job, args=(t,)) for t in range(4)]

@@ -137,9 +137,11 @@ static_assert(sizeof(DecodeArgs::items) == kBatchMax * kMaxSplits * sizeof(uint1
 // launch.  They are written and read with agent-scope relaxed atomics: on
 // gfx950 those are write-through stores / L2-coherent loads (sc1), so the data
 // itself never sits dirty in one XCD's L2.  Ordering against the ticket comes
-// from waiting for the stores to be acknowledged (workgroup-scope release =
-// s_waitcnt vmcnt(0)) and a workgroup barrier before one thread takes the
-// ticket.  A device-wide release fence instead would write back the whole L2
+// from every thread waiting until its own stores have been acknowledged
+// (s_waitcnt vmcnt(0), written out below: a workgroup-scope release fence
+// compiles to no wait at all here, because the waves of a workgroup share one
+// CU) and a workgroup barrier before one thread takes the ticket.  A
+// device-wide release fence instead would write back the whole L2
 // (buffer_wbl2) from every workgroup: measured at 5-10x the kernel's run time.
 #if defined(__HIP_DEVICE_COMPILE__) && !defined(__gfx950__)
 #error "the cross-workgroup exchange below relies on how gfx950 executes agent-scope relaxed atomics (sc1 write-through stores, L2-coherent loads); it has not been argued for any other target"
@@ -204,7 +206,10 @@ __device__ __forceinline__ void publish_and_merge(const DecodeArgs& a, uint32_t 
                                                   uint32_t counter_idx, float* scratch)
 {
     __shared__ uint32_t s_ticket;
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");   // own partial stores acknowledged
+    // own partial stores acknowledged: the ticket below must not be drawn while
+    // one of them is still on its way (the workgroup that merges would read
+    // what the address held before)
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (threadIdx.x == 0)
         s_ticket = __hip_atomic_fetch_add(&a.counters[counter_idx], 1u, __ATOMIC_RELAXED,

@@ -366,7 +366,12 @@ int decode_locked(uint32_t n, wr_hip_kv* const* kv, uint32_t layer, const uint32
     // (one session of 8192 keys: 27 -> 17 us); from
     // 8K keys up an eighth of the session per workgroup measured better
     // (fewer partials and workgroup turnovers: 82 % -> 86 % of HBM peak at
-    // 16 x 32768).  The session's tiles are spread evenly over the workgroups,
+    // 16 x 32768).  A short session (up to 2048 keys at head_dim 128) takes a
+    // quarter of that per workgroup: its launch is a chain of latencies, and a
+    // workgroup that has all its tiles in flight at once ends sooner than one
+    // that walks eight of them per wave (one session of 1024 keys: 12.0 -> 7.8 us,
+    // of 2048: 13.8 -> 8.2 us; 16 sessions of ~520: the step of a 28-layer model
+    // 2.03 -> 1.89 ms).  The session's tiles are spread evenly over the workgroups,
     // and the floor keeps the in-kernel merge within kMaxSplits partials.
     // A single long session gets few workgroups this way; a caller that serves
     // one session at a time can lower the figure with wr_hip_attn_set_tuning.
@@ -381,6 +386,7 @@ int decode_locked(uint32_t n, wr_hip_kv* const* kv, uint32_t layer, const uint32
         } else {
             uint32_t cap = kDefaultTilesPerWg * 128u / (hd < 32 ? 32 : hd);
             if (cap == 0) cap = 1;
+            if (tiles[i] <= 2 * cap) cap = cap >= 4 ? cap / 4 : 1;      // a short session: see above
             if (cap < tiles[i] / 8) cap = tiles[i] / 8;
             const uint32_t want = (tiles[i] + cap - 1) / cap;          // workgroups
             tpw = (tiles[i] + want - 1) / want;                        // even share
