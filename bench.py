@@ -491,6 +491,26 @@ def main() -> None:
         except Exception as exc:
             read_probe = {"error": repr(exc)[:200]}
 
+    # ---- what one launch costs inside a chain of dependent launches (the
+    # device walk's decode step is such a chain): a floor, from kernels that
+    # only read their predecessor's row, reduce it and store (secondary figure)
+    chain_probe = None
+    chain_exe = os.path.join(ROOT, "wayruntime_amd", "calib_chain")
+    if not args.no_e2e and os.path.exists(chain_exe):
+        import subprocess
+        try:
+            res = subprocess.run([chain_exe, "400"], capture_output=True, text=True, timeout=120)
+            chain_probe = []
+            for ln in res.stdout.splitlines():
+                if "us per launch" in ln:
+                    f = ln.split()
+                    chain_probe.append({"kernel": ln.split("  grid")[0].strip(), "workgroups": int(f[f.index("grid") + 1]),
+                                        "us_per_launch": float(f[-1])})
+            if res.returncode != 0 or not chain_probe:
+                chain_probe = {"error": "exit %d: %s" % (res.returncode, (res.stderr or res.stdout)[-200:])}
+        except Exception as exc:
+            chain_probe = {"error": repr(exc)[:200]}
+
     # ---- the host engine end to end on a random-init Qwen3-0.6B-shaped model
     # (secondary figures): a child process, so this process's device state and
     # the engine's do not meet.  A failure is reported, not fatal.
@@ -522,6 +542,7 @@ def main() -> None:
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
         "roofline": roofline, "cpu_baseline": cpu, "prefill": prefill, "decode_configs": decode_configs,
         "hbm_read_probe": read_probe,
+        "launch_chain_probe": chain_probe,
         "projection": proj,
         "end_to_end": e2e,
         "check": {"max_abs": max_abs, "rel_l2": rel_l2},

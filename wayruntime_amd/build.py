@@ -61,13 +61,14 @@ def build_host() -> str:
     return HOST_SO
 
 
-CALIB_BINS = {"calib_copy": "calib_copy.hip", "calib_read": "calib_read.hip"}
+CALIB_BINS = {"calib_copy": "calib_copy.hip", "calib_read": "calib_read.hip", "calib_chain": "calib_chain.hip"}
 CALIB_BIN = os.path.join(PKG, "calib_copy")
 
 
 def build_calib() -> str:
-    """Measurement aids: the counter-calibration copy program and the read-only
-    bandwidth probe (see csrc/calib_copy.hip, csrc/calib_read.hip)."""
+    """Measurement aids: the counter-calibration copy program, the read-only
+    bandwidth probe and the launch-chain probe (see csrc/calib_copy.hip,
+    csrc/calib_read.hip, csrc/calib_chain.hip)."""
     for name, src in CALIB_BINS.items():
         out = os.path.join(PKG, name)
         res = subprocess.run(["hipcc", "-O3", "--offload-arch=gfx950", "-o", out,

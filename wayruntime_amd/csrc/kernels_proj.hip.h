@@ -616,22 +616,28 @@ __global__ __launch_bounds__(kProjThreads) void proj_rows_kernel(const ProjArgs 
 // One row (a decode step): proj_rows_kernel<1, 1> with the fragment kernel
 // folded in.  Every workgroup builds the row's operand terms in its own LDS
 // (4 bytes per input: hi and lo of the one live column pair) while its first
-// batch of weights is on the way, instead of reading fragments a launch before
+// batches of weights are on the way, instead of reading fragments a launch before
 // it wrote: a decode step is a chain of dependent launches of a few
 // microseconds each, and this removes four of ten per layer.  The row's values,
 // the scale and the order of every sum are those of proj_prep_kernel followed
 // by proj_rows_kernel<1, 1> (same helpers, same loops), so the result has the
 // same bits: a serial step still equals its row of a batched step.
-template <int SRC>
-__global__ __launch_bounds__(kProjThreads) void proj_row1_kernel(const ProjArgs a, const ProjPrepArgs p)
+//
+// Order of the requests: the row (with the norm's weights, the gate's partner
+// values and the residual) FIRST, then up to three batches of weights (24
+// k-steps: the whole share of a wave for inputs up to 3072 at four waves per
+// tile).  A wave's loads come back in the order they were asked for, so a row
+// asked for after the weights is not there before them (2.0 us after the
+// workgroup's start, measured, against 0.8); asked for first, the sums over the
+// row run while the weights travel.  NB0 = batches asked for up front, a
+// template parameter so that every load before the first wait is unconditional
+// and the compiler's count of loads in flight is exact.
+template <int SRC, int NB0>
+__device__ __forceinline__ void proj_row1_body(const ProjArgs& a, const ProjPrepArgs& p, half8* sfrag,
+                                               f32x4* s_part, float* s4, float* s_scale)
 {
     constexpr int KB = kProjKBatch;
-    extern __shared__ __attribute__((aligned(16))) unsigned char row1_smem[];
-    half8* sfrag = reinterpret_cast<half8*>(row1_smem);           // [K/8][2]: hi, lo of chunk q
-    __shared__ f32x4 s_part[3 * 64];
-    __shared__ float s4[4];
-    __shared__ float s_scale;
-
+    constexpr int CH = 2;                                        // chunks of eight inputs a thread can hold
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint32_t t = threadIdx.x;
     const uint32_t S = a.ksplit;
@@ -643,24 +649,40 @@ __global__ __launch_bounds__(kProjThreads) void proj_row1_kernel(const ProjArgs 
     const uint32_t kper = ktiles / S;
     const uint32_t k_begin = part * kper, k_end = k_begin + kper;
     const half8* wp = a.w + (size_t)(live ? nt0 : ntiles - 1) * ktiles * 64 + lane;
+    const float* xr = p.x;
+    const bool in_regs = a.K <= 2048u * CH;                      // uniform
 
-    // Up to three batches of weights leave before the row is touched (24 k-steps:
-    // the whole share of a wave for inputs up to 3072 at four waves per tile), so
-    // that they arrive while the row's terms are being made; a launch of this
-    // kernel is a chain of latencies, not of bytes.
+    // 1. the row and what goes with it (a chunk past the end re-reads the last one; dropped below)
+    f32x4 xl[CH], xh[CH];
+    f32x4 el[SRC == kProjSrcPlain ? 1 : CH], eh[SRC == kProjSrcPlain ? 1 : CH];     // norm weights / gate partners
+    if (in_regs) {
+#pragma unroll
+        for (int i = 0; i < CH; i++) {
+            const uint32_t qc = min(t + 256u * i, nchunks - 1);
+            xl[i] = *reinterpret_cast<const f32x4*>(xr + qc * 8);
+            xh[i] = *reinterpret_cast<const f32x4*>(xr + qc * 8 + 4);
+            if constexpr (SRC == kProjSrcRmsNorm) {
+                el[i] = *reinterpret_cast<const f32x4*>(p.norm_w + qc * 8);
+                eh[i] = *reinterpret_cast<const f32x4*>(p.norm_w + qc * 8 + 4);
+            } else if constexpr (SRC == kProjSrcSwiglu || SRC == kProjSrcGeglu) {
+                el[i] = *reinterpret_cast<const f32x4*>(xr + a.K + qc * 8);
+                eh[i] = *reinterpret_cast<const f32x4*>(xr + a.K + qc * 8 + 4);
+            }
+        }
+    }
+
+    // 2. the weights: NB0 batches now, the rest as the buffers come free
     half8 wa[KB], wb[KB], wc[KB];
-    uint32_t kt = k_begin;
-    const uint32_t nb = kper / KB;                               // whole batches of this wave
+    const uint32_t nb = kper / KB;                               // whole batches of this wave (>= NB0)
     auto load_batch = [&](half8 (&w)[KB], uint32_t b) {
 #pragma unroll
         for (int u = 0; u < KB; u++) w[u] = __builtin_nontemporal_load(&wp[(size_t)(k_begin + b * KB + u) * 64]);
     };
-    if (nb > 0) load_batch(wa, 0);
-    if (nb > 1) load_batch(wb, 1);
-    if (nb > 2) load_batch(wc, 2);
+    if constexpr (NB0 > 0) load_batch(wa, 0);
+    if constexpr (NB0 > 1) load_batch(wb, 1);
+    if constexpr (NB0 > 2) load_batch(wc, 2);
 
-    // the row's terms, as proj_prep_kernel forms them
-    const float* xr = p.x;
+    // 3. the row's terms, as proj_prep_kernel forms them
     auto put_chunk = [&](uint32_t q, const float (&v)[8], float inv) {
         half8 hi, lo;
 #pragma unroll
@@ -674,29 +696,20 @@ __global__ __launch_bounds__(kProjThreads) void proj_row1_kernel(const ProjArgs 
         sfrag[q * 2] = hi;
         sfrag[q * 2 + 1] = lo;
     };
-    constexpr int CH = 2;                                        // chunks of eight inputs a thread can hold
-    if (a.K <= 2048u * CH) {
+    if (in_regs) {
         // One read of the row: its values stay in registers between the passes
-        // (sum of squares, largest magnitude, terms).  Every pass over memory is a
-        // round trip, and a launch of this kernel is little else.  Same values,
-        // same order of the sum as the passes below (thread t takes the chunks t,
+        // (sum of squares, largest magnitude, terms).  Same values, same order of
+        // the sum as the passes of the other branch (thread t takes the chunks t,
         // t + 256, ... in order).
         float v[CH][8];
         float ss = 0.f;
 #pragma unroll
         for (int i = 0; i < CH; i++) {
-            const uint32_t q = t + 256u * i;
-            if (q < nchunks) {
-                const f32x4 lo4 = *reinterpret_cast<const f32x4*>(xr + q * 8),
-                            hi4 = *reinterpret_cast<const f32x4*>(xr + q * 8 + 4);
+            const bool has = t + 256u * i < nchunks;
 #pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    v[i][j] = lo4[j];
-                    v[i][4 + j] = hi4[j];
-                }
-            } else {
-#pragma unroll
-                for (int j = 0; j < 8; j++) v[i][j] = 0.f;
+            for (int j = 0; j < 4; j++) {
+                v[i][j] = has ? xl[i][j] : 0.f;
+                v[i][4 + j] = has ? xh[i][j] : 0.f;
             }
             if constexpr (SRC == kProjSrcRmsNorm) {
 #pragma unroll
@@ -707,26 +720,20 @@ __global__ __launch_bounds__(kProjThreads) void proj_row1_kernel(const ProjArgs 
             const float inv_rms = 1.0f / sqrtf(block_sum_256(ss, s4) / (float)a.K + p.eps);
 #pragma unroll
             for (int i = 0; i < CH; i++) {
-                const uint32_t q = t + 256u * i;
-                if (q < nchunks) {
-                    const f32x4 wl = *reinterpret_cast<const f32x4*>(p.norm_w + q * 8),
-                                wh = *reinterpret_cast<const f32x4*>(p.norm_w + q * 8 + 4);
+                if (t + 256u * i < nchunks) {
 #pragma unroll
                     for (int j = 0; j < 4; j++) {
-                        v[i][j] = v[i][j] * inv_rms * wl[j];
-                        v[i][4 + j] = v[i][4 + j] * inv_rms * wh[j];
+                        v[i][j] = v[i][j] * inv_rms * el[i][j];
+                        v[i][4 + j] = v[i][4 + j] * inv_rms * eh[i][j];
                     }
                 }
             }
         } else if constexpr (SRC == kProjSrcSwiglu || SRC == kProjSrcGeglu) {
 #pragma unroll
             for (int i = 0; i < CH; i++) {
-                const uint32_t q = t + 256u * i;
-                if (q < nchunks) {
-                    const f32x4 ul = *reinterpret_cast<const f32x4*>(xr + a.K + q * 8),
-                                uh = *reinterpret_cast<const f32x4*>(xr + a.K + q * 8 + 4);
+                if (t + 256u * i < nchunks) {
 #pragma unroll
-                    for (int j = 0; j < 8; j++) v[i][j] = proj_gated<SRC>(v[i][j], j < 4 ? ul[j] : uh[j - 4]);
+                    for (int j = 0; j < 8; j++) v[i][j] = proj_gated<SRC>(v[i][j], j < 4 ? el[i][j] : eh[i][j - 4]);
                 }
             }
         }
@@ -739,7 +746,7 @@ __global__ __launch_bounds__(kProjThreads) void proj_row1_kernel(const ProjArgs 
         uint32_t ex = (__float_as_uint(mx) >> 23) & 0xFFu;
         if (ex == 0 || ex == 0xFF) ex = 127;
         if (ex > 253) ex = 253;
-        if (t == 0) s_scale = __uint_as_float(ex << 23);
+        if (t == 0) *s_scale = __uint_as_float(ex << 23);
         const float inv = __uint_as_float((254u - ex) << 23);
 #pragma unroll
         for (int i = 0; i < CH; i++) {
@@ -756,7 +763,7 @@ __global__ __launch_bounds__(kProjThreads) void proj_row1_kernel(const ProjArgs 
         uint32_t ex = (__float_as_uint(mx) >> 23) & 0xFFu;
         if (ex == 0 || ex == 0xFF) ex = 127;
         if (ex > 253) ex = 253;
-        if (t == 0) s_scale = __uint_as_float(ex << 23);
+        if (t == 0) *s_scale = __uint_as_float(ex << 23);
         const float inv = __uint_as_float((254u - ex) << 23);
         for (uint32_t q = t; q < nchunks; q += 256) {
             float v[8];
@@ -785,14 +792,16 @@ __global__ __launch_bounds__(kProjThreads) void proj_row1_kernel(const ProjArgs 
 #pragma unroll
         for (int u = 0; u < KB; u++) step(w[u], k_begin + b * KB + u);
     };
-    if (nb > 0) {
+    if constexpr (NB0 > 0) {
         steps(wa, 0);
-        if (nb > 3) load_batch(wa, 3);
-        if (nb > 1) {
-            steps(wb, 1);
-            if (nb > 4) load_batch(wb, 4);
-        }
-        if (nb > 2) steps(wc, 2);
+        if (NB0 > 2 && nb > 3) load_batch(wa, 3);
+    }
+    if constexpr (NB0 > 1) {
+        steps(wb, 1);
+        if (NB0 > 2 && nb > 4) load_batch(wb, 4);
+    }
+    if constexpr (NB0 > 2) {
+        steps(wc, 2);
         for (uint32_t b = 3; b < nb; b += 2) {                   // wa holds batch b, wb batch b + 1
             steps(wa, b);
             if (b + 2 < nb) load_batch(wa, b + 2);
@@ -802,7 +811,7 @@ __global__ __launch_bounds__(kProjThreads) void proj_row1_kernel(const ProjArgs 
             }
         }
     }
-    for (kt = k_begin + nb * KB; kt < k_end; kt++) step(__builtin_nontemporal_load(&wp[(size_t)kt * 64]), kt);
+    for (uint32_t kt = k_begin + nb * KB; kt < k_end; kt++) step(__builtin_nontemporal_load(&wp[(size_t)kt * 64]), kt);
 
     if (S > 1) {                                                 // uniform over the workgroup
         if (part > 0) s_part[(slot * (S - 1) + (part - 1)) * 64 + lane] = acc;
@@ -815,7 +824,26 @@ __global__ __launch_bounds__(kProjThreads) void proj_row1_kernel(const ProjArgs 
         }
     }
     if (!live) return;
-    proj_store_tile(a, acc, nt0, 0, lane, &s_scale);
+    proj_store_tile(a, acc, nt0, 0, lane, s_scale);
+}
+
+template <int SRC>
+__global__ __launch_bounds__(kProjThreads) void proj_row1_kernel(const ProjArgs a, const ProjPrepArgs p)
+{
+    extern __shared__ __attribute__((aligned(16))) unsigned char row1_smem[];
+    half8* sfrag = reinterpret_cast<half8*>(row1_smem);           // [K/8][2]: hi, lo of chunk q
+    __shared__ f32x4 s_part[3 * 64];
+    __shared__ float s4[4];
+    __shared__ float s_scale;
+    const uint32_t nb = a.K / 32 / a.ksplit / kProjKBatch;        // whole batches of weights per wave: uniform
+    if (nb >= 3)
+        proj_row1_body<SRC, 3>(a, p, sfrag, s_part, s4, &s_scale);
+    else if (nb == 2)
+        proj_row1_body<SRC, 2>(a, p, sfrag, s_part, s4, &s_scale);
+    else if (nb == 1)
+        proj_row1_body<SRC, 1>(a, p, sfrag, s_part, s4, &s_scale);
+    else
+        proj_row1_body<SRC, 0>(a, p, sfrag, s_part, s4, &s_scale);
 }
 
 // Many rows (prefill chunks), products too small to fill the chip with the
