@@ -492,7 +492,10 @@ def test_append_and_decode_in_one_launch_equals_the_two_calls(nq, nkv, norm, rot
         hipattn.sync()
         hipattn.set_tuning(0, False)
         got_a, got_b = o_a.to_host((n, nq, hd)), o_b.to_host((n, nq, hd))
-        assert np.array_equal(got_a, got_b), "outputs differ from the two-call path"
+        differ = [(i, pos[i], float(np.abs(got_a[i] - got_b[i]).max()),
+                   [int(h) for h in np.argwhere(np.abs(got_a[i] - got_b[i]).max(axis=1) > 0)[:, 0]])
+                  for i in range(n) if not np.array_equal(got_a[i], got_b[i])]
+        assert differ == [], f"outputs differ from the two-call path: (session, position, max diff, heads) {differ}"
         for i in range(n):
             ka, va = twins[i][0].read_f16(0, 0, pos[i] + 1)
             kb, vb = twins[i][1].read_f16(0, 0, pos[i] + 1)

@@ -275,6 +275,19 @@ __device__ __forceinline__ void publish_and_merge(const DecodeArgs& a, uint32_t 
     if (threadIdx.x == 0) a.counters[counter_idx] = 0;
 }
 
+// A query element scaled and split into the two half-precision terms the first
+// contraction takes (x = hi + lo).  One place, with contraction of the product
+// into the subtraction switched off: the kernel that makes the new row itself
+// and the one that is handed finished Q rows must produce the same bits, and
+// left to itself the compiler fuses "v * qscale - hi" in one and not the other.
+__device__ __forceinline__ void q_hi_lo(float v, float qscale, _Float16& hi, _Float16& lo)
+{
+#pragma clang fp contract(off)
+    const float x = v * qscale;
+    hi = (_Float16)x;
+    lo = (_Float16)(x - (float)hi);
+}
+
 // ------------------------------------------------------------------ MFMA --
 
 template <int HD>
@@ -523,16 +536,19 @@ void decode_mfma_kernel(const DecodeArgs a, const DecodeFusedArgs fz)
     const uint32_t patch_tile =
         (owner && (new_tile - tr.t_begin) % kDecodeWaves == (uint32_t)wave) ? new_tile : 0xFFFFFFFFu;
     const uint32_t hslot = threadIdx.x >> 3, part = threadIdx.x & 7;   // FUSED: head slot (Q heads, K, V), lane of eight
+    // FUSED: the new row's values are asked for here, before the tiles, and worked
+    // out after the tiles have been asked for: a wave's loads return in the order
+    // they were issued.  Lanes of eight without a head shadow head slot 0, so that
+    // every load is unconditional and the waits below stay exact.
+    Row8Loads<kNJ> rl;
+    const uint32_t hs = hslot < (uint32_t)G + (owner ? 2u : 0u) ? hslot : 0u;
     if constexpr (FUSED) {
-        if (hslot < (uint32_t)G + (owner ? 2u : 0u)) {
-            const bool is_q = hslot < (uint32_t)G, is_k = hslot == (uint32_t)G;
-            const uint32_t head = is_q ? kvh * G + hslot : (is_k ? a.nq + kvh : a.nq + a.nkv + kvh);
-            const float* src = fz.qkv + (size_t)sess * fz.ld + (size_t)head * HD + part * 8;
-            row8_head_values<kNJ>(xrow, src, true, is_q ? fz.q_norm : (is_k ? fz.k_norm : nullptr), false, fz.eps,
-                                  part, (hslot <= (uint32_t)G && fz.cos_sin) ? fz.cos_sin + (size_t)sess * fz.n_rot * 2
-                                                                              : nullptr,
-                                  fz.n_rot);
-        }
+        const bool is_q = hs < (uint32_t)G, is_k = hs == (uint32_t)G;
+        const uint32_t head = is_q ? kvh * G + hs : (is_k ? a.nq + kvh : a.nq + a.nkv + kvh);
+        const float* src = fz.qkv + (size_t)sess * fz.ld + (size_t)head * HD + part * 8;
+        // (a V head reads the Q norm's weights and the table and uses neither)
+        row8_head_request<kNJ>(rl, src, is_k ? fz.k_norm : fz.q_norm, part,
+                               fz.cos_sin ? fz.cos_sin + (size_t)sess * fz.n_rot * 2 : nullptr, fz.n_rot);
     } else {
         const float* qg = a.q + ((size_t)sess * a.nq + kvh * G) * HD;     // G contiguous rows
 #pragma unroll
@@ -550,6 +566,9 @@ void decode_mfma_kernel(const DecodeArgs a, const DecodeFusedArgs fz)
     uint32_t t = tr.t_begin + wave;
     load_frag<HD>(fa, kbase, vtbase, min(t, tr.t_end - 1), lane);
     if constexpr (!kSingle) load_frag<HD>(fb, kbase, vtbase, min(t + kDecodeWaves, tr.t_end - 1), lane);
+    if constexpr (FUSED)
+        row8_head_finish<kNJ>(xrow, rl, fz.q_norm != nullptr && hs <= (uint32_t)G, false, fz.eps, part,
+                              fz.cos_sin != nullptr && hs <= (uint32_t)G, fz.n_rot);
 
     // Q^T operand through LDS: row c of lds_q is MFMA column c.  Columns
     // 0..G-1 hold the hi terms of the group's heads, G..2G-1 the lo terms,
@@ -559,15 +578,19 @@ void decode_mfma_kernel(const DecodeArgs a, const DecodeFusedArgs fz)
     if constexpr (FUSED) {
         if (hslot < (uint32_t)G) {
             // a Q head: element 64 c + 8 part + e of MFMA columns hslot (hi) and hslot + G (lo)
+            // (element by element: written as two 16-byte vectors the conversions
+            // become packed ones, which round a lo term in the subnormal range of
+            // binary16 differently from the scalar conversion of the kernel that is
+            // handed finished Q rows -- and the two must agree bit for bit)
 #pragma unroll
             for (int c = 0; c < kNJ; c++)
 #pragma unroll
                 for (int e = 0; e < 8; e++) {
                     const int d = c * 64 + (int)part * 8 + e;
-                    const float x = xrow[c][e] * a.qscale;
-                    const _Float16 hi = (_Float16)x;
+                    _Float16 hi, lo;
+                    q_hi_lo(xrow[c][e], a.qscale, hi, lo);
                     lds_q[hslot][d] = hi;
-                    lds_q[hslot + G][d] = (_Float16)(x - (float)hi);
+                    lds_q[hslot + G][d] = lo;
                 }
         } else if (owner && hslot == (uint32_t)G) {
             // the K head: truncated to F16, into the cache and into the workgroup's copy
@@ -604,10 +627,10 @@ void decode_mfma_kernel(const DecodeArgs a, const DecodeFusedArgs fz)
             const int idx = threadIdx.x + i * kDecodeThreads;
             if (idx < G * HD) {
                 const int h = idx / HD, d = idx % HD;
-                const float x = qreg[i] * a.qscale;
-                const _Float16 hi = (_Float16)x;
+                _Float16 hi, lo;
+                q_hi_lo(qreg[i], a.qscale, hi, lo);
                 lds_q[h][d] = hi;
-                lds_q[h + G][d] = (_Float16)(x - (float)hi);
+                lds_q[h + G][d] = lo;
             }
         }
         for (int idx = threadIdx.x; idx < (16 - 2 * G) * HD; idx += kDecodeThreads)

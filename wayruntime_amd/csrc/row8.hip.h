@@ -29,32 +29,71 @@ __device__ __forceinline__ float row8_sum_f32(float (&s)[8])
     return c0 + c1;
 }
 
-// x: the head's elements of this lane, read from src (the head's row + 8 part)
-// when live, zero otherwise.  nw: the norm's weight vector or null; weightless:
-// an RMSNorm without weights (V heads of the Gemma family); cs: the position's
-// (cos, sin) table or null for no rotation; n_rot a multiple of eight.  All
-// eight lanes of a position must call together (the sum crosses them).
+// What a lane reads for one head of one position: its 8 NJ elements, the
+// norm's weights for them and the (cos, sin) pairs of its rotation pairs.  All
+// three are asked for together, before anything is waited for: read where they
+// are used they are three dependent trips to memory (row -> sum -> weights ->
+// rotation table), and a caller with other loads to start (the decode kernel's
+// tiles) can start them in between.
 template <int NJ>
-__device__ __forceinline__ void row8_head_values(float (&x)[NJ][8], const float* src, bool live,
-                                                 const float* nw, bool weightless, float eps, uint32_t part,
-                                                 const float* cs, uint32_t n_rot)
+struct Row8Loads {
+    f32x4 x[NJ][2];
+    f32x4 w[NJ][2];
+    f32x4 t[NJ / 2 > 0 ? NJ / 2 : 1][4];
+};
+
+// src: the head's row + 8 part; nw: the norm's weight vector or null; cs: the
+// position's (cos, sin) table or null; n_rot a multiple of eight.  EVERY load
+// is issued whatever the lane goes on to use, from an address that is valid:
+// without weights or a table the head's own row is read in their place (its
+// 64 NJ floats cover every offset used below), and pairs past n_rot read the
+// table's last eight.  Loads that are only sometimes issued would make the
+// compiler wait for everything in flight where it now waits for these alone.
+template <int NJ>
+__device__ __forceinline__ void row8_head_request(Row8Loads<NJ>& L, const float* src, const float* nw,
+                                                  uint32_t part, const float* cs, uint32_t n_rot)
+{
+    const float* head = src - part * 8;
+    const float* nwp = nw != nullptr ? nw : head;
+    const float* csp = cs != nullptr ? cs : head;
+    const uint32_t last = (cs != nullptr && n_rot >= 8) ? n_rot - 8 : 64u * (NJ / 2 > 0 ? NJ / 2 : 1) - 8;
+#pragma unroll
+    for (int c = 0; c < NJ; c++) {
+        L.x[c][0] = *reinterpret_cast<const f32x4*>(src + c * 64);
+        L.x[c][1] = *reinterpret_cast<const f32x4*>(src + c * 64 + 4);
+    }
+#pragma unroll
+    for (int c = 0; c < NJ; c++) {
+        L.w[c][0] = *reinterpret_cast<const f32x4*>(nwp + c * 64 + part * 8);
+        L.w[c][1] = *reinterpret_cast<const f32x4*>(nwp + c * 64 + part * 8 + 4);
+    }
+#pragma unroll
+    for (int c = 0; c < NJ / 2; c++) {
+        const uint32_t j0 = min((uint32_t)(c * 64 + part * 8), last);
+#pragma unroll
+        for (int q = 0; q < 4; q++) L.t[c][q] = *reinterpret_cast<const f32x4*>(csp + 2 * j0 + 4 * q);
+    }
+}
+
+// x: the head's elements of this lane from what row8_head_request read.
+// norm: RMSNorm with the weights read (weightless: without weights, the V heads
+// of the Gemma family); rotate: apply the rotation read.  All eight lanes of a
+// position must call together with the same flags (the sum crosses them).
+template <int NJ>
+__device__ __forceinline__ void row8_head_finish(float (&x)[NJ][8], const Row8Loads<NJ>& L, bool norm,
+                                                 bool weightless, float eps, uint32_t part, bool rotate,
+                                                 uint32_t n_rot)
 {
 #pragma clang fp contract(off)
     constexpr uint32_t HD = 64 * NJ;
 #pragma unroll
-    for (int c = 0; c < NJ; c++) {
-        f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = lo;
-        if (live) {
-            lo = *reinterpret_cast<const f32x4*>(src + c * 64);
-            hi = *reinterpret_cast<const f32x4*>(src + c * 64 + 4);
-        }
+    for (int c = 0; c < NJ; c++)
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-            x[c][e] = lo[e];
-            x[c][4 + e] = hi[e];
+            x[c][e] = L.x[c][0][e];
+            x[c][4 + e] = L.x[c][1][e];
         }
-    }
-    if (weightless || nw != nullptr) {                    // uniform over the eight lanes
+    if (weightless || norm) {                             // uniform over the eight lanes
         float s[8];
 #pragma unroll
         for (int e = 0; e < 8; e++) {
@@ -70,25 +109,23 @@ __device__ __forceinline__ void row8_head_values(float (&x)[NJ][8], const float*
 #pragma unroll
                 for (int e = 0; e < 8; e++) x[c][e] = x[c][e] * inv_rms;
             } else {
-                const f32x4 wl = *reinterpret_cast<const f32x4*>(nw + c * 64 + part * 8);
-                const f32x4 wh = *reinterpret_cast<const f32x4*>(nw + c * 64 + part * 8 + 4);
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    x[c][e] = x[c][e] * inv_rms * wl[e];
-                    x[c][4 + e] = x[c][4 + e] * inv_rms * wh[e];
+                    x[c][e] = x[c][e] * inv_rms * L.w[c][0][e];
+                    x[c][4 + e] = x[c][4 + e] * inv_rms * L.w[c][1][e];
                 }
             }
         }
     }
-    if (cs == nullptr) return;
+    if (!rotate) return;
     // rotation of the pairs (j, j + hd/2), j = 64 c + 8 part + e for c < NJ / 2
 #pragma unroll
     for (int c = 0; c < NJ / 2; c++) {
         const uint32_t j0 = c * 64 + part * 8;
-        if (live && j0 < n_rot) {
+        if (j0 < n_rot) {
 #pragma unroll
             for (int q = 0; q < 4; q++) {
-                const f32x4 t = *reinterpret_cast<const f32x4*>(cs + 2 * j0 + 4 * q);
+                const f32x4 t = L.t[c][q];
 #pragma unroll
                 for (int u = 0; u < 2; u++) {
                     const float co = t[2 * u], sn = t[2 * u + 1];
@@ -100,6 +137,26 @@ __device__ __forceinline__ void row8_head_values(float (&x)[NJ][8], const float*
             }
         }
     }
+}
+
+// Both steps in one call.  x: the head's elements of this lane, read from src
+// (the head's row + 8 part) when live, zero otherwise.  nw: the norm's weight
+// vector or null; weightless: an RMSNorm without weights; cs: the position's
+// (cos, sin) table or null for no rotation.  All eight lanes of a position must
+// call together.
+template <int NJ>
+__device__ __forceinline__ void row8_head_values(float (&x)[NJ][8], const float* src, bool live,
+                                                 const float* nw, bool weightless, float eps, uint32_t part,
+                                                 const float* cs, uint32_t n_rot)
+{
+    Row8Loads<NJ> L;
+    if (live) {
+        row8_head_request<NJ>(L, src, nw, part, cs, n_rot);
+    } else {
+#pragma unroll
+        for (int c = 0; c < NJ; c++) L.x[c][0] = L.x[c][1] = L.w[c][0] = L.w[c][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    row8_head_finish<NJ>(x, L, nw != nullptr, weightless, eps, part, live && cs != nullptr, n_rot);
 }
 
 }  // namespace wr
