@@ -79,8 +79,18 @@ struct DecodeArgs {
     // round-robin by linear id) serves one KV head of every session and gets
     // the same share of a ragged batch.
     uint32_t n_items;
-    uint16_t items[kBatchMax * 64];
+    alignas(4) uint16_t items[kBatchMax * 64];
 };
+
+// Work-list entry y.  Read as the 32-bit word that holds it: the index is the
+// same for the whole workgroup, and a 32-bit read of a kernel argument is a
+// scalar load, where a 16-bit one is a vector load the whole wave waits for
+// before it can ask for anything else.
+__device__ __forceinline__ uint32_t decode_item(const DecodeArgs& a, uint32_t y)
+{
+    const uint32_t w = reinterpret_cast<const uint32_t*>(a.items)[y >> 1];
+    return (y & 1u) ? (w >> 16) : (w & 0xFFFFu);
+}
 
 // The decode step's new row made inside the attention launch (FUSED form of the
 // MFMA kernel, head dim 128): row i of qkv is session i's stacked projection
@@ -506,7 +516,7 @@ void decode_mfma_kernel(const DecodeArgs a, const DecodeFusedArgs fz)
 {
     static_assert(!FUSED || HD == 128, "the fused form is built for head dim 128");
     const uint32_t kvh = blockIdx.x;
-    const uint32_t item = a.items[blockIdx.y];
+    const uint32_t item = decode_item(a, blockIdx.y);
     const uint32_t sess = item >> 8, split = item & 0xFFu;
     const DecodeSession S = a.s[sess];
 
@@ -850,7 +860,7 @@ __device__ __forceinline__ GenericMerge merge_generic(const GenericShared& sh)
 __global__ __launch_bounds__(kDecodeThreads) void decode_generic_kernel(const DecodeArgs a)
 {
     const uint32_t head = blockIdx.x;
-    const uint32_t item = a.items[blockIdx.y];
+    const uint32_t item = decode_item(a, blockIdx.y);
     const uint32_t sess = item >> 8, split = item & 0xFFu;
     const DecodeSession S = a.s[sess];
     const uint32_t hd = a.hd;

@@ -93,7 +93,10 @@ __device__ __forceinline__ void row8_head_finish(float (&x)[NJ][8], const Row8Lo
             x[c][e] = L.x[c][0][e];
             x[c][4 + e] = L.x[c][1][e];
         }
-    if (weightless || norm) {                             // uniform over the eight lanes
+    // No branches from here on (values are selected, not skipped): a load whose
+    // value is only used inside a branch gets moved down into that branch,
+    // behind whatever the caller has asked for in between.
+    {
         float s[8];
 #pragma unroll
         for (int e = 0; e < 8; e++) {
@@ -103,37 +106,34 @@ __device__ __forceinline__ void row8_head_finish(float (&x)[NJ][8], const Row8Lo
             s[e] = ss;
         }
         const float inv_rms = 1.0f / sqrtf(row8_sum_f32(s) / (float)HD + eps);
+        const bool scaled = weightless || norm;
 #pragma unroll
         for (int c = 0; c < NJ; c++) {
-            if (weightless) {
 #pragma unroll
-                for (int e = 0; e < 8; e++) x[c][e] = x[c][e] * inv_rms;
-            } else {
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    x[c][e] = x[c][e] * inv_rms * L.w[c][0][e];
-                    x[c][4 + e] = x[c][4 + e] * inv_rms * L.w[c][1][e];
-                }
+            for (int e = 0; e < 4; e++) {
+                // weightless: times one, which changes no bit
+                const float w0 = weightless ? 1.0f : L.w[c][0][e], w1 = weightless ? 1.0f : L.w[c][1][e];
+                const float y0 = x[c][e] * inv_rms * w0, y1 = x[c][4 + e] * inv_rms * w1;
+                x[c][e] = scaled ? y0 : x[c][e];
+                x[c][4 + e] = scaled ? y1 : x[c][4 + e];
             }
         }
     }
-    if (!rotate) return;
     // rotation of the pairs (j, j + hd/2), j = 64 c + 8 part + e for c < NJ / 2
 #pragma unroll
     for (int c = 0; c < NJ / 2; c++) {
         const uint32_t j0 = c * 64 + part * 8;
-        if (j0 < n_rot) {
+        const bool turn = rotate && j0 < n_rot;
 #pragma unroll
-            for (int q = 0; q < 4; q++) {
-                const f32x4 t = L.t[c][q];
+        for (int q = 0; q < 4; q++) {
+            const f32x4 t = L.t[c][q];
 #pragma unroll
-                for (int u = 0; u < 2; u++) {
-                    const float co = t[2 * u], sn = t[2 * u + 1];
-                    const float x0 = x[c][2 * q + u], x1 = x[c + NJ / 2][2 * q + u];
-                    const float a0 = x0 * co, b0 = x1 * sn, a1 = x0 * sn, b1 = x1 * co;
-                    x[c][2 * q + u] = a0 - b0;
-                    x[c + NJ / 2][2 * q + u] = a1 + b1;
-                }
+            for (int u = 0; u < 2; u++) {
+                const float co = t[2 * u], sn = t[2 * u + 1];
+                const float x0 = x[c][2 * q + u], x1 = x[c + NJ / 2][2 * q + u];
+                const float a0 = x0 * co, b0 = x1 * sn, a1 = x0 * sn, b1 = x1 * co;
+                x[c][2 * q + u] = turn ? a0 - b0 : x0;
+                x[c + NJ / 2][2 * q + u] = turn ? a1 + b1 : x1;
             }
         }
     }
@@ -155,6 +155,10 @@ __device__ __forceinline__ void row8_head_values(float (&x)[NJ][8], const float*
     } else {
 #pragma unroll
         for (int c = 0; c < NJ; c++) L.x[c][0] = L.x[c][1] = L.w[c][0] = L.w[c][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < NJ / 2; c++)
+#pragma unroll
+            for (int q = 0; q < 4; q++) L.t[c][q] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
     row8_head_finish<NJ>(x, L, nw != nullptr, weightless, eps, part, live && cs != nullptr, n_rot);
 }
