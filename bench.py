@@ -270,7 +270,7 @@ def main() -> None:
     # ---- dominant kernel alone, per-launch events
     kern_avg_ms = work.time_kernel(min(max(args.steps, 100), 512))
     achieved = bytes_per_step / (kern_avg_ms * 1e-3) / 1e9
-    roofline = {"bound": "hbm", "kernel": "decode_mfma_kernel<%d>" % hd, "achieved": round(achieved, 1),
+    roofline = {"bound": "hbm", "kernel": "decode_mfma_kernel<%d, false>" % hd, "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                 "traffic": pmc_traffic_bytes(S, ctx) if not secondary and len(set(ctxs)) == 1 else None,
                 "kernel_avg_us": round(kern_avg_ms * 1e3, 2),
