@@ -371,7 +371,10 @@ int decode_locked(uint32_t n, wr_hip_kv* const* kv, uint32_t layer, const uint32
     // workgroup that has all its tiles in flight at once ends sooner than one
     // that walks eight of them per wave (one session of 1024 keys: 12.0 -> 7.8 us,
     // of 2048: 13.8 -> 8.2 us; 16 sessions of ~520: the step of a 28-layer model
-    // 2.03 -> 1.89 ms).  The session's tiles are spread evenly over the workgroups,
+    // 2.03 -> 1.89 ms).  A medium session (more than 2048 and fewer than 4096 keys)
+    // takes half: one session of 3000 keys 14 -> 10.6 us, the ragged batch of 16
+    // 35.2 -> 34.6 us; at 4096 keys and beyond the full figure stands (16 x 4096
+    // loses 4-8 % with halves).  The session's tiles are spread evenly over the workgroups,
     // and the floor keeps the in-kernel merge within kMaxSplits partials.
     // A single long session gets few workgroups this way; a caller that serves
     // one session at a time can lower the figure with wr_hip_attn_set_tuning.
@@ -387,6 +390,7 @@ int decode_locked(uint32_t n, wr_hip_kv* const* kv, uint32_t layer, const uint32
             uint32_t cap = kDefaultTilesPerWg * 128u / (hd < 32 ? 32 : hd);
             if (cap == 0) cap = 1;
             if (tiles[i] <= 2 * cap) cap = cap >= 4 ? cap / 4 : 1;      // a short session: see above
+            else if (tiles[i] < 4 * cap) cap = cap >= 2 ? cap / 2 : 1;  // a medium one: see above
             if (cap < tiles[i] / 8) cap = tiles[i] / 8;
             const uint32_t want = (tiles[i] + cap - 1) / cap;          // workgroups
             tpw = (tiles[i] + want - 1) / want;                        // even share
