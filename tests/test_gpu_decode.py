@@ -520,3 +520,47 @@ def test_append_and_decode_in_one_launch_equals_the_two_calls(nq, nkv, norm, rot
     for b in (qwd, kwd):
         if b is not None:
             b.free()
+
+
+def test_append_and_decode_in_one_launch_refuses_what_it_must():
+    # argument contract of wr_hip_attn_append_decode_batched_dev: pointers, counts,
+    # head shapes and strides are checked before anything is counted or written
+    import ctypes as C
+    lib = hipattn.lib()
+    nq, nkv, hd, cap = 16, 8, 128, 96
+    width = (nq + 2 * nkv) * hd
+    kv = hipattn.KVCache(1, hd, nkv, cap)
+    D = hipattn.DeviceBuffer
+    x = D.from_host(synth.normal(9701, (1, width)))
+    w = D.from_host(np.ones(hd, dtype=np.float32))
+    tab = D.from_host(oracle.rope_table(1, hd, 5, 1e6, 0))
+    out = D.from_host(np.full((1, nq, hd), 3.0, dtype=np.float32))
+    kvs = (C.c_void_p * 1)(kv.h)
+    pos = (C.c_uint32 * 1)(5)
+    call = lambda n=1, k=kvs, p=pos, xp=x.p, ld=width, q=nq, qn=w.p, kn=w.p, cs=tab.p, nr=hd // 2, o=out.p, layer=0: \
+        lib.wr_hip_attn_append_decode_batched_dev(n, k, layer, p, xp, ld, q, qn, kn, 1e-6, cs, nr, o, 0.0, 0)   # noqa: E731
+    calls = int(lib.wr_hip_attn_calls())
+    assert call(k=None) == hipattn.ERR_INVAL
+    assert call(p=None) == hipattn.ERR_INVAL
+    assert call(xp=None) == hipattn.ERR_INVAL
+    assert call(o=None) == hipattn.ERR_INVAL
+    assert call(n=0) == hipattn.ERR_LIMIT
+    assert call(n=17) == hipattn.ERR_LIMIT
+    assert call(layer=1) == hipattn.ERR_INVAL               # the cache has one layer
+    assert call(q=12) == hipattn.ERR_INVAL                  # 12 query heads over 8 KV heads
+    assert call(qn=None) == hipattn.ERR_INVAL               # one norm vector without the other
+    assert call(cs=None) == hipattn.ERR_INVAL               # a rotation without its table
+    assert call(nr=hd) == hipattn.ERR_INVAL                 # more pairs than half the head
+    assert call(ld=width - 4) == hipattn.ERR_INVAL          # rows shorter than Q + K + V
+    assert call(nr=4) == hipattn.ERR_UNSUPPORTED            # pairs not a multiple of eight: the two calls take it
+    assert int(lib.wr_hip_attn_calls()) == calls            # nothing counted
+    hipattn.sync()
+    assert np.all(out.to_host((1, nq, hd)) == 3.0)          # nothing written
+    k_now, v_now = kv.read_f16(0, 0, 6)
+    assert not k_now.any() and not v_now.any()
+    # and the call itself, for the record
+    assert call() == hipattn.OK
+    assert int(lib.wr_hip_attn_calls()) == calls + 1
+    for b in (x, w, tab, out):
+        b.free()
+    kv.close()
