@@ -91,6 +91,22 @@ __device__ __forceinline__ size_t vt_offset(uint32_t kvh, uint32_t ctx_pad, uint
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// silu(g) * u, silu(g) = g / (1 + exp(-g)) (reference: src/core/kernels.c:963-967),
+// with exp(-g) = 2^(-g log2 e) from the hardware's exp2 and the reciprocal from
+// v_rcp_f32: six instructions where expf and an IEEE division are about forty,
+// in kernels whose time IS their instruction count (the gated products of a decode
+// step spend a microsecond of vector ALU on sixteen of these per lane, and the
+// unrolled library calls are a third of the code they have to fetch).  Relative
+// error about 2^-23 + |g| 2^-24 (the rounded product in the exponent): for the
+// |g| < 20 that contribute anything, within 1.3e-6.  One definition for every
+// kernel that gates: the fused and the separate forms must agree bit for bit.
+__device__ __forceinline__ float silu_mul(float g, float u)
+{
+    const float e = __builtin_amdgcn_exp2f(-g * 1.44269504088896340736f);
+    const float sig = __builtin_amdgcn_rcpf(1.0f + e);        // e = inf: 0
+    return (g * sig) * u;
+}
+
 __device__ __forceinline__ float wave_xor_f32(float v, int mask)
 {
     return __shfl_xor(v, mask, 64);

@@ -145,8 +145,7 @@ __device__ __forceinline__ float proj_gated(float g, float u)
         const float th = 2.0f / (1.0f + expf(-2.0f * z)) - 1.0f;
         return 0.5f * g * (1.0f + th) * u;
     } else {
-        const float sig = 1.0f / (1.0f + expf(-g));
-        return (g * sig) * u;
+        return silu_mul(g, u);
     }
 }
 

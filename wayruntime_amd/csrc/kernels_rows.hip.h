@@ -311,8 +311,7 @@ __global__ __launch_bounds__(256) void swiglu_rows_kernel(const float* __restric
     if (idx >= (size_t)rows * ffn) return;
     const uint32_t r = (uint32_t)(idx / ffn), j = (uint32_t)(idx % ffn);
     const float g = gu[(size_t)r * ld + j], u = gu[(size_t)r * ld + ffn + j];
-    const float sig = 1.0f / (1.0f + expf(-g));
-    act[(size_t)r * ldo + j] = (g * sig) * u;
+    act[(size_t)r * ldo + j] = silu_mul(g, u);
 }
 
 }  // namespace wr
