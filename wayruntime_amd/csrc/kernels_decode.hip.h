@@ -551,9 +551,17 @@ void decode_mfma_kernel(const DecodeArgs a, const DecodeFusedArgs fz)
     // they were issued.  Lanes of eight without a head shadow head slot 0, so that
     // every load is unconditional and the waits below stay exact.
     Row8Loads<kNJ> rl;
-    const uint32_t hs = hslot < (uint32_t)G + (owner ? 2u : 0u) ? hslot : 0u;
+    // Head slots: the group's Q heads in wave 0 (slots 0 .. G-1), the K head in wave
+    // 1 (slot 8), the V head in wave 2 (slot 16): three waves work on them side by
+    // side, where one wave would run the three branches one after the other (and
+    // fetch their code one after the other) with the workgroup waiting at the
+    // barrier behind it.
+    constexpr uint32_t kSlotK = 8, kSlotV = 16;
+    static_assert(kMaxGroupMfma <= (int)kSlotK, "Q heads fit before the K slot");
+    const bool slot_q = hslot < (uint32_t)G, slot_k = owner && hslot == kSlotK, slot_v = owner && hslot == kSlotV;
+    const uint32_t hs = (slot_q || slot_k || slot_v) ? hslot : 0u;
     if constexpr (FUSED) {
-        const bool is_q = hs < (uint32_t)G, is_k = hs == (uint32_t)G;
+        const bool is_q = hs < (uint32_t)G, is_k = hs == kSlotK;
         const uint32_t head = is_q ? kvh * G + hs : (is_k ? a.nq + kvh : a.nq + a.nkv + kvh);
         const float* src = fz.qkv + (size_t)sess * fz.ld + (size_t)head * HD + part * 8;
         // (a V head reads the Q norm's weights and the table and uses neither)
@@ -577,8 +585,8 @@ void decode_mfma_kernel(const DecodeArgs a, const DecodeFusedArgs fz)
     load_frag<HD>(fa, kbase, vtbase, min(t, tr.t_end - 1), lane);
     if constexpr (!kSingle) load_frag<HD>(fb, kbase, vtbase, min(t + kDecodeWaves, tr.t_end - 1), lane);
     if constexpr (FUSED)
-        row8_head_finish<kNJ>(xrow, rl, fz.q_norm != nullptr && hs <= (uint32_t)G, false, fz.eps, part,
-                              fz.cos_sin != nullptr && hs <= (uint32_t)G, fz.n_rot);
+        row8_head_finish<kNJ>(xrow, rl, fz.q_norm != nullptr && hs != kSlotV, false, fz.eps, part,
+                              fz.cos_sin != nullptr && hs != kSlotV, fz.n_rot);
 
     // Q^T operand through LDS: row c of lds_q is MFMA column c.  Columns
     // 0..G-1 hold the hi terms of the group's heads, G..2G-1 the lo terms,
@@ -602,7 +610,7 @@ void decode_mfma_kernel(const DecodeArgs a, const DecodeFusedArgs fz)
                     lds_q[hslot][d] = hi;
                     lds_q[hslot + G][d] = lo;
                 }
-        } else if (owner && hslot == (uint32_t)G) {
+        } else if (slot_k) {
             // the K head: truncated to F16, into the cache and into the workgroup's copy
             uint16_t* kw = const_cast<uint16_t*>(S.k);
 #pragma unroll
@@ -616,7 +624,7 @@ void decode_mfma_kernel(const DecodeArgs a, const DecodeFusedArgs fz)
                 *reinterpret_cast<u32x4*>(kw + k_offset(kvh, S.ctx_pad, new_pos, c * 64 + part * 8, HD)) = packed;
                 *reinterpret_cast<u32x4*>(&new_row.k[c * 64 + part * 8]) = packed;
             }
-        } else if (owner && hslot == (uint32_t)G + 1) {
+        } else if (slot_v) {
             // the V head: truncated, into the block-transposed Vt and the workgroup's copy
             uint16_t* vw = const_cast<uint16_t*>(S.vt);
 #pragma unroll
