@@ -475,14 +475,23 @@ __device__ __forceinline__ void patch_new_row(DecodeFrag<HD>& f, const DecodeNew
         }
     }
     if (g == (p >> 3)) {
-        const uint32_t e = p & 7;
+        // element p % 8 of eight halves = one half of 32-bit word (p % 8) / 2: a
+        // bit-field insert per word and a select on the word index, not a chain
+        // of selects per half (this runs once per launch, in one wave, with the
+        // rest of the workgroup waiting for that wave's tile: its length in
+        // instructions is what it costs)
+        const uint32_t e = p & 7, w = e >> 1;
+        const uint32_t keep = (e & 1) ? 0x0000FFFFu : 0xFFFF0000u;
 #pragma unroll
         for (int dt = 0; dt < HD / 16; dt++) {
-            const uint16_t bits = nr.v[dt * 16 + m];
-            const _Float16 val = *reinterpret_cast<const _Float16*>(&bits);
+            const uint32_t both = (uint32_t)nr.v[dt * 16 + m] * 0x10001u;
+            u32x4 words = __builtin_bit_cast(u32x4, f.v[dt]);
 #pragma unroll
-            for (int j = 0; j < 8; j++)
-                if ((uint32_t)j == e) f.v[dt][j] = val;
+            for (int wi = 0; wi < 4; wi++) {
+                const uint32_t nw = (words[wi] & keep) | (both & ~keep);
+                words[wi] = ((uint32_t)wi == w) ? nw : words[wi];
+            }
+            f.v[dt] = __builtin_bit_cast(half8, words);
         }
     }
 }
