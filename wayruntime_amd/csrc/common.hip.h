@@ -107,9 +107,42 @@ __device__ __forceinline__ float silu_mul(float g, float u)
     return (g * sig) * u;
 }
 
+// The value lane ^ mask holds, mask a power of two below 64.  Through the
+// vector ALU's own lane crossings where there is one (a swap of wave halves or
+// of rows of sixteen, a rotation inside a row, a quad permutation), not through
+// the LDS crossbar: a reduction over the wave is six of these in a dependent
+// chain, each about a hundred cycles by way of ds_bpermute and about ten this
+// way, and the kernels of a decode step are chains of exactly such things.  The
+// partner is the same lane either way, so every sum keeps its bits.  (Callers
+// pass literal masks or unrolled loop counters: the switch folds away.)
 __device__ __forceinline__ float wave_xor_f32(float v, int mask)
 {
-    return __shfl_xor(v, mask, 64);
+    const uint32_t u = __float_as_uint(v);
+    const uint32_t lane = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+    switch (mask) {
+    case 32: {
+        const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+        return __uint_as_float((lane & 32u) ? r[0] : r[1]);
+    }
+    case 16: {
+        const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+        return __uint_as_float((lane & 16u) ? r[0] : r[1]);
+    }
+    case 8:                                               // row_ror:8
+        return __int_as_float(__builtin_amdgcn_update_dpp(0, (int)u, 0x128, 0xF, 0xF, false));
+    case 4: {
+        // banks 0 and 2 of a row (lanes 0-3, 8-11) take the lane four up (row_shl:4),
+        // banks 1 and 3 the lane four down (row_shr:4)
+        const int up = __builtin_amdgcn_update_dpp(0, (int)u, 0x104, 0xF, 0x5, false);
+        return __int_as_float(__builtin_amdgcn_update_dpp(up, (int)u, 0x114, 0xF, 0xA, false));
+    }
+    case 2:                                               // quad_perm:[2,3,0,1]
+        return __int_as_float(__builtin_amdgcn_update_dpp(0, (int)u, 0x4E, 0xF, 0xF, false));
+    case 1:                                               // quad_perm:[1,0,3,2]
+        return __int_as_float(__builtin_amdgcn_update_dpp(0, (int)u, 0xB1, 0xF, 0xF, false));
+    default:
+        return __shfl_xor(v, mask, 64);
+    }
 }
 
 // The value lane ^ 32 holds, without going through LDS: v_permlane32_swap
