@@ -95,15 +95,16 @@ struct ProjPrepArgs {
 // (The barriers in these two wait for LDS traffic only: __syncthreads() would
 // also wait for every global load in flight, and the one-row product has its
 // weights on the way while it reduces.)
+// s4 must not be written again before the workgroup's next barrier (the two
+// reductions of a row use the two halves of an array of eight): one barrier
+// each, not two.
 __device__ __forceinline__ float block_sum_256(float v, float* s4)
 {
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) v += wave_xor_f32(v, off);
     if ((threadIdx.x & 63) == 0) s4[threadIdx.x >> 6] = v;
     lds_barrier();
-    const float t = (s4[0] + s4[1]) + (s4[2] + s4[3]);
-    lds_barrier();
-    return t;
+    return (s4[0] + s4[1]) + (s4[2] + s4[3]);
 }
 
 __device__ __forceinline__ float block_max_256(float v, float* s4)
@@ -112,9 +113,7 @@ __device__ __forceinline__ float block_max_256(float v, float* s4)
     for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, wave_xor_f32(v, off));
     if ((threadIdx.x & 63) == 0) s4[threadIdx.x >> 6] = v;
     lds_barrier();
-    const float t = fmaxf(fmaxf(s4[0], s4[1]), fmaxf(s4[2], s4[3]));
-    lds_barrier();
-    return t;
+    return fmaxf(fmaxf(s4[0], s4[1]), fmaxf(s4[2], s4[3]));
 }
 
 // Sum of squares of a row by a 256-thread workgroup.  Thread t takes the
@@ -186,7 +185,7 @@ __device__ __forceinline__ void proj_write_chunk(half8* frow, uint32_t q, uint32
 template <int SRC, int CH>
 __global__ __launch_bounds__(256) void proj_prep_kernel(const ProjPrepArgs a)
 {
-    __shared__ float s4[4];
+    __shared__ float s4[8];
     const uint32_t row = blockIdx.x, t = threadIdx.x;
     const uint32_t ktiles = a.K / 32, nchunks = a.K / 8;
     const uint32_t grp = row / 8, c = row % 8;
@@ -242,7 +241,7 @@ __global__ __launch_bounds__(256) void proj_prep_kernel(const ProjPrepArgs a)
         for (int i = 0; i < CH; i++)
 #pragma unroll
             for (int j = 0; j < 8; j++) mx = fmaxf(mx, fabsf(v[i][j]));
-        mx = block_max_256(mx, s4);
+        mx = block_max_256(mx, s4 + 4);
         uint32_t ex = (__float_as_uint(mx) >> 23) & 0xFFu;
         if (ex == 0 || ex == 0xFF) ex = 127;              // zeros, subnormals, inf / NaN rows: no scaling
         if (ex > 253) ex = 253;                           // keeps the inverse 2^-e a normal number
@@ -259,7 +258,7 @@ __global__ __launch_bounds__(256) void proj_prep_kernel(const ProjPrepArgs a)
             inv_rms = 1.0f / sqrtf(row_sumsq_256(xr, a.K, s4) / (float)a.K + a.eps);
         float mx = 0.f;
         for (uint32_t k = t; k < a.K; k += 256) mx = fmaxf(mx, fabsf(proj_src_value<SRC>(a, xr, k, inv_rms)));
-        mx = block_max_256(mx, s4);
+        mx = block_max_256(mx, s4 + 4);
         uint32_t ex = (__float_as_uint(mx) >> 23) & 0xFFu;
         if (ex == 0 || ex == 0xFF) ex = 127;
         if (ex > 253) ex = 253;
@@ -741,7 +740,7 @@ __device__ __forceinline__ void proj_row1_body(const ProjArgs& a, const ProjPrep
         for (int i = 0; i < CH; i++)
 #pragma unroll
             for (int j = 0; j < 8; j++) mx = fmaxf(mx, fabsf(v[i][j]));
-        mx = block_max_256(mx, s4);
+        mx = block_max_256(mx, s4 + 4);
         uint32_t ex = (__float_as_uint(mx) >> 23) & 0xFFu;
         if (ex == 0 || ex == 0xFF) ex = 127;
         if (ex > 253) ex = 253;
@@ -758,7 +757,7 @@ __device__ __forceinline__ void proj_row1_body(const ProjArgs& a, const ProjPrep
             inv_rms = 1.0f / sqrtf(row_sumsq_256(xr, a.K, s4) / (float)a.K + p.eps);
         float mx = 0.f;
         for (uint32_t k = t; k < a.K; k += 256) mx = fmaxf(mx, fabsf(proj_src_value<SRC>(p, xr, k, inv_rms)));
-        mx = block_max_256(mx, s4);
+        mx = block_max_256(mx, s4 + 4);
         uint32_t ex = (__float_as_uint(mx) >> 23) & 0xFFu;
         if (ex == 0 || ex == 0xFF) ex = 127;
         if (ex > 253) ex = 253;
@@ -832,7 +831,7 @@ __global__ __launch_bounds__(kProjThreads) void proj_row1_kernel(const ProjArgs 
     extern __shared__ __attribute__((aligned(16))) unsigned char row1_smem[];
     half8* sfrag = reinterpret_cast<half8*>(row1_smem);           // [K/8][2]: hi, lo of chunk q
     __shared__ f32x4 s_part[3 * 64];
-    __shared__ float s4[4];
+    __shared__ float s4[8];
     __shared__ float s_scale;
     const uint32_t nb = a.K / 32 / a.ksplit / kProjKBatch;        // whole batches of weights per wave: uniform
     if (nb >= 3)
