@@ -432,7 +432,8 @@ struct ProjArgs {
 // its lo term.  The two are combined, the row's scale undone, the optional
 // residual added.  Tiles past N and rows past R are dropped.
 __device__ __forceinline__ void proj_store_tile(const ProjArgs& a, f32x4 v, uint32_t nt, uint32_t group,
-                                                int lane, const float* scales = nullptr)
+                                                int lane, const float* scales = nullptr,
+                                                const f32x4* residual = nullptr)
 {
     if (!scales) scales = a.scales;
     const int c = lane & 15, g = lane >> 4;
@@ -452,7 +453,8 @@ __device__ __forceinline__ void proj_store_tile(const ProjArgs& a, f32x4 v, uint
 #pragma unroll
         for (int i = 0; i < 4; i++) r[i] = v[i] * sc;
         if (a.bias_rows) {
-            const f32x4 b = *reinterpret_cast<const f32x4*>(a.bias_rows + o);
+            // (residual: the same values, read earlier by the caller)
+            const f32x4 b = residual ? *residual : *reinterpret_cast<const f32x4*>(a.bias_rows + o);
 #pragma unroll
             for (int i = 0; i < 4; i++) r[i] += b[i];
         }
@@ -669,6 +671,18 @@ __device__ __forceinline__ void proj_row1_body(const ProjArgs& a, const ProjPrep
         }
     }
 
+    // 1b. the residual values the store at the very end will add, for every lane
+    // and whether or not there is a residual (the row's start stands in): a load
+    // that is only sometimes issued would turn the exact waits below into waits
+    // for everything in flight
+    f32x4 resid;
+    {
+        const int rc = lane & 15, rg = lane >> 4;
+        const uint32_t rrow = min((uint32_t)(rc & 7), a.R - 1), rnt = min(nt0, ntiles - 1);
+        const float* rp = a.bias_rows ? a.bias_rows + (size_t)rrow * a.ldy + rnt * 16 + rg * 4 : xr + rg * 4;
+        resid = *reinterpret_cast<const f32x4*>(rp);
+    }
+
     // 2. the weights: NB0 batches now, the rest as the buffers come free
     half8 wa[KB], wb[KB], wc[KB];
     const uint32_t nb = kper / KB;                               // whole batches of this wave (>= NB0)
@@ -822,7 +836,7 @@ __device__ __forceinline__ void proj_row1_body(const ProjArgs& a, const ProjPrep
         }
     }
     if (!live) return;
-    proj_store_tile(a, acc, nt0, 0, lane, s_scale);
+    proj_store_tile(a, acc, nt0, 0, lane, s_scale, &resid);
 }
 
 template <int SRC>
