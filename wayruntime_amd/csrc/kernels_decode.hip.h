@@ -60,7 +60,7 @@ struct DecodeSession {
     uint32_t ctx_pad;        // rows allocated per KV head (multiple of 32)
     uint32_t n_splits;       // workgroups along the key axis
     uint32_t tiles_per_wg;   // 32-key tiles per workgroup (a function of this session only)
-    uint32_t pad_;
+    uint32_t tail_tiles;     // the session's last tiles that form the last split on their own (0: none)
 };
 
 struct DecodeArgs {
@@ -128,8 +128,13 @@ __device__ __forceinline__ TileRange split_tiles(const DecodeSession& S, uint32_
     const uint32_t first = S.key_lo / kTileKeys;
     const uint32_t last = (S.seq_k + kTileKeys - 1) / kTileKeys;
     TileRange r;
+    if (S.tail_tiles != 0 && split == S.n_splits - 1) {   // the tail: a split of its own
+        r.t_begin = last - S.tail_tiles;
+        r.t_end = last;
+        return r;
+    }
     r.t_begin = first + split * tiles_per_wg;
-    r.t_end = min(r.t_begin + tiles_per_wg, last);
+    r.t_end = min(r.t_begin + tiles_per_wg, last - S.tail_tiles);
     return r;
 }
 
