@@ -144,7 +144,7 @@ __device__ __forceinline__ TileRange split_tiles(const DecodeSession& S, uint32_
 // heads (log-sum-exp over the split maxima, one normalisation), writes the
 // final rows and puts the counter back to zero for the next launch.
 constexpr int kMaxSplits = 64;        // key splits per session (host picks tiles_per_wg to respect it)
-constexpr int kMergeInRegs = 8;       // up to this many partials a merge holds in registers
+constexpr int kMergeInRegs = 12;      // up to this many partials a merge holds in registers
 static_assert(kTileKeys == kKTile, "decode tiles are the cache's K tiles");
 static_assert(sizeof(DecodeArgs::items) == kBatchMax * kMaxSplits * sizeof(uint16_t), "work list size");
 
@@ -237,6 +237,8 @@ __device__ __forceinline__ void publish_and_merge(const DecodeArgs& a, uint32_t 
     if (n_splits <= kMergeInRegs) {
         if (n_splits <= 4)
             merge_in_regs<4>(a, sess, head0, nh, n_splits);
+        else if (n_splits <= 8)
+            merge_in_regs<8>(a, sess, head0, nh, n_splits);
         else
             merge_in_regs<kMergeInRegs>(a, sess, head0, nh, n_splits);
         if (threadIdx.x == 0) a.counters[counter_idx] = 0;

@@ -400,7 +400,9 @@ int decode_locked(uint32_t n, wr_hip_kv* const* kv, uint32_t layer, const uint32
                 // that is done anyway merges: the decode step of a 28-layer model at
                 // ~520 keys 1.02 -> 1.00 ms, sixteen sessions 1.90 -> 1.87 ms.  (A tail
                 // of ONE tile does the same for one session and costs sixteen 2-3 %:
-                // it adds a workgroup per session and KV head.)
+                // it adds a workgroup per session and KV head.)  A caller that has
+                // appended the row itself pays for the extra split instead: one
+                // session of 1024 keys 7.8 -> 8.2 us, of 2048 keys 8.1 -> 8.8 us.
                 if (tiles[i] >= 6) tail = 4;
             } else if (tiles[i] < 4 * cap) {
                 cap = cap >= 2 ? cap / 2 : 1;                           // a medium one: see above
