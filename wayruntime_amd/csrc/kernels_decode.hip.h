@@ -516,18 +516,26 @@ __device__ __forceinline__ void process_tile(DecodeState<HD>& st, DecodeFrag<HD>
     tile_update<HD>(st, f, c, tile, key_lo, seq_k, lane, partner_addr, col_kind);
 }
 
-// Two waves per SIMD for every shape.  Up to head_dim 128 a wave double-buffers
-// whole tiles in registers.  One tile of a 256-wide head is already 128
-// registers, so that shape keeps a single tile and asks for the next tile's K
-// as soon as the scores are out and for its V as soon as P.V is done; the
-// other wave of the SIMD computes while those loads are in flight.  (Double
-// buffering it with one wave per SIMD and 512 registers spilled addresses, and
-// a spill reload waits for every load in flight.)
+// Head dims 128 and 256 keep ONE tile per wave in registers and ask for the next
+// tile's K as soon as the scores are out and for its V as soon as P.V is done;
+// the other waves of the SIMD compute while those loads are in flight.  At 256
+// a tile is 128 registers and two waves share a SIMD (double buffering it with
+// one wave per SIMD and 512 registers spilled addresses, and a spill reload
+// waits for every load in flight).  At 128 the single tile makes room for three
+// workgroups per CU (142 registers) where two tiles per wave allowed two (218):
+// measured against the double-buffered form, 16 x 4096 keys 44.7 -> 44.4 us, the
+// ragged batch of 16 34.7 -> 33.7, one session of 2048 keys 8.5 -> 7.9 and of
+// 8192 keys 15.3 -> 14.7, the fused decode launch at ~520 keys 10.4 -> 8.9 (four
+// workgroups per CU spill: 46 us at 16 x 4096).  The arithmetic of a wave is the
+// same in both forms (same tiles, same order, same chains).  Head dim 64 holds
+// two tiles per wave at 126 registers.
 template <int HD>
-constexpr bool decode_single_buffered() { return HD >= 256; }
+constexpr bool decode_single_buffered() { return HD >= 128; }
+template <int HD>
+constexpr int decode_wgs_per_cu() { return HD >= 256 ? 2 : 3; }
 
 template <int HD, bool FUSED = false>
-__global__ __launch_bounds__(kDecodeThreads, 2)
+__global__ __launch_bounds__(kDecodeThreads, decode_wgs_per_cu<HD>())
 void decode_mfma_kernel(const DecodeArgs a, const DecodeFusedArgs fz)
 {
     static_assert(!FUSED || HD == 128, "the fused form is built for head dim 128");
@@ -706,6 +714,8 @@ void decode_mfma_kernel(const DecodeArgs a, const DecodeFusedArgs fz)
                 load_frag_v<HD>(fa, vtbase, t + kDecodeWaves, lane);
                 t += kDecodeWaves;
             }
+            // (the new position's tile is the last of its wave)
+            if (nrp != nullptr && t == patch_tile) patch_new_row<HD>(fa, *nrp, (S.seq_k - 1) % kTileKeys, lane);
             tile_scores_lds<HD>(c, fa, qrow);
             tile_update<HD>(st, fa, c, t, S.key_lo, S.seq_k, lane, partner_addr, col_kind);
         }
