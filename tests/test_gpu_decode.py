@@ -431,14 +431,16 @@ def test_threads_that_come_and_go_get_a_working_stream():
 
 # ---------------------------------------------- row step inside the attention launch --
 
-@pytest.mark.parametrize("nq,nkv,norm,rot_pairs,window,kpw", [
-    (16, 8, True, 0, 0, 0),          # Qwen3: per-head norms, full rotation
-    (32, 8, False, 0, 0, 0),         # Llama: no norms
-    (32, 8, True, 24, 0, 0),         # partial rotation
-    (16, 8, True, 0, 300, 0),        # sliding window
-    (16, 8, True, 0, 0, 64),         # forced fine key splits: the new row's tile is the last split's
+@pytest.mark.parametrize("nq,nkv,norm,rot_pairs,window,kpw,base", [
+    (16, 8, True, 0, 0, 0, 0),       # Qwen3: per-head norms, full rotation
+    (32, 8, False, 0, 0, 0, 0),      # Llama: no norms
+    (32, 8, True, 24, 0, 0, 0),      # partial rotation
+    (16, 8, True, 0, 300, 0, 0),     # sliding window
+    (16, 8, True, 0, 0, 64, 0),      # forced fine key splits: the new row's tile is the last split's
+    (16, 8, True, 0, 0, 0, 8150),    # long sessions: a workgroup of the batch works through two splits,
+                                     # one of the lone session through one; the new row's tile is in the second
 ])
-def test_append_and_decode_in_one_launch_equals_the_two_calls(nq, nkv, norm, rot_pairs, window, kpw):
+def test_append_and_decode_in_one_launch_equals_the_two_calls(nq, nkv, norm, rot_pairs, window, kpw, base):
     # wr_hip_attn_append_decode_batched_dev against wr_hip_rows_qkv_append_dev +
     # wr_hip_attn_decode_batched_dev on twin caches: the same output bits and
     # the same cache bytes, for one session and for a ragged batch, at positions
@@ -446,8 +448,8 @@ def test_append_and_decode_in_one_launch_equals_the_two_calls(nq, nkv, norm, rot
     import ctypes as C
     hd, eps, theta = 128, 1e-6, 1e6
     lib = hipattn.lib()
-    positions = [0, 1, 31, 32, 33, 63, 64, 500, 1023, 1024, 2047, 2500, 95, 96, 1999, 7]
-    cap = 2600
+    positions = [base + p for p in (0, 1, 31, 32, 33, 63, 64, 500, 1023, 1024, 2047, 2500, 95, 96, 1999, 7)]
+    cap = base + 2600
     n_rot = rot_pairs if rot_pairs else hd // 2
     width = (nq + 2 * nkv) * hd
     qw = synth.normal(9300, (hd,), std=1.0) if norm else None
@@ -455,8 +457,8 @@ def test_append_and_decode_in_one_launch_equals_the_two_calls(nq, nkv, norm, rot
     qwd = hipattn.DeviceBuffer.from_host(qw) if norm else None
     kwd = hipattn.DeviceBuffer.from_host(kw) if norm else None
     for n in (1, 16):
-        pos = positions[:n] if n > 1 else [777]
-        print("fused step", nq, nkv, norm, rot_pairs, window, kpw, "n", n, flush=True)
+        pos = positions[:n] if n > 1 else [base + 777]
+        print("fused step", nq, nkv, norm, rot_pairs, window, kpw, base, "n", n, flush=True)
         twins = []
         for i in range(n):
             _a, _b, k16, v16 = util.make_kv(9400 + 2 * i, cap, nkv, hd)

@@ -83,3 +83,34 @@ def test_long_context_step_loop_at_full_size(nq, nkv, hd):
     finally:
         for kv in caches:
             kv.close()
+
+
+def test_long_sessions_keep_their_bits_whatever_launch_they_are_in():
+    # From 8K keys up a session is cut into twice as many splits as it gets
+    # workgroups in a launch that fills the device: a workgroup there works through
+    # two consecutive splits, in a small launch every split has a workgroup of its
+    # own.  The split is the unit of arithmetic, so the three launches below must
+    # agree byte for byte (reference contract: src/core/batch.c:15-19).
+    nq, nkv, hd = 16, 8, 128
+    ctxs = [8192, 8193, 8223, 8224, 9000, 10000, 12288, 16384, 8255, 11111, 13000, 15000, 8500, 9999, 14000, 16000]
+    caches, qs, kvs = [], [], []
+    for i, ctx in enumerate(ctxs):
+        q = synth.normal(7700 + i, (nq, hd))
+        _a, _b, k16, v16 = util.make_kv(7800 + 2 * i, ctx, nkv, hd)
+        kv = hipattn.KVCache(1, hd, nkv, ctx)
+        kv.write_f16(0, 0, k16, v16)
+        caches.append(kv); qs.append(q); kvs.append((k16, v16))
+    print("long sessions: batch of 16", flush=True)
+    outs = hipattn.decode_batched(caches, 0, ctxs, qs)
+    for i in (0, 7):
+        util.assert_close(outs[i], util.oracle_decode(qs[i], kvs[i][0], kvs[i][1], ctxs[i]), f"session {i}")
+    print("long sessions: alone", flush=True)
+    for i in range(len(ctxs)):
+        single = caches[i].decode(0, ctxs[i], qs[i])
+        assert np.array_equal(single, outs[i]), f"session {i} alone"
+    print("long sessions: pairs", flush=True)
+    for i in range(0, len(ctxs), 2):
+        two = hipattn.decode_batched(caches[i:i + 2], 0, ctxs[i:i + 2], qs[i:i + 2])
+        assert np.array_equal(two[0], outs[i]) and np.array_equal(two[1], outs[i + 1]), f"sessions {i}, {i + 1}"
+    for kv in caches:
+        kv.close()

@@ -60,7 +60,8 @@ struct DecodeSession {
     uint32_t ctx_pad;        // rows allocated per KV head (multiple of 32)
     uint32_t n_splits;       // workgroups along the key axis
     uint32_t tiles_per_wg;   // 32-key tiles per workgroup (a function of this session only)
-    uint32_t tail_tiles;     // the session's last tiles that form the last split on their own (0: none)
+    uint16_t tail_tiles;     // the session's last tiles that form the last split on their own (0: none)
+    uint16_t parts_per_wg;   // consecutive splits one workgroup works through (1 or 2; 1 with a tail)
 };
 
 struct DecodeArgs {
@@ -144,7 +145,7 @@ __device__ __forceinline__ TileRange split_tiles(const DecodeSession& S, uint32_
 // heads (log-sum-exp over the split maxima, one normalisation), writes the
 // final rows and puts the counter back to zero for the next launch.
 constexpr int kMaxSplits = 64;        // key splits per session (host picks tiles_per_wg to respect it)
-constexpr int kMergeInRegs = 12;      // up to this many partials a merge holds in registers
+constexpr int kMergeInRegs = 16;      // up to this many partials a merge holds in registers
 static_assert(kTileKeys == kKTile, "decode tiles are the cache's K tiles");
 static_assert(sizeof(DecodeArgs::items) == kBatchMax * kMaxSplits * sizeof(uint16_t), "work list size");
 
@@ -211,14 +212,15 @@ __device__ __forceinline__ void merge_in_regs(const DecodeArgs& a, uint32_t sess
 }
 
 // Called by every thread of a workgroup after it has stored its partial rows
-// for heads [head0, head0 + nh) of `sess` at its split index.  The workgroup
-// that draws the last of the n_splits tickets merges the partials of those
+// for heads [head0, head0 + nh) of `sess` at its split indices.  The workgroup
+// that draws the last of the n_wgs tickets (the workgroups that share the
+// session's n_splits partials between them) merges the partials of those
 // heads (log-sum-exp over the split maxima, one normalisation), writes the
 // final rows and puts the counter back to zero for the next launch.
 // `scratch` is LDS the caller no longer needs: 3 * nh * kMaxSplits floats.
 __device__ __forceinline__ void publish_and_merge(const DecodeArgs& a, uint32_t sess,
                                                   uint32_t head0, uint32_t nh, uint32_t n_splits,
-                                                  uint32_t counter_idx, float* scratch)
+                                                  uint32_t n_wgs, uint32_t counter_idx, float* scratch)
 {
     __shared__ uint32_t s_ticket;
     // own partial stores acknowledged: the ticket below must not be drawn while
@@ -230,7 +232,7 @@ __device__ __forceinline__ void publish_and_merge(const DecodeArgs& a, uint32_t 
         s_ticket = __hip_atomic_fetch_add(&a.counters[counter_idx], 1u, __ATOMIC_RELAXED,
                                           __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
-    if (s_ticket != n_splits - 1) return;
+    if (s_ticket != n_wgs - 1) return;
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
 
     const uint32_t hd = a.hd;
@@ -239,6 +241,8 @@ __device__ __forceinline__ void publish_and_merge(const DecodeArgs& a, uint32_t 
             merge_in_regs<4>(a, sess, head0, nh, n_splits);
         else if (n_splits <= 8)
             merge_in_regs<8>(a, sess, head0, nh, n_splits);
+        else if (n_splits <= 12)
+            merge_in_regs<12>(a, sess, head0, nh, n_splits);
         else
             merge_in_regs<kMergeInRegs>(a, sess, head0, nh, n_splits);
         if (threadIdx.x == 0) a.counters[counter_idx] = 0;
@@ -547,7 +551,14 @@ void decode_mfma_kernel(const DecodeArgs a, const DecodeFusedArgs fz)
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n = lane & 15, g = lane >> 4;
     const int G = (int)a.group;
-    const TileRange tr = split_tiles(S, split);
+    // The splits this workgroup works through, one after the other: [sp0, sp1).
+    // A split is the unit of arithmetic (one partial) and a function of the
+    // session alone; how many consecutive ones a workgroup takes is the host's
+    // choice per launch and changes no bit.
+    const uint32_t ppw = S.parts_per_wg;
+    const uint32_t sp0 = split * ppw, sp1 = min(sp0 + ppw, S.n_splits);
+    TileRange tr = split_tiles(S, sp0);
+    const TileRange tr_last = split_tiles(S, sp1 - 1);
 
     const uint16_t* kbase = S.k + (size_t)kvh * S.ctx_pad * HD;
     const uint16_t* vtbase = S.vt + (size_t)kvh * (S.ctx_pad / kVBlock) * HD * kVBlock;
@@ -566,9 +577,9 @@ void decode_mfma_kernel(const DecodeArgs a, const DecodeFusedArgs fz)
     // FUSED: the new position's tile, whether this workgroup's range holds it,
     // and the wave that has it (its last tile)
     const uint32_t new_pos = S.seq_k - 1, new_tile = new_pos / kTileKeys;
-    const bool owner = FUSED && new_tile >= tr.t_begin && new_tile < tr.t_end;
+    const bool owner = FUSED && new_tile >= tr.t_begin && new_tile < tr_last.t_end;
     const uint32_t patch_tile =
-        (owner && (new_tile - tr.t_begin) % kDecodeWaves == (uint32_t)wave) ? new_tile : 0xFFFFFFFFu;
+        (owner && (new_tile - tr_last.t_begin) % kDecodeWaves == (uint32_t)wave) ? new_tile : 0xFFFFFFFFu;
     const uint32_t hslot = threadIdx.x >> 3, part = threadIdx.x & 7;   // FUSED: head slot (Q heads, K, V), lane of eight
     // FUSED: the new row's values are asked for here, before the tiles, and worked
     // out after the tiles have been asked for: a wave's loads return in the order
@@ -692,111 +703,134 @@ void decode_mfma_kernel(const DecodeArgs a, const DecodeFusedArgs fz)
     const int partner = (n < G) ? lane + G : ((n < 2 * G) ? lane - G : lane);
     const int partner_addr = partner * 4;
 
-    DecodeState<HD> st;
-#pragma unroll
-    for (int dt = 0; dt < HD / 16; dt++) st.o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
-    st.m = -INFINITY;
-    st.l = 0.f;
-
-    // Loads inside the loops below are unconditional too, and the last tiles
-    // are peeled off, for the same reason.
-    if constexpr (kSingle) {
-        const _Float16* qrow = &lds_q[n][g * 8];
-        if (t < tr.t_end) {
-            f32x4 c[2];
-            while (t + kDecodeWaves < tr.t_end) {
-                // keeps the Q^T reads inside the loop: hoisted, they would cost
-                // the registers this path does not have
-                asm volatile("" ::: "memory");
-                tile_scores_lds<HD>(c, fa, qrow);
-                load_frag_k<HD>(fa, kbase, t + kDecodeWaves, lane);
-                tile_update<HD>(st, fa, c, t, S.key_lo, S.seq_k, lane, partner_addr, col_kind);
-                load_frag_v<HD>(fa, vtbase, t + kDecodeWaves, lane);
-                t += kDecodeWaves;
-            }
-            // (the new position's tile is the last of its wave)
-            if (nrp != nullptr && t == patch_tile) patch_new_row<HD>(fa, *nrp, (S.seq_k - 1) % kTileKeys, lane);
-            tile_scores_lds<HD>(c, fa, qrow);
-            tile_update<HD>(st, fa, c, t, S.key_lo, S.seq_k, lane, partner_addr, col_kind);
-        }
-    } else if (t < tr.t_end) {
-        // fa holds tile t, fb tile t + W (both asked for above); each tile's
-        // buffer is refilled with the tile two rounds on as soon as it is used
-        while (t + 3 * kDecodeWaves < tr.t_end) {
-            process_tile<HD>(st, fa, qop, t, S.key_lo, S.seq_k, lane, partner_addr, col_kind, nrp, patch_tile);
-            load_frag<HD>(fa, kbase, vtbase, t + 2 * kDecodeWaves, lane);
-            process_tile<HD>(st, fb, qop, t + kDecodeWaves, S.key_lo, S.seq_k, lane, partner_addr,
-                             col_kind, nrp, patch_tile);
-            load_frag<HD>(fb, kbase, vtbase, t + 3 * kDecodeWaves, lane);
-            t += 2 * kDecodeWaves;
-        }
-        // one, two or three tiles left; the first two are in flight
-        process_tile<HD>(st, fa, qop, t, S.key_lo, S.seq_k, lane, partner_addr, col_kind, nrp, patch_tile);
-        if (t + 2 * kDecodeWaves < tr.t_end) {
-            load_frag<HD>(fa, kbase, vtbase, t + 2 * kDecodeWaves, lane);
-            process_tile<HD>(st, fb, qop, t + kDecodeWaves, S.key_lo, S.seq_k, lane, partner_addr,
-                             col_kind, nrp, patch_tile);
-            process_tile<HD>(st, fa, qop, t + 2 * kDecodeWaves, S.key_lo, S.seq_k, lane, partner_addr,
-                             col_kind, nrp, patch_tile);
-        } else if (t + kDecodeWaves < tr.t_end) {
-            process_tile<HD>(st, fb, qop, t + kDecodeWaves, S.key_lo, S.seq_k, lane, partner_addr,
-                             col_kind, nrp, patch_tile);
-        }
-    }
-    // denominator: add the four lane groups' shares
-    st.l += wave_xor_f32(st.l, 16);
-    st.l += wave_xor_f32(st.l, 32);
-    // outputs: hi column + lo column
-#pragma unroll
-    for (int dt = 0; dt < HD / 16; dt++)
-#pragma unroll
-        for (int r = 0; r < 4; r++)
-            st.o[dt][r] += __int_as_float(
-                __builtin_amdgcn_ds_bpermute(partner_addr, __float_as_int(st.o[dt][r])));
-
     __shared__ float lds_o[kDecodeWaves][kMaxGroupMfma][HD];
     __shared__ float lds_m[kDecodeWaves][kMaxGroupMfma];
     __shared__ float lds_l[kDecodeWaves][kMaxGroupMfma];
-    if (n < G) {
+    const bool direct = (S.n_splits == 1);
+    for (uint32_t sp = sp0;;) {
+        DecodeState<HD> st;
+#pragma unroll
+        for (int dt = 0; dt < HD / 16; dt++) st.o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        st.m = -INFINITY;
+        st.l = 0.f;
+
+        // Loads inside the loops below are unconditional too, and the last tiles
+        // are peeled off, for the same reason.
+        if constexpr (kSingle) {
+            const _Float16* qrow = &lds_q[n][g * 8];
+            if (t < tr.t_end) {
+                f32x4 c[2];
+                while (t + kDecodeWaves < tr.t_end) {
+                    // keeps the Q^T reads inside the loop: hoisted, they would cost
+                    // the registers this path does not have
+                    asm volatile("" ::: "memory");
+                    tile_scores_lds<HD>(c, fa, qrow);
+                    load_frag_k<HD>(fa, kbase, t + kDecodeWaves, lane);
+                    tile_update<HD>(st, fa, c, t, S.key_lo, S.seq_k, lane, partner_addr, col_kind);
+                    load_frag_v<HD>(fa, vtbase, t + kDecodeWaves, lane);
+                    t += kDecodeWaves;
+                }
+                // (the new position's tile is the last of its wave)
+                if (nrp != nullptr && t == patch_tile) patch_new_row<HD>(fa, *nrp, (S.seq_k - 1) % kTileKeys, lane);
+                tile_scores_lds<HD>(c, fa, qrow);
+                tile_update<HD>(st, fa, c, t, S.key_lo, S.seq_k, lane, partner_addr, col_kind);
+            }
+        } else if (t < tr.t_end) {
+            // fa holds tile t, fb tile t + W (both asked for above); each tile's
+            // buffer is refilled with the tile two rounds on as soon as it is used
+            while (t + 3 * kDecodeWaves < tr.t_end) {
+                process_tile<HD>(st, fa, qop, t, S.key_lo, S.seq_k, lane, partner_addr, col_kind, nrp, patch_tile);
+                load_frag<HD>(fa, kbase, vtbase, t + 2 * kDecodeWaves, lane);
+                process_tile<HD>(st, fb, qop, t + kDecodeWaves, S.key_lo, S.seq_k, lane, partner_addr,
+                                 col_kind, nrp, patch_tile);
+                load_frag<HD>(fb, kbase, vtbase, t + 3 * kDecodeWaves, lane);
+                t += 2 * kDecodeWaves;
+            }
+            // one, two or three tiles left; the first two are in flight
+            process_tile<HD>(st, fa, qop, t, S.key_lo, S.seq_k, lane, partner_addr, col_kind, nrp, patch_tile);
+            if (t + 2 * kDecodeWaves < tr.t_end) {
+                load_frag<HD>(fa, kbase, vtbase, t + 2 * kDecodeWaves, lane);
+                process_tile<HD>(st, fb, qop, t + kDecodeWaves, S.key_lo, S.seq_k, lane, partner_addr,
+                                 col_kind, nrp, patch_tile);
+                process_tile<HD>(st, fa, qop, t + 2 * kDecodeWaves, S.key_lo, S.seq_k, lane, partner_addr,
+                                 col_kind, nrp, patch_tile);
+            } else if (t + kDecodeWaves < tr.t_end) {
+                process_tile<HD>(st, fb, qop, t + kDecodeWaves, S.key_lo, S.seq_k, lane, partner_addr,
+                                 col_kind, nrp, patch_tile);
+            }
+        }
+        // the next split's first tiles travel while this one's waves are merged
+        // (not at head_dim 256: that shape has no register to spare for a loop
+        // around its tile loop, and the host never gives it two splits)
+        const bool more = HD < 256 && sp + 1 < sp1;
+        TileRange tr_next = tr;
+        if (more) {
+            tr_next = split_tiles(S, sp + 1);
+            t = tr_next.t_begin + wave;
+            load_frag<HD>(fa, kbase, vtbase, min(t, tr_next.t_end - 1), lane);
+            if constexpr (!kSingle) load_frag<HD>(fb, kbase, vtbase, min(t + kDecodeWaves, tr_next.t_end - 1), lane);
+        }
+        // denominator: add the four lane groups' shares
+        st.l += wave_xor_f32(st.l, 16);
+        st.l += wave_xor_f32(st.l, 32);
+        // outputs: hi column + lo column
 #pragma unroll
         for (int dt = 0; dt < HD / 16; dt++)
 #pragma unroll
-            for (int r = 0; r < 4; r++) lds_o[wave][n][dt * 16 + 4 * g + r] = st.o[dt][r];
-        if (g == 0) {
-            lds_m[wave][n] = st.m;
-            lds_l[wave][n] = st.l;
-        }
-    }
-    __syncthreads();
+            for (int r = 0; r < 4; r++)
+                st.o[dt][r] += __int_as_float(
+                    __builtin_amdgcn_ds_bpermute(partner_addr, __float_as_int(st.o[dt][r])));
 
-    const bool direct = (S.n_splits == 1);
-    for (uint32_t idx = threadIdx.x; idx < (uint32_t)G * HD; idx += kDecodeThreads) {
-        const uint32_t h = idx / HD, d = idx % HD;
-        float M = lds_m[0][h];
+        if (n < G) {
 #pragma unroll
-        for (int w = 1; w < kDecodeWaves; w++) M = fmaxf(M, lds_m[w][h]);
-        float acc = 0.f, L = 0.f;
+            for (int dt = 0; dt < HD / 16; dt++)
 #pragma unroll
-        for (int w = 0; w < kDecodeWaves; w++) {
-            const float fct = fast_exp2(lds_m[w][h] - M);   // idle wave: exp2(-inf) = 0
-            acc += lds_o[w][h][d] * fct;
-            L += lds_l[w][h] * fct;
-        }
-        const uint32_t head = kvh * G + h;
-        if (direct) {
-            a.out[((size_t)sess * a.nq + head) * HD + d] = (L > 0.f) ? acc / L : 0.f;
-        } else {
-            const size_t pi = ((size_t)sess * a.nq + head) * a.max_splits + split;
-            part_store(&a.part_o[pi * HD + d], acc);
-            if (d == 0) {
-                part_store(&a.part_ml[pi * 2 + 0], M);
-                part_store(&a.part_ml[pi * 2 + 1], L);
+                for (int r = 0; r < 4; r++) lds_o[wave][n][dt * 16 + 4 * g + r] = st.o[dt][r];
+            if (g == 0) {
+                lds_m[wave][n] = st.m;
+                lds_l[wave][n] = st.l;
             }
         }
+        lds_barrier();            // LDS only: the next split's tiles stay in flight
+
+        for (uint32_t idx = threadIdx.x; idx < (uint32_t)G * HD; idx += kDecodeThreads) {
+            const uint32_t h = idx / HD, d = idx % HD;
+            float M = lds_m[0][h];
+#pragma unroll
+            for (int w = 1; w < kDecodeWaves; w++) M = fmaxf(M, lds_m[w][h]);
+            float acc = 0.f, L = 0.f;
+#pragma unroll
+            for (int w = 0; w < kDecodeWaves; w++) {
+                const float fct = fast_exp2(lds_m[w][h] - M);   // idle wave: exp2(-inf) = 0
+                acc += lds_o[w][h][d] * fct;
+                L += lds_l[w][h] * fct;
+            }
+            const uint32_t head = kvh * G + h;
+            if (direct) {
+                a.out[((size_t)sess * a.nq + head) * HD + d] = (L > 0.f) ? acc / L : 0.f;
+            } else {
+                const size_t pi = ((size_t)sess * a.nq + head) * a.max_splits + sp;
+                part_store(&a.part_o[pi * HD + d], acc);
+                if (d == 0) {
+                    part_store(&a.part_ml[pi * 2 + 0], M);
+                    part_store(&a.part_ml[pi * 2 + 1], L);
+                }
+            }
+        }
+        if (!more) break;
+        // lds_o, lds_m, lds_l are written again by the next split.  (This barrier
+        // also waits for the partial stores above and for the tile asked for:
+        // with stores still pending the compiler could no longer count on loads
+        // returning in order, and every wait of the tile loop would become a
+        // wait for everything.)
+        __syncthreads();
+        tr = tr_next;
+        sp++;
     }
     if (!direct) {
         __syncthreads();      // lds_o is reused as merge scratch
-        publish_and_merge(a, sess, kvh * G, G, S.n_splits, sess * a.nkv + kvh, &lds_o[0][0][0]);
+        publish_and_merge(a, sess, kvh * G, G, S.n_splits, (S.n_splits + ppw - 1) / ppw, sess * a.nkv + kvh,
+                          &lds_o[0][0][0]);
     }
 }
 
@@ -926,7 +960,7 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_generic_kernel(const De
     }
     if (!direct) {
         __syncthreads();      // sh.o is reused as merge scratch
-        publish_and_merge(a, sess, head, 1, S.n_splits, sess * a.nq + head, &sh.o[0][0]);
+        publish_and_merge(a, sess, head, 1, S.n_splits, S.n_splits, sess * a.nq + head, &sh.o[0][0]);
     }
 }
 

@@ -376,13 +376,27 @@ int decode_locked(uint32_t n, wr_hip_kv* const* kv, uint32_t layer, const uint32
     // 35.2 -> 34.6 us; at 4096 keys and beyond the full figure stands (16 x 4096
     // loses 4-8 % with halves).  The session's tiles are spread evenly over the workgroups,
     // and the floor keeps the in-kernel merge within kMaxSplits partials.
-    // A single long session gets few workgroups this way; a caller that serves
-    // one session at a time can lower the figure with wr_hip_attn_set_tuning.
+    // A long session (from 8K keys up at head_dim 128) is cut into twice as
+    // many splits as it gets workgroups in a full launch, and a workgroup there
+    // works through two consecutive splits, one after the other: the unit of
+    // arithmetic (a split: one partial, the tiles dealt to the four waves in
+    // turn) stays a function of the session alone, while a launch too small to
+    // give every CU a workgroup sends each split to a workgroup of its own.
+    // One session of 8192 keys: 64 -> 128 workgroups, 14.8 -> 11.2 us; of 16384:
+    // 24.5 -> 16.2; of 32768: 43.9 -> 26.9.  The price in a full launch is one
+    // extra merge of the four waves per workgroup: not measurable at 16 x 32768.
+    // (The same from 4096 keys up costs 16 x 4096 4.5 %: those workgroups have
+    // 32 tiles, and the waves meeting in the middle is 2 us of their 40.)
+    // A caller that serves one session at a time can go further with
+    // wr_hip_attn_set_tuning.
     (void)tiles_total;
     uint32_t max_splits = 1;
     const uint32_t tune = g.tune_keys_per_wg.load(std::memory_order_relaxed);
+    bool pairs[kBatchMax];
+    uint32_t wgs_paired = 0;
     for (uint32_t i = 0; i < n; i++) {
         uint32_t tpw, tail = 0;
+        pairs[i] = false;
         if (tune) {
             tpw = tune / kTileKeys;
             if (tpw == 0) tpw = 1;
@@ -407,35 +421,51 @@ int decode_locked(uint32_t n, wr_hip_kv* const* kv, uint32_t layer, const uint32
             } else if (tiles[i] < 4 * cap) {
                 cap = cap >= 2 ? cap / 2 : 1;                           // a medium one: see above
             }
-            if (cap < tiles[i] / 8) cap = tiles[i] / 8;
+            if (cap <= tiles[i] / 8) {
+                cap = tiles[i] / 8;
+                pairs[i] = use_mfma && hd <= 128;                       // a long session: see above
+            }
             const uint32_t body = tiles[i] - tail;
             const uint32_t want = (body + cap - 1) / cap;              // workgroups
             tpw = (body + want - 1) / want;                            // even share
+            if (pairs[i]) tpw = (tpw + 1) / 2;                         // two splits per workgroup
         }
         const uint32_t body = tiles[i] - tail;
         const uint32_t room = kMaxSplits - (tail ? 1u : 0u);
         const uint32_t floor_tiles = (body + room - 1) / room;
         if (tpw < floor_tiles) tpw = floor_tiles;
         a.s[i].tiles_per_wg = tpw;
-        a.s[i].tail_tiles = tail;
+        a.s[i].tail_tiles = (uint16_t)tail;
+        a.s[i].parts_per_wg = 1;
         a.s[i].n_splits = (body + tpw - 1) / tpw + (tail ? 1u : 0u);
         if (a.s[i].n_splits > max_splits) max_splits = a.s[i].n_splits;
+        wgs_paired += pairs[i] ? (a.s[i].n_splits + 1) / 2 : a.s[i].n_splits;
     }
+    // (the launch as a whole decides this, not the session: it changes which
+    // workgroup does a split, never the split)
+    if ((uint64_t)wgs_paired * nkv >= g.n_cus)
+        for (uint32_t i = 0; i < n; i++)
+            if (pairs[i]) a.s[i].parts_per_wg = 2;
     // work list, longest entries first (ties keep session, split order)
     {
         uint32_t len[kBatchMax * kMaxSplits];
         uint32_t cnt = 0;
         for (uint32_t i = 0; i < n; i++) {
             const uint32_t body = tiles[i] - a.s[i].tail_tiles;
-            for (uint32_t sp = 0; sp < a.s[i].n_splits; sp++) {
-                if (a.s[i].tail_tiles && sp == a.s[i].n_splits - 1) {
-                    len[cnt] = a.s[i].tail_tiles;
-                } else {
-                    const uint32_t begin = sp * a.s[i].tiles_per_wg;
-                    const uint32_t left = body - begin;
-                    len[cnt] = left < a.s[i].tiles_per_wg ? left : a.s[i].tiles_per_wg;
+            const uint32_t ppw = a.s[i].parts_per_wg;
+            for (uint32_t wg = 0; wg * ppw < a.s[i].n_splits; wg++) {
+                uint32_t l = 0;
+                for (uint32_t sp = wg * ppw; sp < (wg + 1) * ppw && sp < a.s[i].n_splits; sp++) {
+                    if (a.s[i].tail_tiles && sp == a.s[i].n_splits - 1) {
+                        l += a.s[i].tail_tiles;
+                    } else {
+                        const uint32_t begin = sp * a.s[i].tiles_per_wg;
+                        const uint32_t left = body - begin;
+                        l += left < a.s[i].tiles_per_wg ? left : a.s[i].tiles_per_wg;
+                    }
                 }
-                a.items[cnt++] = (uint16_t)((i << 8) | sp);
+                len[cnt] = l;
+                a.items[cnt++] = (uint16_t)((i << 8) | wg);
             }
         }
         for (uint32_t i = 1; i < cnt; i++) {           // insertion sort: at most 1024 entries
