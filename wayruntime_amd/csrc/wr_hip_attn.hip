@@ -420,10 +420,9 @@ int decode_locked(uint32_t n, wr_hip_kv* const* kv, uint32_t layer, const uint32
                 if (tiles[i] >= 6) tail = 4;
             } else if (tiles[i] < 4 * cap) {
                 cap = cap >= 2 ? cap / 2 : 1;                           // a medium one: see above
-            }
-            if (cap <= tiles[i] / 8) {
+            } else if (cap <= tiles[i] / 8) {
                 cap = tiles[i] / 8;
-                pairs[i] = use_mfma && hd <= 128;                       // a long session: see above
+                pairs[i] = use_mfma && hd <= 128;                       // a long one: see above
             }
             const uint32_t body = tiles[i] - tail;
             const uint32_t want = (body + cap - 1) / cap;              // workgroups
