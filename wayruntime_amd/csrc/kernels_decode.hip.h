@@ -545,8 +545,22 @@ void decode_mfma_kernel(const DecodeArgs a, const DecodeFusedArgs fz)
     static_assert(!FUSED || HD == 128, "the fused form is built for head dim 128");
     const uint32_t kvh = blockIdx.x;
     const uint32_t item = decode_item(a, blockIdx.y);
+    // Kernel arguments are read through the scalar cache, which starts every
+    // launch empty: each read of a line not yet seen is a trip to memory, and
+    // left to the compiler there were four of them in a row before the first
+    // tile could be asked for (the entry; the session's sizes; the launch's
+    // scalars; the session's pointers: 2 us).  Two are needed: the entry together
+    // with the line that holds the launch's scalars (and the one with the new
+    // row's arguments), then the whole session record at once.  The empty asm
+    // statements pin where the values must have arrived.
+    const float* args_line = a.q;
+    const float* fused_line = FUSED ? fz.qkv : nullptr;
+    asm volatile("" ::"s"(item), "s"(args_line), "s"(fused_line));
     const uint32_t sess = item >> 8, split = item & 0xFFu;
     const DecodeSession S = a.s[sess];
+    if constexpr (!FUSED)
+        asm volatile("" ::"s"(S.k), "s"(S.vt), "s"(S.seq_k), "s"(S.key_lo), "s"(S.ctx_pad), "s"(S.n_splits),
+                     "s"(S.tiles_per_wg), "s"((uint32_t)S.tail_tiles), "s"((uint32_t)S.parts_per_wg));
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n = lane & 15, g = lane >> 4;
