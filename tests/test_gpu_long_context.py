@@ -114,3 +114,27 @@ def test_long_sessions_keep_their_bits_whatever_launch_they_are_in():
         assert np.array_equal(two[0], outs[i]) and np.array_equal(two[1], outs[i + 1]), f"sessions {i}, {i + 1}"
     for kv in caches:
         kv.close()
+
+
+def test_long_sessions_at_head_dim_64_keep_their_bits_too():
+    # head_dim 64 keeps two tiles per wave in registers and has its own form of
+    # the step from one split to the next inside a workgroup; its sessions are
+    # "long" from 16K keys up (64 tiles per workgroup otherwise)
+    nq, nkv, hd = 16, 8, 64
+    ctxs = [16384, 16385, 17000, 20000]
+    caches, qs, kvs = [], [], []
+    for i, ctx in enumerate(ctxs):
+        q = synth.normal(7900 + i, (nq, hd))
+        _a, _b, k16, v16 = util.make_kv(7950 + 2 * i, ctx, nkv, hd)
+        kv = hipattn.KVCache(1, hd, nkv, ctx)
+        kv.write_f16(0, 0, k16, v16)
+        caches.append(kv); qs.append(q); kvs.append((k16, v16))
+    print("long sessions, head_dim 64: four in one launch", flush=True)
+    outs = hipattn.decode_batched(caches, 0, ctxs, qs)
+    util.assert_close(outs[2], util.oracle_decode(qs[2], kvs[2][0], kvs[2][1], ctxs[2]), "session 2")
+    print("long sessions, head_dim 64: alone", flush=True)
+    for i in range(len(ctxs)):
+        single = caches[i].decode(0, ctxs[i], qs[i])
+        assert np.array_equal(single, outs[i]), f"session {i} alone"
+    for kv in caches:
+        kv.close()
