@@ -253,7 +253,7 @@ int wr_hip_attn_append_decode_batched_dev(uint32_t n, wr_hip_kv *const *kv,
  * hipFree or other allocating call.  Limits: nq <= WR_HIP_NOALLOC_MAX_HEADS,
  * and n * nq * max_splits * (hd + 2) * 4 bytes of partials must fit the array
  * behind its first 64 KiB (with the automatic split rule a session has at most
- * 8 key splits: 16 sessions of 32 heads x 128 need 2.1 MB); beyond either,
+ * 18 key splits: 16 sessions of 32 heads x 128 need 4.8 MB); beyond either,
  * WR_HIP_ERR_LIMIT and nothing is launched.  All calls on one device share the
  * array: the library runs them one after the other, also when they come from
  * different threads (each launch waits for an event the previous one
