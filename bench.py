@@ -299,6 +299,28 @@ def main() -> None:
         prefill = {"workload": "causal prefill, 32/8/128, T=2048, empty cache", "tflops": round(tfl, 2),
                    "ms": round(p_avg, 4), "frac_of_f16_mfma_peak": round(tfl / MFMA_F16_PEAK_TFLOPS, 4),
                    "max_abs_err_sampled_rows": perr}
+        # the form for callers whose Q never leaves the device: Q as the binary16
+        # operand the kernel would round it to (same output bits, half the Q bytes)
+        qscale = np.float32(np.float32(1.0) / np.sqrt(np.float32(hd))) * np.float32(1.4426950408889634)
+        q16_dev = hipattn.DeviceBuffer.from_host((qp * qscale).astype(np.float16))
+        o16_dev = hipattn.DeviceBuffer(qp.nbytes)
+        lib = hipattn.lib()
+        def q16_launch():
+            rc = lib.wr_hip_attn_prefill_q16_dev(caches[0].h, 0, 0, T, q16_dev.p, o16_dev.p, nq, 0.0, 0)
+            if rc != hipattn.OK:
+                raise RuntimeError("wr_hip_attn_prefill_q16_dev: %d" % rc)
+        q16_launch()
+        hipattn.profile_begin(reps)
+        for _ in range(reps):
+            q16_launch()
+        qms, qn_ = hipattn.profile_end()
+        q_avg = qms / max(qn_, 1)
+        got16 = o16_dev.to_host((T, nq, hd))
+        prefill["q16_dev"] = {"ms": round(q_avg, 4), "tflops": round(flops / (q_avg * 1e-3) / 1e12, 2),
+                              "frac_of_f16_mfma_peak": round(flops / (q_avg * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
+                              "same_bits_as_f32_rows": bool(got16.tobytes() == gotp.tobytes())}
+        q16_dev.free()
+        o16_dev.free()
         qp_dev.free()
         op_dev.free()
         # the same launch at other head shapes and lengths (timing only: their

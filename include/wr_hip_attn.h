@@ -219,6 +219,19 @@ int wr_hip_attn_prefill_dev(wr_hip_kv *kv, uint32_t layer, uint32_t p0,
                             uint32_t T, const float *q_dev, float *out_dev,
                             uint32_t nq, float scale_override,
                             uint32_t window);
+/* wr_hip_attn_prefill_dev for a caller whose Q rows never leave the device:
+ * q16_dev [T][nq][hd] holds them as binary16, already multiplied by the
+ * softmax scale times log2(e) -- exactly what the kernel makes of F32 rows
+ * before its first contraction (it rounds Q to binary16 once), so the output equals wr_hip_attn_prefill_dev's bit for bit
+ * at half the Q bytes.  wr_hip_rows_qkv_append_q16_dev writes that form.
+ * Replaces the same reference call sites (src/core/session.c:599-630 with
+ * src/core/kernels.c:1475-1523).  head_dim 64 and 128 with the matrix-core group
+ * sizes; WR_HIP_ERR_UNSUPPORTED otherwise (the caller keeps the F32 form).
+ * q16_dev must be 8-byte aligned. */
+int wr_hip_attn_prefill_q16_dev(wr_hip_kv *kv, uint32_t layer, uint32_t p0,
+                                uint32_t T, const uint16_t *q16_dev,
+                                float *out_dev, uint32_t nq,
+                                float scale_override, uint32_t window);
 
 /* A decode step's row work and attention in one launch: row i of qkv_dev
  * [n][ld] is session i's stacked projection (nq Q heads, then nkv K heads, then
@@ -386,6 +399,17 @@ int wr_hip_rows_qkv_append_dev(const float *qkv_dev, uint32_t ld, uint32_t rows,
                                const float *cos_sin_dev, uint32_t n_rot, uint32_t n_kv,
                                wr_hip_kv *const *kv, uint32_t layer, const uint32_t *pos,
                                float *q_out_dev, uint32_t flags);
+/* The same (src/core/session.c:459-486), with Q written as binary16 rows
+ * multiplied by the softmax scale (scale_override > 0, else 1/sqrt(hd)) times
+ * log2(e): the operand wr_hip_attn_prefill_q16_dev takes.  K and V are appended
+ * exactly as above.  head_dim 128 with the alignment of the eight-lane form
+ * (16-byte aligned pointers, ld % 4 == 0, n_rot % 8 == 0);
+ * WR_HIP_ERR_UNSUPPORTED otherwise, before anything is written. */
+int wr_hip_rows_qkv_append_q16_dev(const float *qkv_dev, uint32_t ld, uint32_t rows, uint32_t nq,
+                                   const float *q_norm_dev, const float *k_norm_dev, float eps,
+                                   const float *cos_sin_dev, uint32_t n_rot, uint32_t n_kv,
+                                   wr_hip_kv *const *kv, uint32_t layer, const uint32_t *pos,
+                                   uint16_t *q16_out_dev, float scale_override, uint32_t flags);
 
 /* swiglu: act[r][j] = silu(gu[r][j]) * gu[r][ffn + j] for rows of a stacked
  * gate/up projection (wri_op_fused_silu_mul, src/core/kernels.c:1243-1258 with

@@ -331,6 +331,22 @@ int wr_hip_rows_qkv_append_dev(const float *qkv, uint32_t ld, uint32_t rows, uin
     (void)n_kv; (void)kv; (void)layer; (void)pos; (void)q; (void)flags;
     return WR_HIP_ERR_STATE;
 }
+int wr_hip_rows_qkv_append_q16_dev(const float *qkv, uint32_t ld, uint32_t rows, uint32_t nq,
+                                   const float *qn, const float *kn, float eps, const float *cs,
+                                   uint32_t n_rot, uint32_t n_kv, wr_hip_kv *const *kv, uint32_t layer,
+                                   const uint32_t *pos, uint16_t *q16, float scale_override, uint32_t flags)
+{
+    (void)qkv; (void)ld; (void)rows; (void)nq; (void)qn; (void)kn; (void)eps; (void)cs; (void)n_rot;
+    (void)n_kv; (void)kv; (void)layer; (void)pos; (void)q16; (void)scale_override; (void)flags;
+    return WR_HIP_ERR_STATE;
+}
+int wr_hip_attn_prefill_q16_dev(wr_hip_kv *kv, uint32_t layer, uint32_t p0, uint32_t T, const uint16_t *q16,
+                                float *out, uint32_t nq, float scale_override, uint32_t window)
+{
+    (void)kv; (void)layer; (void)p0; (void)T; (void)q16; (void)out; (void)nq; (void)scale_override;
+    (void)window;
+    return WR_HIP_ERR_STATE;
+}
 int wr_hip_rows_rmsnorm_add_dev(const float *x, uint32_t ldx, const float *w, uint32_t wn, float *acc,
                                 uint32_t lda, uint32_t rows, uint32_t dim, float eps)
 {

@@ -221,3 +221,71 @@ def test_prefill_error_contract():
     assert pre(0, 4) == hipattn.OK
     assert lib.wr_hip_attn_calls() == calls + 4            # one per token, as the serial loop counts
     kv.close()
+
+
+@pytest.mark.parametrize("nq,nkv,T,p0,norm,scale,window", [
+    (16, 8, 600, 0, True, 0.0, 0),       # Qwen3 shape: per-head norms, one block per workgroup
+    (32, 8, 2048, 0, False, 0.0, 0),     # Llama shape: paired blocks
+    (16, 8, 300, 500, True, 0.25, 0),    # a later chunk of a prompt, scale override
+    (32, 8, 700, 0, False, 0.0, 256),    # sliding window
+])
+def test_prefill_from_f16_query_rows_equals_the_f32_form(nq, nkv, T, p0, norm, scale, window):
+    # wr_hip_rows_qkv_append_q16_dev + wr_hip_attn_prefill_q16_dev against
+    # wr_hip_rows_qkv_append_dev + wr_hip_attn_prefill_dev on twin caches: the
+    # kernel rounds Q to binary16 once in either form, so the outputs must agree
+    # byte for byte, as must the caches; the F16 rows themselves are checked against
+    # the F32 rows times the scale, rounded to nearest
+    import ctypes as C
+    hd, eps, theta = 128, 1e-6, 1e6
+    lib = hipattn.lib()
+    print("prefill q16", nq, nkv, T, p0, norm, scale, window, flush=True)
+    width = (nq + 2 * nkv) * hd
+    x = synth.normal(8800 + T, (T, width), std=1.5)
+    qw = synth.normal(8801, (hd,), std=1.0) if norm else None
+    kw = synth.normal(8802, (hd,), std=1.0) if norm else None
+    tab = oracle.rope_table(T, hd, p0, theta, 0)
+    n_rot = tab.shape[1]
+    xd = hipattn.DeviceBuffer.from_host(x)
+    td = hipattn.DeviceBuffer.from_host(tab)
+    qwd = hipattn.DeviceBuffer.from_host(qw) if norm else None
+    kwd = hipattn.DeviceBuffer.from_host(kw) if norm else None
+    qn = qwd.p if norm else None
+    kn = kwd.p if norm else None
+    _a, _b, k16, v16 = util.make_kv(8810, p0 + T, nkv, hd)
+    twins = []
+    for _ in range(2):
+        kv = hipattn.KVCache(1, hd, nkv, p0 + T)
+        kv.write_f16(0, 0, k16, v16)
+        twins.append(kv)
+    pp = (C.c_uint32 * 1)(p0)
+    q32 = hipattn.DeviceBuffer(T * nq * hd * 4)
+    q16 = hipattn.DeviceBuffer(T * nq * hd * 2)
+    o32 = hipattn.DeviceBuffer.from_host(np.full((T, nq, hd), 3.0, dtype=np.float32))
+    o16 = hipattn.DeviceBuffer.from_host(np.full((T, nq, hd), -4.0, dtype=np.float32))
+    kva = (C.c_void_p * 1)(twins[0].h)
+    kvb = (C.c_void_p * 1)(twins[1].h)
+    assert lib.wr_hip_rows_qkv_append_dev(xd.p, width, T, nq, qn, kn, eps, td.p, n_rot, 1, kva, 0, pp,
+                                          q32.p, 0) == hipattn.OK
+    assert lib.wr_hip_attn_prefill_dev(twins[0].h, 0, p0, T, q32.p, o32.p, nq, scale, window) == hipattn.OK
+    assert lib.wr_hip_rows_qkv_append_q16_dev(xd.p, width, T, nq, qn, kn, eps, td.p, n_rot, 1, kvb, 0, pp,
+                                              q16.p, scale, 0) == hipattn.OK
+    assert lib.wr_hip_attn_prefill_q16_dev(twins[1].h, 0, p0, T, q16.p, o16.p, nq, scale, window) == hipattn.OK
+    hipattn.sync()
+    a, b = o32.to_host((T, nq, hd)), o16.to_host((T, nq, hd))
+    rows_off = np.argwhere(np.abs(a - b).reshape(T, -1).max(axis=1) > 0)[:, 0]
+    assert a.tobytes() == b.tobytes(), f"rows that differ: {rows_off[:8].tolist()} of {len(rows_off)}"
+    ka, va = twins[0].read_f16(0, 0, p0 + T)
+    kb, vb = twins[1].read_f16(0, 0, p0 + T)
+    assert ka.tobytes() == kb.tobytes() and va.tobytes() == vb.tobytes()
+    qs = np.float32((scale if scale > 0 else 1.0 / np.sqrt(np.float32(hd))) * np.float32(1.4426950408889634))
+    want = (q32.to_host((T, nq, hd)) * qs).astype(np.float16)
+    got = q16.to_host((T, nq, hd), dtype=np.float16)
+    assert got.tobytes() == want.tobytes()
+    # shapes the form does not take are refused before anything is written
+    assert lib.wr_hip_rows_qkv_append_q16_dev(xd.p, width + 2, T, nq, qn, kn, eps, td.p, n_rot, 1, kvb, 0, pp,
+                                              q16.p, scale, 0) == hipattn.ERR_UNSUPPORTED
+    for kv in twins:
+        kv.close()
+    for buf in (xd, td, qwd, kwd, q32, q16, o32, o16):
+        if buf is not None:
+            buf.free()

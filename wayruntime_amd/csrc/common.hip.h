@@ -196,6 +196,21 @@ __device__ __forceinline__ void lds_direct_load(uint32_t lds_addr, const unsigne
                  : "memory");
 }
 
+// Four query values multiplied by the softmax scale (times log2 e) and rounded
+// to binary16: what the prefill kernel's first contraction takes.  One
+// function for the kernel that is handed F32 rows and for the row kernel that
+// writes the rounded form for it, so that the two give the same bits.
+__device__ __forceinline__ half4 q_scaled_f16(float4 x, float qscale)
+{
+#pragma clang fp contract(off)
+    half4 h;
+    h[0] = (_Float16)(x.x * qscale);
+    h[1] = (_Float16)(x.y * qscale);
+    h[2] = (_Float16)(x.z * qscale);
+    h[3] = (_Float16)(x.w * qscale);
+    return h;
+}
+
 // Workgroup barrier that waits for this wave's LDS traffic only.  __syncthreads()
 // also drains outstanding global loads, which would pull the tiles being
 // prefetched for later iterations back onto the critical path.

@@ -15,6 +15,7 @@ struct PrefillArgs {
     const uint16_t* k;
     const uint16_t* vt;
     const float* q;          // [T][nq][hd]
+    const uint16_t* q16;     // or: the same rows as binary16, already multiplied by qscale (prefill_il_kernel only)
     float* out;              // [T][nq][hd]
     uint32_t p0, T, nq, nkv, group, hd, ctx_pad, window;
     float qscale;            // softmax scale * log2(e)

@@ -415,7 +415,13 @@ __device__ __forceinline__ void il_load_q(IlQRows<HD>& q, const PrefillArgs& a, 
     for (int j = 0; j < 16 / Q::RPI; j++) {
         const int r = kg * 16 + j * Q::RPI + lane / Q::LPR;
         const uint32_t row = min(row0 + r, a.T - 1);      // idle rows re-read the last one
-        q.x[j] = *reinterpret_cast<const float4*>(a.q + ((size_t)row * a.nq + head) * HD + (lane % Q::LPR) * 4);
+        const size_t at = ((size_t)row * a.nq + head) * HD + (lane % Q::LPR) * 4;
+        if (a.q16 != nullptr) {                           // four finished halves: 8 bytes in .x and .y
+            const uint2 h = *reinterpret_cast<const uint2*>(a.q16 + at);
+            q.x[j] = make_float4(__uint_as_float(h.x), __uint_as_float(h.y), 0.f, 0.f);
+        } else {
+            q.x[j] = *reinterpret_cast<const float4*>(a.q + at);
+        }
     }
 }
 
@@ -550,12 +556,12 @@ __device__ __forceinline__ void il_block(const PrefillArgs& a, unsigned char* sm
         for (int j = 0; j < 16 / Q::RPI; j++) {
             const int r = kg * 16 + j * Q::RPI + lane / Q::LPR;
             const float4 x = q.x[j];
-            half4 h;
-            h[0] = (_Float16)(x.x * a.qscale);
-            h[1] = (_Float16)(x.y * a.qscale);
-            h[2] = (_Float16)(x.z * a.qscale);
-            h[3] = (_Float16)(x.w * a.qscale);
-            *reinterpret_cast<half4*>(&qs[sub][r][(lane % Q::LPR) * 4]) = h;
+            if (a.q16 != nullptr) {
+                *reinterpret_cast<uint2*>(&qs[sub][r][(lane % Q::LPR) * 4]) =
+                    make_uint2(__float_as_uint(x.x), __float_as_uint(x.y));
+            } else {
+                *reinterpret_cast<half4*>(&qs[sub][r][(lane % Q::LPR) * 4]) = q_scaled_f16(x, a.qscale);
+            }
             q.x[j] = make_float4(0.f, 0.f, 0.f, 0.f);      // consumed: nothing of it has to outlive the step loop
         }
     }

@@ -125,6 +125,8 @@ struct QkvAppendArgs {
     const float* k_norm;
     const float* cos_sin;    // [rows][n_rot][2]
     float* q_out;            // [rows][nq][hd]
+    uint16_t* q16_out;       // or (eight-lane form only): the Q rows as binary16, multiplied by q16_scale
+    float q16_scale;
     uint16_t* k[16];
     uint16_t* vt[16];
     uint32_t pos[16];
@@ -179,7 +181,17 @@ __device__ __forceinline__ void qkv_append_row8(const QkvAppendArgs& a, unsigned
     }
 
     if (!live) return;
-    if (is_q) {
+    if (is_q && a.q16_out != nullptr) {
+        // what the prefill kernel would make of the F32 row itself (q_scaled_f16)
+        uint16_t* dst = a.q16_out + ((size_t)r * a.nq + h) * HD + part * 8;
+#pragma unroll
+        for (int c = 0; c < NJ; c++) {
+            const half4 lo = q_scaled_f16(make_float4(x[c][0], x[c][1], x[c][2], x[c][3]), a.q16_scale);
+            const half4 hi = q_scaled_f16(make_float4(x[c][4], x[c][5], x[c][6], x[c][7]), a.q16_scale);
+            *reinterpret_cast<half4*>(dst + c * 64) = lo;
+            *reinterpret_cast<half4*>(dst + c * 64 + 4) = hi;
+        }
+    } else if (is_q) {
         float* dst = a.q_out + ((size_t)r * a.nq + h) * HD + part * 8;
 #pragma unroll
         for (int c = 0; c < NJ; c++) {

@@ -585,7 +585,8 @@ int check_decode(uint32_t n, wr_hip_kv* const* kv, uint32_t layer, const uint32_
 }
 
 int prefill_locked(wr_hip_kv* kv, uint32_t layer, uint32_t p0, uint32_t T, const float* q_dev,
-                   float* out_dev, uint32_t nq, float scale_override, uint32_t window)
+                   float* out_dev, uint32_t nq, float scale_override, uint32_t window,
+                   const uint16_t* q16_dev = nullptr)
 {
     const uint32_t hd = kv->hd[layer];
     PrefillArgs a;
@@ -593,6 +594,7 @@ int prefill_locked(wr_hip_kv* kv, uint32_t layer, uint32_t p0, uint32_t T, const
     a.k = reinterpret_cast<const uint16_t*>(kv->slab + kv->k_off[layer]);
     a.vt = reinterpret_cast<const uint16_t*>(kv->slab + kv->vt_off[layer]);
     a.q = q_dev;
+    a.q16 = q16_dev;
     a.out = out_dev;
     a.p0 = p0;
     a.T = T;
@@ -607,6 +609,7 @@ int prefill_locked(wr_hip_kv* kv, uint32_t layer, uint32_t p0, uint32_t T, const
     const uint32_t G = a.group;
     const bool mfma = !g.force_generic && (hd == 64 || hd == 128 || hd == 256) &&
                       (G == 1 || G == 2 || G == 4 || G == 8);
+    if (q16_dev && !(mfma && (hd == 64 || hd == 128))) return WR_HIP_ERR_UNSUPPORTED;
     if (mfma) {
         const uint32_t Gw = G < 4 ? G : 4;
         const uint32_t BP = 32 * (4 / Gw);
@@ -1461,6 +1464,17 @@ int wr_hip_attn_prefill_dev(wr_hip_kv* kv, uint32_t layer, uint32_t p0, uint32_t
     return prefill_locked(kv, layer, p0, T, q_dev, out_dev, nq, scale_override, window);
 }
 
+int wr_hip_attn_prefill_q16_dev(wr_hip_kv* kv, uint32_t layer, uint32_t p0, uint32_t T,
+                                const uint16_t* q16_dev, float* out_dev, uint32_t nq, float scale_override,
+                                uint32_t window)
+{
+    int rc = check_prefill(kv, layer, p0, T, q16_dev, out_dev, nq);
+    if (rc) return rc;
+    if (((uintptr_t)q16_dev & 7) != 0) return WR_HIP_ERR_INVAL;
+    ENTER();
+    return prefill_locked(kv, layer, p0, T, nullptr, out_dev, nq, scale_override, window, q16_dev);
+}
+
 int wr_hip_attn_prefill(wr_hip_kv* kv, uint32_t layer, uint32_t p0, uint32_t T, const float* q,
                         float* out, uint32_t nq, float scale_override, uint32_t window)
 {
@@ -1756,14 +1770,16 @@ int wr_hip_rows_qkv_prep_dev(const float* qkv_dev, uint32_t ld, uint32_t rows, u
     return WR_HIP_OK;
 }
 
-int wr_hip_rows_qkv_append_dev(const float* qkv_dev, uint32_t ld, uint32_t rows, uint32_t nq,
-                               const float* q_norm_dev, const float* k_norm_dev, float eps,
-                               const float* cos_sin_dev, uint32_t n_rot, uint32_t n_kv,
-                               wr_hip_kv* const* kv, uint32_t layer, const uint32_t* pos,
-                               float* q_out_dev, uint32_t flags)
+// q16_out_dev != nullptr: Q leaves as binary16 rows multiplied by the softmax
+// scale times log2(e) (what wr_hip_attn_prefill_q16_dev takes) instead of F32.
+static int qkv_append_common(const float* qkv_dev, uint32_t ld, uint32_t rows, uint32_t nq,
+                             const float* q_norm_dev, const float* k_norm_dev, float eps,
+                             const float* cos_sin_dev, uint32_t n_rot, uint32_t n_kv,
+                             wr_hip_kv* const* kv, uint32_t layer, const uint32_t* pos,
+                             float* q_out_dev, uint16_t* q16_out_dev, float scale_override, uint32_t flags)
 {
     if (!g.inited) return WR_HIP_ERR_STATE;
-    if (!qkv_dev || !q_out_dev || !kv || !pos || nq == 0) return WR_HIP_ERR_INVAL;
+    if (!qkv_dev || (!q_out_dev && !q16_out_dev) || !kv || !pos || nq == 0) return WR_HIP_ERR_INVAL;
     if (flags & ~(uint32_t)(WR_HIP_QKV_V_NORM | WR_HIP_QKV_Q_ONLY)) return WR_HIP_ERR_INVAL;
     const bool q_only = (flags & WR_HIP_QKV_Q_ONLY) != 0;
     if (n_kv == 0 || (n_kv != 1 && n_kv != rows)) return WR_HIP_ERR_INVAL;
@@ -1807,9 +1823,17 @@ int wr_hip_rows_qkv_append_dev(const float* qkv_dev, uint32_t ld, uint32_t rows,
     {
         // eight lanes per position with 16-byte accesses where the shapes and
         // the addresses allow it (every model on the device walk does)
-        const uintptr_t addrs = (uintptr_t)qkv_dev | (uintptr_t)q_out_dev | (uintptr_t)cos_sin_dev |
-                                (uintptr_t)q_norm_dev | (uintptr_t)k_norm_dev;
+        const uintptr_t addrs = (uintptr_t)qkv_dev | (uintptr_t)q_out_dev | (uintptr_t)q16_out_dev |
+                                (uintptr_t)cos_sin_dev | (uintptr_t)q_norm_dev | (uintptr_t)k_norm_dev;
         if ((hd == 128 || hd == 256) && n_rot % 8 == 0 && ld % 4 == 0 && addrs % 16 == 0) a.row8 = hd / 64;
+    }
+    if (q16_out_dev) {
+        // only the eight-lane form writes it, and only the 128-wide head has a
+        // prefill kernel that reads it
+        if (a.row8 != 2) return WR_HIP_ERR_UNSUPPORTED;
+        const float scale = (scale_override > 0.0f) ? scale_override : 1.0f / sqrtf((float)hd);
+        a.q16_out = q16_out_dev;
+        a.q16_scale = scale * kLog2e;                     // prefill_locked's qscale, by the same expression
     }
     const uint32_t gx = a.per_session ? rows : (pos[0] + rows - 1) / kVBlock - pos[0] / kVBlock + 1;
     const size_t lds = std::max((size_t)4 * hd * sizeof(float), (size_t)hd * (kVBlock + 2) * sizeof(uint16_t));
@@ -1817,6 +1841,28 @@ int wr_hip_rows_qkv_append_dev(const float* qkv_dev, uint32_t ld, uint32_t rows,
     hipLaunchKernelGGL(qkv_append_kernel, dim3(gx, nq + (q_only ? 0 : 2 * nkv)), dim3(256), lds, cx->stream, a);
     HIP_TRY(hipGetLastError(), "qkv append launch", layer);
     return WR_HIP_OK;
+}
+
+int wr_hip_rows_qkv_append_dev(const float* qkv_dev, uint32_t ld, uint32_t rows, uint32_t nq,
+                               const float* q_norm_dev, const float* k_norm_dev, float eps,
+                               const float* cos_sin_dev, uint32_t n_rot, uint32_t n_kv,
+                               wr_hip_kv* const* kv, uint32_t layer, const uint32_t* pos,
+                               float* q_out_dev, uint32_t flags)
+{
+    if (!q_out_dev) return g.inited ? WR_HIP_ERR_INVAL : WR_HIP_ERR_STATE;
+    return qkv_append_common(qkv_dev, ld, rows, nq, q_norm_dev, k_norm_dev, eps, cos_sin_dev, n_rot, n_kv, kv,
+                             layer, pos, q_out_dev, nullptr, 0.0f, flags);
+}
+
+int wr_hip_rows_qkv_append_q16_dev(const float* qkv_dev, uint32_t ld, uint32_t rows, uint32_t nq,
+                                   const float* q_norm_dev, const float* k_norm_dev, float eps,
+                                   const float* cos_sin_dev, uint32_t n_rot, uint32_t n_kv,
+                                   wr_hip_kv* const* kv, uint32_t layer, const uint32_t* pos,
+                                   uint16_t* q16_out_dev, float scale_override, uint32_t flags)
+{
+    if (!q16_out_dev) return g.inited ? WR_HIP_ERR_INVAL : WR_HIP_ERR_STATE;
+    return qkv_append_common(qkv_dev, ld, rows, nq, q_norm_dev, k_norm_dev, eps, cos_sin_dev, n_rot, n_kv, kv,
+                             layer, pos, nullptr, q16_out_dev, scale_override, flags);
 }
 
 int wr_hip_rows_swiglu_dev(const float* gate_up_dev, uint32_t ld, float* act_dev, uint32_t ldo,

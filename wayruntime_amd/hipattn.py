@@ -90,6 +90,9 @@ def load() -> C.CDLL:
                                                _vp, _u32, _vp, _vp, _vp]),
         "wr_hip_rows_qkv_append_dev": (C.c_int, [_vp, _u32, _u32, _u32, _vp, _vp, C.c_float, _vp, _u32, _u32,
                                                  C.POINTER(_vp), _u32, C.POINTER(_u32), _vp, _u32]),
+        "wr_hip_rows_qkv_append_q16_dev": (C.c_int, [_vp, _u32, _u32, _u32, _vp, _vp, C.c_float, _vp, _u32, _u32,
+                                                     C.POINTER(_vp), _u32, C.POINTER(_u32), _vp, C.c_float, _u32]),
+        "wr_hip_attn_prefill_q16_dev": (C.c_int, [_vp, _u32, _u32, _u32, _vp, _vp, _u32, C.c_float, _u32]),
         "wr_hip_rows_rmsnorm_add_dev": (C.c_int, [_vp, _u32, _vp, _u32, _vp, _u32, _u32, _u32, C.c_float]),
         "wr_hip_proj_rows_geglu_dev": (C.c_int, [_vp, _u32, _vp, _u32, _vp, _vp, _u32]),
         "wr_hip_rows_swiglu_dev": (C.c_int, [_vp, _u32, _vp, _u32, _u32, _u32]),

@@ -41,6 +41,9 @@ struct wrh_dev_model {
      * 1 = yes, -1 = no (the two calls are made).  Read and written atomically:
      * sessions step from several threads. */
     int            step_in_one_launch;
+    /* prompt passes: does the library take Q as binary16 rows for this model's
+     * attention (same meaning of 0 / 1 / -1)? */
+    int            prefill_q16;
 };
 
 static int proj_dims_ok(const wrh_weight *w)
@@ -102,6 +105,9 @@ wr_status wrh_device_model_init(wr_model *m)
     /* WAYRT_STEP_TWO_LAUNCHES=1: a decode step's row step and attention stay two calls */
     env = getenv("WAYRT_STEP_TWO_LAUNCHES");
     if (env && env[0] == '1') d->step_in_one_launch = -1;
+    /* WAYRT_PREFILL_Q_F32=1: prompt passes hand the attention kernel F32 Q rows */
+    env = getenv("WAYRT_PREFILL_Q_F32");
+    if (env && env[0] == '1') d->prefill_q16 = -1;
     int rc = WR_HIP_OK;
     /* norm vectors: [final | per layer: attn, ffn, (q, k), (post-attn, post-ffn)] */
     size_t n_vec = m->hidden;
@@ -421,11 +427,30 @@ wr_status wrh_forward_rows_device(wr_model *m, wrh_workspace *hs, wrh_devspace *
         } else {
             wr_session *s = ss[0];
             wr_hip_kv *one[1] = {s->kv};
-            TRY(wr_hip_rows_qkv_append_dev(ds->qkv, width, R, nq, dl->q_norm, shared ? NULL : dl->k_norm,
-                                           m->rms_eps, tab, nr, 1, one, ksrc, &pos0, ds->q, flags),
-                "qkv split + kv append");
+            /* Prompt rows: Q goes to the attention kernel as the binary16 operand the
+             * kernel would make of it anyway (same bits, half the bytes); shapes that
+             * form does not take keep F32 rows. */
+            int q16 = 0;
+            if (prefill && __atomic_load_n(&m->dev->prefill_q16, __ATOMIC_RELAXED) >= 0) {
+                const int r16 = wr_hip_rows_qkv_append_q16_dev(ds->qkv, width, R, nq, dl->q_norm,
+                                                               shared ? NULL : dl->k_norm, m->rms_eps, tab, nr, 1,
+                                                               one, ksrc, &pos0, (uint16_t *)ds->q, scale, flags);
+                if (r16 == WR_HIP_ERR_UNSUPPORTED) {
+                    __atomic_store_n(&m->dev->prefill_q16, -1, __ATOMIC_RELAXED);
+                } else {
+                    if (r16 != WR_HIP_OK) return dev_fail(e, "qkv split + kv append", L, r16);
+                    q16 = 1;
+                }
+            }
+            if (!q16)
+                TRY(wr_hip_rows_qkv_append_dev(ds->qkv, width, R, nq, dl->q_norm, shared ? NULL : dl->k_norm,
+                                               m->rms_eps, tab, nr, 1, one, ksrc, &pos0, ds->q, flags),
+                    "qkv split + kv append");
             if (!shared) s->kv_rows[L] = pos0 + R;
-            if (prefill) {
+            if (q16) {
+                TRY(wr_hip_attn_prefill_q16_dev(s->kv, ksrc, pos0, R, (const uint16_t *)ds->q, ds->attn, nq, scale,
+                                                window), "gqa");
+            } else if (prefill) {
                 TRY(wr_hip_attn_prefill_dev(s->kv, ksrc, pos0, R, ds->q, ds->attn, nq, scale, window), "gqa");
             } else {
                 const uint32_t sk = pos0 + 1;
