@@ -64,15 +64,18 @@ def main() -> int:
         tok, steps = int(toks[-1]), (16 if args.host else 64)
         for _ in range(4):
             tok = int(np.argmax(s.step(tok)))
-        dt = 0.0                                  # the engine call alone: the greedy pick over 150 000
+        per_step = []                             # the engine call alone: the greedy pick over 150 000
         for _ in range(steps):                    # logits in numpy costs 50 us a row and is not the engine's
             t = time.perf_counter()
             logits = s.step(tok)
-            dt += time.perf_counter() - t
+            per_step.append(time.perf_counter() - t)
             tok = int(np.argmax(logits))
-        dt /= steps
-        print(f"{walk}: decode step at context ~520: {dt * 1e3:.2f} ms/token ({1 / dt:.0f} tok/s)", flush=True)
+        dt = sum(per_step) / steps
+        med = float(np.median(per_step))
+        print(f"{walk}: decode step at context ~520: {dt * 1e3:.2f} ms/token ({1 / dt:.0f} tok/s), "
+              f"median {med * 1e3:.2f}, slowest {max(per_step) * 1e3:.2f}", flush=True)
         figures["decode_ms_per_token"] = round(dt * 1e3, 3)
+        figures["decode_ms_per_token_median"] = round(med * 1e3, 3)
         ss = [m.session(1024) for _ in range(16)]
         for i, x in enumerate(ss):
             assert x.prefill(toks[:100 + i]) == 100 + i
