@@ -109,6 +109,25 @@ def test_no_alloc_decode_with_the_finest_partition_and_a_window():
             kv.close()
 
 
+def test_no_alloc_decode_of_long_sessions_whose_workgroups_take_two_splits():
+    # sessions of 8K keys and more are cut into sixteen splits; in a launch that
+    # fills the device a workgroup works through two of them and the merging
+    # workgroup is the last of eight, not of sixteen, to draw its ticket from the
+    # array.  Then one of them alone (a workgroup per split) on the same array.
+    nq, nkv, hd = 16, 8, 128
+    ctxs = [8192, 9000, 12288, 16384, 8223, 10000, 8255, 11111]
+    caches, kvs = _sessions(7400, ctxs, nkv, hd)
+    q = synth.normal(7450, (len(ctxs), nq, hd))
+    ref, new = _both(caches, ctxs, q, nq, hd)
+    assert np.array_equal(ref, new)
+    util.assert_close(new[3], util.oracle_decode(q[3], kvs[3][0], kvs[3][1], ctxs[3]), "session 3")
+    ref1, new1 = _both(caches[4:5], ctxs[4:5], q[4:5], nq, hd)
+    assert np.array_equal(ref1, new1)
+    assert np.array_equal(new1[0], new[4])            # alone or in the full launch: the same bits
+    for kv in caches:
+        kv.close()
+
+
 def test_no_alloc_decode_refuses_what_does_not_fit():
     # 16 sessions x 32 heads x 64 splits x (256 + 2) floats = 33.8 MB of partials:
     # more than the fixed array; refused with WR_HIP_ERR_LIMIT, nothing launched,
