@@ -14,7 +14,9 @@
 //            owns a run of 16 KiB tiles (8 KiB of "K" in one region, 8 KiB of
 //            "V" in another, as the cache stores them), waves take tiles
 //            round-robin with two tiles in flight each, 256 registers a wave
-//            so that two workgroups share a compute unit, as there.
+//            so that two workgroups share a compute unit (the decode kernel's
+//            earlier form); and the same with one tile per wave and three
+//            workgroups to a compute unit (its present form at head dim 128).
 // Every figure is the average kernel time between the kernel's own start and
 // stop events (hipExtLaunchKernelGGL), as the bench times the decode kernel.
 #include <hip/hip_runtime.h>
@@ -78,6 +80,44 @@ __global__ __launch_bounds__(256, 2) void read_tiles_kernel(const f4* __restrict
     if (acc[0] + acc[1] + acc[2] + acc[3] == 12345.678f) *sink = 1.f;
 }
 
+// The same run of tiles with ONE tile per wave in registers, the next one asked
+// for once the present one has been used, and three workgroups to a compute
+// unit: what the decode kernel does at head dim 128.
+__global__ __launch_bounds__(256, 3) void read_tiles1_kernel(const f4* __restrict__ base, int tiles_per_wave,
+                                                             float* sink)
+{
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int tiles = 4 * tiles_per_wave;
+    const f4* wg = base + (size_t)blockIdx.x * tiles * 1024;
+    f4 acc = {0, 0, 0, 0};
+    f4 a[16];
+    auto load_k = [&](int t) {
+        const f4* k = wg + (size_t)t * 512;
+#pragma unroll
+        for (int i = 0; i < 8; i++) a[i] = __builtin_nontemporal_load(&k[i * 64 + lane]);
+    };
+    auto load_v = [&](int t) {
+        const f4* v = wg + (size_t)tiles * 512 + (size_t)t * 512;
+#pragma unroll
+        for (int i = 0; i < 8; i++) a[8 + i] = __builtin_nontemporal_load(&v[i * 64 + lane]);
+    };
+    int t = wave;
+    load_k(t);
+    load_v(t);
+#pragma unroll 1
+    for (; t + 4 < tiles; t += 4) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) acc += a[i];          // the K half is used, and refilled, first
+        load_k(t + 4);
+#pragma unroll
+        for (int i = 8; i < 16; i++) acc += a[i];
+        load_v(t + 4);
+    }
+#pragma unroll
+    for (int i = 0; i < 16; i++) acc += a[i];
+    if (acc[0] + acc[1] + acc[2] + acc[3] == 12345.678f) *sink = 1.f;
+}
+
 int main(int argc, char** argv)
 {
     const size_t mib = argc > 1 ? strtoull(argv[1], nullptr, 10) : 256;
@@ -129,6 +169,13 @@ int main(int argc, char** argv)
         char name[64];
         snprintf(name, sizeof name, "tiles, %d per workgroup (decode-like)", 4 * tpw);
         TIMED(hipExtLaunchKernelGGL(read_tiles_kernel, dim3(grid), dim3(256), 0, st, e0, e1, 0, p, tpw, sink),
+              name, grid, (double)grid * 4 * tpw * 16384);
+    }
+    for (int tpw : {8, 4}) {
+        const int grid = (int)(window / ((size_t)4 * tpw * 16384));
+        char name[64];
+        snprintf(name, sizeof name, "tiles, %d per workgroup, one in flight", 4 * tpw);
+        TIMED(hipExtLaunchKernelGGL(read_tiles1_kernel, dim3(grid), dim3(256), 0, st, e0, e1, 0, p, tpw, sink),
               name, grid, (double)grid * 4 * tpw * 16384);
     }
     return 0;
