@@ -24,6 +24,7 @@
 #include "kernels_decode.hip.h"
 #include "kernels_prefill.hip.h"
 #include "kernels_prefill_il.hip.h"
+#include "kernels_prefill_pair.hip.h"
 #include "kernels_proj.hip.h"
 #include "kernels_rows.hip.h"
 
@@ -116,6 +117,7 @@ struct Lib {
     void* log_user = nullptr;
     std::atomic<uint32_t> tune_keys_per_wg{0};
     std::atomic<int> force_generic{0};
+    int prefill_two_waves = 0;        // WR_HIP_PREFILL_TWO_WAVES=1: head dim 128 keeps the two-waves-per-SIMD prefill kernel
 } g;
 
 // The calling thread's context (set by Entered, below).
@@ -625,7 +627,14 @@ int prefill_locked(wr_hip_kv* kv, uint32_t layer, uint32_t p0, uint32_t T, const
         if (hd == 64)
             launch_main(prefill_il_kernel<64>, dim3(ny, nwg), dim3(kSplitThreads), a,
                         split_smem_bytes<64>());
-        else if (hd == 128)
+        else if (hd == 128 && !g.prefill_two_waves) {
+            if (q16_dev)
+                launch_main(prefill_pair_kernel<128, true>, dim3(ny, nwg), dim3(kPairThreads), a,
+                            pair_smem_bytes<128>());
+            else
+                launch_main(prefill_pair_kernel<128, false>, dim3(ny, nwg), dim3(kPairThreads), a,
+                            pair_smem_bytes<128>());
+        } else if (hd == 128)
             launch_main(prefill_il_kernel<128>, dim3(ny, nwg), dim3(kSplitThreads), a,
                         split_smem_bytes<128>());
         else   // 256: one wave per SIMD (the accumulators alone need 256 registers)
@@ -990,6 +999,10 @@ int wr_hip_attn_init(int device)
              prop.multiProcessorCount, (double)prop.totalGlobalMem / (1024.0 * 1024.0 * 1024.0));
     g.inited = true;
     g.calls.store(0);
+    {
+        const char* e = getenv("WR_HIP_PREFILL_TWO_WAVES");
+        g.prefill_two_waves = (e && e[0] == '1') ? 1 : 0;
+    }
     g.generation++;
     int rc = WR_HIP_OK;
     {
@@ -1021,6 +1034,14 @@ int wr_hip_attn_init(int device)
             e = hipFuncSetAttribute(reinterpret_cast<const void*>(prefill_il_kernel<128>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize,
                                     (int)split_smem_bytes<128>());
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute(reinterpret_cast<const void*>(prefill_pair_kernel<128, false>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)pair_smem_bytes<128>());
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute(reinterpret_cast<const void*>(prefill_pair_kernel<128, true>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)pair_smem_bytes<128>());
         if (e == hipSuccess)
             e = hipFuncSetAttribute(reinterpret_cast<const void*>(proj_gemm_lds_kernel<8, 2, 3>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)gemm_lds_bytes<8, 2, 3>());
