@@ -203,11 +203,17 @@ __device__ __forceinline__ void lds_direct_load(uint32_t lds_addr, const unsigne
 __device__ __forceinline__ half4 q_scaled_f16(float4 x, float qscale)
 {
 #pragma clang fp contract(off)
+    // Two roundings, product then conversion.  The products pass through an empty
+    // statement: where it cannot pair two conversions the compiler otherwise
+    // folds product and conversion into one mixed-precision instruction
+    // (v_fma_mixlo_f16), which rounds once and differs in the tie cases.
+    float p0 = x.x * qscale, p1 = x.y * qscale, p2 = x.z * qscale, p3 = x.w * qscale;
+    asm("" : "+v"(p0), "+v"(p1), "+v"(p2), "+v"(p3));
     half4 h;
-    h[0] = (_Float16)(x.x * qscale);
-    h[1] = (_Float16)(x.y * qscale);
-    h[2] = (_Float16)(x.z * qscale);
-    h[3] = (_Float16)(x.w * qscale);
+    h[0] = (_Float16)p0;
+    h[1] = (_Float16)p1;
+    h[2] = (_Float16)p2;
+    h[3] = (_Float16)p3;
     return h;
 }
 

@@ -56,6 +56,18 @@
 
 namespace wr {
 
+#ifdef WR_PAIR_STAMPS
+// timing build only: segment durations of the step loop, summed over the steps of
+// one wave (100 MHz ticks): chain, products, end of step, barrier; and the count
+__device__ unsigned long long pair_stamp_acc[8];
+__device__ unsigned long long pair_stamp_blk[2][8];
+// (the wait is part of the statement: the counter arrives like a load, and a
+// destination the compiler believes written at once may be reused before it is)
+#define WR_STAMP(v) asm volatile("s_memrealtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(v)::"memory")
+#else
+#define WR_STAMP(v)
+#endif
+
 constexpr int kPairThreads = 256;
 
 template <int HD>
@@ -76,8 +88,17 @@ struct PairLds {
     // (m, l) of the exchanged units: in the odd set's third Vt slot, which no copy
     // of a block's prologue goes to
     static constexpr int ML_OFF = SET_BYTES + V_IN_SET + 2 * VTILE;
+    static constexpr int ML_WAVE = 256;                   // floats per wave: m[64], l[64], w0[32], w1[32], spare
+    // Q staging (start of a block, before anything is exchanged): the block's
+    // rows as pre-scaled F16, [4 units][32 rows][HD + 8], over the exchange scratch
+    static constexpr int QS_OFF = X_OFF;
+    static constexpr int QS_ROW = (HD + 8) * 2;
+    static constexpr int QS_BYTES = 4 * 32 * QS_ROW;
+    // per-wave scratch of the rare rescale (32 floats), clear of the Q staging
+    static constexpr int RS_OFF = X_OFF + 3 * X_WAVE + X_WAVE / 2;
     static_assert(KTILE == VTILE && NLW >= 1, "one piece schedule serves K and Vt");
-    static_assert(4 * 2 * 64 * 4 <= VTILE, "(m, l) of four waves fit a Vt slot");
+    static_assert(4 * ML_WAVE * 4 <= VTILE, "the exchange's scalars of four waves fit a Vt slot");
+    static_assert(QS_BYTES <= 3 * X_WAVE + X_WAVE / 2, "Q staging ends below the rescale scratch");
     static_assert(TOTAL <= 160 * 1024, "LDS of one compute unit");
     __device__ static constexpr int fk(int row) { return (row / RPB) & (CPR - 1); }
     __device__ static constexpr int fv(int row) { return (row >> 2) & 3; }
@@ -163,7 +184,7 @@ __device__ __forceinline__ void pair_patch_tail(unsigned char* smem, const PairC
 {
     using L = PairLds<HD>;
     const uint32_t tile = pair_tile(cx, jt);
-    if (tile < cx.tail_tile) return;
+    if (__builtin_expect(tile < cx.tail_tile, 1)) return;
 #pragma unroll
     for (int u = 0; u < L::NLW; u++) {
         const int row = lane / 4;                         // Vt row (dimension) inside the piece: fv sees its low bits only
@@ -205,19 +226,40 @@ __device__ __forceinline__ void pair_mask_special(const PairUnit<HD>& U, f32x16&
     }
 }
 
-// The softmax reference of a row moves (rare, wave-uniform branch).
+// The softmax reference of a row moves (rare, wave-uniform branch).  The output
+// accumulators hold O[query][dim] (a lane: one dimension of sixteen queries), the
+// factors belong to queries (a lane of the score layout: one query): they cross
+// over through 32 floats of LDS, and only when some row that already has a
+// reference moves it (a row without one has an all-zero accumulator).
 template <int HD>
-__device__ __forceinline__ void pair_move_reference(PairUnit<HD>& U, f32x16& c, float tmax, bool jump)
+__device__ __forceinline__ void pair_move_reference(PairUnit<HD>& U, f32x16& c, float tmax, bool jump,
+                                                    unsigned char* smem)
 {
+    using L = PairLds<HD>;
     PrefillRows<HD>& R = U.R;
     const bool unset = (R.m_run == -INFINITY);
     const float delta = jump ? tmax : 0.f;
     const float alpha = jump ? (unset ? 0.f : fast_exp2(-delta)) : 1.0f;
     R.l_run *= alpha;
+    if (__builtin_amdgcn_ballot_w64(jump && !unset) != 0) {
+        // The accumulators are results of hand-written matrix instructions, the
+        // last of them issued just before this branch, and the compiler puts no
+        // wait states in front of the reads below: wait for the matrix pipe here.
+        asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+        const int lane = il_fresh_lane();
+        const int n = lane & 31, g = lane >> 5;
+        const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+        float* sc = reinterpret_cast<float*>(smem + L::RS_OFF) + wave * 32;
+        if (g == 0) sc[n] = alpha;
 #pragma unroll
-    for (int dt = 0; dt < HD / 32; dt++)
+        for (int q4 = 0; q4 < 4; q4++) {
+            const f32x4 av = *reinterpret_cast<const f32x4*>(sc + 8 * q4 + 4 * g);
 #pragma unroll
-        for (int r = 0; r < 16; r++) R.o[dt][r] *= alpha;
+            for (int dt = 0; dt < HD / 32; dt++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) R.o[dt][4 * q4 + e] *= av[e];
+        }
+    }
 #pragma unroll
     for (int r = 0; r < 16; r++) asm volatile("v_sub_f32 %0, %0, %1" : "+v"(c[r]) : "v"(delta));
     if (jump) R.m_run = (unset ? 0.f : R.m_run) + delta;
@@ -228,24 +270,53 @@ __device__ __forceinline__ void pair_move_reference(PairUnit<HD>& U, f32x16& c, 
     asm volatile("v_mov_b32 %0, %1" : "+v"(U.thr) : "v"(still ? -INFINITY : kLazyLog2));
 }
 
-// Row maximum of `c` (taken as if the tile were plain), masks where it is not,
-// the maximum joined across the two lanes of a row and, rarely, a move of the
-// row's reference.
+// Settling the scores of a tile, first half: masks where the tile is not plain
+// for the unit (rare, wave-uniform branch), then the row maximum of the sixteen
+// scores a lane holds.
 template <int HD>
-__device__ __forceinline__ void pair_settle(PairUnit<HD>& U, const PairCtx<HD>& cx, f32x16& c, uint32_t jt, int g)
+__device__ __forceinline__ void pair_settle_a(PairUnit<HD>& U, const PairCtx<HD>& cx, f32x16& c, uint32_t jt, int g,
+                                              float& tmax)
 {
-    float tmax = il_max16(c);
-    if (jt < U.pl_lo || jt > U.pl_hi) {
-        pair_mask_special<HD>(U, c, cx.t0 + 2 * jt, jt, g, tmax);
-        tmax = il_max16(c);
-    }
-    {
-        const uint32_t u = __float_as_uint(tmax);
-        const auto sw = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-        tmax = max3_raw(__uint_as_float(sw[0]), __uint_as_float(sw[1]), tmax);
-    }
+    if (jt < U.pl_lo || jt > U.pl_hi) pair_mask_special<HD>(U, c, cx.t0 + 2 * jt, jt, g, 0.f);
+    tmax = il_max16(c);
+}
+
+// Second half: the maximum joined across the two lanes of a row and, rarely, a
+// move of the row's reference.
+template <int HD>
+__device__ __forceinline__ void pair_settle_b(float& tmax)
+{
+    const uint32_t u = __float_as_uint(tmax);
+    const auto sw = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    tmax = max3_raw(__uint_as_float(sw[0]), __uint_as_float(sw[1]), tmax);
+}
+
+// Third part: which rows' maxima exceed the threshold, as a lane mask in scalar
+// registers, made slots before the step's end looks at it (a scalar branch on a
+// comparison made just before it waits for the vector pipe to drain).
+__device__ __forceinline__ uint64_t pair_settle_jumps(float tmax, float thr)
+{
+    uint64_t m;
+    asm volatile("v_cmp_gt_f32 %0, %1, %2" : "=s"(m) : "v"(tmax), "v"(thr));
+    return m;
+}
+
+// Last part, behind the step's products: the rare move.
+template <int HD>
+__device__ __forceinline__ void pair_settle_c(PairUnit<HD>& U, f32x16& c, float tmax, unsigned char* smem)
+{
     const bool jump = tmax > U.thr;
-    if (__builtin_amdgcn_ballot_w64(jump) != 0) pair_move_reference<HD>(U, c, tmax, jump);
+    if (__builtin_amdgcn_ballot_w64(jump) != 0) pair_move_reference<HD>(U, c, tmax, jump, smem);
+}
+
+template <int HD>
+__device__ __forceinline__ void pair_settle(PairUnit<HD>& U, const PairCtx<HD>& cx, f32x16& c, uint32_t jt, int g,
+                                            unsigned char* smem)
+{
+    float tmax;
+    pair_settle_a<HD>(U, cx, c, jt, g, tmax);
+    pair_settle_b<HD>(tmax);
+    pair_settle_c<HD>(U, c, tmax, smem);
 }
 
 // The matrix instructions, spelled out so that each operand sits in the register
@@ -284,12 +355,75 @@ __device__ __forceinline__ void pair_mfma_acc(f32x16& d, half8 a, half8 b)
     asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(d) : "v"(a), "v"(b));
 }
 
+// A link of a score chain and, in its shadow, a pair of scores of the tile before
+// turned into probabilities: two exponentials (in place), their sum into the row
+// sum, the rounded pair.  An exponential's result may be read by another kind of
+// vector instruction only one instruction later: the order below keeps that.
+__device__ __forceinline__ void pair_slot_chain(f32x16& d, half8 a, half8 b, f32x16& sc, int r, float& ps,
+                                                u32x4& pk4, int e)
+{
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %5, %6, %0\n\t"
+                 "v_exp_f32 %1, %1\n\t"
+                 "v_exp_f32 %2, %2\n\t"
+                 "v_add_f32 %3, %3, %1\n\t"
+                 "v_add_f32 %3, %3, %2\n\t"
+                 "v_cvt_pk_f16_f32 %4, %1, %2"
+                 : "+v"(d), "+v"(sc[r]), "+v"(sc[r + 1]), "+v"(ps), "=v"(pk4[e])
+                 : "a"(a), "a"(b));
+}
+
+__device__ __forceinline__ void pair_slot_chain_first(f32x16& d, half8 a, half8 b, const f32x16& c, f32x16& sc,
+                                                      int r, float& ps, u32x4& pk4, int e)
+{
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %5, %6, %7\n\t"
+                 "v_exp_f32 %1, %1\n\t"
+                 "v_exp_f32 %2, %2\n\t"
+                 "v_add_f32 %3, %3, %1\n\t"
+                 "v_add_f32 %3, %3, %2\n\t"
+                 "v_cvt_pk_f16_f32 %4, %1, %2"
+                 : "=&v"(d), "+v"(sc[r]), "+v"(sc[r + 1]), "+v"(ps), "=v"(pk4[e])
+                 : "a"(a), "a"(b), "v"(c));
+}
+
+// A product and, in its shadow, the first / second half of the row maximum of
+// sixteen scores.
+__device__ __forceinline__ void pair_slot_pv_max_a(f32x16& o, half8 a, half8 b, float& t, const f32x16& c)
+{
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %2, %3, %0\n\t"
+                 "v_max3_f32 %1, %4, %5, %6\n\t"
+                 "v_max3_f32 %1, %1, %7, %8\n\t"
+                 "v_max3_f32 %1, %1, %9, %10\n\t"
+                 "v_max3_f32 %1, %1, %11, %12"
+                 : "+a"(o), "=&v"(t)
+                 : "v"(a), "v"(b), "v"(c[0]), "v"(c[1]), "v"(c[2]), "v"(c[3]), "v"(c[4]), "v"(c[5]), "v"(c[6]),
+                   "v"(c[7]), "v"(c[8]));
+}
+
+__device__ __forceinline__ void pair_slot_pv_max_b(f32x16& o, half8 a, half8 b, float& t, const f32x16& c)
+{
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %2, %3, %0\n\t"
+                 "v_max3_f32 %1, %1, %4, %5\n\t"
+                 "v_max3_f32 %1, %1, %6, %7\n\t"
+                 "v_max3_f32 %1, %1, %8, %9\n\t"
+                 "v_max_f32 %1, %1, %10"
+                 : "+a"(o), "+v"(t)
+                 : "v"(a), "v"(b), "v"(c[9]), "v"(c[10]), "v"(c[11]), "v"(c[12]), "v"(c[13]), "v"(c[14]),
+                   "v"(c[15]));
+}
+
+// A product that names a value made by the statements before it, so that those
+// stay in front of it.
+__device__ __forceinline__ void pair_mfma_acc_after(f32x16& d, half8 a, half8 b, float& after)
+{
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %2, %3, %0" : "+a"(d), "+v"(after) : "v"(a), "v"(b));
+}
+
 // Step j of a wave (P == j % kRing).  On entry cur[u] holds unit u's scores of the
 // set's tile j (masked, reference settled), kf the K operands of tile j+1; on exit
 // nxt[u] holds the scores of tile j+1 in the same state and kf the operands of
 // tile j+2.
 template <int HD, int P>
-__device__ __forceinline__ void pair_step(PairUnit<HD> (&U)[2], const PairCtx<HD>& cx, const f32x16 (&cur)[2],
+__device__ __forceinline__ void pair_step(PairUnit<HD> (&U)[2], const PairCtx<HD>& cx, f32x16 (&cur)[2],
                                           f32x16 (&nxt)[2], u32x4 (&pop)[2][2], half8 (&kf)[HD / 16],
                                           half8 (&vf)[HD / 16], unsigned char* smem, uint32_t j, int lane, int g,
                                           uint32_t kv_valid)
@@ -304,113 +438,190 @@ __device__ __forceinline__ void pair_step(PairUnit<HD> (&U)[2], const PairCtx<HD
     constexpr int VC = (P + 2) % 3;       // Vt of tile j+2 replaces Vt of tile j-1 (read in the previous step)
     constexpr int TS = (P + 1) % 3;       // slot of Vt of tile j+1, whose tail is patched once it has landed
 
+    // One slot per matrix instruction, each slot one block of hand-ordered
+    // instructions: what follows a matrix instruction in its block is issued in
+    // that instruction's shadow.  (Left as ordinary statements between pinned
+    // matrix instructions, the additions and part of the exponentials were sunk
+    // to the end of the step by the compiler, where nothing overlaps them.)
+    //
+    // Row sums by plain additions of the unrounded exponentials: a dot-product
+    // instruction (v_dot2c_f32_f16 on the rounded pair) runs on the matrix pipe
+    // and waits for the matrix instruction in front of it, which a lone wave
+    // cannot afford (measured: MFMA + 2 dot2c = 55 clocks, MFMA + 6 additions = 36).
+    static_assert(PAIRS == 1, "slot blocks below are written for one pair of scores per link");
+#ifdef WR_PAIR_STAMPS
+    unsigned long long st_a, st_b, st_c, st_d, st_e;
+    WR_STAMP(st_a);
+#endif
     float psum[2] = {0.f, 0.f};
-    const half2v ones = {(_Float16)1.0f, (_Float16)1.0f};
 #pragma unroll
     for (int i = 0; i < NS; i++) {
 #pragma unroll
         for (int u = 0; u < 2; u++) {
-            if (i == 0)
-                nxt[u] = pair_mfma_first(kf[0], U[u].R.qop[0], U[u].negm);
+            const int r = 2 * i;
+            if (WR_PAIR_PROBE & 1) {
+                if (i == 0) nxt[u] = pair_mfma_first(kf[0], U[u].R.qop[0], U[u].negm);
+                else pair_mfma_link(nxt[u], kf[i], U[u].R.qop[i]);
+            } else if (i == 0)
+                pair_slot_chain_first(nxt[u], kf[0], U[u].R.qop[0], U[u].negm, cur[u], r, psum[u], pop[u][r >> 3],
+                                      (r & 7) >> 1);
             else
-                pair_mfma_link(nxt[u], kf[i], U[u].R.qop[i]);
+                pair_slot_chain(nxt[u], kf[i], U[u].R.qop[i], cur[u], r, psum[u], pop[u][r >> 3], (r & 7) >> 1);
             if (u == 0 && !(WR_PAIR_PROBE & 8))
                 vf[i] = *reinterpret_cast<const half8*>(smem + cx.vop[i / ND] + VS * L::VTILE + (i % ND) * 2048);
-#pragma unroll
-            for (int q = 0; q < ((WR_PAIR_PROBE & 1) ? 0 : PAIRS); q++) {
-                const int r = 2 * (i * PAIRS + q);
-                const half2v ph = {(_Float16)fast_exp2(cur[u][r]), (_Float16)fast_exp2(cur[u][r + 1])};
-                psum[u] = __builtin_amdgcn_fdot2(ph, ones, psum[u], false);
-                pop[u][r >> 3][(r & 7) >> 1] = __builtin_bit_cast(uint32_t, ph);
+#ifdef WR_PAIR_EARLY_COPIES
+            if (u == 1 && !(WR_PAIR_PROBE & 2)) {
+                if (i < L::NLW) pair_issue_k1<HD, KC>(cx, j + 4, i);
+                else if (i < 2 * L::NLW) pair_issue_v1<HD, VC>(cx, j + 2, i - L::NLW);
             }
+#endif
             __builtin_amdgcn_sched_barrier(0);
         }
     }
     U[0].R.l_run += psum[0];
     U[1].R.l_run += psum[1];
+    WR_STAMP(st_b);
+    // The products, and in their shadows the K operand reads of tile j+2, the
+    // step's copies and the settling of S(j+1).  The scores of tile j+1 are results
+    // of hand-written matrix instructions: nothing may read them before two more
+    // matrix instructions have been issued behind the last link (the compiler knows
+    // of no wait states here).
+    float tmax[2] = {0.f, 0.f};
+    uint64_t jumps[2] = {0, 0};
+    constexpr int S0 = 2, S1 = 6;         // slots behind which unit 0 / unit 1 settle (three slots each)
 #pragma unroll
-    for (int i = 0; i < NS; i++) {
+    for (int s = 0; s < 2 * NS; s++) {
+        const int i = s / 2, u = s % 2;
         const int t = i / ND, dt = i % ND;
-#pragma unroll
-        for (int u = 0; u < 2; u++) pair_mfma_acc(U[u].R.o[dt], vf[i], __builtin_bit_cast(half8, pop[u][t]));
-        if (!(WR_PAIR_PROBE & 8)) kf[i] = *reinterpret_cast<const half8*>(smem + cx.kop[i] + KS * L::KTILE);
-        if (!(WR_PAIR_PROBE & 2)) {
+        const half8 pp = __builtin_bit_cast(half8, pop[u][t]);
+        if (s == S0 || s == S1) {
+            const int w = (s == S0) ? 0 : 1;
+            if (!(WR_PAIR_PROBE & 16)) {
+                const uint32_t jt = j + 1;
+                if (__builtin_expect(jt < U[w].pl_lo || jt > U[w].pl_hi, 0))
+                    pair_mask_special<HD>(U[w], nxt[w], cx.t0 + 2 * jt, jt, g, 0.f);
+            }
+            pair_slot_pv_max_a(U[u].R.o[dt], pp, vf[i], tmax[w], nxt[w]);
+        } else if (s == S0 + 1 || s == S1 + 1) {
+            const int w = (s == S0 + 1) ? 0 : 1;
+            pair_slot_pv_max_b(U[u].R.o[dt], pp, vf[i], tmax[w], nxt[w]);
+        } else if (s == S0 + 2 || s == S1 + 2) {
+            const int w = (s == S0 + 2) ? 0 : 1;
+            pair_mfma_acc(U[u].R.o[dt], pp, vf[i]);
+            pair_settle_b<HD>(tmax[w]);
+        } else if (s == S0 + 3 || s == S1 + 3) {
+            // (the joined maximum is an operand, so that it is made in the slot before)
+            const int w = (s == S0 + 3) ? 0 : 1;
+            pair_mfma_acc_after(U[u].R.o[dt], pp, vf[i], tmax[w]);
+            jumps[w] = pair_settle_jumps(tmax[w], U[w].thr);
+        } else {
+            pair_mfma_acc(U[u].R.o[dt], pp, vf[i]);
+        }
+        if (u == 0) {
+            if (!(WR_PAIR_PROBE & 8)) kf[i] = *reinterpret_cast<const half8*>(smem + cx.kop[i] + KS * L::KTILE);
+        }
+#ifndef WR_PAIR_EARLY_COPIES
+        else if (!(WR_PAIR_PROBE & 2)) {
             if (i < L::NLW) pair_issue_k1<HD, KC>(cx, j + 4, i);
             else if (i < 2 * L::NLW) pair_issue_v1<HD, VC>(cx, j + 2, i - L::NLW);
         }
-        // The scores of tile j+1 are results of hand-written matrix instructions:
-        // nothing may read them before two more matrix instructions have been
-        // issued behind the last link (the compiler knows of no wait states here).
-        if (i == 0) __builtin_amdgcn_sched_barrier(0);
+#endif
+        __builtin_amdgcn_sched_barrier(0);
     }
+    WR_STAMP(st_c);
     if (!(WR_PAIR_PROBE & 16)) {
-        pair_settle<HD>(U[0], cx, nxt[0], j + 1, g);
-        pair_settle<HD>(U[1], cx, nxt[1], j + 1, g);
+        if (__builtin_expect((jumps[0] | jumps[1]) != 0, 0)) {
+            pair_settle_c<HD>(U[0], nxt[0], tmax[0], smem);
+            pair_settle_c<HD>(U[1], nxt[1], tmax[1], smem);
+        }
     }
     // all copies but this step's have landed: K of tile j+3 and Vt of tile j+1,
     // which the next step reads once the barrier has published them
     if (!(WR_PAIR_PROBE & 2)) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * L::NLW) : "memory");
     pair_patch_tail<HD, TS>(smem, cx, j + 1, lane, kv_valid);
     __builtin_amdgcn_sched_barrier(0);
+    WR_STAMP(st_d);
     if (!(WR_PAIR_PROBE & 4)) asm volatile("s_barrier" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
+#ifdef WR_PAIR_STAMPS
+    WR_STAMP(st_e);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) {
+        pair_stamp_acc[0] += st_b - st_a;
+        pair_stamp_acc[1] += st_c - st_b;
+        pair_stamp_acc[2] += st_d - st_c;
+        pair_stamp_acc[3] += st_e - st_d;
+        pair_stamp_acc[4] += 1;
+    }
+#endif
 }
 
-// Q rows of one unit as read from global memory, already in operand order: the
-// lane's own row, eight consecutive dimensions per contraction step.
-template <int HD>
+// Q rows as read from global memory: wave w brings in the 32 rows of unit w with
+// whole-row coalesced loads (a lane per row reads 64 different cache lines per
+// instruction and takes four times as long to get through the vector cache).
+template <int HD, bool Q16>
 struct PairQ {
-    float4 x[HD / 16][2];
+    static constexpr int LPR = Q16 ? HD / 8 : HD / 4;     // lanes per row (16 bytes each)
+    static constexpr int RPI = 64 / LPR;                  // rows per load instruction
+    static constexpr int NI = 32 / RPI;
+    float4 x[NI];
 };
 
 template <int HD, bool Q16>
-__device__ __forceinline__ void pair_load_q(PairQ<HD>& q, const PrefillArgs& a, uint32_t row0, uint32_t head,
-                                            int n, int g)
+__device__ __forceinline__ void pair_load_q(PairQ<HD, Q16>& q, const PrefillArgs& a, uint32_t row0, uint32_t head,
+                                            int lane)
 {
-    const uint32_t row = min(row0 + n, a.T - 1);          // idle rows re-read the last one
-    const size_t at = ((size_t)row * a.nq + head) * HD + g * 8;
-    if (WR_PAIR_PROBE & 32) {
+    using Q = PairQ<HD, Q16>;
 #pragma unroll
-        for (int i = 0; i < HD / 16; i++) q.x[i][0] = q.x[i][1] = make_float4(0.f, 0.f, 0.f, 0.f);
-        return;
-    }
-    if constexpr (Q16) {                                  // eight finished halves: 16 bytes
-        const uint16_t* src = a.q16 + at;
-#pragma unroll
-        for (int i = 0; i < HD / 16; i++) {
-            const uint4 h = *reinterpret_cast<const uint4*>(src + i * 16);
-            q.x[i][0] = make_float4(__uint_as_float(h.x), __uint_as_float(h.y), __uint_as_float(h.z),
-                                    __uint_as_float(h.w));
+    for (int j = 0; j < Q::NI; j++) {
+        if (WR_PAIR_PROBE & 32) {
+            q.x[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+            continue;
         }
-    } else {
-        const float* src = a.q + at;
-#pragma unroll
-        for (int i = 0; i < HD / 16; i++) {
-            q.x[i][0] = *reinterpret_cast<const float4*>(src + i * 16);
-            q.x[i][1] = *reinterpret_cast<const float4*>(src + i * 16 + 4);
+        const int r = j * Q::RPI + lane / Q::LPR;
+        const uint32_t row = min(row0 + r, a.T - 1);      // idle rows re-read the last one
+        if constexpr (Q16) {
+            const size_t at = ((size_t)row * a.nq + head) * HD + (lane % Q::LPR) * 8;
+            const uint4 h = *reinterpret_cast<const uint4*>(a.q16 + at);
+            q.x[j] = make_float4(__uint_as_float(h.x), __uint_as_float(h.y), __uint_as_float(h.z),
+                                 __uint_as_float(h.w));
+        } else {
+            const size_t at = ((size_t)row * a.nq + head) * HD + (lane % Q::LPR) * 4;
+            q.x[j] = *reinterpret_cast<const float4*>(a.q + at);
         }
     }
 }
 
+// The rows of unit `unit` (this wave's index) scaled, rounded and written into
+// the staging image, [unit][row][HD + 8] halves.
 template <int HD, bool Q16>
-__device__ __forceinline__ void pair_convert_q(PrefillRows<HD>& R, PairQ<HD>& q, const PrefillArgs& a)
+__device__ __forceinline__ void pair_stage_q(PairQ<HD, Q16>& q, const PrefillArgs& a, unsigned char* smem, int unit,
+                                             int lane)
 {
-    if constexpr (Q16) {
+    using L = PairLds<HD>;
+    using Q = PairQ<HD, Q16>;
 #pragma unroll
-        for (int i = 0; i < HD / 16; i++) {
-            const u32x4 h = {__float_as_uint(q.x[i][0].x), __float_as_uint(q.x[i][0].y),
-                             __float_as_uint(q.x[i][0].z), __float_as_uint(q.x[i][0].w)};
-            R.qop[i] = pair_to_acc(__builtin_bit_cast(half8, h));
-            q.x[i][0] = make_float4(0.f, 0.f, 0.f, 0.f);  // consumed: nothing of it has to outlive the step loop
-        }
-    } else {
-#pragma unroll
-        for (int i = 0; i < HD / 16; i++) {
-            const half4 lo = q_scaled_f16(q.x[i][0], a.qscale), hi = q_scaled_f16(q.x[i][1], a.qscale);
-            R.qop[i] = pair_to_acc(half8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]});
-            q.x[i][0] = q.x[i][1] = make_float4(0.f, 0.f, 0.f, 0.f);
-        }
+    for (int j = 0; j < Q::NI; j++) {
+        const int r = j * Q::RPI + lane / Q::LPR;
+        unsigned char* at = smem + L::QS_OFF + (unit * 32 + r) * L::QS_ROW + (lane % Q::LPR) * (Q16 ? 16 : 8);
+        if constexpr (Q16)
+            *reinterpret_cast<float4*>(at) = q.x[j];
+        else
+            *reinterpret_cast<half4*>(at) = q_scaled_f16(q.x[j], a.qscale);
+        q.x[j] = make_float4(0.f, 0.f, 0.f, 0.f);          // consumed: nothing of it has to outlive the step loop
     }
+}
+
+// The Q^T operand of a unit out of the staging image: the lane's row, eight
+// consecutive dimensions per contraction step.
+template <int HD>
+__device__ __forceinline__ void pair_read_q(PrefillRows<HD>& R, const unsigned char* smem, int unit, int n, int g)
+{
+    using L = PairLds<HD>;
+#pragma unroll
+    for (int i = 0; i < HD / 16; i++)
+        R.qop[i] = pair_to_acc(*reinterpret_cast<const half8*>(smem + L::QS_OFF + (unit * 32 + n) * L::QS_ROW +
+                                                               (i * 16 + g * 8) * 2));
 }
 
 // The tile range of position block pb for key set kg, into the context.
@@ -455,23 +666,26 @@ __device__ __forceinline__ void pair_unit_ranges(PairUnit<HD>& U, const PairCtx<
 }
 
 // The copies and loads a block starts with: the first three K tiles and two Vt
-// blocks of the set into their ring slots, in order of need, and the wave's Q rows.
+// blocks of the set into their ring slots, in order of need, and the wave's share
+// of the Q rows.
 template <int HD, bool Q16>
-__device__ __forceinline__ void pair_first_loads(const PairCtx<HD>& cx, PairQ<HD> (&q)[2], const PrefillArgs& a,
-                                                 const uint32_t (&row0)[2], const uint32_t (&head)[2], int n, int g)
+__device__ __forceinline__ void pair_first_loads(const PairCtx<HD>& cx, PairQ<HD, Q16>& q, const PrefillArgs& a,
+                                                 uint32_t qrow0, uint32_t qhead, int lane)
 {
-    pair_load_q<HD, Q16>(q[0], a, row0[0], head[0], n, g);
     pair_issue_k<HD, 0>(cx, 0);
+    pair_load_q<HD, Q16>(q, a, qrow0, qhead, lane);
     pair_issue_v<HD, 0>(cx, 0);
-    pair_load_q<HD, Q16>(q[1], a, row0[1], head[1], n, g);
     pair_issue_k<HD, 1>(cx, 1);
     pair_issue_k<HD, 2>(cx, 2);
     pair_issue_v<HD, 1>(cx, 1);
 }
 
-// Unit `mine` of the pair is finished by this wave: its partial is merged with
-// the partner wave's (read from the partner's scratch), normalised and stored;
-// unit `theirs` went into this wave's scratch before the barrier.
+// End of a block.  The wave of key set s finishes unit s of its pair: the other
+// unit's partial goes into this wave's scratch for the partner (pair_send), and
+// after the barrier the partner's partial of this wave's unit is merged in,
+// normalised and stored (pair_finish).  The accumulators hold O[query][dim], so a
+// store instruction writes 128 contiguous bytes of two rows; the per-query
+// weights cross over from the score layout through 64 floats of LDS.
 template <int HD>
 __device__ __forceinline__ void pair_send(const PairUnit<HD>& U, unsigned char* smem, int wave, int lane)
 {
@@ -487,42 +701,61 @@ __device__ __forceinline__ void pair_send(const PairUnit<HD>& U, unsigned char* 
             // a few registers at a time: the next block's Q rows are in flight in the others
             __builtin_amdgcn_sched_barrier(0);
         }
-    float* ml = reinterpret_cast<float*>(smem + L::ML_OFF) + wave * 128;
+    float* ml = reinterpret_cast<float*>(smem + L::ML_OFF) + wave * L::ML_WAVE;
     ml[lane] = U.R.m_run;
     ml[64 + lane] = U.R.l_run;
 }
 
+template <int HD, bool GUARD>
+__device__ __forceinline__ void pair_finish_rows(PairUnit<HD>& U, const PrefillArgs& a, const f32x4* x,
+                                                 const float* wsc, int lane, int n, int g)
+{
+    PrefillRows<HD>& R = U.R;
+    const size_t rowstride = (size_t)a.nq * HD;
+    float* ob = a.out + ((size_t)min(U.row0 + 4 * g, a.T - 1) * a.nq + U.head) * HD + n;
+#pragma unroll
+    for (int q4 = 0; q4 < 4; q4++) {
+        const f32x4 w0v = *reinterpret_cast<const f32x4*>(wsc + 8 * q4 + 4 * g);
+        const f32x4 w1v = *reinterpret_cast<const f32x4*>(wsc + 32 + 8 * q4 + 4 * g);
+#pragma unroll
+        for (int dt = 0; dt < HD / 32; dt++) {
+            const f32x4 p = x[(dt * 4 + q4) * 64 + lane];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const float v = R.o[dt][4 * q4 + e] * w0v[e] + p[e] * w1v[e];
+                const uint32_t row = U.row0 + 8 * q4 + 4 * g + e;
+                if (!GUARD || row < a.T) ob[(size_t)(8 * q4 + e) * rowstride + dt * 32] = v;
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);                // a quarter of the registers at a time
+    }
+}
+
 template <int HD>
-__device__ __forceinline__ void pair_finish(PairUnit<HD>& U, const PrefillArgs& a, unsigned char* smem,
-                                            int partner, int lane, int n, int g)
+__device__ __forceinline__ void pair_finish(PairUnit<HD>& U, const PrefillArgs& a, unsigned char* smem, int wave,
+                                            int lane, int n, int g)
 {
     using L = PairLds<HD>;
     PrefillRows<HD>& R = U.R;
+    const int partner = wave ^ 2;
     const f32x4* x = reinterpret_cast<const f32x4*>(smem + L::X_OFF + partner * L::X_WAVE);
-    const float* ml = reinterpret_cast<const float*>(smem + L::ML_OFF) + partner * 128;
+    const float* ml = reinterpret_cast<const float*>(smem + L::ML_OFF) + partner * L::ML_WAVE;
     const float m1 = ml[lane], l1 = ml[64 + lane];
     const float m = fmaxf(R.m_run, m1);
     const float f0m = (R.m_run == -INFINITY) ? 0.f : fast_exp2(R.m_run - m);
     const float f1m = (m1 == -INFINITY) ? 0.f : fast_exp2(m1 - m);
     const float l_tot = wave_pair32_sum(R.l_run * f0m + l1 * f1m);
     const float inv = (l_tot > 0.f) ? 1.0f / l_tot : 0.f;
-    const float w0 = f0m * inv, w1 = f1m * inv;
-    const uint32_t my_row = U.row0 + n;
-    float* orow = a.out + ((size_t)min(my_row, a.T - 1) * a.nq + U.head) * HD + 4 * g;
-    const bool live = my_row < a.T;
-#pragma unroll
-    for (int dt = 0; dt < HD / 32; dt++)
-#pragma unroll
-        for (int q4 = 0; q4 < 4; q4++) {
-            const f32x4 p = x[(dt * 4 + q4) * 64 + lane];
-            float4 v;
-            v.x = R.o[dt][4 * q4 + 0] * w0 + p[0] * w1;
-            v.y = R.o[dt][4 * q4 + 1] * w0 + p[1] * w1;
-            v.z = R.o[dt][4 * q4 + 2] * w0 + p[2] * w1;
-            v.w = R.o[dt][4 * q4 + 3] * w0 + p[3] * w1;
-            if (live) *reinterpret_cast<float4*>(orow + dt * 32 + 8 * q4) = v;
-            if (q4 & 1) __builtin_amdgcn_sched_barrier(0);    // two lines of registers at a time
-        }
+    // the weights of query n, to where the lanes that hold its outputs read them
+    float* wsc = reinterpret_cast<float*>(smem + L::ML_OFF) + wave * L::ML_WAVE + 128;
+    if (g == 0) {
+        wsc[n] = f0m * inv;
+        wsc[32 + n] = f1m * inv;
+    }
+    if (U.row0 + 32 <= a.T)
+        pair_finish_rows<HD, false>(U, a, x, wsc, lane, n, g);
+    else
+        pair_finish_rows<HD, true>(U, a, x, wsc, lane, n, g);
 }
 
 // One position block.  started: the block's first loads are already on their way
@@ -532,7 +765,7 @@ __device__ __forceinline__ void pair_finish(PairUnit<HD>& U, const PrefillArgs& 
 template <int HD, bool Q16>
 __device__ __forceinline__ void pair_block(const PrefillArgs& a, unsigned char* smem, uint32_t pb, uint32_t kvh,
                                            uint32_t hc, const unsigned char* kbase, const unsigned char* vtbase,
-                                           bool started, PairQ<HD> (&q)[2], int next_pb)
+                                           bool started, PairQ<HD, Q16>& q, int next_pb)
 {
     using L = PairLds<HD>;
     const int tid = threadIdx.x;
@@ -602,16 +835,26 @@ __device__ __forceinline__ void pair_block(const PrefillArgs& a, unsigned char* 
     // fewer and spends its last step on probabilities of zero); the same in every wave
     const uint32_t nsteps = (t_last - t_first) / 2 + 1;
 
-    if (!started) pair_first_loads<HD, Q16>(cx, q, a, row0, head, n, g);
+#ifdef WR_PAIR_STAMPS
+    unsigned long long bt0, bt1, bt2, bt3, bt4, bt5;
+    WR_STAMP(bt0);
+#endif
+    // Q rows: wave w brings in unit w
+    const uint32_t qhead = (uint32_t)__builtin_amdgcn_readfirstlane(kvh * G + hc * Gw + ((uint32_t)wave % Gw));
+    const uint32_t qsub = (uint32_t)__builtin_amdgcn_readfirstlane(((uint32_t)wave / Gw) * 32);
+    if (!started) pair_first_loads<HD, Q16>(cx, q, a, pb * BP + qsub, qhead, lane);
+    WR_STAMP(bt1);
 
     f32x16 sa[2], sb[2];
     u32x4 pop[2][2];
     half8 kf[HD / 16], vf[HD / 16];
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    pair_convert_q<HD, Q16>(U[0].R, q[0], a);
-    pair_convert_q<HD, Q16>(U[1].R, q[1], a);
+    pair_stage_q<HD, Q16>(q, a, smem, wave, lane);
     pair_patch_tail<HD, 0>(smem, cx, 0, lane, kv_valid);
-    il_barrier();                                         // first tiles visible to all
+    il_barrier();                                         // first tiles and Q rows visible to all
+    WR_STAMP(bt2);
+    pair_read_q<HD>(U[0].R, smem, 2 * hp, n, g);
+    pair_read_q<HD>(U[1].R, smem, 2 * hp + 1, n, g);
     // scores of the set's first tile
 #pragma unroll
     for (int i = 0; i < HD / 16; i++) kf[i] = *reinterpret_cast<const half8*>(smem + cx.kop[i]);
@@ -628,9 +871,10 @@ __device__ __forceinline__ void pair_block(const PrefillArgs& a, unsigned char* 
     pair_issue_k<HD, 0>(cx, 3);
 #pragma unroll
     for (int i = 0; i < HD / 16; i++) kf[i] = *reinterpret_cast<const half8*>(smem + cx.kop[i] + L::KTILE);
-    pair_settle<HD>(U[0], cx, sa[0], 0, g);
-    pair_settle<HD>(U[1], cx, sa[1], 0, g);
+    pair_settle<HD>(U[0], cx, sa[0], 0, g, smem);
+    pair_settle<HD>(U[1], cx, sa[1], 0, g, smem);
     il_barrier();                                         // slot 1 of K has been read by all: step 0 refills it
+    WR_STAMP(bt3);
 
 #define WR_PAIR_STEP(PHASE, CUR, NXT)                                                  \
     pair_step<HD, PHASE>(U, cx, CUR, NXT, pop, kf, vf, smem, j, lane, g, kv_valid);    \
@@ -646,6 +890,7 @@ __device__ __forceinline__ void pair_block(const PrefillArgs& a, unsigned char* 
     }
 #undef WR_PAIR_STEP
 
+    WR_STAMP(bt4);
     // the ring must be quiet before anything else lands in it (the last steps'
     // copies still target it)
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -656,9 +901,19 @@ __device__ __forceinline__ void pair_block(const PrefillArgs& a, unsigned char* 
         PairCtx<HD> cn = cx;
         uint32_t nf, nl;
         pair_ctx_tiles<HD>(cn, a, (uint32_t)next_pb, BP, kg, nf, nl);
-        const uint32_t nrow0[2] = {(uint32_t)next_pb * BP + sub_rows[0], (uint32_t)next_pb * BP + sub_rows[1]};
-        pair_first_loads<HD, Q16>(cn, q, a, nrow0, head, n_e, g_e);
+        pair_first_loads<HD, Q16>(cn, q, a, (uint32_t)next_pb * BP + qsub, qhead, lane_e);
     }
+#ifdef WR_PAIR_STAMPS
+    if (WR_PAIR_PROBE & 64) {
+        WR_STAMP(bt5);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) {
+            const int b = started ? 1 : 0;
+            pair_stamp_blk[b][0] += bt1 - bt0; pair_stamp_blk[b][1] += bt2 - bt1; pair_stamp_blk[b][2] += bt3 - bt2;
+            pair_stamp_blk[b][3] += bt4 - bt3; pair_stamp_blk[b][4] += bt5 - bt4; pair_stamp_blk[b][5] += 1;
+        }
+    }
+#endif
     if (WR_PAIR_PROBE & 64) return;
     // the wave of key set s finishes unit s of its pair and hands the other one over
     if (kg == 0)
@@ -667,9 +922,18 @@ __device__ __forceinline__ void pair_block(const PrefillArgs& a, unsigned char* 
         pair_send<HD>(U[0], smem, wave, lane_e);
     lds_barrier();                                        // LDS traffic only: the next block's loads stay in flight
     if (kg == 0)
-        pair_finish<HD>(U[0], a, smem, wave ^ 2, lane_e, n_e, g_e);
+        pair_finish<HD>(U[0], a, smem, wave, lane_e, n_e, g_e);
     else
-        pair_finish<HD>(U[1], a, smem, wave ^ 2, lane_e, n_e, g_e);
+        pair_finish<HD>(U[1], a, smem, wave, lane_e, n_e, g_e);
+#ifdef WR_PAIR_STAMPS
+    WR_STAMP(bt5);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) {
+        const int b = started ? 1 : 0;
+        pair_stamp_blk[b][0] += bt1 - bt0; pair_stamp_blk[b][1] += bt2 - bt1; pair_stamp_blk[b][2] += bt3 - bt2;
+        pair_stamp_blk[b][3] += bt4 - bt3; pair_stamp_blk[b][4] += bt5 - bt4; pair_stamp_blk[b][5] += 1;
+    }
+#endif
 }
 
 // grid = (KV heads x head chunks, ceil(blocks / 2)): consecutive workgroups (which
@@ -694,7 +958,7 @@ __global__ __launch_bounds__(kPairThreads, 1) void prefill_pair_kernel(const Pre
         uniform_ptr(reinterpret_cast<const unsigned char*>(a.k + (size_t)kvh * a.ctx_pad * HD));
     const unsigned char* vtbase = uniform_ptr(reinterpret_cast<const unsigned char*>(
         a.vt + (size_t)kvh * (a.ctx_pad / kVBlock) * HD * kVBlock));
-    PairQ<HD> q[2];
+    PairQ<HD, Q16> q;
     if (a.single || hi == lo) {
         pair_block<HD, Q16>(a, prefill_smem_raw, hi, kvh, hc, kbase, vtbase, false, q, -1);
     } else {
