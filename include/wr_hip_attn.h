@@ -422,6 +422,14 @@ int wr_hip_rows_swiglu_dev(const float *gate_up_dev, uint32_t ld, float *act_dev
  * kernels.  Not needed by a normal caller. */
 void wr_hip_attn_set_tuning(uint32_t decode_keys_per_wg, int force_generic);
 
+/* Measurement knob without a counterpart in the reference: which of the two
+ * causal-prefill kernels head dim 128 takes.  0 (the default, also set by
+ * WR_HIP_PREFILL_TWO_WAVES unset or "1" at init): eight waves per workgroup,
+ * two per SIMD, one 32-row unit per wave.  1 (WR_HIP_PREFILL_TWO_WAVES=0): four
+ * waves, one per SIMD, two units per wave.  Same results to rounding; the
+ * second form is kept for comparison and is the slower one at present. */
+void wr_hip_attn_set_prefill_one_wave(int on);
+
 /* Kernel timing for the roofline figure.  Between profile_begin and
  * profile_end every launch of the MAIN kernel of a call (the split-K decode
  * kernel, or the prefill kernel; not the small combine / append kernels) is

@@ -232,6 +232,7 @@ int wr_hip_attn_prefill(wr_hip_kv *kv, uint32_t layer, uint32_t p0, uint32_t T, 
  * its own CPU walk when the answer is 0; they exist so the engine links. */
 uint32_t wr_hip_attn_caps(void) { return 0; }
 void wr_hip_attn_set_tuning(uint32_t keys_per_wg, int force_generic) { (void)keys_per_wg; (void)force_generic; }
+void wr_hip_attn_set_prefill_one_wave(int on) { (void)on; }
 void *wr_hip_attn_dev_alloc(size_t bytes) { (void)bytes; return NULL; }
 void wr_hip_attn_dev_free(void *p) { (void)p; }
 int wr_hip_attn_h2d(void *d, const void *s, size_t n) { (void)d; (void)s; (void)n; return WR_HIP_ERR_STATE; }

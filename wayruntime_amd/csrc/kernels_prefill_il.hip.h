@@ -344,15 +344,8 @@ __device__ __forceinline__ void il_step(PrefillRows<HD>& R, IlCtx<HD>& cx, f32x1
             // two exp2, one pack to F16, one dot product with (1, 1): the normaliser
             // is the sum of exactly the rounded values P.V multiplies
             const int r = 2 * (i * PAIRS + q);
-#ifdef WR_IL_ADDS
-            const float e0 = fast_exp2(cur[r]), e1 = fast_exp2(cur[r + 1]);
-            const half2v ph = {(_Float16)e0, (_Float16)e1};
-            psum += e0;
-            psum += e1;
-#else
             const half2v ph = {(_Float16)fast_exp2(cur[r]), (_Float16)fast_exp2(cur[r + 1])};
             psum = __builtin_amdgcn_fdot2(ph, ones, psum, false);
-#endif
             pop[r >> 3][(r & 7) >> 1] = __builtin_bit_cast(uint32_t, ph);
         }
         // every link keeps its own share of the vector work behind it (left to

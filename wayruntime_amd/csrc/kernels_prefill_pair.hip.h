@@ -50,23 +50,7 @@
 
 #include "kernels_prefill_il.hip.h"
 
-#ifndef WR_PAIR_PROBE
-#define WR_PAIR_PROBE 0
-#endif
-
 namespace wr {
-
-#ifdef WR_PAIR_STAMPS
-// timing build only: segment durations of the step loop, summed over the steps of
-// one wave (100 MHz ticks): chain, products, end of step, barrier; and the count
-__device__ unsigned long long pair_stamp_acc[8];
-__device__ unsigned long long pair_stamp_blk[2][8];
-// (the wait is part of the statement: the counter arrives like a load, and a
-// destination the compiler believes written at once may be reused before it is)
-#define WR_STAMP(v) asm volatile("s_memrealtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(v)::"memory")
-#else
-#define WR_STAMP(v)
-#endif
 
 constexpr int kPairThreads = 256;
 
@@ -449,38 +433,24 @@ __device__ __forceinline__ void pair_step(PairUnit<HD> (&U)[2], const PairCtx<HD
     // and waits for the matrix instruction in front of it, which a lone wave
     // cannot afford (measured: MFMA + 2 dot2c = 55 clocks, MFMA + 6 additions = 36).
     static_assert(PAIRS == 1, "slot blocks below are written for one pair of scores per link");
-#ifdef WR_PAIR_STAMPS
-    unsigned long long st_a, st_b, st_c, st_d, st_e;
-    WR_STAMP(st_a);
-#endif
     float psum[2] = {0.f, 0.f};
 #pragma unroll
     for (int i = 0; i < NS; i++) {
 #pragma unroll
         for (int u = 0; u < 2; u++) {
             const int r = 2 * i;
-            if (WR_PAIR_PROBE & 1) {
-                if (i == 0) nxt[u] = pair_mfma_first(kf[0], U[u].R.qop[0], U[u].negm);
-                else pair_mfma_link(nxt[u], kf[i], U[u].R.qop[i]);
-            } else if (i == 0)
+            if (i == 0)
                 pair_slot_chain_first(nxt[u], kf[0], U[u].R.qop[0], U[u].negm, cur[u], r, psum[u], pop[u][r >> 3],
                                       (r & 7) >> 1);
             else
                 pair_slot_chain(nxt[u], kf[i], U[u].R.qop[i], cur[u], r, psum[u], pop[u][r >> 3], (r & 7) >> 1);
-            if (u == 0 && !(WR_PAIR_PROBE & 8))
+            if (u == 0)
                 vf[i] = *reinterpret_cast<const half8*>(smem + cx.vop[i / ND] + VS * L::VTILE + (i % ND) * 2048);
-#ifdef WR_PAIR_EARLY_COPIES
-            if (u == 1 && !(WR_PAIR_PROBE & 2)) {
-                if (i < L::NLW) pair_issue_k1<HD, KC>(cx, j + 4, i);
-                else if (i < 2 * L::NLW) pair_issue_v1<HD, VC>(cx, j + 2, i - L::NLW);
-            }
-#endif
             __builtin_amdgcn_sched_barrier(0);
         }
     }
     U[0].R.l_run += psum[0];
     U[1].R.l_run += psum[1];
-    WR_STAMP(st_b);
     // The products, and in their shadows the K operand reads of tile j+2, the
     // step's copies and the settling of S(j+1).  The scores of tile j+1 are results
     // of hand-written matrix instructions: nothing may read them before two more
@@ -496,11 +466,9 @@ __device__ __forceinline__ void pair_step(PairUnit<HD> (&U)[2], const PairCtx<HD
         const half8 pp = __builtin_bit_cast(half8, pop[u][t]);
         if (s == S0 || s == S1) {
             const int w = (s == S0) ? 0 : 1;
-            if (!(WR_PAIR_PROBE & 16)) {
-                const uint32_t jt = j + 1;
-                if (__builtin_expect(jt < U[w].pl_lo || jt > U[w].pl_hi, 0))
-                    pair_mask_special<HD>(U[w], nxt[w], cx.t0 + 2 * jt, jt, g, 0.f);
-            }
+            const uint32_t jt = j + 1;
+            if (__builtin_expect(jt < U[w].pl_lo || jt > U[w].pl_hi, 0))
+                pair_mask_special<HD>(U[w], nxt[w], cx.t0 + 2 * jt, jt, g, 0.f);
             pair_slot_pv_max_a(U[u].R.o[dt], pp, vf[i], tmax[w], nxt[w]);
         } else if (s == S0 + 1 || s == S1 + 1) {
             const int w = (s == S0 + 1) ? 0 : 1;
@@ -518,42 +486,24 @@ __device__ __forceinline__ void pair_step(PairUnit<HD> (&U)[2], const PairCtx<HD
             pair_mfma_acc(U[u].R.o[dt], pp, vf[i]);
         }
         if (u == 0) {
-            if (!(WR_PAIR_PROBE & 8)) kf[i] = *reinterpret_cast<const half8*>(smem + cx.kop[i] + KS * L::KTILE);
-        }
-#ifndef WR_PAIR_EARLY_COPIES
-        else if (!(WR_PAIR_PROBE & 2)) {
+            kf[i] = *reinterpret_cast<const half8*>(smem + cx.kop[i] + KS * L::KTILE);
+        } else {
             if (i < L::NLW) pair_issue_k1<HD, KC>(cx, j + 4, i);
             else if (i < 2 * L::NLW) pair_issue_v1<HD, VC>(cx, j + 2, i - L::NLW);
         }
-#endif
         __builtin_amdgcn_sched_barrier(0);
     }
-    WR_STAMP(st_c);
-    if (!(WR_PAIR_PROBE & 16)) {
-        if (__builtin_expect((jumps[0] | jumps[1]) != 0, 0)) {
-            pair_settle_c<HD>(U[0], nxt[0], tmax[0], smem);
-            pair_settle_c<HD>(U[1], nxt[1], tmax[1], smem);
-        }
+    if (__builtin_expect((jumps[0] | jumps[1]) != 0, 0)) {
+        pair_settle_c<HD>(U[0], nxt[0], tmax[0], smem);
+        pair_settle_c<HD>(U[1], nxt[1], tmax[1], smem);
     }
     // all copies but this step's have landed: K of tile j+3 and Vt of tile j+1,
     // which the next step reads once the barrier has published them
-    if (!(WR_PAIR_PROBE & 2)) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * L::NLW) : "memory");
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * L::NLW) : "memory");
     pair_patch_tail<HD, TS>(smem, cx, j + 1, lane, kv_valid);
     __builtin_amdgcn_sched_barrier(0);
-    WR_STAMP(st_d);
-    if (!(WR_PAIR_PROBE & 4)) asm volatile("s_barrier" ::: "memory");
+    asm volatile("s_barrier" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
-#ifdef WR_PAIR_STAMPS
-    WR_STAMP(st_e);
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) {
-        pair_stamp_acc[0] += st_b - st_a;
-        pair_stamp_acc[1] += st_c - st_b;
-        pair_stamp_acc[2] += st_d - st_c;
-        pair_stamp_acc[3] += st_e - st_d;
-        pair_stamp_acc[4] += 1;
-    }
-#endif
 }
 
 // Q rows as read from global memory: wave w brings in the 32 rows of unit w with
@@ -574,10 +524,6 @@ __device__ __forceinline__ void pair_load_q(PairQ<HD, Q16>& q, const PrefillArgs
     using Q = PairQ<HD, Q16>;
 #pragma unroll
     for (int j = 0; j < Q::NI; j++) {
-        if (WR_PAIR_PROBE & 32) {
-            q.x[j] = make_float4(0.f, 0.f, 0.f, 0.f);
-            continue;
-        }
         const int r = j * Q::RPI + lane / Q::LPR;
         const uint32_t row = min(row0 + r, a.T - 1);      // idle rows re-read the last one
         if constexpr (Q16) {
@@ -835,15 +781,10 @@ __device__ __forceinline__ void pair_block(const PrefillArgs& a, unsigned char* 
     // fewer and spends its last step on probabilities of zero); the same in every wave
     const uint32_t nsteps = (t_last - t_first) / 2 + 1;
 
-#ifdef WR_PAIR_STAMPS
-    unsigned long long bt0, bt1, bt2, bt3, bt4, bt5;
-    WR_STAMP(bt0);
-#endif
     // Q rows: wave w brings in unit w
     const uint32_t qhead = (uint32_t)__builtin_amdgcn_readfirstlane(kvh * G + hc * Gw + ((uint32_t)wave % Gw));
     const uint32_t qsub = (uint32_t)__builtin_amdgcn_readfirstlane(((uint32_t)wave / Gw) * 32);
     if (!started) pair_first_loads<HD, Q16>(cx, q, a, pb * BP + qsub, qhead, lane);
-    WR_STAMP(bt1);
 
     f32x16 sa[2], sb[2];
     u32x4 pop[2][2];
@@ -852,7 +793,6 @@ __device__ __forceinline__ void pair_block(const PrefillArgs& a, unsigned char* 
     pair_stage_q<HD, Q16>(q, a, smem, wave, lane);
     pair_patch_tail<HD, 0>(smem, cx, 0, lane, kv_valid);
     il_barrier();                                         // first tiles and Q rows visible to all
-    WR_STAMP(bt2);
     pair_read_q<HD>(U[0].R, smem, 2 * hp, n, g);
     pair_read_q<HD>(U[1].R, smem, 2 * hp + 1, n, g);
     // scores of the set's first tile
@@ -874,7 +814,6 @@ __device__ __forceinline__ void pair_block(const PrefillArgs& a, unsigned char* 
     pair_settle<HD>(U[0], cx, sa[0], 0, g, smem);
     pair_settle<HD>(U[1], cx, sa[1], 0, g, smem);
     il_barrier();                                         // slot 1 of K has been read by all: step 0 refills it
-    WR_STAMP(bt3);
 
 #define WR_PAIR_STEP(PHASE, CUR, NXT)                                                  \
     pair_step<HD, PHASE>(U, cx, CUR, NXT, pop, kf, vf, smem, j, lane, g, kv_valid);    \
@@ -890,7 +829,6 @@ __device__ __forceinline__ void pair_block(const PrefillArgs& a, unsigned char* 
     }
 #undef WR_PAIR_STEP
 
-    WR_STAMP(bt4);
     // the ring must be quiet before anything else lands in it (the last steps'
     // copies still target it)
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -903,18 +841,6 @@ __device__ __forceinline__ void pair_block(const PrefillArgs& a, unsigned char* 
         pair_ctx_tiles<HD>(cn, a, (uint32_t)next_pb, BP, kg, nf, nl);
         pair_first_loads<HD, Q16>(cn, q, a, (uint32_t)next_pb * BP + qsub, qhead, lane_e);
     }
-#ifdef WR_PAIR_STAMPS
-    if (WR_PAIR_PROBE & 64) {
-        WR_STAMP(bt5);
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) {
-            const int b = started ? 1 : 0;
-            pair_stamp_blk[b][0] += bt1 - bt0; pair_stamp_blk[b][1] += bt2 - bt1; pair_stamp_blk[b][2] += bt3 - bt2;
-            pair_stamp_blk[b][3] += bt4 - bt3; pair_stamp_blk[b][4] += bt5 - bt4; pair_stamp_blk[b][5] += 1;
-        }
-    }
-#endif
-    if (WR_PAIR_PROBE & 64) return;
     // the wave of key set s finishes unit s of its pair and hands the other one over
     if (kg == 0)
         pair_send<HD>(U[1], smem, wave, lane_e);
@@ -925,15 +851,6 @@ __device__ __forceinline__ void pair_block(const PrefillArgs& a, unsigned char* 
         pair_finish<HD>(U[0], a, smem, wave, lane_e, n_e, g_e);
     else
         pair_finish<HD>(U[1], a, smem, wave, lane_e, n_e, g_e);
-#ifdef WR_PAIR_STAMPS
-    WR_STAMP(bt5);
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) {
-        const int b = started ? 1 : 0;
-        pair_stamp_blk[b][0] += bt1 - bt0; pair_stamp_blk[b][1] += bt2 - bt1; pair_stamp_blk[b][2] += bt3 - bt2;
-        pair_stamp_blk[b][3] += bt4 - bt3; pair_stamp_blk[b][4] += bt5 - bt4; pair_stamp_blk[b][5] += 1;
-    }
-#endif
 }
 
 // grid = (KV heads x head chunks, ceil(blocks / 2)): consecutive workgroups (which
@@ -959,12 +876,19 @@ __global__ __launch_bounds__(kPairThreads, 1) void prefill_pair_kernel(const Pre
     const unsigned char* vtbase = uniform_ptr(reinterpret_cast<const unsigned char*>(
         a.vt + (size_t)kvh * (a.ctx_pad / kVBlock) * HD * kVBlock));
     PairQ<HD, Q16> q;
-    if (a.single || hi == lo) {
-        pair_block<HD, Q16>(a, prefill_smem_raw, hi, kvh, hc, kbase, vtbase, false, q, -1);
-    } else {
-        pair_block<HD, Q16>(a, prefill_smem_raw, hi, kvh, hc, kbase, vtbase, false, q, (int)lo);
+    const bool two = !(a.single || hi == lo);
+    // one copy of the block's code for both blocks: the kernel's instructions
+    // have to come through an instruction cache two compute units share
+    uint32_t pb = hi;
+    bool started = false;
+#pragma unroll 1
+    for (int b = 0;; b++) {
+        const int next = (b == 0 && two) ? (int)lo : -1;
+        pair_block<HD, Q16>(a, prefill_smem_raw, pb, kvh, hc, kbase, vtbase, started, q, next);
+        if (next < 0) break;
         lds_barrier();                                    // LDS changes hands
-        pair_block<HD, Q16>(a, prefill_smem_raw, lo, kvh, hc, kbase, vtbase, true, q, -1);
+        pb = lo;
+        started = true;
     }
 }
 

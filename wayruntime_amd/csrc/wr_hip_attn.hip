@@ -117,7 +117,7 @@ struct Lib {
     void* log_user = nullptr;
     std::atomic<uint32_t> tune_keys_per_wg{0};
     std::atomic<int> force_generic{0};
-    int prefill_two_waves = 1;        // WR_HIP_PREFILL_TWO_WAVES=0: head dim 128 takes the one-wave-per-SIMD prefill kernel
+    std::atomic<int> prefill_two_waves{1};        // WR_HIP_PREFILL_TWO_WAVES=0: head dim 128 takes the one-wave-per-SIMD prefill kernel
 } g;
 
 // The calling thread's context (set by Entered, below).
@@ -1090,19 +1090,10 @@ const char* wr_hip_attn_device_name(void) { return g.name; }
 
 uint32_t wr_hip_attn_caps(void) { return WR_HIP_CAP_PROJ; }
 
-#ifdef WR_PAIR_STAMPS
-extern "C" int wr_hip_debug_pair_stamps(unsigned long long* out8, int reset)
+void wr_hip_attn_set_prefill_one_wave(int on)
 {
-    if (reset) {
-        unsigned long long z[16] = {0};
-        (void)hipMemcpyToSymbol(HIP_SYMBOL(wr::pair_stamp_blk), z, sizeof z);
-        return (int)hipMemcpyToSymbol(HIP_SYMBOL(wr::pair_stamp_acc), z, 64);
-    }
-    (void)hipDeviceSynchronize();
-    (void)hipMemcpyFromSymbol(out8 + 8, HIP_SYMBOL(wr::pair_stamp_blk), 128);
-    return (int)hipMemcpyFromSymbol(out8, HIP_SYMBOL(wr::pair_stamp_acc), 64);
+    g.prefill_two_waves = on ? 0 : 1;
 }
-#endif
 
 void wr_hip_attn_set_tuning(uint32_t decode_keys_per_wg, int force_generic)
 {

@@ -99,6 +99,7 @@ def load() -> C.CDLL:
         "wr_hip_attn_host_alloc": (_vp, [C.c_size_t]),
         "wr_hip_attn_host_free": (None, [_vp]),
         "wr_hip_attn_set_tuning": (None, [_u32, C.c_int]),
+        "wr_hip_attn_set_prefill_one_wave": (None, [C.c_int]),
         "wr_hip_attn_profile_begin": (C.c_int, [_u32]),
         "wr_hip_attn_profile_end": (C.c_int, [C.POINTER(C.c_double), C.POINTER(_u32)]),
     }
@@ -376,6 +377,10 @@ def sync() -> None:
 
 def set_tuning(decode_keys_per_wg: int = 0, force_generic: bool = False) -> None:
     lib().wr_hip_attn_set_tuning(decode_keys_per_wg, 1 if force_generic else 0)
+
+
+def set_prefill_one_wave(on: bool) -> None:
+    lib().wr_hip_attn_set_prefill_one_wave(1 if on else 0)
 
 
 def profile_begin(max_launches: int) -> None:
