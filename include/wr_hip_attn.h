@@ -206,7 +206,10 @@ int wr_hip_attn_rope_dev(void *x_dev, const void *cos_sin_dev, uint32_t rows,
  * stands for 10000 (the angle of wri_op_rope, src/core/kernels.c:1384-1404,
  * through the polynomials and the range reduction of src/core/mathx.c:37-57,
  * :72-86 and :112-147 operation for operation: the bytes equal what the
- * reference computes per element).  Asynchronous on the stream. */
+ * reference computes per element).  Every position must lie below
+ * WR_HIP_ATTN_MAX_SEQ (the bound of the reference's callers; the range
+ * reduction's loop does not end for angles beyond 2^27): WR_HIP_ERR_LIMIT
+ * otherwise, before anything is launched.  Asynchronous on the stream. */
 int wr_hip_attn_rope_table_dev(float *cos_sin_dev, uint32_t rows, uint32_t pos0,
                                const uint32_t *pos, uint32_t hd,
                                float theta_base, uint32_t n_rot_pairs);
@@ -256,14 +259,20 @@ int wr_hip_attn_append_decode_batched_dev(uint32_t n, wr_hip_kv *const *kv,
                                           uint32_t window);
 
 /* wr_hip_attn_decode_batched_dev for callers that cannot allocate device
- * memory (code under HIP graph capture, tight serving loops, harnesses that
- * forbid hipMalloc).  It has no counterpart in the reference.  Same arguments,
- * same kernels and the same results bit for bit; the difference is where the
- * split-K tickets and partial rows live: in a fixed array of
+ * memory while they run (tight serving loops with a fixed memory budget,
+ * harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * Same arguments, same kernels and the same results bit for bit; the difference
+ * is where the split-K tickets and partial rows live: in a fixed array of
  * WR_HIP_NOALLOC_SCRATCH_BYTES that is part of the library's device image
  * (every device the library runs on holds it until the process ends) instead
  * of a buffer the library grows on demand.  The call makes no hipMalloc,
- * hipFree or other allocating call.  Limits: nq <= WR_HIP_NOALLOC_MAX_HEADS,
+ * hipFree or other allocating call.  A thread's FIRST call into the library
+ * creates that thread's stream and staging buffers, which does allocate: this
+ * entry point refuses to be that call (WR_HIP_ERR_STATE; any other entry point,
+ * wr_hip_attn_sync for one, from the same thread beforehand is enough).  The
+ * launch goes to the library's own stream of the calling thread, like every
+ * other *_dev call, so it is not something a caller's stream capture records.
+ * Limits: nq <= WR_HIP_NOALLOC_MAX_HEADS,
  * and n * nq * max_splits * (hd + 2) * 4 bytes of partials must fit the array
  * behind its first 64 KiB (with the automatic split rule a session has at most
  * 18 key splits: 16 sessions of 32 heads x 128 need 4.8 MB); beyond either,
@@ -271,8 +280,7 @@ int wr_hip_attn_append_decode_batched_dev(uint32_t n, wr_hip_kv *const *kv,
  * array: the library runs them one after the other, also when they come from
  * different threads (each launch waits for an event the previous one
  * recorded), but a caller must not let two of them overlap on one device by
- * other means (two processes' worth of streams replaying captured launches,
- * say): they would race. */
+ * other means (two processes on one device, say): they would race. */
 #define WR_HIP_NOALLOC_SCRATCH_BYTES (20u * 1024u * 1024u)
 #define WR_HIP_NOALLOC_MAX_HEADS     1024u
 int wr_hip_attn_decode_batched_dev_noalloc(uint32_t n, wr_hip_kv *const *kv,

@@ -524,6 +524,59 @@ def test_append_and_decode_in_one_launch_equals_the_two_calls(nq, nkv, norm, rot
             b.free()
 
 
+def test_append_and_decode_in_one_launch_with_sixteen_short_sessions_paired_splits():
+    # Sixteen sessions of 500 to 640 keys at the Llama shape: a launch that fills
+    # the device, so a workgroup of a short session takes two consecutive splits,
+    # and the one that makes the new row runs a body split followed by the tail
+    # split.  Same output bits and cache bytes as the two-call path, and the oracle.
+    import ctypes as C
+    nq, nkv, hd, eps, theta, n = 32, 8, 128, 1e-6, 5e5, 16
+    lib = hipattn.lib()
+    pos = [500 + 9 * i + (i % 3) for i in range(n)]           # 500 .. 637, on both sides of tile edges
+    cap = 700
+    width = (nq + 2 * nkv) * hd
+    twins = []
+    for i in range(n):
+        _a, _b, k16, v16 = util.make_kv(9800 + 2 * i, cap, nkv, hd)
+        pair = []
+        for _ in range(2):
+            kv = hipattn.KVCache(1, hd, nkv, cap)
+            kv.write_f16(0, 0, k16, v16)
+            pair.append(kv)
+        twins.append(pair)
+    x = synth.normal(9850, (n, width), std=1.5)
+    xd = hipattn.DeviceBuffer.from_host(x)
+    td = hipattn.DeviceBuffer.from_host(np.concatenate([oracle.rope_table(1, hd, p, theta, 0) for p in pos]))
+    pp = (C.c_uint32 * n)(*pos)
+    sk = (C.c_uint32 * n)(*[p + 1 for p in pos])
+    kv_a = (C.c_void_p * n)(*[t[0].h for t in twins])
+    kv_b = (C.c_void_p * n)(*[t[1].h for t in twins])
+    q_dev = hipattn.DeviceBuffer(n * nq * hd * 4)
+    o_a = hipattn.DeviceBuffer.from_host(np.full((n, nq, hd), 3.0, dtype=np.float32))
+    o_b = hipattn.DeviceBuffer.from_host(np.full((n, nq, hd), -4.0, dtype=np.float32))
+    assert lib.wr_hip_rows_qkv_append_dev(xd.p, width, n, nq, None, None, eps, td.p, hd // 2, n, kv_a, 0, pp,
+                                          q_dev.p, 0) == hipattn.OK
+    assert lib.wr_hip_attn_decode_batched_dev(n, kv_a, 0, sk, q_dev.p, o_a.p, nq, 0.0, 0) == hipattn.OK
+    assert lib.wr_hip_attn_append_decode_batched_dev(n, kv_b, 0, pp, xd.p, width, nq, None, None, eps, td.p, hd // 2,
+                                                     o_b.p, 0.0, 0) == hipattn.OK
+    hipattn.sync()
+    got_a, got_b = o_a.to_host((n, nq, hd)), o_b.to_host((n, nq, hd))
+    differ = [(i, pos[i], float(np.abs(got_a[i] - got_b[i]).max())) for i in range(n)
+              if not np.array_equal(got_a[i], got_b[i])]
+    assert differ == [], f"outputs differ from the two-call path: (session, position, max diff) {differ}"
+    qh = q_dev.to_host((n, nq, hd))
+    for i in range(n):
+        ka, va = twins[i][0].read_f16(0, 0, pos[i] + 1)
+        kb, vb = twins[i][1].read_f16(0, 0, pos[i] + 1)
+        assert np.array_equal(ka, kb) and np.array_equal(va, vb), f"cache of session {i} differs"
+        util.assert_close(got_b[i], util.oracle_decode(qh[i], ka, va, pos[i] + 1, 0.0, 0), f"session {i}")
+    for b in (xd, td, q_dev, o_a, o_b):
+        b.free()
+    for pair in twins:
+        for kv in pair:
+            kv.close()
+
+
 def test_append_and_decode_in_one_launch_refuses_what_it_must():
     # argument contract of wr_hip_attn_append_decode_batched_dev: pointers, counts,
     # head shapes and strides are checked before anything is counted or written

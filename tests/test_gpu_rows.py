@@ -319,3 +319,55 @@ def test_rope_table_on_device_listed_positions():
     assert lib.wr_hip_attn_rope_table_dev(None, 1, 0, None, 128, 1e6, 0) == hipattn.ERR_INVAL
     assert lib.wr_hip_attn_rope_table_dev(buf.p, 0, 0, None, 128, 1e6, 0) == hipattn.ERR_INVAL
     buf.free()
+
+
+def test_rope_table_on_device_refuses_positions_beyond_the_sequence_limit():
+    # The range reduction subtracts 2 pi in a loop that does not end for angles
+    # beyond 2^27: the entry point takes positions below WR_HIP_ATTN_MAX_SEQ only
+    # and refuses the rest before any kernel runs (nothing is launched here).
+    import ctypes as C
+    lib = hipattn.lib()
+    buf = hipattn.DeviceBuffer.from_host(np.full((4, 64, 2), 9.0, dtype=np.float32))
+    lim = hipattn.ATTN_MAX_SEQ
+    assert lib.wr_hip_attn_rope_table_dev(buf.p, 4, lim - 3, None, 128, 1e6, 0) == hipattn.ERR_LIMIT
+    assert lib.wr_hip_attn_rope_table_dev(buf.p, 1, 2 ** 31, None, 128, 1e6, 0) == hipattn.ERR_LIMIT
+    assert lib.wr_hip_attn_rope_table_dev(buf.p, 4, 2 ** 32 - 2, None, 128, 1e6, 0) == hipattn.ERR_LIMIT
+    plist = (C.c_uint32 * 3)(5, lim, 7)
+    assert lib.wr_hip_attn_rope_table_dev(buf.p, 3, 0, plist, 128, 1e6, 0) == hipattn.ERR_LIMIT
+    plist = (C.c_uint32 * 2)(2 ** 32 - 1, 1)
+    assert lib.wr_hip_attn_rope_table_dev(buf.p, 2, 0, plist, 128, 1e6, 0) == hipattn.ERR_LIMIT
+    hipattn.sync()
+    assert np.all(buf.to_host((4, 64, 2)) == 9.0)            # nothing written
+    # the last positions inside the limit are served
+    got = hipattn.rope_table_dev(2, 128, 1e6, 0, pos0=lim - 2)
+    assert np.isfinite(got).all()
+    buf.free()
+
+
+def test_row_step_without_rotation_ignores_the_table_pointer():
+    # n_rot = 0 with a table pointer given: the eight-lane path must not read a
+    # table that holds zero pairs per row (head dim 128, aligned operands)
+    import ctypes as C
+    lib = hipattn.lib()
+    nq, nkv, hd, rows = 16, 8, 128, 40
+    width = (nq + 2 * nkv) * hd
+    x = synth.normal(8700, (rows, width))
+    xd = hipattn.DeviceBuffer.from_host(x)
+    tiny = hipattn.DeviceBuffer.from_host(np.zeros(4, dtype=np.float32))   # far smaller than a table would be
+    outs = []
+    for tab in (tiny.p, None):
+        kv = hipattn.KVCache(1, hd, nkv, rows)
+        q = hipattn.DeviceBuffer.from_host(np.full((rows, nq, hd), 2.0, dtype=np.float32))
+        kvs = (C.c_void_p * 1)(kv.h)
+        pos = (C.c_uint32 * 1)(0)
+        assert lib.wr_hip_rows_qkv_append_dev(xd.p, width, rows, nq, None, None, 1e-6, tab, 0, 1, kvs, 0, pos,
+                                              q.p, 0) == hipattn.OK
+        hipattn.sync()
+        outs.append((q.to_host((rows, nq, hd)),) + tuple(kv.read_f16(0, 0, rows)))
+        q.free()
+        kv.close()
+    for a, b in zip(outs[0], outs[1]):
+        assert np.array_equal(a, b)
+    assert np.array_equal(outs[0][0], x[:, :nq * hd].reshape(rows, nq, hd))   # Q passes through unrotated
+    xd.free()
+    tiny.free()

@@ -244,3 +244,43 @@ def test_no_alloc_decode_from_several_threads_shares_the_one_array():
         for caches, _ in groups:
             for kv in caches:
                 kv.close()
+
+
+def test_no_alloc_decode_refuses_to_be_a_threads_first_library_call():
+    # A thread's first call into the library creates its stream and staging
+    # buffers (that allocates); the no-alloc entry point must not be that call:
+    # WR_HIP_ERR_STATE, nothing launched, the output untouched.  After any other
+    # call from the same thread it runs and equals the ordinary entry point.
+    import threading
+    nq, nkv, hd = 16, 8, 128
+    ctxs = [700, 130]
+    caches, _ = _sessions(7950, ctxs, nkv, hd)
+    q = synth.normal(7951, (len(ctxs), nq, hd))
+    q_dev = hipattn.DeviceBuffer.from_host(q)
+    o_ref = hipattn.DeviceBuffer(q.nbytes)
+    o_new = hipattn.DeviceBuffer.from_host(np.full(q.shape, 5.0, dtype=np.float32))
+    hipattn.decode_batched_dev(caches, 0, ctxs, q_dev, o_ref, nq)
+    hipattn.sync()
+    want = o_ref.to_host(q.shape)
+    seen = {}
+
+    def job():
+        try:
+            seen["first"] = hipattn.decode_batched_dev_noalloc(caches, 0, ctxs, q_dev, o_new, nq)
+            hipattn.sync()                                    # this thread's context is made here
+            seen["untouched"] = bool((o_new.to_host(q.shape) == 5.0).all())
+            seen["second"] = hipattn.decode_batched_dev_noalloc(caches, 0, ctxs, q_dev, o_new, nq)
+            hipattn.sync()
+            seen["equal"] = bool(np.array_equal(o_new.to_host(q.shape), want))
+        except Exception as e:                                # noqa: BLE001
+            seen["error"] = repr(e)
+    th = threading.Thread(target=job)
+    th.start()
+    th.join()
+    try:
+        assert seen == {"first": hipattn.ERR_STATE, "untouched": True, "second": hipattn.OK, "equal": True}, seen
+    finally:
+        for b in (q_dev, o_ref, o_new):
+            b.free()
+        for kv in caches:
+            kv.close()

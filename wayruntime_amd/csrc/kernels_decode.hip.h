@@ -61,7 +61,9 @@ struct DecodeSession {
     uint32_t n_splits;       // workgroups along the key axis
     uint32_t tiles_per_wg;   // 32-key tiles per workgroup (a function of this session only)
     uint16_t tail_tiles;     // the session's last tiles that form the last split on their own (0: none)
-    uint16_t parts_per_wg;   // consecutive splits one workgroup works through (1 or 2; 1 with a tail)
+    uint16_t parts_per_wg;   // consecutive splits one workgroup works through (1 or 2: in a launch that fills
+                             // the device a short session's workgroups take two, and the last of them then
+                             // runs a body split followed by the tail split)
 };
 
 struct DecodeArgs {

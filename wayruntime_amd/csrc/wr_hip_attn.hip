@@ -98,10 +98,10 @@ struct Ctx {
 
 struct Lib {
     std::mutex mu;               // init / shutdown, the set of thread contexts, the knobs
-    bool inited = false;
+    std::atomic<bool> inited{false};   // read without the lock by every entry point
     int device = -1;
     uint32_t n_cus = 256;        // compute units of the device in use
-    uint64_t generation = 0;     // bumped by every init: contexts of an earlier one are gone
+    std::atomic<uint64_t> generation{0};   // bumped by every init: contexts of an earlier one are gone
     std::vector<Ctx*> ctxs;      // every context of this generation
     std::vector<Ctx*> idle;      // contexts whose thread has ended, for the next new thread
     char name[320] = "uninitialised";
@@ -1239,7 +1239,14 @@ int wr_hip_attn_rope_table_dev(float* cos_sin_dev, uint32_t rows, uint32_t pos0,
     if (!cos_sin_dev || rows == 0) return WR_HIP_ERR_INVAL;
     if (hd < 2 || (hd & 1)) return WR_HIP_ERR_INVAL;
     if (pos && rows > WR_HIP_BATCH_MAX) return WR_HIP_ERR_INVAL;
-    if (!pos && (uint64_t)pos0 + rows > (1ull << 32)) return WR_HIP_ERR_INVAL;
+    // The kernel folds an angle into [-pi, pi] by subtracting 2 pi in a loop, as
+    // the reference does (src/core/mathx.c:112-147); from an angle of 2^27 on a
+    // float's spacing exceeds 2 pi, the subtraction rounds back to itself and the
+    // loop never ends.  The reference's callers stay below WR_ATTN_MAX_SEQ: the
+    // same bound here, before anything is launched.
+    if (!pos && (uint64_t)pos0 + rows > WR_HIP_ATTN_MAX_SEQ) return WR_HIP_ERR_LIMIT;
+    for (uint32_t i = 0; pos && i < rows; i++)
+        if (pos[i] >= WR_HIP_ATTN_MAX_SEQ) return WR_HIP_ERR_LIMIT;
     RopeTableArgs a{};
     a.out = cos_sin_dev;
     a.rows = rows;
@@ -1376,6 +1383,14 @@ int wr_hip_attn_decode_batched_dev_noalloc(uint32_t n, wr_hip_kv* const* kv, uin
         logmsg(0, "decode (no-alloc form): %u query heads exceed the %u the fixed ticket array holds",
                nq, kNoAllocMaxHeads);
         return WR_HIP_ERR_LIMIT;
+    }
+    // A thread's first call into the library makes its stream and staging
+    // buffers (hipStreamCreate, hipMalloc, hipHostMalloc): that call cannot be
+    // this one.  Any other entry point (wr_hip_attn_sync is enough) does it.
+    if (!t_slot.c || t_slot.generation != g.generation) {
+        logmsg(0, "decode (no-alloc form): the calling thread has no stream context yet; "
+                  "make one other library call from it first (wr_hip_attn_sync will do)");
+        return WR_HIP_ERR_STATE;
     }
     ENTER();
     DecodeWorkspace fixed;
@@ -1836,7 +1851,7 @@ static int qkv_append_common(const float* qkv_dev, uint32_t ld, uint32_t rows, u
     a.qkv = qkv_dev;
     a.q_norm = q_norm_dev;
     a.k_norm = k_norm_dev;
-    a.cos_sin = cos_sin_dev;
+    a.cos_sin = n_rot ? cos_sin_dev : nullptr;           // a table of zero pairs per row holds nothing to read
     a.q_out = q_out_dev;
     a.ld = ld;
     a.nq = nq;

@@ -399,7 +399,12 @@ wr_status wrh_forward_rows_device(wr_model *m, wrh_workspace *hs, wrh_devspace *
             rc = wr_hip_attn_append_decode_batched_dev(R, kvs, ksrc, at, ds->qkv, width, nq, dl->q_norm, dl->k_norm,
                                                        m->rms_eps, tab, nr, ds->attn, scale, window);
             if (rc == WR_HIP_ERR_UNSUPPORTED) {
-                __atomic_store_n(&m->dev->step_in_one_launch, -1, __ATOMIC_RELAXED);
+                /* remembered for the model (the refusal is about its shapes as a
+                 * rule); said once, because the step is slower from here on */
+                if (__atomic_exchange_n(&m->dev->step_in_one_launch, -1, __ATOMIC_RELAXED) != -1)
+                    wrh_logf(e, 1, "device layers: the decode step's row is not made inside the attention launch "
+                                   "(shape or alignment not taken, or generic kernels forced): two launches per "
+                                   "layer from here on");
             } else {
                 if (rc != WR_HIP_OK) return dev_fail(e, "kv append + gqa", L, rc);
                 __atomic_store_n(&m->dev->step_in_one_launch, 1, __ATOMIC_RELAXED);
@@ -436,7 +441,9 @@ wr_status wrh_forward_rows_device(wr_model *m, wrh_workspace *hs, wrh_devspace *
                                                                shared ? NULL : dl->k_norm, m->rms_eps, tab, nr, 1,
                                                                one, ksrc, &pos0, (uint16_t *)ds->q, scale, flags);
                 if (r16 == WR_HIP_ERR_UNSUPPORTED) {
-                    __atomic_store_n(&m->dev->prefill_q16, -1, __ATOMIC_RELAXED);
+                    if (__atomic_exchange_n(&m->dev->prefill_q16, -1, __ATOMIC_RELAXED) != -1)
+                        wrh_logf(e, 1, "device layers: prompt rows keep F32 query rows (the binary16 form does not "
+                                       "take this shape or alignment, or generic kernels are forced)");
                 } else {
                     if (r16 != WR_HIP_OK) return dev_fail(e, "qkv split + kv append", L, r16);
                     q16 = 1;
