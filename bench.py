@@ -283,7 +283,7 @@ def main() -> None:
         qp = synth.normal(synth.config_seed(4, 1), (T, nq, hd))
         qp_dev = hipattn.DeviceBuffer.from_host(qp)
         op_dev = hipattn.DeviceBuffer(qp.nbytes)
-        reps = 5
+        reps = 60                                          # whatever --steps says: a stable mean
         hipattn.prefill_dev(caches[0], 0, 0, T, qp_dev, op_dev, nq)
         hipattn.profile_begin(reps)
         for _ in range(reps):
@@ -319,6 +319,23 @@ def main() -> None:
         prefill["q16_dev"] = {"ms": round(q_avg, 4), "tflops": round(flops / (q_avg * 1e-3) / 1e12, 2),
                               "frac_of_f16_mfma_peak": round(flops / (q_avg * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
                               "same_bits_as_f32_rows": bool(got16.tobytes() == gotp.tobytes())}
+        # the other kernel for this head dim (one wave per SIMD, two units per wave),
+        # kept for comparison: same workload, F32 rows
+        hipattn.set_prefill_one_wave(True)
+        try:
+            hipattn.prefill_dev(caches[0], 0, 0, T, qp_dev, op_dev, nq)
+            hipattn.profile_begin(reps)
+            for _ in range(reps):
+                hipattn.prefill_dev(caches[0], 0, 0, T, qp_dev, op_dev, nq)
+            wms, wn = hipattn.profile_end()
+            w_avg = wms / max(wn, 1)
+            goto = op_dev.to_host((T, nq, hd))
+            prefill["one_wave_kernel"] = {
+                "ms": round(w_avg, 4), "tflops": round(flops / (w_avg * 1e-3) / 1e12, 2),
+                "frac_of_f16_mfma_peak": round(flops / (w_avg * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
+                "max_abs_err_sampled_rows": float(np.max(np.abs(goto[rows] - wantp[rows])))}
+        finally:
+            hipattn.set_prefill_one_wave(False)
         q16_dev.free()
         o16_dev.free()
         qp_dev.free()
@@ -336,8 +353,9 @@ def main() -> None:
             oq_dev = hipattn.DeviceBuffer.from_host(oq)
             oo_dev = hipattn.DeviceBuffer(oq.nbytes)
             hipattn.prefill_dev(okv, 0, 0, oT, oq_dev, oo_dev, onq)
-            hipattn.profile_begin(reps)
-            for _ in range(reps):
+            oreps = 50
+            hipattn.profile_begin(oreps)
+            for _ in range(oreps):
                 hipattn.prefill_dev(okv, 0, 0, oT, oq_dev, oo_dev, onq)
             oms, on = hipattn.profile_end()
             o_avg = oms / max(on, 1)

@@ -138,3 +138,49 @@ def test_long_sessions_at_head_dim_64_keep_their_bits_too():
         assert np.array_equal(single, outs[i]), f"session {i} alone"
     for kv in caches:
         kv.close()
+
+
+def test_sixteen_sessions_with_the_whole_models_cache_footprint():
+    # The cache of the long-context workload's model as a serving process holds it
+    # (src/core/session.c:640-733): Llama-3-8B geometry, 32 layers x 8 KV heads x
+    # head_dim 128 at 32768 positions = 4 GiB per session, 16 sessions = 64 GiB of
+    # ordinary device allocations on one 288 GB device.  Appends and decode calls
+    # on the first and the last layer of the first and the last session against the
+    # CPU oracle at a short cursor, the byte count of every slab, then everything
+    # is destroyed and allocated once more (a leak of 64 GiB per round would not
+    # fit a third time; no allocation here runs the device out of memory).
+    layers, nq, nkv, hd, ctx, n = 32, 32, 8, 128, 32768, 16
+    per_session = 2 * layers * nkv * ctx * hd * 2
+    assert per_session == 4 << 30
+    for round_ in range(2):
+        caches = [hipattn.KVCache(layers, hd, nkv, ctx) for _ in range(n)]
+        try:
+            total = sum(c.bytes for c in caches)
+            print("footprint round %d: %d sessions, %.1f GiB" % (round_, n, total / 2.0 ** 30), flush=True)
+            assert all(c.bytes >= per_session for c in caches)
+            assert total < 1.02 * n * per_session            # alignment only, no hidden copies
+            rows = 77
+            for si in (0, n - 1):
+                for layer in (0, layers - 1):
+                    seed = synth.config_seed(5, 9000 + 100 * round_ + 10 * si + layer)
+                    k32 = synth.normal(seed, (rows, nkv, hd))
+                    v32 = synth.normal(seed + 1, (rows, nkv, hd))
+                    q = synth.normal(seed + 2, (nq, hd))
+                    assert caches[si].append(layer, 0, k32, v32) == hipattn.OK
+                    got = caches[si].decode(layer, rows, q)
+                    k16, v16 = synth.f32_to_f16_trunc(k32), synth.f32_to_f16_trunc(v32)
+                    util.assert_close(got, util.oracle_decode(q, k16, v16, rows), f"session {si} layer {layer}")
+                    kb, vb = caches[si].read_f16(layer, 0, rows)
+                    assert np.array_equal(kb, k16) and np.array_equal(vb, v16)
+            # the slabs are zero-filled at creation: an untouched layer of an untouched
+            # session reads back zeros, also at the far end of the context
+            kz, vz = caches[5].read_f16(17, ctx - 64, 64)
+            assert not kz.any() and not vz.any()
+            # the two sessions in one batched launch, last layer
+            qs = [synth.normal(synth.config_seed(5, 9900 + i), (nq, hd)) for i in range(2)]
+            outs = hipattn.decode_batched([caches[0], caches[n - 1]], layers - 1, [rows, rows], qs)
+            for o, c, qq in zip(outs, (caches[0], caches[n - 1]), qs):
+                assert np.array_equal(o, c.decode(layers - 1, rows, qq))
+        finally:
+            for c in caches:
+                c.close()

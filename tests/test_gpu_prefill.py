@@ -51,7 +51,10 @@ def _setup(nq, nkv, hd, p0, T, seed, theta=None, extra_rows=0):
 ])
 def test_prefill_matches_serial_stepping_oracle(nq, nkv, hd, p0, T, win):
     print("prefill", nq, nkv, hd, p0, T, win, flush=True)
-    kv, q, k16, v16 = _setup(nq, nkv, hd, p0, T, seed=1000 + T + p0)
+    # the two workload shapes at T = 512 take their inputs after RoPE, as the
+    # workload says (base 1e6 for the Qwen3 shape, 5e5 for the Llama-3 shape)
+    theta = {(16, 512): 1e6, (32, 512): 5e5}.get((nq, T)) if (hd == 128 and p0 == 0 and win == 0) else None
+    kv, q, k16, v16 = _setup(nq, nkv, hd, p0, T, seed=1000 + T + p0, theta=theta)
     got = kv.prefill(0, p0, q, 0.0, win)
     want = oracle.causal_prefill(q, k16, v16, p0=p0, window=win, threads=8)
     print("  errors", util.assert_close(got, want), flush=True)
@@ -140,6 +143,7 @@ def test_prefill_workload_sizes_after_rope_sampled_rows(nq, nkv, theta, T, hd):
     (32, 8, 5e5, 2048),             # Llama-3: the paired-block launch form
     (16, 8, 1e6, 2048),             # Qwen3: the one-block-per-workgroup form
     (16, 8, 1e6, 4096),             # Qwen3 at the longest chunk of the workload
+    (32, 8, 5e5, 4096),             # Llama-3 at the longest chunk: two rounds of paired workgroups
 ])
 def test_prefill_workload_sizes_after_rope_every_row(nq, nkv, theta, T):
     # the prefill workload at full size with EVERY row checked against the serial
