@@ -563,8 +563,53 @@ def main() -> None:
             last = [ln for ln in res.stdout.splitlines() if ln.startswith("{")]
             e2e = json.loads(last[-1]) if res.returncode == 0 and last else {
                 "error": "exit %d: %s" % (res.returncode, (res.stderr or res.stdout)[-200:])}
+            # the same model on the host walk: the host does the layer, the library
+            # only the cache append and the attention (what a reference build with
+            # this library behind its two call sites does per layer)
+            if "error" not in e2e:
+                res = subprocess.run([sys.executable, "-m", "wayruntime_amd.e2e_timing", "--json", "--host",
+                                      "--prompt", "511", "--reps", "1"],
+                                     cwd=ROOT, capture_output=True, text=True, timeout=240)
+                last = [ln for ln in res.stdout.splitlines() if ln.startswith("{")]
+                if res.returncode == 0 and last:
+                    hw = json.loads(last[-1])
+                    for key in ("decode_ms_per_token", "batch16_ms_per_step", "prefill_511_ms"):
+                        e2e["host_walk_" + key] = hw.get(key)
+                else:
+                    e2e["host_walk_error"] = "exit %d: %s" % (res.returncode, (res.stderr or res.stdout)[-200:])
         except Exception as exc:                      # timeout, missing model space, ...
-            e2e = {"error": repr(exc)[:200]}
+            e2e = e2e if isinstance(e2e, dict) else {}
+            e2e["error"] = repr(exc)[:200]
+
+    # ---- what the two call sites cost a host-resident caller per layer of a decode
+    # step (Qwen3 head shape, context 520): cache append then attention as two
+    # synchronous calls, and the one call that does both
+    if isinstance(e2e, dict):
+        try:
+            hkv = hipattn.KVCache(1, 128, 8, 1024)
+            hkv.append(0, 0, synth.normal(11, (520, 8, 128)), synth.normal(12, (520, 8, 128)))
+            hk, hv, hq = synth.normal(13, (8, 128)), synth.normal(14, (8, 128)), synth.normal(15, (16, 128))
+            hout = np.empty_like(hq)
+            hlib = hipattn.lib()
+
+            def hop_two(pos):
+                hlib.wr_hip_attn_append(hkv.h, 0, pos, 1, hk.ctypes.data, hv.ctypes.data)
+                hlib.wr_hip_attn_decode(hkv.h, 0, pos + 1, hq.ctypes.data, hout.ctypes.data, 16, 0.0, 0)
+
+            def hop_one(pos):
+                hlib.wr_hip_attn_append_decode(hkv.h, 0, pos, hk.ctypes.data, hv.ctypes.data, hq.ctypes.data,
+                                               hout.ctypes.data, 16, 0.0, 0)
+
+            for key, fn in (("host_rows_append_then_decode_us", hop_two), ("host_rows_append_decode_us", hop_one)):
+                ts = []
+                for i in range(220):
+                    t0 = time.perf_counter()
+                    fn(520 + i)
+                    ts.append(time.perf_counter() - t0)
+                e2e[key] = round(float(np.median(ts[20:])) * 1e6, 1)
+            hkv.close()
+        except Exception as exc:
+            e2e["host_rows_error"] = repr(exc)[:200]
 
     line = {
         "metric": "decode-attn HBM GB/s (% peak) at 16 sess x 4K ctx; prefill attn TFLOP/s",

@@ -152,6 +152,36 @@ int wr_hip_attn_decode_batched(uint32_t n, wr_hip_kv *const *kv,
                                uint32_t nq, float scale_override,
                                uint32_t window);
 
+/* ---- a decode step's append and attention in one call ---------------------
+ * Replaces the pair the reference makes per layer of a decode step,
+ * kv_append_row then wri_op_gqa_attention (src/core/session.c:483-496): row
+ * k_f32 / v_f32 [nkv, hd_layer] is truncated to F16 and stored at `pos`, then
+ * the nq heads of q attend keys 0 .. pos (with `window` > 0, the last `window`
+ * of them) into out.  All four are host F32 and taken as they stand (K and Q
+ * already normed and rotated, as at that call site).  Cache bytes and output
+ * are those of wr_hip_attn_append followed by wr_hip_attn_decode with
+ * seq_k = pos + 1, bit for bit; what changes is the traffic: one copy up, one
+ * launch where the shape allows it (head dim 128 with the matrix-core group
+ * sizes; two launches back to back otherwise), one copy down, one wait --
+ * half the synchronous round trips of the two calls.  pos >= max_ctx is
+ * WR_HIP_ERR_CTX_FULL and nothing is written. */
+int wr_hip_attn_append_decode(wr_hip_kv *kv, uint32_t layer, uint32_t pos,
+                              const float *k_f32, const float *v_f32,
+                              const float *q, float *out, uint32_t nq,
+                              float scale_override, uint32_t window);
+
+/* The same for n <= WR_HIP_BATCH_MAX sessions at once (the per-session appends
+ * and the one batched attention of src/core/batch.c:152-196): row pointers per
+ * session, pos[i] the position session i's row goes to.  Any pos[i] >= max_ctx
+ * is WR_HIP_ERR_CTX_FULL with nothing written for any session. */
+int wr_hip_attn_append_decode_batched(uint32_t n, wr_hip_kv *const *kv,
+                                      uint32_t layer, const uint32_t *pos,
+                                      const float *const *k_f32,
+                                      const float *const *v_f32,
+                                      const float *const *q, float *const *out,
+                                      uint32_t nq, float scale_override,
+                                      uint32_t window);
+
 /* ---- causal prefill -----------------------------------------------------
  * Replaces the loop of seq_q = 1 attention calls that prefill runs
  * (src/core/session.c:615-625): rows p0 .. p0+T-1 have already been appended;

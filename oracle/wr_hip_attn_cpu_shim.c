@@ -212,6 +212,45 @@ int wr_hip_attn_decode_batched(uint32_t n, wr_hip_kv *const *kv, uint32_t layer,
     return late_error();
 }
 
+int wr_hip_attn_append_decode_batched(uint32_t n, wr_hip_kv *const *kv, uint32_t layer,
+                                      const uint32_t *pos, const float *const *k,
+                                      const float *const *v, const float *const *q,
+                                      float *const *out, uint32_t nq, float scale_override,
+                                      uint32_t window)
+{
+    if (!g_inited) return WR_HIP_ERR_STATE;
+    if (!kv || !pos || !k || !v || !q || !out) return WR_HIP_ERR_INVAL;
+    if (n == 0 || n > WR_HIP_BATCH_MAX) return WR_HIP_ERR_LIMIT;
+    uint32_t seq_k[WR_HIP_BATCH_MAX];
+    for (uint32_t i = 0; i < n; i++) {
+        if (!k[i] || !v[i] || !q[i] || !out[i] || !layer_ok(kv[i], layer)) return WR_HIP_ERR_INVAL;
+        if (pos[i] >= kv[i]->max_ctx) return WR_HIP_ERR_CTX_FULL;
+        seq_k[i] = pos[i] + 1;
+    }
+    g_calls += n;
+    for (uint32_t i = 0; i < n; i++) {
+        int rc = check_decode(kv[i], layer, seq_k[i], nq);
+        if (rc) return rc;
+        for (uint32_t j = 0; j < i; j++)
+            if (kv[i] == kv[j]) return WR_HIP_ERR_INVAL;
+    }
+    for (uint32_t i = 0; i < n; i++) {
+        int rc = wr_hip_attn_append(kv[i], layer, pos[i], 1, k[i], v[i]);
+        if (rc) return rc;
+        wro_attention_f16kv(q[i], kv[i]->k[layer], kv[i]->v[layer], out[i], 1, nq, kv[i]->nkv,
+                            kv[i]->hd[layer], seq_k[i], scale_override, window);
+    }
+    return late_error();
+}
+
+int wr_hip_attn_append_decode(wr_hip_kv *kv, uint32_t layer, uint32_t pos, const float *k,
+                              const float *v, const float *q, float *out, uint32_t nq,
+                              float scale_override, uint32_t window)
+{
+    return wr_hip_attn_append_decode_batched(1, &kv, layer, &pos, &k, &v, &q, &out, nq, scale_override,
+                                             window);
+}
+
 int wr_hip_attn_prefill(wr_hip_kv *kv, uint32_t layer, uint32_t p0, uint32_t T, const float *q,
                         float *out, uint32_t nq, float scale_override, uint32_t window)
 {

@@ -619,3 +619,121 @@ def test_append_and_decode_in_one_launch_refuses_what_it_must():
     for b in (x, w, tab, out):
         b.free()
     kv.close()
+
+
+# ---------------------- append + decode in one call, rows from host memory --
+
+@pytest.mark.parametrize("nq,nkv,hd,base,steps,sc,win", [
+    (32, 8, 128, 700, 3, 0.0, 0),        # one launch (head dim 128, group 4)
+    (16, 8, 128, 0, 4, 0.0, 0),          # from an empty cache: the first key is the row itself
+    (64, 8, 128, 333, 2, 0.07, 100),     # group 8, scale override, sliding window
+    (8, 8, 128, 31, 3, 0.0, 0),          # group 1, across a 32-position block edge
+    (8, 4, 256, 250, 2, 0.0, 0),         # two launches back to back: head dim 256
+    (8, 2, 64, 95, 3, 0.0, 16),          # head dim 64
+    (6, 2, 80, 17, 2, 0.0, 0),           # a shape the generic kernels take
+])
+def test_append_decode_from_host_rows_equals_the_two_calls(nq, nkv, hd, base, steps, sc, win):
+    cap = base + steps
+    _a, _b, k16, v16 = util.make_kv(7100 + nq + hd, cap, nkv, hd)
+    one = hipattn.KVCache(1, hd, nkv, cap)
+    two = hipattn.KVCache(1, hd, nkv, cap)
+    if base:
+        one.write_f16(0, 0, k16[:base], v16[:base])
+        two.write_f16(0, 0, k16[:base], v16[:base])
+    calls0 = hipattn.lib().wr_hip_attn_calls()
+    for s in range(steps):
+        pos = base + s
+        print("append+decode", nq, nkv, hd, "pos", pos, flush=True)
+        kn = synth.normal(7200 + 3 * s, (nkv, hd), std=2.0)
+        vn = synth.normal(7201 + 3 * s, (nkv, hd), std=2.0)
+        q = synth.normal(7202 + 3 * s, (nq, hd))
+        got = one.append_decode(0, pos, kn, vn, q, sc, win)
+        assert two.append(0, pos, kn[None], vn[None]) == hipattn.OK
+        want = two.decode(0, pos + 1, q, sc, win)
+        assert np.array_equal(got, want), f"step {s}"
+        k16[pos] = synth.f32_to_f16_trunc(kn)
+        v16[pos] = synth.f32_to_f16_trunc(vn)
+        util.assert_close(got, util.oracle_decode(q, k16, v16, pos + 1, sc, win), f"step {s}")
+    gk, gv = one.read_f16(0, 0, cap)
+    assert np.array_equal(gk, k16) and np.array_equal(gv, v16)
+    # one attention call counted per step by each form
+    assert hipattn.lib().wr_hip_attn_calls() == calls0 + 2 * steps
+    one.close(); two.close()
+
+
+@pytest.mark.parametrize("nq,nkv,hd", [(32, 8, 128), (8, 4, 256)])
+def test_append_decode_batched_from_host_rows_equals_the_two_calls(nq, nkv, hd):
+    S = 16 if hd == 128 else 5
+    ctxs = synth.ragged_contexts(synth.config_seed(5, 1), S, 1, 3000)
+    ctxs[0] = 1                                   # a session whose cache is empty before the step
+    print("append+decode batched", nq, nkv, hd, ctxs.tolist(), flush=True)
+    ones, twos, ks, vs, qs, kv16 = [], [], [], [], [], []
+    for i, ctx in enumerate(int(c) for c in ctxs):
+        _a, _b, k16, v16 = util.make_kv(7300 + i, ctx, nkv, hd)
+        a = hipattn.KVCache(1, hd, nkv, ctx)
+        b = hipattn.KVCache(1, hd, nkv, ctx)
+        if ctx > 1:
+            a.write_f16(0, 0, k16[:ctx - 1], v16[:ctx - 1])
+            b.write_f16(0, 0, k16[:ctx - 1], v16[:ctx - 1])
+        kn = synth.normal(7400 + i, (nkv, hd))
+        vn = synth.normal(7500 + i, (nkv, hd))
+        k16[ctx - 1] = synth.f32_to_f16_trunc(kn)
+        v16[ctx - 1] = synth.f32_to_f16_trunc(vn)
+        ones.append(a); twos.append(b); ks.append(kn); vs.append(vn); kv16.append((k16, v16))
+        qs.append(synth.normal(7600 + i, (nq, hd)))
+    got = hipattn.append_decode_batched(ones, 0, [int(c) - 1 for c in ctxs], ks, vs, qs)
+    for i, ctx in enumerate(int(c) for c in ctxs):
+        assert twos[i].append(0, ctx - 1, ks[i][None], vs[i][None]) == hipattn.OK
+    want = hipattn.decode_batched(twos, 0, ctxs, qs)
+    for i, ctx in enumerate(int(c) for c in ctxs):
+        assert np.array_equal(got[i], want[i]), f"session {i}"
+        util.assert_close(got[i], util.oracle_decode(qs[i], kv16[i][0], kv16[i][1], ctx), f"session {i}")
+        gk, gv = ones[i].read_f16(0, 0, ctx)
+        assert np.array_equal(gk, kv16[i][0]) and np.array_equal(gv, kv16[i][1]), f"session {i}"
+    for kv in ones + twos:
+        kv.close()
+
+
+def test_append_decode_from_host_rows_refuses_what_it_must():
+    import ctypes as C
+    lib = hipattn.lib()
+    nq, nkv, hd, cap = 16, 8, 128, 12
+    kv = hipattn.KVCache(2, [hd, 0], nkv, cap)
+    other = hipattn.KVCache(1, hd, nkv, 4)
+    _a, _b, k16, v16 = util.make_kv(7700, cap, nkv, hd)
+    kv.write_f16(0, 0, k16, v16)
+    k = synth.normal(7701, (nkv, hd)); v = synth.normal(7702, (nkv, hd))
+    q = synth.normal(7703, (nq, hd)); out = np.zeros_like(q)
+    p = lambda a: a.ctypes.data                                        # noqa: E731
+    call = lambda layer, pos, nq_=nq, kk=p(k), qq=p(q), oo=p(out): lib.wr_hip_attn_append_decode(   # noqa: E731
+        kv.h, layer, pos, kk, p(v), qq, oo, nq_, 0.0, 0)
+    calls0 = lib.wr_hip_attn_calls()
+    assert call(0, cap) == hipattn.ERR_CTX_FULL                        # a full cache: refused ...
+    assert call(0, cap + 5) == hipattn.ERR_CTX_FULL
+    assert call(1, 3) == hipattn.ERR_INVAL                             # layer without storage
+    assert call(2, 3) == hipattn.ERR_INVAL
+    assert call(0, 3, nq_=12) == hipattn.ERR_INVAL                     # nq % nkv != 0
+    assert call(0, 3, kk=None) == hipattn.ERR_INVAL
+    assert call(0, 3, qq=None) == hipattn.ERR_INVAL
+    assert call(0, 3, oo=None) == hipattn.ERR_INVAL
+    assert lib.wr_hip_attn_append_decode(None, 0, 3, p(k), p(v), p(q), p(out), nq, 0.0, 0) == hipattn.ERR_INVAL
+    assert lib.wr_hip_attn_calls() == calls0                           # ... none of them counted
+    gk, gv = kv.read_f16(0, 0, cap)
+    assert np.array_equal(gk, k16) and np.array_equal(gv, v16)         # ... and nothing written
+    # batch: 0 and 17 sessions, the same session twice, one full session among good ones
+    kvp = (C.c_void_p * 17)(*([kv.h] * 17))
+    pos = (C.c_uint32 * 17)(*([3] * 17))
+    arr = lambda a: (C.c_void_p * 17)(*([p(a)] * 17))                  # noqa: E731
+    bat = lambda n, kvs=kvp, ps=pos: lib.wr_hip_attn_append_decode_batched(     # noqa: E731
+        n, kvs, 0, ps, arr(k), arr(v), arr(q), arr(out), nq, 0.0, 0)
+    assert bat(0) == hipattn.ERR_LIMIT
+    assert bat(17) == hipattn.ERR_LIMIT
+    assert bat(2) == hipattn.ERR_INVAL
+    two = (C.c_void_p * 17)(kv.h, other.h, *([None] * 15))
+    assert bat(2, two, (C.c_uint32 * 17)(3, 4, *([0] * 15))) == hipattn.ERR_CTX_FULL
+    gk, gv = kv.read_f16(0, 0, cap)
+    assert np.array_equal(gk, k16) and np.array_equal(gv, v16)         # the good session's row was not written
+    assert bat(2, two, (C.c_uint32 * 17)(3, 3, *([0] * 15))) == hipattn.OK
+    gk, _gv = kv.read_f16(0, 3, 1)
+    assert np.array_equal(gk[0], synth.f32_to_f16_trunc(k))
+    kv.close(); other.close()

@@ -1493,6 +1493,93 @@ int wr_hip_attn_decode(wr_hip_kv* kv, uint32_t layer, uint32_t seq_k, const floa
     return wr_hip_attn_decode_batched(1, kvs, layer, &seq_k, qs, outs, nq, scale_override, window);
 }
 
+int wr_hip_attn_append_decode_batched(uint32_t n, wr_hip_kv* const* kv, uint32_t layer,
+                                      const uint32_t* pos, const float* const* k_f32,
+                                      const float* const* v_f32, const float* const* q,
+                                      float* const* out, uint32_t nq, float scale_override,
+                                      uint32_t window)
+{
+    if (!g.inited) return WR_HIP_ERR_STATE;
+    if (!kv || !pos || !k_f32 || !v_f32 || !q || !out) return WR_HIP_ERR_INVAL;
+    if (n == 0 || n > WR_HIP_BATCH_MAX) return WR_HIP_ERR_LIMIT;
+    for (uint32_t i = 0; i < n; i++) {
+        if (!k_f32[i] || !v_f32[i] || !q[i] || !out[i]) return WR_HIP_ERR_INVAL;
+        int rc = check_layer(kv[i], layer);
+        if (rc) return rc;
+    }
+    const uint32_t hd = kv[0]->hd[layer], nkv = kv[0]->nkv;
+    if (nq == 0 || nq % nkv != 0) return WR_HIP_ERR_INVAL;
+    uint32_t seq_k[WR_HIP_BATCH_MAX];
+    for (uint32_t i = 0; i < n; i++) {
+        if (pos[i] >= kv[i]->max_ctx) return WR_HIP_ERR_CTX_FULL;          // as the append: nothing is written
+        seq_k[i] = pos[i] + 1;
+    }
+    int rc = check_decode(n, kv, layer, seq_k, q, out, nq);
+    if (rc) return rc;
+    // One staged image, one copy up, the output rows behind it.  For the one-launch
+    // kernel session i's rows lie as [nq Q | nkv K | nkv V], the stacked-projection
+    // form it reads; for the two-step form the Q rows are packed in front (what the
+    // attention reads) and the [K | V] pairs follow.
+    const size_t qrow = (size_t)nq * hd, krow = (size_t)nkv * hd;
+    const uint32_t ld = (uint32_t)(qrow + 2 * krow);
+    const bool one_launch = hd == 128 && mfma_shape(hd, nq / nkv);
+    const size_t in_bytes = (size_t)n * ld * sizeof(float), out_bytes = n * qrow * sizeof(float);
+    ENTER();
+    rc = ensure_device(cx->d_stage, in_bytes + out_bytes);
+    if (rc) return rc;
+    rc = ensure_pinned(cx->h_pin, in_bytes);
+    if (rc) return rc;
+    float* din = reinterpret_cast<float*>(cx->d_stage.p);
+    float* dout = reinterpret_cast<float*>((uint8_t*)cx->d_stage.p + in_bytes);
+    float* pin = reinterpret_cast<float*>(cx->h_pin.p);
+    for (uint32_t i = 0; i < n; i++) {
+        float* qdst = one_launch ? pin + (size_t)i * ld : pin + (size_t)i * qrow;
+        float* kdst = one_launch ? qdst + qrow : pin + (size_t)n * qrow + (size_t)i * 2 * krow;
+        memcpy(qdst, q[i], qrow * sizeof(float));
+        memcpy(kdst, k_f32[i], krow * sizeof(float));
+        memcpy(kdst + krow, v_f32[i], krow * sizeof(float));
+    }
+    HIP_TRY(hipMemcpyAsync(din, pin, in_bytes, hipMemcpyHostToDevice, cx->stream), "rows h2d", layer);
+    if (one_launch) {
+        // rows taken as they stand: no norm weights, no rotation
+        DecodeFusedArgs fz;
+        memset(&fz, 0, sizeof fz);
+        fz.qkv = din;
+        fz.ld = ld;
+        rc = decode_locked(n, kv, layer, seq_k, nullptr, dout, nq, scale_override, window,
+                           DecodeWorkspace(), &fz);
+    } else {
+        // the same two steps as separate launches on the one stream, no wait between them
+        const float* dkv = din + (size_t)n * qrow;
+        for (uint32_t i = 0; i < n && rc == WR_HIP_OK; i++)
+            rc = append_rows_locked<float>(kv[i], layer, pos[i], 1, dkv + (size_t)i * 2 * krow,
+                                           dkv + (size_t)i * 2 * krow + krow);
+        if (rc == WR_HIP_OK)
+            rc = decode_locked(n, kv, layer, seq_k, din, dout, nq, scale_override, window);
+    }
+    if (rc) return rc;
+    HIP_TRY(hipMemcpyAsync(cx->h_pin.p, dout, out_bytes, hipMemcpyDeviceToHost, cx->stream), "out d2h",
+            layer);
+    rc = sync_checked("append+decode sync", layer);
+    if (rc) return rc;
+    for (uint32_t i = 0; i < n; i++)
+        memcpy(out[i], (uint8_t*)cx->h_pin.p + i * qrow * sizeof(float), qrow * sizeof(float));
+    return WR_HIP_OK;
+}
+
+int wr_hip_attn_append_decode(wr_hip_kv* kv, uint32_t layer, uint32_t pos, const float* k_f32,
+                              const float* v_f32, const float* q, float* out, uint32_t nq,
+                              float scale_override, uint32_t window)
+{
+    wr_hip_kv* kvs[1] = {kv};
+    const float* ks[1] = {k_f32};
+    const float* vs[1] = {v_f32};
+    const float* qs[1] = {q};
+    float* outs[1] = {out};
+    return wr_hip_attn_append_decode_batched(1, kvs, layer, &pos, ks, vs, qs, outs, nq, scale_override,
+                                             window);
+}
+
 // ---------------------------------------------------------------- prefill --
 
 int wr_hip_attn_prefill_dev(wr_hip_kv* kv, uint32_t layer, uint32_t p0, uint32_t T,

@@ -53,6 +53,12 @@ def load() -> C.CDLL:
                                                  C.POINTER(_vp), C.POINTER(_vp), _u32, C.c_float,
                                                  _u32]),
         "wr_hip_attn_prefill": (C.c_int, [_vp, _u32, _u32, _u32, _vp, _vp, _u32, C.c_float, _u32]),
+        "wr_hip_attn_append_decode": (C.c_int, [_vp, _u32, _u32, _vp, _vp, _vp, _vp, _u32, C.c_float,
+                                                _u32]),
+        "wr_hip_attn_append_decode_batched": (C.c_int, [_u32, C.POINTER(_vp), _u32, C.POINTER(_u32),
+                                                        C.POINTER(_vp), C.POINTER(_vp),
+                                                        C.POINTER(_vp), C.POINTER(_vp), _u32,
+                                                        C.c_float, _u32]),
         "wr_hip_attn_dev_alloc": (_vp, [C.c_size_t]),
         "wr_hip_attn_dev_free": (None, [_vp]),
         "wr_hip_attn_h2d": (C.c_int, [_vp, _vp, C.c_size_t]),
@@ -221,6 +227,19 @@ class KVCache:
                                         scale_override, window), "decode")
         return out
 
+    def append_decode(self, layer: int, pos: int, k: np.ndarray, v: np.ndarray, q: np.ndarray,
+                      scale_override: float = 0.0, window: int = 0) -> np.ndarray:
+        """Row k, v float32 [nkv, hd] stored at pos, then q float32 [nq, hd] attends keys
+        0 .. pos: append + decode in one call."""
+        k = np.ascontiguousarray(k, dtype=np.float32)
+        v = np.ascontiguousarray(v, dtype=np.float32)
+        q = np.ascontiguousarray(q, dtype=np.float32)
+        out = np.empty_like(q)
+        _check(lib().wr_hip_attn_append_decode(self.h, layer, pos, _ptr(k), _ptr(v), _ptr(q),
+                                               _ptr(out), q.shape[0], scale_override, window),
+               "append_decode")
+        return out
+
     def prefill(self, layer: int, p0: int, q: np.ndarray, scale_override: float = 0.0,
                 window: int = 0) -> np.ndarray:
         """q float32 [T, nq, hd] -> float32 [T, nq, hd]."""
@@ -242,6 +261,27 @@ def decode_batched(caches, layer: int, seq_k, qs, scale_override: float = 0.0, w
     op = (_vp * n)(*[_ptr(o) for o in outs])
     _check(lib().wr_hip_attn_decode_batched(n, kvp, layer, sk, qp, op, qs[0].shape[0],
                                             scale_override, window), "decode_batched")
+    return outs
+
+
+def append_decode_batched(caches, layer: int, pos, ks, vs, qs, scale_override: float = 0.0,
+                          window: int = 0):
+    """Session i's row ks[i], vs[i] stored at pos[i], then qs[i] attends keys 0 .. pos[i];
+    returns the list of outputs."""
+    n = len(caches)
+    ks = [np.ascontiguousarray(a, dtype=np.float32) for a in ks]
+    vs = [np.ascontiguousarray(a, dtype=np.float32) for a in vs]
+    qs = [np.ascontiguousarray(a, dtype=np.float32) for a in qs]
+    outs = [np.empty_like(q) for q in qs]
+    kvp = (_vp * n)(*[c.h for c in caches])
+    pp = (_u32 * n)(*[int(p) for p in pos])
+
+    def arr(xs):
+        return (_vp * n)(*[_ptr(x) for x in xs])
+
+    _check(lib().wr_hip_attn_append_decode_batched(n, kvp, layer, pp, arr(ks), arr(vs), arr(qs),
+                                                   arr(outs), qs[0].shape[0], scale_override,
+                                                   window), "append_decode_batched")
     return outs
 
 

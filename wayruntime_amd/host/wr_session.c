@@ -12,11 +12,14 @@
  * device:
  *
  *   reference kv_append_row (session.c:139-154, called :483-486)
- *                                  -> wr_hip_attn_append
+ *                                  -> wr_hip_attn_append_rope     (wr_prefill)
  *   reference wri_op_gqa_attention (kernels.c:1414, called session.c:493)
- *                                  -> wr_hip_attn_decode          (wr_step)
  *                                  -> wr_hip_attn_prefill         (wr_prefill)
- *                                  -> wr_hip_attn_decode_batched  (wr_batch_step)
+ *   the two back to back, a decode step's pair (session.c:483-496)
+ *                                  -> wr_hip_attn_append_decode          (wr_step)
+ *                                  -> wr_hip_attn_append_decode_batched  (wr_batch_step)
+ *   (a layer that reads another layer's cache appends nothing and calls
+ *    wr_hip_attn_decode / wr_hip_attn_decode_batched)
  *
  * Contracts kept from the reference: one mutex per session held for the whole
  * call (session.c:581-595); a call that cannot complete consumes nothing —
@@ -148,20 +151,37 @@ static wr_status forward_rows_gemma(wr_model *m, wrh_workspace *ws, uint32_t R,
             uint32_t seq_k[WR_BATCH_MAX];
             const float *qp[WR_BATCH_MAX];
             float *op[WR_BATCH_MAX];
+            const float *kp[WR_BATCH_MAX], *vp[WR_BATCH_MAX];
+            uint32_t at[WR_BATCH_MAX];
             for (uint32_t r = 0; r < R; r++) {
-                if (!shared) {
-                    rc = wr_hip_attn_append_rope(ss[r]->kv, L, ss[r]->pos, 1, ws->k + (size_t)r * kd,
-                                                 ws->v + (size_t)r * kd, tab + r * ts, n_rot);
-                    if (rc != WR_HIP_OK) return (rc == WR_HIP_ERR_CTX_FULL) ? WR_ERR_CTX_FULL
-                                                                             : op_fail(e, "kv append", L, rc);
-                    ss[r]->kv_rows[L] = ss[r]->pos + 1;
-                }
                 kvs[r] = ss[r]->kv;
+                at[r] = ss[r]->pos;
                 seq_k[r] = ss[r]->pos + 1;
                 qp[r] = ws->q + (size_t)r * qd;
                 op[r] = ws->attn + (size_t)r * qd;
+                kp[r] = ws->k + (size_t)r * kd;
+                vp[r] = ws->v + (size_t)r * kd;
             }
-            rc = wr_hip_attn_decode_batched(R, kvs, ksrc, seq_k, qp, op, nq, m->attn_scale, window);
+            if (!shared) {
+                /* the rows' K rotated here like Q, then every session's append and the
+                 * batched attention in one call: one round trip to the device per layer */
+                for (uint32_t r = 0; r < R; r++)
+                    wrh_rope_apply(ws->k + (size_t)r * kd, nkv, hd, tab + r * ts, n_rot);
+                rc = wr_hip_attn_append_decode_batched(R, kvs, L, at, kp, vp, qp, op, nq, m->attn_scale,
+                                                       window);
+                if (rc == WR_HIP_ERR_CTX_FULL) return WR_ERR_CTX_FULL;
+                if (rc == WR_HIP_OK)
+                    for (uint32_t r = 0; r < R; r++) ss[r]->kv_rows[L] = ss[r]->pos + 1;
+            } else {
+                rc = wr_hip_attn_decode_batched(R, kvs, ksrc, seq_k, qp, op, nq, m->attn_scale, window);
+            }
+        } else if (mode == FWD_STEP && !shared) {
+            wr_session *s = ss[0];
+            wrh_rope_apply(ws->k, nkv, hd, tab, n_rot);
+            rc = wr_hip_attn_append_decode(s->kv, L, pos0, ws->k, ws->v, ws->q, ws->attn, nq, m->attn_scale,
+                                           window);
+            if (rc == WR_HIP_ERR_CTX_FULL) return WR_ERR_CTX_FULL;
+            if (rc == WR_HIP_OK) s->kv_rows[L] = pos0 + 1;
         } else {
             wr_session *s = ss[0];
             if (!shared) {
@@ -231,8 +251,10 @@ static wr_status forward_rows(wr_model *m, wrh_workspace *ws, uint32_t R, wr_ses
             wrh_rmsnorm(ws->k, m->k_norm[L].data, m->k_norm[L].n, ws->k, R * nkv, hd, m->rms_eps);
         }
         /* RoPE (reference: session.c:475-478): the rows' angles are worked out
-         * once here; Q is rotated on the host, K on the device inside the
-         * append (same arithmetic, same bits), so K goes up as projected. */
+         * once here and Q is rotated on the host.  A decode step rotates K here
+         * too and hands both rows to the one append-and-attend call; a prompt's K
+         * goes up as projected and is rotated on the device inside the append
+         * (same arithmetic, same bits). */
         const uint32_t n_rot =
             (m->n_rot_pairs >= 1 && m->n_rot_pairs < hd / 2) ? m->n_rot_pairs : hd / 2;
         const size_t ts = (size_t)2 * n_rot;              /* table row: n_rot (cos, sin) pairs */
@@ -249,31 +271,37 @@ static wr_status forward_rows(wr_model *m, wrh_workspace *ws, uint32_t R, wr_ses
         }
         if (mode == FWD_BATCH) {
             wr_hip_kv *kvs[WR_BATCH_MAX];
-            uint32_t seq_k[WR_BATCH_MAX];
             const float *qp[WR_BATCH_MAX];
             float *op[WR_BATCH_MAX];
+            const float *kp[WR_BATCH_MAX], *vp[WR_BATCH_MAX];
+            uint32_t at[WR_BATCH_MAX];
             for (uint32_t r = 0; r < R; r++) {
-                rc = wr_hip_attn_append_rope(ss[r]->kv, L, ss[r]->pos, 1, ws->k + (size_t)r * kd,
-                                             ws->v + (size_t)r * kd, ws->rope + r * ts, n_rot);
-                if (rc != WR_HIP_OK) return (rc == WR_HIP_ERR_CTX_FULL) ? WR_ERR_CTX_FULL
-                                                                         : op_fail(e, "kv append", L, rc);
-                ss[r]->kv_rows[L] = ss[r]->pos + 1;
+                wrh_rope_apply(ws->k + (size_t)r * kd, nkv, hd, ws->rope + r * ts, n_rot);
                 kvs[r] = ss[r]->kv;
-                seq_k[r] = ss[r]->pos + 1;
+                at[r] = ss[r]->pos;
                 qp[r] = ws->q + (size_t)r * qd;
                 op[r] = ws->attn + (size_t)r * qd;
+                kp[r] = ws->k + (size_t)r * kd;
+                vp[r] = ws->v + (size_t)r * kd;
             }
-            rc = wr_hip_attn_decode_batched(R, kvs, L, seq_k, qp, op, nq, 0.0f, 0);
+            /* every session's append and the batched attention in one call */
+            rc = wr_hip_attn_append_decode_batched(R, kvs, L, at, kp, vp, qp, op, nq, 0.0f, 0);
+            if (rc == WR_HIP_ERR_CTX_FULL) return WR_ERR_CTX_FULL;
+            if (rc == WR_HIP_OK)
+                for (uint32_t r = 0; r < R; r++) ss[r]->kv_rows[L] = ss[r]->pos + 1;
+        } else if (mode == FWD_STEP) {
+            wr_session *s = ss[0];
+            wrh_rope_apply(ws->k, nkv, hd, ws->rope, n_rot);
+            rc = wr_hip_attn_append_decode(s->kv, L, pos0, ws->k, ws->v, ws->q, ws->attn, nq, 0.0f, 0);
+            if (rc == WR_HIP_ERR_CTX_FULL) return WR_ERR_CTX_FULL;
+            if (rc == WR_HIP_OK) s->kv_rows[L] = pos0 + 1;
         } else {
             wr_session *s = ss[0];
             rc = wr_hip_attn_append_rope(s->kv, L, pos0, R, ws->k, ws->v, ws->rope, n_rot);
             if (rc != WR_HIP_OK) return (rc == WR_HIP_ERR_CTX_FULL) ? WR_ERR_CTX_FULL
                                                                      : op_fail(e, "kv append", L, rc);
             s->kv_rows[L] = pos0 + R;
-            if (mode == FWD_STEP)
-                rc = wr_hip_attn_decode(s->kv, L, pos0 + 1, ws->q, ws->attn, nq, 0.0f, 0);
-            else
-                rc = wr_hip_attn_prefill(s->kv, L, pos0, R, ws->q, ws->attn, nq, 0.0f, 0);
+            rc = wr_hip_attn_prefill(s->kv, L, pos0, R, ws->q, ws->attn, nq, 0.0f, 0);
         }
         if (rc != WR_HIP_OK) return op_fail(e, "gqa", L, rc);
 
