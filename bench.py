@@ -531,6 +531,32 @@ def main() -> None:
         except Exception as exc:
             read_probe = {"error": repr(exc)[:200]}
 
+    # ---- what the matrix pipes sustain with nothing but MFMAs in flight, with
+    # operands of zeros and with operands drawn from N(0, 1): the clock the device
+    # grants depends on the data (secondary figure: the prefill fraction above stays
+    # priced against the published peak)
+    mfma_probe = None
+    mfma_exe = os.path.join(ROOT, "wayruntime_amd", "calib_mfma")
+    if not args.no_prefill and os.path.exists(mfma_exe):
+        import subprocess
+        try:
+            res = subprocess.run([mfma_exe, "32"], capture_output=True, text=True, timeout=120)
+            mfma_probe = []
+            for ln in res.stdout.splitlines():
+                f = ln.split()
+                if ln.startswith("operands") and "TFLOP/s" in f:
+                    mfma_probe.append({"operands": f[1], "launch_us": float(f[f.index("launch_us") + 1]),
+                                       "TFLOP/s": float(f[f.index("TFLOP/s") + 1]),
+                                       "shader_GHz": float(f[f.index("GHz") + 1])})
+            if res.returncode != 0 or not mfma_probe:
+                mfma_probe = {"error": "exit %d: %s" % (res.returncode, (res.stderr or res.stdout)[-200:])}
+            elif isinstance(prefill, dict) and prefill.get("tflops"):
+                normal = [m["TFLOP/s"] for m in mfma_probe if m["operands"] == "normal"]
+                if normal:
+                    prefill["frac_of_mfma_probe_normal_operands"] = round(prefill["tflops"] / normal[0], 4)
+        except Exception as exc:
+            mfma_probe = {"error": repr(exc)[:200]}
+
     # ---- what one launch costs inside a chain of dependent launches (the
     # device walk's decode step is such a chain): a floor, from kernels that
     # only read their predecessor's row, reduce it and store (secondary figure)
@@ -628,6 +654,7 @@ def main() -> None:
         "roofline": roofline, "cpu_baseline": cpu, "prefill": prefill, "decode_configs": decode_configs,
         "hbm_read_probe": read_probe,
         "launch_chain_probe": chain_probe,
+        "mfma_probe": mfma_probe,
         "projection": proj,
         "end_to_end": e2e,
         "check": {"max_abs": max_abs, "rel_l2": rel_l2},

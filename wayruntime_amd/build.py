@@ -61,17 +61,20 @@ def build_host() -> str:
     return HOST_SO
 
 
-CALIB_BINS = {"calib_copy": "calib_copy.hip", "calib_read": "calib_read.hip", "calib_chain": "calib_chain.hip"}
+CALIB_BINS = {"calib_copy": "calib_copy.hip", "calib_read": "calib_read.hip", "calib_chain": "calib_chain.hip",
+              "calib_mfma": "calib_mfma.hip"}
 CALIB_BIN = os.path.join(PKG, "calib_copy")
 
 
 def build_calib() -> str:
     """Measurement aids: the counter-calibration copy program, the read-only
-    bandwidth probe and the launch-chain probe (see csrc/calib_copy.hip,
-    csrc/calib_read.hip, csrc/calib_chain.hip)."""
+    bandwidth probe, the launch-chain probe and the matrix-pipe probe (see
+    csrc/calib_copy.hip, csrc/calib_read.hip, csrc/calib_chain.hip,
+    csrc/calib_mfma.hip)."""
     for name, src in CALIB_BINS.items():
         out = os.path.join(PKG, name)
-        res = subprocess.run(["hipcc", "-O3", "--offload-arch=gfx950", "-o", out,
+        res = subprocess.run(["hipcc", "-O3", "--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang",
+                              "-packed-fp32-ops", "-o", out,
                               os.path.join(PKG, "csrc", src)], capture_output=True, text=True)
         if res.returncode != 0:
             sys.stderr.write(res.stderr)
