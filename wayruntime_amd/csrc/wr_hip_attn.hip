@@ -25,6 +25,7 @@
 #include "kernels_prefill.hip.h"
 #include "kernels_prefill_il.hip.h"
 #include "kernels_prefill_pair.hip.h"
+#include "kernels_prefill_ild.hip.h"
 #include "kernels_proj.hip.h"
 #include "kernels_rows.hip.h"
 
@@ -117,6 +118,7 @@ struct Lib {
     void* log_user = nullptr;
     std::atomic<uint32_t> tune_keys_per_wg{0};
     std::atomic<int> force_generic{0};
+    std::atomic<int> prefill_256_four_waves{0};   // WR_HIP_PREFILL_256_FOUR_WAVES=1: head dim 256 keeps the earlier four-wave prefill kernel
     std::atomic<int> prefill_two_waves{1};        // WR_HIP_PREFILL_TWO_WAVES=0: head dim 128 takes the one-wave-per-SIMD prefill kernel
 } g;
 
@@ -637,7 +639,9 @@ int prefill_locked(wr_hip_kv* kv, uint32_t layer, uint32_t p0, uint32_t T, const
         } else if (hd == 128)
             launch_main(prefill_il_kernel<128>, dim3(ny, nwg), dim3(kSplitThreads), a,
                         split_smem_bytes<128>());
-        else   // 256: one wave per SIMD (the accumulators alone need 256 registers)
+        else if (!g.prefill_256_four_waves)   // 256: the wave sets divide the dimensions
+            launch_main(prefill_ild_kernel, dim3(ny, nwg), dim3(kSplitThreads), a, ild_smem_bytes());
+        else   // the earlier form: one wave per SIMD owns all 256 dimensions of its rows
             launch_main(prefill_mfma_kernel<256>, dim3(nwg, ny), dim3(kPrefillThreads), a);
     } else {
         launch_main(prefill_generic_kernel, dim3(T, nq), dim3(kDecodeThreads), a);
@@ -1002,6 +1006,8 @@ int wr_hip_attn_init(int device)
     {
         const char* e = getenv("WR_HIP_PREFILL_TWO_WAVES");
         g.prefill_two_waves = (e && e[0] == '0') ? 0 : 1;
+        e = getenv("WR_HIP_PREFILL_256_FOUR_WAVES");
+        g.prefill_256_four_waves = (e && e[0] == '1') ? 1 : 0;
     }
     g.generation++;
     int rc = WR_HIP_OK;
@@ -1042,6 +1048,9 @@ int wr_hip_attn_init(int device)
             e = hipFuncSetAttribute(reinterpret_cast<const void*>(prefill_pair_kernel<128, true>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize,
                                     (int)pair_smem_bytes<128>());
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute(reinterpret_cast<const void*>(prefill_ild_kernel),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)ild_smem_bytes());
         if (e == hipSuccess)
             e = hipFuncSetAttribute(reinterpret_cast<const void*>(proj_gemm_lds_kernel<8, 2, 3>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)gemm_lds_bytes<8, 2, 3>());
