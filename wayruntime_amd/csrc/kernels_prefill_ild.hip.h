@@ -29,20 +29,27 @@
 // slots: the ring geometry, the slot permutations, the operand reads and the
 // copy schedule are those of the 128-dimension kernel (SplitLds<128>).
 //
-// Step j.  On entry `cur` holds the scores of tile j (complete, masked,
-// reference settled), kf the K operands of tile j+1.
-//   first half:   the partial chain S'(j+1), with the Vt operand reads of tile j
-//                 and the exponentials and packs of S(j) behind its links;
-//   the partial scores go to the exchange buffer; barrier (the other half's are
-//   there, and everybody has read tile j+1's K slot);
-//   second half:  O^T += Vt(j).P(j)^T, with the other half's partial scores, the
-//                 K operand reads of tile j+2 and the step's copies between the
-//                 products; then the sum, its row maximum, masks and reference;
-//   barrier (copies that have landed are published, the ring slots and the
-//   exchange buffer change hands).
-// Two hardware barriers per step where the 128-dimension kernel has one: the
-// price of the exchange; no buffer is read and written between the same two
-// barriers, so nothing here depends on how far one wave runs ahead of another.
+// Step j.  On entry `cur` holds the wave's partial scores of tile j, kf the K
+// operands of tile j+1; the other half's partial scores of tile j are in the
+// exchange buffer of parity j.
+//   first half:   the partial chain S'(j+1); behind its first links the scores of
+//                 tile j are completed (sum of the two partials, row maximum,
+//                 masks, reference), behind the others go the Vt operand reads of
+//                 tile j and the exponentials and packs of S(j);
+//   second half:  O^T += Vt(j).P(j)^T, and between the products the K operand
+//                 reads of tile j+2, the step's copies and the partial scores of
+//                 tile j+1 on their way to the exchange buffer of parity j+1;
+//   one hardware barrier per step, as in the 128-dimension kernel: it publishes
+//   the copies that have landed and the partial scores, and frees the ring slots
+//   and the exchange buffer the next step overwrites.  A buffer of either parity
+//   is written in one step, read in the next and written again in the step after
+//   that, with a barrier between each two: nothing here depends on how far one
+//   wave runs ahead of another.
+//
+// The chain of tile j+1 has started (from the block of -m) when the reference of
+// tile j is settled.  If that moves m by delta, the scores of tile j+1 come out
+// delta too high; the move leaves delta in `pend`, and the completion of tile j+1
+// subtracts it (rare, wave-uniform branch; the same in both halves).
 //
 // The halves share the accumulated reference: the chain of the lower half starts
 // from the block of -m, the upper half's from zero, and their sum is S - m.
@@ -56,9 +63,10 @@ constexpr int kIldHalf = 128;                             // dimensions a wave o
 
 struct IldLds {
     using L = SplitLds<kIldHalf>;
-    static constexpr int X_OFF = 2 * L::SET_BYTES;        // exchange of partial scores: [4 pairs][2 halves][16][64] floats
+    static constexpr int X_OFF = 2 * L::SET_BYTES;        // exchange of partial scores: [2 parities][4 pairs][2 halves][16][64] floats
     static constexpr int X_WAVE = 16 * 64 * 4;
-    static constexpr int X_BYTES = 8 * X_WAVE;
+    static constexpr int X_PARITY = 8 * X_WAVE;
+    static constexpr int X_BYTES = 2 * X_PARITY;
     // rows leave through LDS, row-major, once the rings are quiet: [8 waves][32][128 + 4] floats from 0
     static constexpr int O_WAVE = 32 * (kIldHalf + 4) * 4;
     static constexpr int TOTAL = (X_OFF + X_BYTES > 8 * O_WAVE) ? X_OFF + X_BYTES : 8 * O_WAVE;
@@ -138,7 +146,8 @@ __device__ __forceinline__ void ild_patch_tail(unsigned char* smem, const IlCtx<
 // il_move_reference with the upper half's chain starting from zero: only the
 // lower half keeps -m in the block its chain starts from.
 __device__ __forceinline__ void ild_move_reference(PrefillRows<kIldHalf>& R, IlCtx<kIldHalf>& cx, f32x16& negm,
-                                                   f32x16& c, float tmax, bool jump, bool upper)
+                                                   f32x16& c, float tmax, bool jump, bool upper, float& pend,
+                                                   uint32_t& pend_on)
 {
     const bool unset = (R.m_run == -INFINITY);
     const float delta = jump ? tmax : 0.f;
@@ -150,6 +159,10 @@ __device__ __forceinline__ void ild_move_reference(PrefillRows<kIldHalf>& R, IlC
         for (int r = 0; r < 16; r++) R.o[dt][r] *= alpha;
 #pragma unroll
     for (int r = 0; r < 16; r++) asm volatile("v_sub_f32 %0, %0, %1" : "+v"(c[r]) : "v"(delta));
+    // the chain in flight started from the reference as it was (from zero while
+    // the row had none): its scores come out delta too high
+    pend = delta;
+    pend_on = 1;
     if (jump) R.m_run = (unset ? 0.f : R.m_run) + delta;
     const bool still = (R.m_run == -INFINITY);
     const float nm = (still || upper) ? 0.f : -R.m_run;
@@ -159,7 +172,7 @@ __device__ __forceinline__ void ild_move_reference(PrefillRows<kIldHalf>& R, IlC
 }
 
 __device__ __forceinline__ void ild_settle(PrefillRows<kIldHalf>& R, IlCtx<kIldHalf>& cx, f32x16& negm, f32x16& c,
-                                           float tmax, bool upper)
+                                           float tmax, bool upper, float& pend, uint32_t& pend_on)
 {
     {
         const uint32_t u = __float_as_uint(tmax);
@@ -167,43 +180,55 @@ __device__ __forceinline__ void ild_settle(PrefillRows<kIldHalf>& R, IlCtx<kIldH
         tmax = max3_raw(__uint_as_float(sw[0]), __uint_as_float(sw[1]), tmax);   // same in both lanes of a row
     }
     const bool jump = tmax > cx.thr;
-    if (__builtin_amdgcn_ballot_w64(jump) != 0) ild_move_reference(R, cx, negm, c, tmax, jump, upper);
+    if (__builtin_amdgcn_ballot_w64(jump) != 0) ild_move_reference(R, cx, negm, c, tmax, jump, upper, pend, pend_on);
 }
 
 // The wave's partial scores into the exchange buffer, register r of lane l at
 // float (r / 4 * 64 + l) * 4 + r % 4: 16-byte writes, lane-contiguous.
+__device__ __forceinline__ void ild_send1(float* xw, const f32x16& c, int lane, int q4)
+{
+    *reinterpret_cast<f32x4*>(xw + (q4 * 64 + lane) * 4) = f32x4{c[4 * q4], c[4 * q4 + 1], c[4 * q4 + 2],
+                                                              c[4 * q4 + 3]};
+}
+
 __device__ __forceinline__ void ild_send(float* xw, const f32x16& c, int lane)
 {
 #pragma unroll
-    for (int q4 = 0; q4 < 4; q4++)
-        *reinterpret_cast<f32x4*>(xw + (q4 * 64 + lane) * 4) = f32x4{c[4 * q4], c[4 * q4 + 1], c[4 * q4 + 2],
-                                                                  c[4 * q4 + 3]};
+    for (int q4 = 0; q4 < 4; q4++) ild_send1(xw, c, lane, q4);
 }
 
 // Completes the scores of a tile from the two halves' partial sums and settles
-// them: sum, row maximum, masks of a tile that is not plain, reference.
+// them: sum, what a reference move left pending, row maximum, masks of a tile
+// that is not plain, reference.
 __device__ __forceinline__ void ild_complete(PrefillRows<kIldHalf>& R, IlCtx<kIldHalf>& cx, f32x16& negm, f32x16& c,
-                                             const f32x4 (&xr)[4], uint32_t jt, int g, bool upper)
+                                             const f32x4 (&xr)[4], uint32_t jt, int g, bool upper, float& pend,
+                                             uint32_t& pend_on)
 {
 #pragma unroll
     for (int r = 0; r < 16; r++) c[r] += xr[r >> 2][r & 3];
+    if (pend_on) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) asm volatile("v_sub_f32 %0, %0, %1" : "+v"(c[r]) : "v"(pend));
+        pend_on = 0;
+    }
     float tmax = il_max16(c);
     if (jt < cx.pl_lo || jt > cx.pl_hi) {
         il_mask_special<kIldHalf>(R, cx, c, cx.t0 + jt, jt, g, tmax);
         tmax = il_max16(c);
     }
-    ild_settle(R, cx, negm, c, tmax, upper);
+    ild_settle(R, cx, negm, c, tmax, upper, pend, pend_on);
 }
 
-// Step j of a wave (P == j % kRing).  On entry `cur` holds the scores of tile j
-// (complete, masked, reference settled), kf the K operands of tile j+1; on exit
-// `nxt` holds the scores of tile j+1 in the same state and kf the operands of
-// tile j+2.
-template <int P>
-__device__ __forceinline__ void ild_step(PrefillRows<kIldHalf>& R, IlCtx<kIldHalf>& cx, f32x16& negm,
-                                         const f32x16& cur, f32x16& nxt, u32x4 (&pop)[2], half8 (&kf)[8],
-                                         half8 (&vf)[8], unsigned char* smem, float* xw, const float* xr_at,
-                                         uint32_t j, int sub, int lane, int g, uint32_t kv_valid, bool upper)
+// Step j of a wave (P == j % kRing, XB == j % 2).  On entry `cur` holds the
+// wave's partial scores of tile j and kf the K operands of tile j+1; on exit
+// `nxt` holds the partial scores of tile j+1 (sent to the exchange buffer of the
+// other parity) and kf the operands of tile j+2.
+template <int P, int XB>
+__device__ __forceinline__ void ild_step(PrefillRows<kIldHalf>& R, IlCtx<kIldHalf>& cx, f32x16& negm, f32x16& cur,
+                                         f32x16& nxt, u32x4 (&pop)[2], half8 (&kf)[8], half8 (&vf)[8],
+                                         unsigned char* smem, float* xw, const float* xr_at, uint32_t j, int sub,
+                                         int lane, int g, uint32_t kv_valid, bool upper, float& pend,
+                                         uint32_t& pend_on)
 {
     using L = SplitLds<kIldHalf>;
     constexpr int NS = 8, ND = 4;
@@ -212,49 +237,79 @@ __device__ __forceinline__ void ild_step(PrefillRows<kIldHalf>& R, IlCtx<kIldHal
     constexpr int KC = (P + 1) % 3;       // K of tile j+4 replaces K of tile j+1 (read in the previous step)
     constexpr int VC = (P + 2) % 3;       // Vt of tile j+2 replaces Vt of tile j-1 (read in the previous step)
     constexpr int TS = (P + 1) % 3;       // slot of Vt of tile j+1, whose tail is patched once it has landed
+    constexpr int XF = IldLds::X_PARITY / 4;              // floats between the two exchange buffers
 
     float psum = 0.f;
     const half2v ones = {(_Float16)1.0f, (_Float16)1.0f};
-#pragma unroll
-    for (int i = 0; i < NS; i++) {
-        if (i == 0)
-            nxt = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[0], R.qop[0], negm, 0, 0, 0);
-        else
-            nxt = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[i], R.qop[i], nxt, 0, 0, 0);
-        vf[i] = *reinterpret_cast<const half8*>(cx.vop[i / ND] + VS * L::VTILE + (i % ND) * 2048);
-        {
-            const int r = 2 * i;
-            const half2v ph = {(_Float16)fast_exp2(cur[r]), (_Float16)fast_exp2(cur[r + 1])};
-            psum = __builtin_amdgcn_fdot2(ph, ones, psum, false);
-            pop[r >> 3][(r & 7) >> 1] = __builtin_bit_cast(uint32_t, ph);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-    }
-    R.l_run += psum;
-    // the partial scores of tile j+1 meet the other half's
-    ild_send(xw, nxt, lane);
-    __builtin_amdgcn_sched_barrier(0);
-    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    __builtin_amdgcn_sched_barrier(0);
+    auto pair = [&](int p) {
+        // two exp2, one pack to F16, one dot product with (1, 1): the normaliser
+        // is the sum of exactly the rounded values P.V multiplies
+        const int r = 2 * p;
+        const half2v ph = {(_Float16)fast_exp2(cur[r]), (_Float16)fast_exp2(cur[r + 1])};
+        psum = __builtin_amdgcn_fdot2(ph, ones, psum, false);
+        pop[r >> 3][(r & 7) >> 1] = __builtin_bit_cast(uint32_t, ph);
+    };
     f32x4 xr[4];
 #pragma unroll
-    for (int q4 = 0; q4 < 4; q4++) xr[q4] = *reinterpret_cast<const f32x4*>(xr_at + (q4 * 64 + lane) * 4);
+    for (int q4 = 0; q4 < 4; q4++)
+        xr[q4] = *reinterpret_cast<const f32x4*>(xr_at + XB * XF + (q4 * 64 + lane) * 4);
+    // the completion of tile j's scores is spread behind the first three links, so
+    // that neither wave of the SIMD leaves the matrix pipe waiting for it
+    nxt = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[0], R.qop[0], negm, 0, 0, 0);
+    vf[0] = *reinterpret_cast<const half8*>(cx.vop[0] + VS * L::VTILE);
+#pragma unroll
+    for (int r = 0; r < 16; r++) cur[r] += xr[r >> 2][r & 3];
+    if (pend_on) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) asm volatile("v_sub_f32 %0, %0, %1" : "+v"(cur[r]) : "v"(pend));
+        pend_on = 0;
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    nxt = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[1], R.qop[1], nxt, 0, 0, 0);
+    vf[1] = *reinterpret_cast<const half8*>(cx.vop[0] + VS * L::VTILE + 2048);
+    float tmax = il_max16(cur);
+    if (j < cx.pl_lo || j > cx.pl_hi) {
+        il_mask_special<kIldHalf>(R, cx, cur, cx.t0 + j, j, g, tmax);
+        tmax = il_max16(cur);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    nxt = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[2], R.qop[2], nxt, 0, 0, 0);
+    vf[2] = *reinterpret_cast<const half8*>(cx.vop[0] + VS * L::VTILE + 2 * 2048);
+    ild_settle(R, cx, negm, cur, tmax, upper, pend, pend_on);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 3; i < NS; i++) {
+        nxt = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[i], R.qop[i], nxt, 0, 0, 0);
+        vf[i] = *reinterpret_cast<const half8*>(cx.vop[i / ND] + VS * L::VTILE + (i % ND) * 2048);
+        pair(i - 3);
+        if (i == NS - 1) pair(5);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    // products; the partial scores of tile j+1 leave behind the first of them, ahead
+    // of the last operand reads, so that the wait before the barrier can name them
 #pragma unroll
     for (int i = 0; i < NS; i++) {
         const int t = i / ND, dt = i % ND;
         R.o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[i], __builtin_bit_cast(half8, pop[t]), R.o[dt], 0, 0,
                                                            0);
         kf[i] = *reinterpret_cast<const half8*>(cx.kop[i] + KS * L::KTILE);
+        if (i < 2) pair(6 + i);                           // the second half of P is first used by product 4
+        if (i >= 1 && i <= 4) ild_send1(xw + (XB ^ 1) * XF, nxt, lane, i - 1);
         if (i < L::NL) ild_issue_k1<KC>(cx, j + 4, i);
         else if (i < 2 * L::NL) ild_issue_v1<VC>(cx, j + 2, i - L::NL);
+        __builtin_amdgcn_sched_barrier(0);
     }
-    ild_complete(R, cx, negm, nxt, xr, j + 1, g, upper);
+    R.l_run += psum;
     // all copies but this step's have landed: K of tile j+3 and Vt of tile j+1,
     // which the next step reads once the barrier has published them
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * L::NL) : "memory");
     ild_patch_tail<TS>(smem, cx, j + 1, sub, lane, kv_valid);
     __builtin_amdgcn_sched_barrier(0);
-    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");   // the exchange buffer has been read
+    // LDS operations complete in the order issued: with at most the three operand
+    // reads issued after the last piece of the partial scores outstanding, those
+    // are in the exchange buffer (the operand reads' slot is not refilled before
+    // the next step's products, long after the next chain has consumed them)
+    asm volatile("s_waitcnt lgkmcnt(3)\n\ts_barrier" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
 }
 
@@ -378,30 +433,27 @@ __device__ __forceinline__ void ild_block(const PrefillArgs& a, unsigned char* s
     for (int i = 0; i < 8; i++) kf[i] = *reinterpret_cast<const half8*>(cx.kop[i]);
 #pragma unroll
     for (int i = 0; i < 8; i++) sa = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[i], R.qop[i], sa, 0, 0, 0);
-    ild_send(xw, sa, lane);
+    ild_send(xw, sa, lane);                               // tile 0: the exchange buffer of parity 0
     il_barrier();                                         // partial scores out; slot 0 of K has been read by all
     ild_issue_k<0>(cx, 3);
 #pragma unroll
     for (int i = 0; i < 8; i++) kf[i] = *reinterpret_cast<const half8*>(cx.kop[i] + L::KTILE);
-    {
-        f32x4 xr[4];
-#pragma unroll
-        for (int q4 = 0; q4 < 4; q4++) xr[q4] = *reinterpret_cast<const f32x4*>(xr_at + (q4 * 64 + lane) * 4);
-        ild_complete(R, cx, negm, sa, xr, 0, g, upper);
-    }
-    il_barrier();                                         // slot 1 of K and the exchange buffer have been read by all
+    il_barrier();                                         // slot 1 of K has been read by all: step 0 refills it
+    float pend = 0.f;
+    uint32_t pend_on = 0;
 
-#define WR_ILD_STEP(PHASE, CUR, NXT)                                                                    \
-    ild_step<PHASE>(R, cx, negm, CUR, NXT, pop, kf, vf, smem, xw, xr_at, j, sub, lane, g, kv_valid, upper); \
+#define WR_ILD_STEP(PHASE, XB, CUR, NXT)                                                                     \
+    ild_step<PHASE, XB>(R, cx, negm, CUR, NXT, pop, kf, vf, smem, xw, xr_at, j, sub, lane, g, kv_valid, upper, \
+                        pend, pend_on);                                                                      \
     if (++j >= nsteps) break;
 #pragma unroll 1
     for (uint32_t j = 0;;) {
-        WR_ILD_STEP(0, sa, sb)
-        WR_ILD_STEP(1, sb, sa)
-        WR_ILD_STEP(2, sa, sb)
-        WR_ILD_STEP(0, sb, sa)
-        WR_ILD_STEP(1, sa, sb)
-        WR_ILD_STEP(2, sb, sa)
+        WR_ILD_STEP(0, 0, sa, sb)
+        WR_ILD_STEP(1, 1, sb, sa)
+        WR_ILD_STEP(2, 0, sa, sb)
+        WR_ILD_STEP(0, 1, sb, sa)
+        WR_ILD_STEP(1, 0, sa, sb)
+        WR_ILD_STEP(2, 1, sb, sa)
     }
 #undef WR_ILD_STEP
 
