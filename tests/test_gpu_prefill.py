@@ -181,6 +181,33 @@ def test_prefill_paired_blocks_with_offset_and_window_sampled_rows(nq, nkv, hd, 
     kv.close()
 
 
+@pytest.mark.parametrize("every", [1, 3])
+@pytest.mark.parametrize("nq,nkv,hd,p0", [(16, 8, 256, 0), (8, 4, 256, 70), (32, 8, 128, 0), (4, 2, 64, 0)])
+def test_prefill_with_a_softmax_reference_that_moves_from_tile_to_tile(nq, nkv, hd, p0, every):
+    # scores that climb by 8 (11.5 in log2 units, above the 2^8 the lazy reference
+    # tolerates) every `every` tiles of 32 keys: each row's reference moves again
+    # and again, at every tile or with plain tiles between the moves.  In the
+    # head-dim-256 kernel a move finds the next tile's score chain already
+    # started from the old reference.
+    T = 330
+    rows = p0 + T
+    print("prefill moving reference", nq, nkv, hd, p0, every, flush=True)
+    k32 = synth.normal(5100 + hd, (rows, nkv, hd), std=0.05)
+    v32 = synth.normal(5101 + hd, (rows, nkv, hd))
+    q = synth.normal(5102 + hd, (T, nq, hd), std=0.05)
+    k32[:, :, 0] = (np.arange(rows) // (32 * every) * (8.0 * every))[:, None]
+    q[:, :, 0] = np.sqrt(hd)                             # score = ramp(key) + noise
+    kv = hipattn.KVCache(1, hd, nkv, rows)
+    assert kv.append(0, 0, k32, v32) == hipattn.OK
+    k16, v16 = synth.f32_to_f16_trunc(k32), synth.f32_to_f16_trunc(v32)
+    got = kv.prefill(0, p0, q)
+    want = oracle.causal_prefill(q, k16, v16, p0=p0, threads=8)
+    print("  errors", util.assert_close(got, want), flush=True)
+    again = kv.prefill(0, p0, q)
+    assert np.array_equal(got, again)
+    kv.close()
+
+
 @pytest.mark.parametrize("nq,nkv,hd", [(4, 2, 64), (32, 8, 128), (16, 8, 128), (8, 4, 256)])
 def test_prefill_is_bit_identical_from_launch_to_launch(nq, nkv, hd):
     # The same chunk through caches at different addresses and launch after launch
