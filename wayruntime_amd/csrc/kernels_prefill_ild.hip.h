@@ -253,10 +253,14 @@ __device__ __forceinline__ void ild_step(PrefillRows<kIldHalf>& R, IlCtx<kIldHal
 #pragma unroll
     for (int q4 = 0; q4 < 4; q4++)
         xr[q4] = *reinterpret_cast<const f32x4*>(xr_at + XB * XF + (q4 * 64 + lane) * 4);
-    // the completion of tile j's scores is spread behind the first three links, so
-    // that neither wave of the SIMD leaves the matrix pipe waiting for it
+    // the completion of tile j's scores is spread behind links 1 to 3 (the other
+    // half's partial scores, asked for above, are on their way during links 0 and
+    // 1), so that neither wave of the SIMD leaves the matrix pipe waiting for it
     nxt = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[0], R.qop[0], negm, 0, 0, 0);
     vf[0] = *reinterpret_cast<const half8*>(cx.vop[0] + VS * L::VTILE);
+    __builtin_amdgcn_sched_barrier(0);
+    nxt = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[1], R.qop[1], nxt, 0, 0, 0);
+    vf[1] = *reinterpret_cast<const half8*>(cx.vop[0] + VS * L::VTILE + 2048);
 #pragma unroll
     for (int r = 0; r < 16; r++) cur[r] += xr[r >> 2][r & 3];
     if (pend_on) {
@@ -265,24 +269,24 @@ __device__ __forceinline__ void ild_step(PrefillRows<kIldHalf>& R, IlCtx<kIldHal
         pend_on = 0;
     }
     __builtin_amdgcn_sched_barrier(0);
-    nxt = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[1], R.qop[1], nxt, 0, 0, 0);
-    vf[1] = *reinterpret_cast<const half8*>(cx.vop[0] + VS * L::VTILE + 2048);
+    nxt = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[2], R.qop[2], nxt, 0, 0, 0);
+    vf[2] = *reinterpret_cast<const half8*>(cx.vop[0] + VS * L::VTILE + 2 * 2048);
     float tmax = il_max16(cur);
     if (j < cx.pl_lo || j > cx.pl_hi) {
         il_mask_special<kIldHalf>(R, cx, cur, cx.t0 + j, j, g, tmax);
         tmax = il_max16(cur);
     }
     __builtin_amdgcn_sched_barrier(0);
-    nxt = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[2], R.qop[2], nxt, 0, 0, 0);
-    vf[2] = *reinterpret_cast<const half8*>(cx.vop[0] + VS * L::VTILE + 2 * 2048);
+    nxt = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[3], R.qop[3], nxt, 0, 0, 0);
+    vf[3] = *reinterpret_cast<const half8*>(cx.vop[0] + VS * L::VTILE + 3 * 2048);
     ild_settle(R, cx, negm, cur, tmax, upper, pend, pend_on);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int i = 3; i < NS; i++) {
+    for (int i = 4; i < NS; i++) {
         nxt = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[i], R.qop[i], nxt, 0, 0, 0);
         vf[i] = *reinterpret_cast<const half8*>(cx.vop[i / ND] + VS * L::VTILE + (i % ND) * 2048);
-        pair(i - 3);
-        if (i == NS - 1) pair(5);
+        pair(i - 4);
+        if (i == NS - 1) pair(4);                         // the first half of P is complete before the first product
         __builtin_amdgcn_sched_barrier(0);
     }
     // products; the partial scores of tile j+1 leave behind the first of them, ahead
@@ -293,7 +297,7 @@ __device__ __forceinline__ void ild_step(PrefillRows<kIldHalf>& R, IlCtx<kIldHal
         R.o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[i], __builtin_bit_cast(half8, pop[t]), R.o[dt], 0, 0,
                                                            0);
         kf[i] = *reinterpret_cast<const half8*>(cx.kop[i] + KS * L::KTILE);
-        if (i < 2) pair(6 + i);                           // the second half of P is first used by product 4
+        if (i < 3) pair(5 + i);                           // the second half of P is first used by product 4
         if (i >= 1 && i <= 4) ild_send1(xw + (XB ^ 1) * XF, nxt, lane, i - 1);
         if (i < L::NL) ild_issue_k1<KC>(cx, j + 4, i);
         else if (i < 2 * L::NL) ild_issue_v1<VC>(cx, j + 2, i - L::NL);
@@ -405,17 +409,13 @@ __device__ __forceinline__ void ild_block(const PrefillArgs& a, unsigned char* s
     ild_issue_v<0>(cx, 0);
     ild_issue_k<2>(cx, 2);
     ild_issue_v<1>(cx, 1);
-    // Q^T operand of the half's dimensions, each lane its own row, scaled and
-    // rounded once: contraction slots (g, j) = dims 128 kg + 16 i + 8 g + j
-    {
-        const uint32_t my_row = min(row0 + n, a.T - 1);   // idle rows re-read the last one
-        const float* qrow = a.q + ((size_t)my_row * a.nq + head) * HD + kg * H + g * 8;
+    // The wave's Q: 32 rows x its 128 dimensions, read in whole half rows (512
+    // contiguous bytes per 32 lanes)
+    float4 qx[16];
 #pragma unroll
-        for (int i = 0; i < H / 16; i++) {
-            const half4 lo = q_scaled_f16(*reinterpret_cast<const float4*>(qrow + i * 16), a.qscale);
-            const half4 hi = q_scaled_f16(*reinterpret_cast<const float4*>(qrow + i * 16 + 4), a.qscale);
-            R.qop[i] = half8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        }
+    for (int jj = 0; jj < 16; jj++) {
+        const uint32_t row = min(row0 + 2 * jj + (lane >> 5), a.T - 1);   // idle rows re-read the last one
+        qx[jj] = *reinterpret_cast<const float4*>(a.q + ((size_t)row * a.nq + head) * HD + kg * H + (lane & 31) * 4);
     }
     float* xw = reinterpret_cast<float*>(smem + IldLds::X_OFF + (sub * 2 + kg) * IldLds::X_WAVE);
     const float* xr_at = reinterpret_cast<const float*>(smem + IldLds::X_OFF + (sub * 2 + (kg ^ 1)) * IldLds::X_WAVE);
@@ -426,6 +426,26 @@ __device__ __forceinline__ void ild_block(const PrefillArgs& a, unsigned char* s
 #pragma unroll
     for (int r = 0; r < 16; r++) sa[r] = sb[r] = negm[r] = 0.f;
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    {
+        // Q is scaled, rounded once and turned into the per-lane operand layout
+        // (contraction slots (g, j) of link i = dims 128 kg + 16 i + 8 g + j of the
+        // lane's own row) through the wave's share of the exchange buffers, which
+        // nothing uses before the first step: rows of 256 bytes, the 16-byte chunk
+        // c of row r at slot c ^ (r % 16).  Nobody else reads it: no barrier.
+        unsigned char* qs = smem + IldLds::X_OFF + wave * 8192;
+        static_assert(8 * 8192 <= IldLds::X_BYTES, "the staged Q operands fit the exchange buffers");
+#pragma unroll
+        for (int jj = 0; jj < 16; jj++) {
+            const int r = 2 * jj + (lane >> 5), c = (lane & 31) >> 1;
+            *reinterpret_cast<half4*>(qs + r * 256 + ((c ^ (r & 15)) * 16) + (lane & 1) * 8) =
+                q_scaled_f16(qx[jj], a.qscale);
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int i = 0; i < H / 16; i++)
+            R.qop[i] = *reinterpret_cast<const half8*>(qs + n * 256 + (((2 * i + g) ^ (n & 15)) * 16));
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // read back before the first partial scores land there
+    }
     ild_patch_tail<0>(smem, cx, 0, sub, lane, kv_valid);
     il_barrier();                                         // first tiles visible to all
     // scores of the first tile
