@@ -48,6 +48,12 @@ def _setup(nq, nkv, hd, p0, T, seed, theta=None, extra_rows=0):
     (32, 8, 128, 50, 300, 33),
     (8, 4, 256, 0, 300, 100),
     (16, 8, 256, 40, 700, 0),       # head_dim 256 behind a non-empty cache: blocks of 2 to 24 tiles, odd and even
+    (4, 4, 256, 5, 131, 0),         # head_dim 256, MHA: four 32-row blocks per workgroup
+    (16, 2, 256, 0, 97, 0),         # head_dim 256, group of 8: two head chunks per KV head
+    (16, 4, 256, 33, 260, 70),      # head_dim 256, group of 4, window, chunk that starts inside a tile
+    (8, 4, 256, 0, 1, 0),           # head_dim 256, a single row
+    (8, 4, 256, 63, 2, 0),
+    (8, 4, 256, 0, 33, 0),
 ])
 def test_prefill_matches_serial_stepping_oracle(nq, nkv, hd, p0, T, win):
     print("prefill", nq, nkv, hd, p0, T, win, flush=True)
@@ -100,8 +106,9 @@ def test_prefill_mfma_and_generic_kernels_agree():
     kv.close()
 
 
-def test_prefill_ignores_rows_that_were_never_appended():
-    nq, nkv, hd, T = 16, 8, 128, 70
+@pytest.mark.parametrize("nq,nkv,hd", [(16, 8, 128), (8, 4, 256), (8, 4, 64)])
+def test_prefill_ignores_rows_that_were_never_appended(nq, nkv, hd):
+    T = 70
     kv, q, k16, v16 = _setup(nq, nkv, hd, 0, T, seed=21, extra_rows=58)
     bad = np.full((58, nkv, hd), 0x7E00, dtype=np.uint16)       # NaN patterns above the chunk
     kv.write_f16(0, T, bad, bad)

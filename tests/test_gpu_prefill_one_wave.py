@@ -70,4 +70,4 @@ def test_one_wave_prefill_is_bit_identical_from_launch_to_launch(nq, nkv):
 
 
 def test_one_wave_prefill_ignores_rows_that_were_never_appended():
-    base.test_prefill_ignores_rows_that_were_never_appended()
+    base.test_prefill_ignores_rows_that_were_never_appended(16, 8, 128)
