@@ -64,7 +64,11 @@ def _check(got, x, w16, what):
     (2040, 96, 4112, 0.3),        # LDS-staged GEMM, eight waves, 256 x 128 tiles: partial panels, three input tiles
     (2040, 32, 4112, 0.5),        # ... a single input tile
     (500, 1088, 4112, 0.02),      # ... 34 input tiles, partial panels
-    (2047, 2048, 1024, 0.02),     # the output projection of a 2047-token prompt (Qwen3-0.6B): one 128 x 64 tile per CU
+    (2047, 2048, 1024, 0.02),     # the output projection of a 2047-token prompt (Qwen3-0.6B): one 128 x 64 tile per CU,
+                                  # two sets of waves halving the input range
+    (2047, 3072, 1024, 0.02),     # ... its down projection, 96 input tiles
+    (2000, 2112, 1040, 0.02),     # ... partial panels both ways, 66 input tiles
+    (2000, 2080, 1040, 0.02),     # ... an odd number of input tiles: one set of waves takes the whole range
     (1000, 2048, 1040, 0.02),     # too few LDS tiles for the chip: the register GEMM with a long contraction
 ])
 def test_projection_shapes_vs_oracle(rows, n_in, n_out, std):
@@ -76,7 +80,7 @@ def test_projection_shapes_vs_oracle(rows, n_in, n_out, std):
     w.close()
 
 
-@pytest.mark.parametrize("rows,n_in,n_out", [(2047, 2048, 1024), (1000, 2048, 1040)])
+@pytest.mark.parametrize("rows,n_in,n_out", [(2047, 2048, 1024), (2000, 2112, 1040), (1000, 2048, 1040)])
 def test_repeated_launches_give_the_same_bits(rows, n_in, n_out):
     # no sum in these kernels depends on the order in which waves or workgroups finish
     print("proj repeat", rows, n_in, n_out, flush=True)

@@ -982,27 +982,37 @@ __global__ __launch_bounds__(kProjThreads, 3) void proj_gemm_split_kernel(const 
 // with too few rows to fill the chip with the large one.  <8, 4, 4>: eight
 // waves, 256 outputs x 128 rows, 32 KiB per stage copied three k-steps ahead,
 // one workgroup per CU: a third fewer bytes per MFMA than the four-wave tile.
-template <int GROUPS, int WN, int RING>
+template <int GROUPS, int WN, int RING, int KS = 1>
 constexpr size_t gemm_lds_bytes()
 {
-    return (size_t)RING * (WN * 4 + 2 * GROUPS) * 1024;   // KiB per stage: 4 WN weight tiles, 2 GROUPS fragments
+    return (size_t)KS * RING * (WN * 4 + 2 * GROUPS) * 1024;   // KiB per stage and set of waves: 4 WN weight tiles, 2 GROUPS fragments
 }
 
 // PIPE: the operand reads of the next k-step are issued before this one's MFMAs
 // (two register sets), for launches that leave a SIMD with a single wave and
 // nobody else to cover its LDS latency; needs one more ring stage, because a
 // stage is now read one k-step before it is used.
-template <int GROUPS, int WN, int RING, bool PIPE = false>
-__global__ __launch_bounds__(128 * WN, WN == 2 ? 2 : 1) void proj_gemm_lds_kernel(const ProjArgs a)
+//
+// KS = 2: two such sets of waves in one workgroup, each with its own ring, take
+// one half of the input range each (the host asks for it only when the number of
+// k-steps is even); the upper half's sums pass through LDS at the end and the
+// lower half adds them to its own, always in that order.  For products whose
+// tiles give every CU one workgroup and no more (a SIMD would hold a single wave
+// for a long chain of k-steps): twice the waves per SIMD, half the chain.
+template <int GROUPS, int WN, int RING, bool PIPE = false, int KS = 1>
+__global__ __launch_bounds__(128 * WN * KS, (WN == 2 && KS == 1) ? 2 : 1) void proj_gemm_lds_kernel(const ProjArgs a)
 {
     extern __shared__ __attribute__((aligned(16))) unsigned char gemm_smem[];
     constexpr int NT = 4, WAVES = 2 * WN, CHUNKS = WN * NT + 2 * GROUPS, CPW = CHUNKS / WAVES;
     static_assert(CHUNKS % WAVES == 0, "every wave copies the same number of chunks");
+    static_assert(KS == 1 || KS == 2, "one set of waves, or two that halve the input range");
     constexpr uint32_t STAGE = CHUNKS * 1024;
     const int lane = threadIdx.x & 63;
-    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t wave_wg = (uint32_t)__builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t kh = wave_wg / WAVES, wave = wave_wg % WAVES;      // half of the input range, wave of the set
     const uint32_t wn = wave % WN, wr = wave / WN;
-    const uint32_t ktiles = a.K / 32, ntiles = a.N / 16, ngroups = (a.R + 7) / 8;
+    const uint32_t ktiles_row = a.K / 32, ntiles = a.N / 16, ngroups = (a.R + 7) / 8;
+    const uint32_t ktiles = ktiles_row / KS, kfirst = kh * ktiles;    // this set's k-steps
     const uint32_t klast = ktiles - 1;
     // Workgroup -> tile.  The dispatcher deals consecutive workgroups round-robin
     // to the eight XCDs; XCD x takes the output panels x, x + 8, ..., and runs
@@ -1023,15 +1033,15 @@ __global__ __launch_bounds__(128 * WN, WN == 2 ? 2 : 1) void proj_gemm_lds_kerne
     for (int i = 0; i < CPW; i++) {
         const uint32_t c = wave * CPW + i;
         const unsigned char* p =
-            c < WN * NT ? reinterpret_cast<const unsigned char*>(a.w) + (size_t)min(nt_wg + c, ntiles - 1) * ktiles * 1024
+            c < WN * NT ? reinterpret_cast<const unsigned char*>(a.w) + (size_t)min(nt_wg + c, ntiles - 1) * ktiles_row * 1024
                         : reinterpret_cast<const unsigned char*>(a.xfrag) +
-                              (size_t)min(g_wg + c - WN * NT, ngroups - 1) * ktiles * 1024;
-        src[i] = uniform_ptr(p);
+                              (size_t)min(g_wg + c - WN * NT, ngroups - 1) * ktiles_row * 1024;
+        src[i] = uniform_ptr(p + (size_t)kfirst * 1024);
     }
     const uint32_t lane_off = lane * 16;
     auto issue = [&](uint32_t kt) {                        // a k-step past the end copies the last one again
         const size_t k = (size_t)min(kt, klast) * 1024;
-        const uint32_t to = lds0 + (kt % RING) * STAGE + wave * CPW * 1024;
+        const uint32_t to = lds0 + ((kt % RING) * KS + kh) * STAGE + wave * CPW * 1024;
 #pragma unroll
         for (int i = 0; i < CPW; i++) lds_direct_load(to + i * 1024, src[i] + k, lane_off);
     };
@@ -1050,7 +1060,7 @@ __global__ __launch_bounds__(128 * WN, WN == 2 ? 2 : 1) void proj_gemm_lds_kerne
         static_assert(RING >= 4, "a stage is read while the one before it is multiplied");
         half8 w0[NT], x0[GROUPS], w1[NT], x1[GROUPS];
         auto read_ops = [&](half8 (&wv)[NT], half8 (&xv)[GROUPS], uint32_t kt) {
-            const unsigned char* st = gemm_smem + (kt % RING) * STAGE;
+            const unsigned char* st = gemm_smem + ((kt % RING) * KS + kh) * STAGE;
 #pragma unroll
             for (int t = 0; t < NT; t++) wv[t] = *reinterpret_cast<const half8*>(st + w_off + t * 1024);
 #pragma unroll
@@ -1089,7 +1099,7 @@ __global__ __launch_bounds__(128 * WN, WN == 2 ? 2 : 1) void proj_gemm_lds_kerne
         // this wave's copies of stage kt have landed; those of the RING - 2 stages after it may be in flight
         asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(CPW * (RING - 2)) : "memory");
         issue(kt + RING - 1);
-        const unsigned char* st = gemm_smem + (kt % RING) * STAGE;
+        const unsigned char* st = gemm_smem + ((kt % RING) * KS + kh) * STAGE;
         half8 wv[NT], xv[GROUPS];
 #pragma unroll
         for (int t = 0; t < NT; t++) wv[t] = *reinterpret_cast<const half8*>(st + w_off + t * 1024);
@@ -1108,6 +1118,31 @@ __global__ __launch_bounds__(128 * WN, WN == 2 ? 2 : 1) void proj_gemm_lds_kerne
     }
     // the last steps' copies still target the ring
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+    if constexpr (KS == 2) {
+        // the upper half's sums through LDS (the rings are done with: every wave's
+        // copies have landed and, past the barrier, every wave's reads are over),
+        // added to the lower half's in a fixed order
+        static_assert((size_t)WAVES * NT * GROUPS * 1024 <= (size_t)RING * KS * STAGE, "the partial tiles fit the rings");
+        f32x4* red = reinterpret_cast<f32x4*>(gemm_smem) + (size_t)wave * NT * GROUPS * 64 + lane;
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        if (kh == 1) {
+#pragma unroll
+            for (int t = 0; t < NT; t++)
+#pragma unroll
+                for (int gi = 0; gi < GROUPS; gi++) red[(t * GROUPS + gi) * 64] = acc[t][gi];
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        if (kh == 1) return;
+#pragma unroll
+        for (int t = 0; t < NT; t++)
+#pragma unroll
+            for (int gi = 0; gi < GROUPS; gi++) {
+                const f32x4 o = red[(t * GROUPS + gi) * 64];
+#pragma unroll
+                for (int i = 0; i < 4; i++) acc[t][gi][i] += o[i];
+            }
+    }
 
     const uint32_t nt0 = nt_wg + wn * NT, group0 = g_wg + wr * GROUPS;
     if (nt0 >= ntiles || group0 >= ngroups) return;

@@ -831,6 +831,12 @@ void launch_proj_gemm(const ProjArgs& a, uint32_t groups)
     else if (panels * ((groups + 7) / 8) >= 512)          // two and more per CU cover each other's latency
         launch_main(proj_gemm_lds_kernel<4, 2, 3>, dim3(share * ((groups + 7) / 8)), dim3(kProjThreads), a,
                     gemm_lds_bytes<4, 2, 3>());
+    else if (panels * ((groups + 7) / 8) >= 256 && (a.K / 32) % 2 == 0 && a.K >= 2048)
+        // one per CU and a long input range: two sets of waves halve it (two waves per SIMD, half the
+        // chain of k-steps; 2047 rows x 2048 -> 1024: 40.3 -> 28.3 us, x 3072 -> 1024: 40 -> 36.6; at
+        // 1024 inputs the sum through LDS costs more than the shorter chain gives)
+        launch_main(proj_gemm_lds_kernel<4, 2, 4, true, 2>, dim3(share * ((groups + 7) / 8)), dim3(2 * kProjThreads), a,
+                    gemm_lds_bytes<4, 2, 4, 2>());
     else if (panels * ((groups + 7) / 8) >= 256)          // one per CU, one wave per SIMD: pipelined reads
         launch_main(proj_gemm_lds_kernel<4, 2, 4, true>, dim3(share * ((groups + 7) / 8)), dim3(kProjThreads), a,
                     gemm_lds_bytes<4, 2, 4>());
@@ -1057,6 +1063,9 @@ int wr_hip_attn_init(int device)
         if (e == hipSuccess)
             e = hipFuncSetAttribute(reinterpret_cast<const void*>(proj_gemm_lds_kernel<4, 2, 4, true>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)gemm_lds_bytes<4, 2, 4>());
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute(reinterpret_cast<const void*>(proj_gemm_lds_kernel<4, 2, 4, true, 2>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)gemm_lds_bytes<4, 2, 4, 2>());
         if (e == hipSuccess)
             e = hipFuncSetAttribute(reinterpret_cast<const void*>(proj_gemm_lds_kernel<8, 4, 4>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)gemm_lds_bytes<8, 4, 4>());
