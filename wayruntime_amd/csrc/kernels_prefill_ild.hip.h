@@ -197,28 +197,6 @@ __device__ __forceinline__ void ild_send(float* xw, const f32x16& c, int lane)
     for (int q4 = 0; q4 < 4; q4++) ild_send1(xw, c, lane, q4);
 }
 
-// Completes the scores of a tile from the two halves' partial sums and settles
-// them: sum, what a reference move left pending, row maximum, masks of a tile
-// that is not plain, reference.
-__device__ __forceinline__ void ild_complete(PrefillRows<kIldHalf>& R, IlCtx<kIldHalf>& cx, f32x16& negm, f32x16& c,
-                                             const f32x4 (&xr)[4], uint32_t jt, int g, bool upper, float& pend,
-                                             uint32_t& pend_on)
-{
-#pragma unroll
-    for (int r = 0; r < 16; r++) c[r] += xr[r >> 2][r & 3];
-    if (pend_on) {
-#pragma unroll
-        for (int r = 0; r < 16; r++) asm volatile("v_sub_f32 %0, %0, %1" : "+v"(c[r]) : "v"(pend));
-        pend_on = 0;
-    }
-    float tmax = il_max16(c);
-    if (jt < cx.pl_lo || jt > cx.pl_hi) {
-        il_mask_special<kIldHalf>(R, cx, c, cx.t0 + jt, jt, g, tmax);
-        tmax = il_max16(c);
-    }
-    ild_settle(R, cx, negm, c, tmax, upper, pend, pend_on);
-}
-
 // Step j of a wave (P == j % kRing, XB == j % 2).  On entry `cur` holds the
 // wave's partial scores of tile j and kf the K operands of tile j+1; on exit
 // `nxt` holds the partial scores of tile j+1 (sent to the exchange buffer of the
