@@ -23,7 +23,15 @@ one session; `projection` the row projections either side of the path: 16 rows
 (proj_rows_kernel, HBM-bound on the F16 weight bytes) and a 1024-row prefill
 pass (proj_gemm_lds_kernel, MFMA-bound); `end_to_end` the host engine on a
 random-init Qwen3-0.6B-shaped model (python -m wayruntime_amd.e2e_timing in a
-child process).
+child process): every layer on the device, and (`host_walk_*`) the layers on
+the host with only the cache append and the attention on the device, plus what
+that pair of calls costs per layer as two calls and as one
+(`host_rows_append_then_decode_us`, `host_rows_append_decode_us`).
+`mfma_probe` is what back-to-back MFMAs alone sustain on this device with
+operands of zeros, of ones and of N(0, 1) samples (wayruntime_amd/calib_mfma):
+the clock the device grants depends on the data, and
+`prefill.frac_of_mfma_probe_normal_operands` prices the prefill launch against
+the last of the three beside the published peak.
 """
 from __future__ import annotations
 
