@@ -816,12 +816,14 @@ void launch_proj_gemm(const ProjArgs& a, uint32_t groups)
     const uint32_t share = (panels + 7) / 8 * 8;
     const uint32_t wide = (nt + 15) / 16, wshare = (wide + 7) / 8 * 8;
     // The eight-wave tile runs one workgroup per CU, in rounds of 256: when its
-    // last round would leave more than 15 % of the CUs idle, the four-wave tile
+    // last round would leave more than 10 % of the CUs idle, the four-wave tile
     // (two per CU, half the work each) loses less (2047 rows x 6144 outputs:
-    // 384 eight-wave tiles, 1.5 rounds, 83 us; 768 four-wave tiles 65 us).
+    // 384 eight-wave tiles, 1.5 rounds, 83 us; 768 four-wave tiles 65 us.
+    // 1024 rows x 28672 outputs: 896 eight-wave tiles, 3.5 rounds, 559 us;
+    // 1792 four-wave tiles 530 us).
     const uint32_t n_wide = wide * ((groups + 15) / 16), n_big = panels * ((groups + 15) / 16);
     const uint32_t rounds = (n_wide + 255) / 256;
-    const bool wide_fills = n_wide >= 256 && (n_wide * 100 >= rounds * 256 * 85 || n_big < 512);
+    const bool wide_fills = n_wide >= 256 && (n_wide * 100 >= rounds * 256 * 90 || n_big < 512);
     if (wide_fills)
         launch_main(proj_gemm_lds_kernel<8, 4, 4>, dim3(wshare * ((groups + 15) / 16)), dim3(512), a,
                     gemm_lds_bytes<8, 4, 4>());
