@@ -290,7 +290,10 @@ __device__ __forceinline__ void ild_step(PrefillRows<kIldHalf>& R, IlCtx<kIldHal
     // LDS operations complete in the order issued: with at most the three operand
     // reads issued after the last piece of the partial scores outstanding, those
     // are in the exchange buffer (the operand reads' slot is not refilled before
-    // the next step's products, long after the next chain has consumed them)
+    // the next step's products, long after the next chain has consumed them).
+    // The last piece leaves with product 4, and products 5, 6 and 7 each issue one
+    // operand read behind a scheduling barrier that nothing crosses: three reads
+    // follow it whatever the scheduler does inside a product's group.
     asm volatile("s_waitcnt lgkmcnt(3)\n\ts_barrier" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
 }
