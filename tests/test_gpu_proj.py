@@ -60,6 +60,7 @@ def _check(got, x, w16, what):
     (500, 128, 4112, 0.3),        # ... an even number of them
     (1000, 1056, 4112, 0.02),     # ... the plain 128 x 64 tile (two workgroups per CU), 33 input tiles
     (1000, 96, 8208, 0.3),        # LDS-staged GEMM, 128 x 128 tiles: partial output and row panels, three input tiles
+    (1536, 64, 6144, 0.3),        # ... 576 such tiles would fill 1.1 rounds: the 128 x 64 tile takes over
     (1000, 32, 8208, 0.5),        # ... a single input tile (the ring's prologue covers the whole product)
     (2040, 96, 4112, 0.3),        # LDS-staged GEMM, eight waves, 256 x 128 tiles: partial panels, three input tiles
     (2040, 32, 4112, 0.5),        # ... a single input tile

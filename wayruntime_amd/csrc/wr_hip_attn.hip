@@ -824,10 +824,22 @@ void launch_proj_gemm(const ProjArgs& a, uint32_t groups)
     const uint32_t n_wide = wide * ((groups + 15) / 16), n_big = panels * ((groups + 15) / 16);
     const uint32_t rounds = (n_wide + 255) / 256;
     const bool wide_fills = n_wide >= 256 && (n_wide * 100 >= rounds * 256 * 90 || n_big < 512);
+    // The four-wave tiles run two per CU, in rounds of 512.  The 128 x 128 tile moves
+    // fewer bytes per MFMA than the 128 x 64 one (2048 rows x 4096 -> 6144: 226 against
+    // 243 us) but has half as many workgroups to fill its last round with: where that
+    // round would be thin (under 70 % full) and the smaller tile's is fuller by a tenth
+    // or more, the smaller tile wins (1536 rows x 1024 -> 6144: 576 tiles, 1.1 rounds,
+    // 59.8 us; 1152 smaller ones 49 us.  At three quarters full the larger tile still
+    // holds its own: 2047 rows x 1024 -> 6144 65.6 against 64.8 us, 2048 x 4096 -> 6144
+    // 226 against 243).
+    const uint32_t n_small = panels * ((groups + 7) / 8);
+    const uint32_t rounds_b = (n_big + 511) / 512, rounds_s = (n_small + 511) / 512;
+    const bool small_fills_better = n_small >= 512 && n_big * 100 < rounds_b * 512 * 70 &&
+                                    (uint64_t)n_small * rounds_b * 100 >= (uint64_t)n_big * rounds_s * 100 + (uint64_t)rounds_b * rounds_s * 512 * 10;
     if (wide_fills)
         launch_main(proj_gemm_lds_kernel<8, 4, 4>, dim3(wshare * ((groups + 15) / 16)), dim3(512), a,
                     gemm_lds_bytes<8, 4, 4>());
-    else if (n_big >= 512)
+    else if (n_big >= 512 && !small_fills_better)
         launch_main(proj_gemm_lds_kernel<8, 2, 3>, dim3(share * ((groups + 15) / 16)), dim3(kProjThreads), a,
                     gemm_lds_bytes<8, 2, 3>());
     else if (panels * ((groups + 7) / 8) >= 512)          // two and more per CU cover each other's latency
