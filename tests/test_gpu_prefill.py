@@ -67,6 +67,33 @@ def test_prefill_matches_serial_stepping_oracle(nq, nkv, hd, p0, T, win):
     kv.close()
 
 
+def _drawn_shapes(n, seed):
+    """n (nq, nkv, hd, p0, T, win) tuples drawn from a fixed seed: matrix-core head dims and
+    group sizes, chunks that start and end anywhere in a tile, windows shorter and longer
+    than the chunk."""
+    r = synth.splitmix64(seed, 6 * n).reshape(n, 6)
+    out = []
+    for a in r:
+        hd = (64, 128, 256, 256)[int(a[0] % 4)]
+        group = (1, 2, 4, 8)[int(a[1] % 4)]
+        nkv = (1, 2, 4)[int(a[2] % 3)]
+        p0 = int(a[3] % 150)
+        T = 1 + int(a[4] % 260)
+        win = (0, 0, 1 + int(a[5] % 40), 40 + int(a[5] % 300))[int((a[5] >> 20) % 4)]
+        out.append((group * nkv, nkv, hd, p0, T, win))
+    return out
+
+
+@pytest.mark.parametrize("nq,nkv,hd,p0,T,win", _drawn_shapes(16, 20260))
+def test_prefill_drawn_shapes_against_the_oracle(nq, nkv, hd, p0, T, win):
+    print("prefill drawn", nq, nkv, hd, p0, T, win, flush=True)
+    kv, q, k16, v16 = _setup(nq, nkv, hd, p0, T, seed=3000 + 7 * T + p0)
+    got = kv.prefill(0, p0, q, 0.0, win)
+    want = oracle.causal_prefill(q, k16, v16, p0=p0, window=win, threads=8)
+    util.assert_close(got, want)
+    kv.close()
+
+
 @pytest.mark.parametrize("nq,nkv,hd,p0,T,win", [
     (4, 2, 32, 3, 70, 0),           # head_dim 32: generic kernel
     (6, 2, 64, 0, 40, 0),           # group of 3
